@@ -1,0 +1,257 @@
+// FlashAttention forward entry points: argument checks, kernel choice, launches.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdlib>
+
+#include "ahpc_device.hpp"
+#include "flash_fwd_mfma.hpp"
+
+namespace ahpc {
+
+// ---------------------------------------------------------------------------------------------
+// fp32-FMA kernel: any dtype, any head dimension up to 256, optional dense mask.  One thread owns
+// one query row (q and the output accumulator stay in registers); a workgroup of 128 rows of the
+// same (sequence, head) shares key/value tiles of 16 rows staged in LDS as fp32.  This is the
+// accuracy path (fp32 inputs, 1e-4 tolerance) and the fallback for shapes the MFMA kernel does
+// not take; it is not tuned.
+struct SimpleParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* o;
+    const int32_t* cu_seqlens;
+    const float* mask;          // [B,N,N] or null
+    int64_t stride_b, stride_n, stride_h;
+    int32_t N, H, d;
+    float scale;
+    int32_t causal;
+};
+
+constexpr int kSimpleRows = 128;
+constexpr int kSimpleKeys = 16;
+
+template <typename T, int DP, bool VARLEN>
+__global__ __launch_bounds__(kSimpleRows) void flash_fwd_simple_kernel(const SimpleParams p) {
+    __shared__ float sk[kSimpleKeys][DP];
+    __shared__ float sv[kSimpleKeys][DP];
+
+    const int tid = threadIdx.x;
+    const int h = blockIdx.y, b = blockIdx.z;
+    int L;
+    int64_t base;
+    if (VARLEN) {
+        const int s0 = p.cu_seqlens[b];
+        L = p.cu_seqlens[b + 1] - s0;
+        base = (int64_t)s0 * p.stride_n + (int64_t)h * p.stride_h;
+    } else {
+        L = p.N;
+        base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+    }
+    const int row0 = blockIdx.x * kSimpleRows;
+    if (row0 >= L) return;
+    const int n = row0 + tid;
+    const bool active = n < L;
+    const int d = p.d;
+
+    const T* gq = static_cast<const T*>(p.q) + base;
+    const T* gk = static_cast<const T*>(p.k) + base;
+    const T* gv = static_cast<const T*>(p.v) + base;
+
+    float qv[DP], acc[DP];
+#pragma unroll
+    for (int e = 0; e < DP; ++e) {
+        qv[e] = (active && e < d) ? Storage<T>::load(gq + (int64_t)n * p.stride_n + e) : 0.0f;
+        acc[e] = 0.0f;
+    }
+    float m = -INFINITY, l = 0.0f;
+
+    for (int i = tid; i < kSimpleKeys * DP; i += kSimpleRows) {
+        (&sk[0][0])[i] = 0.0f;
+        (&sv[0][0])[i] = 0.0f;
+    }
+
+    int k_end = L;
+    if (p.causal) k_end = (row0 + kSimpleRows) < L ? (row0 + kSimpleRows) : L;
+    const float* mrow = (p.mask && active) ? p.mask + ((int64_t)b * p.N + n) * p.N : nullptr;
+
+    for (int k0 = 0; k0 < k_end; k0 += kSimpleKeys) {
+        __syncthreads();
+        for (int i = tid; i < kSimpleKeys * d; i += kSimpleRows) {
+            const int kr = i / d, e = i - kr * d;
+            const int key = k0 + kr;
+            float kx = 0.0f, vx = 0.0f;
+            if (key < L) {
+                kx = Storage<T>::load(gk + (int64_t)key * p.stride_n + e);
+                vx = Storage<T>::load(gv + (int64_t)key * p.stride_n + e);
+            }
+            sk[kr][e] = kx;
+            sv[kr][e] = vx;
+        }
+        __syncthreads();
+        if (!active) continue;
+        for (int kr = 0; kr < kSimpleKeys; ++kr) {
+            const int key = k0 + kr;
+            if (key >= L) break;
+            if (p.causal && key > n) break;
+            if (mrow && mrow[key] == 0.0f) continue;
+            float dot = 0.0f;
+#pragma unroll
+            for (int e = 0; e < DP; ++e) dot = __builtin_fmaf(qv[e], sk[kr][e], dot);
+            const float s = dot * p.scale;
+            if (s > m) {
+                const float a = __expf(m - s);  // first key: exp(-inf) = 0
+                l = l * a + 1.0f;
+#pragma unroll
+                for (int e = 0; e < DP; ++e) acc[e] = __builtin_fmaf(acc[e], a, sv[kr][e]);
+                m = s;
+            } else {
+                const float w = __expf(s - m);
+                l += w;
+#pragma unroll
+                for (int e = 0; e < DP; ++e) acc[e] = __builtin_fmaf(w, sv[kr][e], acc[e]);
+            }
+        }
+    }
+    if (!active) return;
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    T* go = static_cast<T*>(p.o) + base + (int64_t)n * p.stride_n;
+#pragma unroll
+    for (int e = 0; e < DP; ++e)
+        if (e < d) Storage<T>::store(go + e, acc[e] * inv);
+}
+
+template <typename T, bool VARLEN>
+static int launch_simple(const SimpleParams& p, int64_t B, hipStream_t stream) {
+    dim3 grid((unsigned)((p.N + kSimpleRows - 1) / kSimpleRows), (unsigned)p.H, (unsigned)B);
+    dim3 block(kSimpleRows);
+    if (p.d <= 16) hipLaunchKernelGGL((flash_fwd_simple_kernel<T, 16, VARLEN>), grid, block, 0, stream, p);
+    else if (p.d <= 32) hipLaunchKernelGGL((flash_fwd_simple_kernel<T, 32, VARLEN>), grid, block, 0, stream, p);
+    else if (p.d <= 64) hipLaunchKernelGGL((flash_fwd_simple_kernel<T, 64, VARLEN>), grid, block, 0, stream, p);
+    else if (p.d <= 128) hipLaunchKernelGGL((flash_fwd_simple_kernel<T, 128, VARLEN>), grid, block, 0, stream, p);
+    else if (p.d <= 256) hipLaunchKernelGGL((flash_fwd_simple_kernel<T, 256, VARLEN>), grid, block, 0, stream, p);
+    else return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+    return static_cast<int>(hipGetLastError());
+}
+
+template <bool VARLEN>
+static int dispatch_simple(int dtype, const SimpleParams& p, int64_t B, hipStream_t stream) {
+    switch (dtype) {
+        case AHPC_F32: return launch_simple<float, VARLEN>(p, B, stream);
+        case AHPC_F16: return launch_simple<f16_t, VARLEN>(p, B, stream);
+        case AHPC_BF16: return launch_simple<bf16_t, VARLEN>(p, B, stream);
+        default: return AHPC_ERR_BAD_DTYPE;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Queries per wavefront of the MFMA kernel, in blocks of 32.  Read once from AHPC_FLASH_QB
+// (1 or 2) so that both tilings can be timed; 0 / unset picks the default.
+static int flash_qb_override() {
+    static const int v = [] {
+        const char* e = std::getenv("AHPC_FLASH_QB");
+        return e ? std::atoi(e) : 0;
+    }();
+    return v;
+}
+
+template <typename T, int D, int QB, bool VARLEN>
+static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
+    constexpr int BM = 128 * QB;
+    p.n_qtiles = (p.N + BM - 1) / BM;
+    const int64_t total = B * p.H * (int64_t)p.n_qtiles;
+    if (total > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
+    p.total_blocks = (int32_t)total;
+    p.blocks_per_xcd = (int32_t)((total + 7) / 8);
+    dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
+    if (causal) hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, QB, true, VARLEN>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, QB, false, VARLEN>), grid, block, 0, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
+template <typename T, bool VARLEN>
+static int dispatch_mfma(const FlashParams& p, int64_t B, int d, bool causal, hipStream_t stream) {
+    int qb = flash_qb_override();
+    if (qb != 1 && qb != 2) qb = 1;
+    if (d == 128) return qb == 2 ? launch_mfma<T, 128, 2, VARLEN>(p, B, causal, stream) : launch_mfma<T, 128, 1, VARLEN>(p, B, causal, stream);
+    if (d == 64) return qb == 2 ? launch_mfma<T, 64, 2, VARLEN>(p, B, causal, stream) : launch_mfma<T, 64, 1, VARLEN>(p, B, causal, stream);
+    return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+}
+
+static bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+static bool mfma_eligible(int dtype, int64_t d, const void* q, const void* k, const void* v, const void* o,
+                          int64_t s0, int64_t s1, int64_t s2) {
+    if (dtype != AHPC_F16 && dtype != AHPC_BF16) return false;
+    if (d != 64 && d != 128) return false;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return false;
+    return (s0 % 8 == 0) && (s1 % 8 == 0) && (s2 % 8 == 0);
+}
+
+static int check_dense(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N, int64_t H,
+                       int64_t d, int64_t sb, int64_t sn, int64_t sh) {
+    if (!q || !k || !v || !o) return AHPC_ERR_NULL_POINTER;
+    if (dtype < AHPC_F32 || dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
+    if (B <= 0 || N <= 0 || H <= 0 || d <= 0) return AHPC_ERR_BAD_SHAPE;
+    if (B > 65535 || H > 65535 || N > 0x7FFFFF00ll) return AHPC_ERR_BAD_SHAPE;
+    if (d > 256) return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+    if (sn < d || sh < d || sb < 0) return AHPC_ERR_BAD_SHAPE;
+    return AHPC_OK;
+}
+
+}  // namespace ahpc
+
+using namespace ahpc;
+
+extern "C" {
+
+int ahpc_hip_flash_fwd_masked(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N,
+                              int64_t H, int64_t d, int64_t stride_b, int64_t stride_n, int64_t stride_h, float scale,
+                              int causal, const float* mask, void* stream) {
+    if (int rc = check_dense(q, k, v, o, dtype, B, N, H, d, stride_b, stride_n, stride_h)) return rc;
+    if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
+    SimpleParams p{q, k, v, o, nullptr, mask, stride_b, stride_n, stride_h, (int32_t)N, (int32_t)H, (int32_t)d, scale, causal ? 1 : 0};
+    return dispatch_simple<false>(dtype, p, B, static_cast<hipStream_t>(stream));
+}
+
+int ahpc_hip_flash_fwd(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N, int64_t H,
+                       int64_t d, int64_t stride_b, int64_t stride_n, int64_t stride_h, float scale, int causal,
+                       void* stream) {
+    if (int rc = check_dense(q, k, v, o, dtype, B, N, H, d, stride_b, stride_n, stride_h)) return rc;
+    if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (mfma_eligible(dtype, d, q, k, v, o, stride_b, stride_n, stride_h)) {
+        FlashParams p{};
+        p.q = q; p.k = k; p.v = v; p.o = o;
+        p.stride_b = stride_b; p.stride_n = stride_n; p.stride_h = stride_h;
+        p.N = (int32_t)N; p.H = (int32_t)H;
+        p.scale_log2 = scale * kLog2e;
+        return dtype == AHPC_F16 ? dispatch_mfma<f16_t, false>(p, B, (int)d, causal != 0, st)
+                                 : dispatch_mfma<bf16_t, false>(p, B, (int)d, causal != 0, st);
+    }
+    SimpleParams p{q, k, v, o, nullptr, nullptr, stride_b, stride_n, stride_h, (int32_t)N, (int32_t)H, (int32_t)d, scale, causal ? 1 : 0};
+    return dispatch_simple<false>(dtype, p, B, st);
+}
+
+int ahpc_hip_flash_fwd_varlen(const void* q, const void* k, const void* v, void* o, int dtype, const int32_t* cu_seqlens,
+                              int64_t n_seqs, int64_t max_len, int64_t H, int64_t d, int64_t stride_t, int64_t stride_h,
+                              float scale, int causal, void* stream) {
+    if (!cu_seqlens) return AHPC_ERR_NULL_POINTER;
+    if (int rc = check_dense(q, k, v, o, dtype, n_seqs, max_len, H, d, 0, stride_t, stride_h)) return rc;
+    if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (mfma_eligible(dtype, d, q, k, v, o, 0, stride_t, stride_h)) {
+        FlashParams p{};
+        p.q = q; p.k = k; p.v = v; p.o = o;
+        p.cu_seqlens = cu_seqlens;
+        p.stride_b = 0; p.stride_n = stride_t; p.stride_h = stride_h;
+        p.N = (int32_t)max_len; p.H = (int32_t)H;
+        p.scale_log2 = scale * kLog2e;
+        return dtype == AHPC_F16 ? dispatch_mfma<f16_t, true>(p, n_seqs, (int)d, causal != 0, st)
+                                 : dispatch_mfma<bf16_t, true>(p, n_seqs, (int)d, causal != 0, st);
+    }
+    SimpleParams p{q, k, v, o, cu_seqlens, nullptr, 0, stride_t, stride_h, (int32_t)max_len, (int32_t)H, (int32_t)d, scale, causal ? 1 : 0};
+    return dispatch_simple<true>(dtype, p, n_seqs, st);
+}
+
+}  // extern "C"

@@ -1,0 +1,159 @@
+// Device, memory, stream and event entry points of the C ABI, and the error strings.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "ahpc_hip.h"
+
+extern "C" {
+
+const char* ahpc_hip_error_string(int code) {
+    switch (code) {
+        case AHPC_OK: return "success";
+        case AHPC_ERR_NULL_POINTER: return "null pointer argument";
+        case AHPC_ERR_BAD_SHAPE: return "invalid shape, stride or size argument";
+        case AHPC_ERR_BAD_DTYPE: return "unknown data type code";
+        case AHPC_ERR_UNSUPPORTED_HEAD_DIM: return "head dimension not supported by this kernel";
+        case AHPC_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";
+        case AHPC_ERR_NO_DEVICE: return "no HIP device available";
+        case AHPC_ERR_BAD_ALIGNMENT: return "pointer or stride not aligned for 16-byte access";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+    return "unknown error code";
+}
+
+int ahpc_hip_device_count(int* count) {
+    if (!count) return AHPC_ERR_NULL_POINTER;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        n = 0;
+    }
+    *count = n;
+    return AHPC_OK;
+}
+
+int ahpc_hip_device_info(int device, ahpc_device_info* out) {
+    if (!out) return AHPC_ERR_NULL_POINTER;
+    int n = 0;
+    ahpc_hip_device_count(&n);
+    if (device < 0 || device >= n) return AHPC_ERR_NO_DEVICE;
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) return static_cast<int>(e);
+    std::memset(out, 0, sizeof(*out));
+    std::strncpy(out->name, prop.name, sizeof(out->name) - 1);
+    std::strncpy(out->arch, prop.gcnArchName, sizeof(out->arch) - 1);
+    if (char* colon = std::strchr(out->arch, ':')) *colon = '\0';
+    out->total_memory_bytes = prop.totalGlobalMem;
+    size_t free_b = 0, total_b = 0;
+    int current = 0;
+    if (hipGetDevice(&current) == hipSuccess && current == device && hipMemGetInfo(&free_b, &total_b) == hipSuccess)
+        out->free_memory_bytes = free_b;
+    out->compute_units = prop.multiProcessorCount;
+    out->wavefront_size = prop.warpSize;
+    out->lds_bytes_per_workgroup = static_cast<int32_t>(prop.sharedMemPerBlock);
+    out->max_threads_per_workgroup = prop.maxThreadsPerBlock;
+    out->clock_khz = prop.clockRate;
+    int rt = 0;
+    if (hipRuntimeGetVersion(&rt) == hipSuccess) out->runtime_version = rt;
+    return AHPC_OK;
+}
+
+int ahpc_hip_malloc(void** ptr, size_t bytes) {
+    if (!ptr) return AHPC_ERR_NULL_POINTER;
+    return static_cast<int>(hipMalloc(ptr, bytes ? bytes : 1));
+}
+
+int ahpc_hip_free(void* ptr) { return ptr ? static_cast<int>(hipFree(ptr)) : AHPC_OK; }
+
+int ahpc_hip_host_malloc(void** ptr, size_t bytes) {
+    if (!ptr) return AHPC_ERR_NULL_POINTER;
+    return static_cast<int>(hipHostMalloc(ptr, bytes ? bytes : 1, hipHostMallocDefault));
+}
+
+int ahpc_hip_host_free(void* ptr) { return ptr ? static_cast<int>(hipHostFree(ptr)) : AHPC_OK; }
+
+int ahpc_hip_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream) {
+    if (!bytes) return AHPC_OK;
+    if (!dst || !src) return AHPC_ERR_NULL_POINTER;
+    return static_cast<int>(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
+}
+
+int ahpc_hip_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream) {
+    if (!bytes) return AHPC_OK;
+    if (!dst || !src) return AHPC_ERR_NULL_POINTER;
+    return static_cast<int>(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
+}
+
+int ahpc_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream) {
+    if (!bytes) return AHPC_OK;
+    if (!dst || !src) return AHPC_ERR_NULL_POINTER;
+    return static_cast<int>(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
+}
+
+int ahpc_hip_memset(void* dst, int byte_value, size_t bytes, void* stream) {
+    if (!bytes) return AHPC_OK;
+    if (!dst) return AHPC_ERR_NULL_POINTER;
+    return static_cast<int>(hipMemsetAsync(dst, byte_value, bytes, static_cast<hipStream_t>(stream)));
+}
+
+int ahpc_hip_ptr_is_device(const void* ptr, int* is_device) {
+    if (!is_device) return AHPC_ERR_NULL_POINTER;
+    *is_device = 0;
+    if (!ptr) return AHPC_OK;
+    hipPointerAttribute_t attr;
+    hipError_t e = hipPointerGetAttributes(&attr, ptr);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();  // ordinary host memory is reported as an error: not one for us
+        return AHPC_OK;
+    }
+    *is_device = (attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged) ? 1 : 0;
+    return AHPC_OK;
+}
+
+int ahpc_hip_stream_create(void** stream) {
+    if (!stream) return AHPC_ERR_NULL_POINTER;
+    hipStream_t s = nullptr;
+    hipError_t e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);
+    *stream = s;
+    return static_cast<int>(e);
+}
+
+int ahpc_hip_stream_destroy(void* stream) {
+    return stream ? static_cast<int>(hipStreamDestroy(static_cast<hipStream_t>(stream))) : AHPC_OK;
+}
+
+int ahpc_hip_stream_synchronize(void* stream) {
+    return static_cast<int>(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+}
+
+int ahpc_hip_event_create(void** event) {
+    if (!event) return AHPC_ERR_NULL_POINTER;
+    hipEvent_t ev = nullptr;
+    hipError_t e = hipEventCreate(&ev);
+    *event = ev;
+    return static_cast<int>(e);
+}
+
+int ahpc_hip_event_destroy(void* event) {
+    return event ? static_cast<int>(hipEventDestroy(static_cast<hipEvent_t>(event))) : AHPC_OK;
+}
+
+int ahpc_hip_event_record(void* event, void* stream) {
+    if (!event) return AHPC_ERR_NULL_POINTER;
+    return static_cast<int>(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
+}
+
+int ahpc_hip_event_synchronize(void* event) {
+    if (!event) return AHPC_ERR_NULL_POINTER;
+    return static_cast<int>(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+}
+
+int ahpc_hip_event_elapsed_ms(void* start, void* stop, float* ms) {
+    if (!start || !stop || !ms) return AHPC_ERR_NULL_POINTER;
+    return static_cast<int>(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+}
+
+}  // extern "C"

@@ -1,0 +1,148 @@
+"""ctypes view of the C ABI in include/ahpc_hip.h (lib/libahpc_hip.so).
+
+Pointers are plain integers (e.g. torch.Tensor.data_ptr()); nothing here allocates or copies
+unless the function name says so.  A non-zero status raises HipError.
+"""
+import ctypes as C
+import os
+
+F32, F16, BF16 = 0, 1, 2
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libahpc_hip.so")
+
+
+class HipError(RuntimeError):
+    def __init__(self, code, what):
+        super().__init__(f"{what}: status {code}: {error_string(code)}")
+        self.code = code
+
+
+class DeviceInfo(C.Structure):
+    _fields_ = [
+        ("name", C.c_char * 128),
+        ("arch", C.c_char * 32),
+        ("total_memory_bytes", C.c_uint64),
+        ("free_memory_bytes", C.c_uint64),
+        ("compute_units", C.c_int32),
+        ("wavefront_size", C.c_int32),
+        ("lds_bytes_per_workgroup", C.c_int32),
+        ("max_threads_per_workgroup", C.c_int32),
+        ("clock_khz", C.c_int32),
+        ("runtime_version", C.c_int32),
+    ]
+
+
+_vp, _i64, _f32, _ci, _sz = C.c_void_p, C.c_int64, C.c_float, C.c_int, C.c_size_t
+
+# name -> (restype, argtypes); every symbol the header declares
+SIGNATURES = {
+    "ahpc_hip_error_string": (C.c_char_p, [_ci]),
+    "ahpc_hip_device_count": (_ci, [C.POINTER(_ci)]),
+    "ahpc_hip_device_info": (_ci, [_ci, C.POINTER(DeviceInfo)]),
+    "ahpc_hip_malloc": (_ci, [C.POINTER(_vp), _sz]),
+    "ahpc_hip_free": (_ci, [_vp]),
+    "ahpc_hip_host_malloc": (_ci, [C.POINTER(_vp), _sz]),
+    "ahpc_hip_host_free": (_ci, [_vp]),
+    "ahpc_hip_memcpy_h2d": (_ci, [_vp, _vp, _sz, _vp]),
+    "ahpc_hip_memcpy_d2h": (_ci, [_vp, _vp, _sz, _vp]),
+    "ahpc_hip_memcpy_d2d": (_ci, [_vp, _vp, _sz, _vp]),
+    "ahpc_hip_memset": (_ci, [_vp, _ci, _sz, _vp]),
+    "ahpc_hip_ptr_is_device": (_ci, [_vp, C.POINTER(_ci)]),
+    "ahpc_hip_stream_create": (_ci, [C.POINTER(_vp)]),
+    "ahpc_hip_stream_destroy": (_ci, [_vp]),
+    "ahpc_hip_stream_synchronize": (_ci, [_vp]),
+    "ahpc_hip_event_create": (_ci, [C.POINTER(_vp)]),
+    "ahpc_hip_event_destroy": (_ci, [_vp]),
+    "ahpc_hip_event_record": (_ci, [_vp, _vp]),
+    "ahpc_hip_event_synchronize": (_ci, [_vp]),
+    "ahpc_hip_event_elapsed_ms": (_ci, [_vp, _vp, C.POINTER(_f32)]),
+    "ahpc_hip_flash_fwd": (_ci, [_vp, _vp, _vp, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp]),
+    "ahpc_hip_flash_fwd_masked": (_ci, [_vp, _vp, _vp, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp, _vp]),
+    "ahpc_hip_flash_fwd_varlen": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp]),
+    "ahpc_hip_kv_scatter": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
+    "ahpc_hip_kv_gather": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
+    "ahpc_hip_paged_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64]),
+    "ahpc_hip_paged_decode": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp, _sz, _vp]),
+    "ahpc_hip_paged_gather_indices": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp]),
+}
+
+_lib = None
+
+
+def load():
+    """Load lib/libahpc_hip.so (once).  Raises if it has not been built: there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(f"{LIB_PATH} is missing: build it with `make -C attention_amd/csrc` "
+                              "(or __graft_entry__.build()); this package has no CPU fallback")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def error_string(code):
+    return load().ahpc_hip_error_string(int(code)).decode()
+
+
+def _check(code, what):
+    if code != 0:
+        raise HipError(code, what)
+
+
+def device_count():
+    n = _ci(0)
+    _check(load().ahpc_hip_device_count(C.byref(n)), "device_count")
+    return n.value
+
+
+def device_info(device=0):
+    info = DeviceInfo()
+    _check(load().ahpc_hip_device_info(device, C.byref(info)), "device_info")
+    return info
+
+
+def flash_fwd(q, k, v, o, dtype, B, N, H, d, strides, scale, causal, stream=None, mask=None):
+    sb, sn, sh = strides
+    if mask is None:
+        rc = load().ahpc_hip_flash_fwd(q, k, v, o, dtype, B, N, H, d, sb, sn, sh, scale, int(causal), stream)
+    else:
+        rc = load().ahpc_hip_flash_fwd_masked(q, k, v, o, dtype, B, N, H, d, sb, sn, sh, scale, int(causal), mask, stream)
+    _check(rc, "flash_fwd")
+
+
+def flash_fwd_varlen(q, k, v, o, dtype, cu_seqlens, n_seqs, max_len, H, d, stride_t, stride_h, scale, causal, stream=None):
+    _check(load().ahpc_hip_flash_fwd_varlen(q, k, v, o, dtype, cu_seqlens, n_seqs, max_len, H, d, stride_t, stride_h,
+                                           scale, int(causal), stream), "flash_fwd_varlen")
+
+
+def kv_scatter(k_new, v_new, in_dtype, k_pool, v_pool, pool_dtype, table, max_pages, n_tokens, H, d, P,
+               token_row=None, token_pos=None, row0=0, pos0=0, stream=None):
+    _check(load().ahpc_hip_kv_scatter(k_new, v_new, in_dtype, k_pool, v_pool, pool_dtype, table, max_pages, token_row,
+                                     token_pos, row0, pos0, n_tokens, H, d, P, stream), "kv_scatter")
+
+
+def kv_gather(k_out, v_out, out_dtype, k_pool, v_pool, pool_dtype, table, max_pages, row, start, n, H, d, P, stream=None):
+    _check(load().ahpc_hip_kv_gather(k_out, v_out, out_dtype, k_pool, v_pool, pool_dtype, table, max_pages, row, start,
+                                    n, H, d, P, stream), "kv_gather")
+
+
+def paged_decode_workspace_bytes(B, H, d, max_len, P, chunk_tokens=0):
+    return load().ahpc_hip_paged_decode_workspace_bytes(B, H, d, max_len, P, chunk_tokens)
+
+
+def paged_decode(q, o, qo_dtype, k_pool, v_pool, pool_dtype, table, seq_lens, batch_rows, B, H, d, P, max_pages, max_len,
+                 scale, chunk_tokens=0, workspace=None, workspace_bytes=0, stream=None):
+    _check(load().ahpc_hip_paged_decode(q, o, qo_dtype, k_pool, v_pool, pool_dtype, table, seq_lens, batch_rows, B, H, d,
+                                       P, max_pages, max_len, scale, chunk_tokens, workspace, workspace_bytes, stream),
+           "paged_decode")
+
+
+def paged_gather_indices(table, seq_lens, batch_rows, B, H, d, P, max_pages, max_len, offsets, stream=None):
+    _check(load().ahpc_hip_paged_gather_indices(table, seq_lens, batch_rows, B, H, d, P, max_pages, max_len, offsets,
+                                               stream), "paged_gather_indices")

@@ -1,0 +1,196 @@
+/*
+ * ahpc_hip.h - C ABI of the gfx950 (MI355X) attention kernels.
+ *
+ * This is the only door between host code and the GPU: plain pointers and sizes, no C++
+ * types, no exceptions.  The C++ classes in include/attention_hpc/ (HipFlashAttention,
+ * HipPagedAttention) call these functions and turn a non-zero return into
+ * AttentionException(COMPUTATION_FAILED), the way the reference's CUDA_CHECK does
+ * (src/backends/cuda/cuda_flash_attention.hpp:16-22).  The reference's precedent for such a
+ * layer is its `extern "C" launch_*` block, src/backends/cuda/cuda_flash_attention.hpp:41-68;
+ * each entry point below cites what it stands in for.  Paths are relative to the reference
+ * checkout.
+ *
+ * Conventions
+ *   - every function returns 0 on success, otherwise an ahpc_status (negative: rejected
+ *     arguments, nothing launched) or a positive hipError_t value;
+ *     ahpc_hip_error_string() explains either.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Launches are
+ *     asynchronous on that stream; nothing here synchronises unless it says so.
+ *   - all tensor pointers are DEVICE pointers unless a parameter says "host".
+ *   - dtype codes equal the reference's DataType enumerators
+ *     (src/api/attention_interface.hpp:16-20): 0 fp32, 1 fp16, 2 bf16.  16-bit values are
+ *     produced with round-to-nearest-even.
+ *   - strides are in elements.
+ */
+#ifndef AHPC_HIP_H
+#define AHPC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { AHPC_F32 = 0, AHPC_F16 = 1, AHPC_BF16 = 2 };
+
+typedef enum ahpc_status {
+    AHPC_OK = 0,
+    AHPC_ERR_NULL_POINTER = -1,
+    AHPC_ERR_BAD_SHAPE = -2,       /* zero / negative / overflowing dimension, stride too small */
+    AHPC_ERR_BAD_DTYPE = -3,
+    AHPC_ERR_UNSUPPORTED_HEAD_DIM = -4,
+    AHPC_ERR_WORKSPACE_TOO_SMALL = -5,
+    AHPC_ERR_NO_DEVICE = -6,
+    AHPC_ERR_BAD_ALIGNMENT = -7    /* pointers/strides must allow 16-byte vector access */
+} ahpc_status;
+
+const char* ahpc_hip_error_string(int code);
+
+/* ---- device, memory, streams, events ------------------------------------------------------
+ * Stand in for CudaMemoryManager / CudaStreamManager,
+ * src/backends/cuda/cuda_flash_attention.hpp:71-122, and for the capability probe
+ * BackendFactory::detectBackendCapabilities, src/api/backend_factory.cpp (BackendCapability,
+ * src/api/backend_factory.hpp:24-37). */
+typedef struct ahpc_device_info {
+    char     name[128];
+    char     arch[32];               /* e.g. "gfx950" */
+    uint64_t total_memory_bytes;
+    uint64_t free_memory_bytes;
+    int32_t  compute_units;
+    int32_t  wavefront_size;
+    int32_t  lds_bytes_per_workgroup;
+    int32_t  max_threads_per_workgroup;
+    int32_t  clock_khz;
+    int32_t  runtime_version;
+} ahpc_device_info;
+
+int ahpc_hip_device_count(int* count);                       /* never fails: count = 0 without a GPU */
+int ahpc_hip_device_info(int device, ahpc_device_info* out);
+int ahpc_hip_malloc(void** ptr, size_t bytes);
+int ahpc_hip_free(void* ptr);
+int ahpc_hip_host_malloc(void** ptr, size_t bytes);           /* pinned host staging memory */
+int ahpc_hip_host_free(void* ptr);
+int ahpc_hip_memcpy_h2d(void* dst, const void* src_host, size_t bytes, void* stream);
+int ahpc_hip_memcpy_d2h(void* dst_host, const void* src, size_t bytes, void* stream);
+int ahpc_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream);
+int ahpc_hip_memset(void* dst, int byte_value, size_t bytes, void* stream);
+int ahpc_hip_ptr_is_device(const void* ptr, int* is_device);  /* 0 for ordinary host memory */
+int ahpc_hip_stream_create(void** stream);
+int ahpc_hip_stream_destroy(void* stream);
+int ahpc_hip_stream_synchronize(void* stream);
+int ahpc_hip_event_create(void** event);
+int ahpc_hip_event_destroy(void* event);
+int ahpc_hip_event_record(void* event, void* stream);
+int ahpc_hip_event_synchronize(void* event);
+int ahpc_hip_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* ---- FlashAttention forward -------------------------------------------------------------------
+ * O = softmax(scale * Q K^T [+ causal]) V in one launch; replaces
+ * FlashAttention::forward -> compute_multihead_attention -> compute_attention_block,
+ * src/algorithms/flash_attention.cpp:68-112, :379-450, :277-350, and the
+ * launch_flash_attention_kernel slot of src/backends/cuda/cuda_flash_attention.hpp:42-48.
+ *
+ * Element (b, n, h, e) is at  b*stride_b + n*stride_n + h*stride_h + e; the last dimension
+ * is contiguous.  The API layout [B,N,H,d] (FlashAttention::validate_inputs,
+ * src/algorithms/flash_attention.cpp:238-275) is stride_b = N*H*d, stride_n = H*d,
+ * stride_h = d; [B,H,N,d] is stride_b = H*N*d, stride_h = N*d, stride_n = d, so no transpose
+ * pass (src/backends/cuda/cuda_kernels.cu:668-687) is ever needed.  Q, K, V and O share one
+ * dtype and one set of strides.  fp16/bf16 with d in {64, 128} run on the MFMA kernel; every
+ * other case (fp32, other d <= 256) runs on the fp32-FMA kernel.  Accumulation is fp32
+ * throughout.  A row with no visible key yields zeros
+ * (OnlineSoftmaxState::get_normalizer, src/algorithms/flash_attention.hpp:59-61).
+ * scale <= 0 means 1/sqrt(d) (AttentionParams::scale_factor,
+ * src/api/attention_interface.hpp:64). */
+int ahpc_hip_flash_fwd(const void* q, const void* k, const void* v, void* o, int dtype,
+                       int64_t B, int64_t N, int64_t H, int64_t d,
+                       int64_t stride_b, int64_t stride_n, int64_t stride_h,
+                       float scale, int causal, void* stream);
+
+/* Same with a dense fp32 mask [B,N,N] shared by all heads, 0.0f removes the key
+ * (FlashAttention::apply_attention_mask, src/algorithms/flash_attention.cpp:596-607;
+ * indexing :432-435).  mask may be NULL.  Always runs on the fp32-FMA kernel. */
+int ahpc_hip_flash_fwd_masked(const void* q, const void* k, const void* v, void* o, int dtype,
+                              int64_t B, int64_t N, int64_t H, int64_t d,
+                              int64_t stride_b, int64_t stride_n, int64_t stride_h,
+                              float scale, int causal, const float* mask, void* stream);
+
+/* Ragged batch packed as [T,H,d] (token stride stride_t, head stride stride_h); sequence i
+ * owns tokens cu_seqlens[i] .. cu_seqlens[i+1]-1 (int32, device, n_seqs+1 entries) and
+ * attends only within itself.  max_len = longest sequence (sizes the grid).  The reference
+ * has no ragged entry point; the nearest declared shape is
+ * CudaFlashAttention::forward_multi_sequence,
+ * src/backends/cuda/cuda_flash_attention.hpp:270-279. */
+int ahpc_hip_flash_fwd_varlen(const void* q, const void* k, const void* v, void* o, int dtype,
+                              const int32_t* cu_seqlens, int64_t n_seqs, int64_t max_len,
+                              int64_t H, int64_t d, int64_t stride_t, int64_t stride_h,
+                              float scale, int causal, void* stream);
+
+/* ---- paged KV pool ---------------------------------------------------------------------------
+ * Pool layout: K and V are separate slabs  [page][slot 0..P-1][head][d]  (the layout
+ * update_kv_cache_kernel writes, src/backends/cuda/cuda_kernels.cu:547-556).
+ * block_table is int32 [n_rows][max_pages], -1 = no page (sentinel of
+ * src/backends/cuda/cuda_kernels.cu:420).  Token t of table row r, head h lives at element
+ *     ((block_table[r*max_pages + t/P] * P + t%P) * H + h) * d.
+ */
+
+/* Write n_tokens new K/V rows ([n_tokens,H,d], dtype in_dtype) into the pool (dtype
+ * pool_dtype, converted with RNE).  Token i goes to table row token_row[i] at position
+ * token_pos[i]; token_row == NULL means every token belongs to `row0`, token_pos == NULL
+ * means positions pos0, pos0+1, ...  Tokens whose table entry is negative are skipped.
+ * Replaces PagedAttention::append_kv_cache -> scatter_keys_values,
+ * src/algorithms/paged_attention.cpp:434-462, and update_kv_cache_kernel with its
+ * slot_mapping, src/backends/cuda/cuda_kernels.cu:518-563. */
+int ahpc_hip_kv_scatter(const void* k_new, const void* v_new, int in_dtype,
+                        void* k_pool, void* v_pool, int pool_dtype,
+                        const int32_t* block_table, int64_t max_pages,
+                        const int32_t* token_row, const int32_t* token_pos,
+                        int64_t row0, int64_t pos0, int64_t n_tokens,
+                        int64_t H, int64_t d, int64_t P, void* stream);
+
+/* Read tokens [start, start+n) of table row `row` back as [n,H,d] in out_dtype.  Replaces
+ * PagedAttention::get_kv_cache -> gather_keys_values,
+ * src/algorithms/paged_attention.cpp:464-490. */
+int ahpc_hip_kv_gather(void* k_out, void* v_out, int out_dtype,
+                       const void* k_pool, const void* v_pool, int pool_dtype,
+                       const int32_t* block_table, int64_t max_pages,
+                       int64_t row, int64_t start, int64_t n,
+                       int64_t H, int64_t d, int64_t P, void* stream);
+
+/* ---- PagedAttention decode --------------------------------------------------------------------
+ * One query token per batch entry attends to all seq_lens[row] cached tokens of its sequence:
+ * replaces PagedAttention::forward_batch -> compute_paged_attention,
+ * src/algorithms/paged_attention.cpp:496-547, :596-680, and paged_attention_kernel,
+ * src/backends/cuda/cuda_kernels.cu:370-515 (with the query at the last position, which that
+ * kernel's causal test :434 reduces to "all cached keys").
+ *
+ * q, o: [B,H,d] in qo_dtype.  batch_rows (int32[B], device, may be NULL = identity) maps
+ * batch entry b to its row of block_table / seq_lens.  seq_lens: int32 per table row.
+ * A sequence of length 0 gets a zero output row (the reference skips it, :613-615).
+ *
+ * Long contexts are cut into chunks of `chunk_tokens` tokens (a multiple of P; 0 = choose),
+ * each chunk reduced by its own workgroup into an fp32 partial (m, l, o[d]) per head, then
+ * merged with the rule of OnlineSoftmaxState::update, src/algorithms/flash_attention.hpp:50-57.
+ * `max_len` bounds seq_lens (it sizes the grid; tokens beyond it are not read).
+ * workspace must hold ahpc_hip_paged_decode_workspace_bytes() bytes. */
+size_t ahpc_hip_paged_decode_workspace_bytes(int64_t B, int64_t H, int64_t d, int64_t max_len,
+                                             int64_t P, int64_t chunk_tokens);
+int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype,
+                          const void* k_pool, const void* v_pool, int pool_dtype,
+                          const int32_t* block_table, const int32_t* seq_lens, const int32_t* batch_rows,
+                          int64_t B, int64_t H, int64_t d, int64_t P, int64_t max_pages, int64_t max_len,
+                          float scale, int64_t chunk_tokens,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
+/* Debug twin of the decode kernel's addressing: offsets[b*max_len + t] = the element offset
+ * of (token t, head 0, lane 0) of batch entry b, computed by the same device function the
+ * decode kernel uses, or -1 for t >= seq_lens[row] or a negative table entry.  Lets a test
+ * compare the gather indices bit for bit with a host computation. */
+int ahpc_hip_paged_gather_indices(const int32_t* block_table, const int32_t* seq_lens, const int32_t* batch_rows,
+                                  int64_t B, int64_t H, int64_t d, int64_t P, int64_t max_pages, int64_t max_len,
+                                  int64_t* offsets, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AHPC_HIP_H */

@@ -1,0 +1,249 @@
+"""FlashAttention forward on the GPU (through the C ABI) against the CPU oracle.
+
+Tolerances: fp32 <= 1e-4 max-abs (tests/test_flash_attention.cpp:174 of the reference), fp16/bf16
+<= 2e-2 max-abs against the fp32 oracle fed the same, already rounded, inputs."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    from attention_amd import hip
+    hip.load()
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return hip
+
+
+def run_dense(hip, q, k, v, dtype, B, N, H, d, scale, causal, layout="BNHD", mask=None):
+    import torch
+    from gpu_util import to_dev, to_host, stream_ptr
+    dq, dk, dv = (to_dev(x, dtype) for x in (q, k, v))
+    do = torch.full_like(dq, float("nan"))
+    strides = (N * H * d, H * d, d) if layout == "BNHD" else (H * N * d, d, N * d)
+    dm = None if mask is None else torch.from_numpy(mask).cuda()
+    hip.flash_fwd(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), do.data_ptr(), dtype, B, N, H, d, strides, scale, causal,
+                  stream_ptr(), None if dm is None else dm.data_ptr())
+    torch.cuda.synchronize()
+    return to_host(do)
+
+
+def make_qkv(shape, seed, dtype, sigma=1.0, uniform=False):
+    gen = (lambda t: O.fill_uniform(shape, seed, t)) if uniform else (lambda t: O.fill_normal(shape, seed, t, sigma))
+    return tuple(O.round_to(gen(t), dtype) for t in (1, 2, 3))
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_reference_fixture_shape_fp32(gpu, causal):
+    # B=2,N=16,H=4,d=64: the fixture of tests/test_flash_attention.cpp:103-108, U(-1,1) inputs
+    B, N, H, d = 2, 16, 4, 64
+    q, k, v = make_qkv((B, N, H, d), 1, O.F32, uniform=True)
+    scale = 1.0 / np.sqrt(d)
+    got = run_dense(gpu, q, k, v, O.F32, B, N, H, d, scale, causal)
+    want = O.attention(q, k, v, B, N, H, d, scale, causal)
+    assert np.abs(got - want).max() <= 1e-4
+
+
+@pytest.mark.parametrize("N", [1, 4, 32, 128, 129, 300])
+def test_sequence_lengths_fp32(gpu, N):
+    # tests/test_flash_attention.cpp:218-260 uses {1,4,32,128}; 129 and 300 add ragged tails
+    B, H, d = 2, 4, 64
+    q, k, v = make_qkv((B, N, H, d), 2, O.F32, uniform=True)
+    got = run_dense(gpu, q, k, v, O.F32, B, N, H, d, 0.125, False)
+    want = O.attention(q, k, v, B, N, H, d, 0.125, False)
+    assert np.abs(got - want).max() <= 1e-4
+    if N == 1:
+        assert np.abs(got - v).max() <= 1e-6  # N = 1 => O = V (tests/test_flash_attention.cpp:585-588)
+
+
+@pytest.mark.parametrize("d", [16, 32, 64, 128, 80, 256])
+def test_head_dimensions_fp32(gpu, d):
+    # tests/test_flash_attention.cpp:263-307, tolerance max(1e-4, 1e-5*sqrt(d)); 80 and 256 are extra
+    B, N, H = 2, 16, 4
+    q, k, v = make_qkv((B, N, H, d), 3, O.F32, uniform=True)
+    scale = 1.0 / np.sqrt(d)
+    got = run_dense(gpu, q, k, v, O.F32, B, N, H, d, scale, True)
+    want = O.attention(q, k, v, B, N, H, d, scale, True)
+    assert np.abs(got - want).max() <= max(1e-4, 1e-5 * np.sqrt(d))
+
+
+def test_config1_fp32_noncausal(gpu):
+    # fp32, non-causal, B=2, N=512, H=8, d=64, N(0,1) inputs
+    B, N, H, d = 2, 512, 8, 64
+    q, k, v = make_qkv((B, N, H, d), 0xA77E0001, O.F32)
+    scale = 1.0 / np.sqrt(d)
+    got = run_dense(gpu, q, k, v, O.F32, B, N, H, d, scale, False)
+    want = O.attention(q, k, v, B, N, H, d, scale, False)
+    assert np.abs(got - want).max() <= 1e-4
+
+
+def test_layout_bhnd_fp32(gpu):
+    B, N, H, d = 2, 40, 3, 32
+    q, k, v = make_qkv((B, H, N, d), 4, O.F32)
+    got = run_dense(gpu, q, k, v, O.F32, B, N, H, d, 0.2, True, layout="BHND")
+    want = O.attention(q, k, v, B, N, H, d, 0.2, True, layout="BHND")
+    assert np.abs(got - want).max() <= 1e-4
+
+
+def test_dense_mask_fp32(gpu):
+    # tests/test_flash_attention.cpp:483-582: mask [B,N,N], 0 = masked; a fully masked row gives zeros
+    B, N, H, d = 2, 48, 2, 32
+    q, k, v = make_qkv((B, N, H, d), 5, O.F32)
+    rng = np.random.default_rng(7)
+    mask = (rng.random((B, N, N)) > 0.5).astype(np.float32)
+    mask[1, 3, :] = 0.0
+    got = run_dense(gpu, q, k, v, O.F32, B, N, H, d, 0.2, False, mask=mask)
+    want = O.attention(q, k, v, B, N, H, d, 0.2, False, mask=mask)
+    assert np.abs(got - want).max() <= 1e-4
+    assert np.all(got[1, 3] == 0.0)
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16])
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("N", [1, 37, 64, 128, 200, 517])
+def test_mfma_small(gpu, dtype, d, causal, N):
+    B, H = 2, 3
+    q, k, v = make_qkv((B, N, H, d), 100 + N, dtype)
+    scale = 1.0 / np.sqrt(d)
+    got = run_dense(gpu, q, k, v, dtype, B, N, H, d, scale, causal)
+    want = O.attention(q, k, v, B, N, H, d, scale, causal)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= 2e-2
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16])
+def test_mfma_closed_forms(gpu, dtype):
+    B, N, H, d = 1, 256, 2, 128
+    q, k, v = make_qkv((B, N, H, d), 9, dtype)
+    # V constant => O constant (exactly representable value)
+    vc = np.full_like(v, 0.625)
+    got = run_dense(gpu, q, k, vc, dtype, B, N, H, d, 0.1, True)
+    assert np.abs(got - 0.625).max() <= 4e-3
+    # Q = 0 => prefix mean of V
+    got = run_dense(gpu, np.zeros_like(q), k, v, dtype, B, N, H, d, 0.1, True)
+    prefix = np.cumsum(v.astype(np.float64), axis=1) / np.arange(1, N + 1)[None, :, None, None]
+    assert np.abs(got - prefix).max() <= 2e-2
+    # one dominant logit => that V row
+    q1 = np.zeros_like(q)
+    k1 = np.zeros_like(k)
+    q1[..., 0] = 1.0
+    k1[:, 77, :, 0] = 80.0
+    got = run_dense(gpu, q1, k1, v, dtype, B, N, H, d, 1.0, False)
+    assert np.abs(got - v[:, 77:78]).max() <= 1e-2
+    # key-permutation invariance (non causal)
+    perm = np.random.default_rng(1).permutation(N)
+    a = run_dense(gpu, q, k, v, dtype, B, N, H, d, 0.1, False)
+    b = run_dense(gpu, q, np.ascontiguousarray(k[:, perm]), np.ascontiguousarray(v[:, perm]), dtype, B, N, H, d, 0.1, False)
+    assert np.abs(a - b).max() <= 1e-2
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16])
+def test_mfma_layout_bhnd(gpu, dtype):
+    B, N, H, d = 2, 96, 2, 64
+    q, k, v = make_qkv((B, H, N, d), 6, dtype)
+    got = run_dense(gpu, q, k, v, dtype, B, N, H, d, 0.125, True, layout="BHND")
+    want = O.attention(q, k, v, B, N, H, d, 0.125, True, layout="BHND")
+    assert np.abs(got - want).max() <= 2e-2
+
+
+def test_config2_shape_bf16_causal_sampled_rows(gpu):
+    # bf16, causal, B=4, N=4096, H=32, d=128 at full size: a seeded sample of rows against the oracle,
+    # plus size-independent properties over the whole output
+    import torch
+    from gpu_util import stream_ptr
+    B, N, H, d = 4, 4096, 32, 128
+    dtype = O.BF16
+    g = torch.Generator(device="cuda").manual_seed(0xA77E0002)
+    dq, dk, dv = (torch.randn((B, N, H, d), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16) for _ in range(3))
+    do = torch.full_like(dq, float("nan"))
+    scale = 1.0 / np.sqrt(d)
+    gpu.flash_fwd(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), do.data_ptr(), dtype, B, N, H, d, (N * H * d, H * d, d),
+                  scale, True, stream_ptr())
+    torch.cuda.synchronize()
+    assert torch.isfinite(do.float()).all()
+    # row 0 of every (b, h) sees only key 0 => equals V row 0 exactly
+    assert torch.equal(do[:, 0], dv[:, 0])
+    # outputs are convex combinations of V rows: bounded by the running min/max of V along the sequence
+    vmax = torch.cummax(dv.float(), dim=1).values
+    vmin = torch.cummin(dv.float(), dim=1).values
+    assert (do.float() <= vmax + 2e-2).all() and (do.float() >= vmin - 2e-2).all()
+    rng = np.random.default_rng(2)
+    rows = np.unique(np.concatenate([rng.integers(0, B * H * N, 384), [N - 1, B * H * N - 1, 127, 128, 4095]])).astype(np.int64)
+    q, k, v = (t.float().cpu().numpy() for t in (dq, dk, dv))
+    want = O.attention_rows(q, k, v, B, N, H, d, scale, rows, True)
+    out = do.float().cpu().numpy()
+    got = np.stack([out[r // (N * H), r % N, (r // N) % H] for r in rows])
+    assert np.abs(got - want).max() <= 2e-2
+
+
+@pytest.mark.parametrize("dtype,d", [(O.F16, 64), (O.BF16, 128), (O.F32, 64), (O.F16, 32)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_varlen_small(gpu, dtype, d, causal):
+    import torch
+    from gpu_util import to_dev, to_host, stream_ptr, dev_i32
+    H = 4
+    lens = [5, 130, 1, 64, 257, 128]
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    q, k, v = make_qkv((T, H, d), 11, dtype, sigma=0.5)
+    dq, dk, dv = (to_dev(x, dtype) for x in (q, k, v))
+    do = torch.full_like(dq, float("nan"))
+    dcu = dev_i32(cu)
+    scale = 1.0 / np.sqrt(d)
+    gpu.flash_fwd_varlen(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), do.data_ptr(), dtype, dcu.data_ptr(), len(lens),
+                         max(lens), H, d, H * d, d, scale, causal, stream_ptr())
+    torch.cuda.synchronize()
+    got = to_host(do)
+    want = O.attention_varlen(q, k, v, cu, H, d, scale, causal)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= (1e-4 if dtype == O.F32 else 2e-2)
+
+
+def test_config5_varlen_fp16_causal_sampled_rows(gpu):
+    # fp16 causal ragged batch: 16 sequences, lengths U[128, 8192], H=32, d=64, sigma = 0.5
+    import torch
+    from gpu_util import stream_ptr, dev_i32
+    H, d = 32, 64
+    lens = O.fill_lengths(16, 0xA77E0005, 4, 128, 8192)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    g = torch.Generator(device="cuda").manual_seed(0xA77E0005)
+    dq, dk, dv = ((0.5 * torch.randn((T, H, d), generator=g, device="cuda", dtype=torch.float32)).to(torch.float16) for _ in range(3))
+    do = torch.full_like(dq, float("nan"))
+    dcu = dev_i32(cu)
+    scale = 1.0 / np.sqrt(d)
+    gpu.flash_fwd_varlen(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), do.data_ptr(), O.F16, dcu.data_ptr(), 16,
+                         int(lens.max()), H, d, H * d, d, scale, True, stream_ptr())
+    torch.cuda.synchronize()
+    assert torch.isfinite(do.float()).all()
+    # first token of every sequence sees only itself
+    first = torch.from_numpy(cu[:-1].astype(np.int64)).cuda()
+    assert torch.equal(do[first], dv[first])
+    rng = np.random.default_rng(5)
+    toks = np.concatenate([rng.integers(0, T, 300), cu[1:] - 1, cu[:-1]])
+    rows = (toks.astype(np.int64) * H + rng.integers(0, H, toks.size)).astype(np.int64)
+    q, k, v = (t.float().cpu().numpy() for t in (dq, dk, dv))
+    want = O.attention_varlen_rows(q, k, v, cu, H, d, scale, rows, True)
+    out = do.float().cpu().numpy()
+    got = np.stack([out[r // H, r % H] for r in rows])
+    assert np.abs(got - want).max() <= 2e-2
+
+
+def test_bad_arguments_are_rejected_without_launch(gpu):
+    import torch
+    x = torch.zeros(2 * 16 * 4 * 64, device="cuda")
+    p = x.data_ptr()
+    with pytest.raises(gpu.HipError):
+        gpu.flash_fwd(0, p, p, p, O.F32, 2, 16, 4, 64, (16 * 4 * 64, 4 * 64, 64), 0.1, False)
+    with pytest.raises(gpu.HipError):
+        gpu.flash_fwd(p, p, p, p, 7, 2, 16, 4, 64, (16 * 4 * 64, 4 * 64, 64), 0.1, False)
+    with pytest.raises(gpu.HipError):
+        gpu.flash_fwd(p, p, p, p, O.F32, 2, 0, 4, 64, (16 * 4 * 64, 4 * 64, 64), 0.1, False)
+    with pytest.raises(gpu.HipError):
+        gpu.flash_fwd(p, p, p, p, O.F32, 2, 16, 4, 512, (16 * 4 * 512, 4 * 512, 512), 0.1, False)
+    torch.cuda.synchronize()
