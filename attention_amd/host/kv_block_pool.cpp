@@ -1,0 +1,126 @@
+// Device KV block pool: FIFO page ids on the host, K/V slabs in HBM.
+#include "memory/kv_block_pool.hpp"
+
+#include <algorithm>
+
+#include "hip_support.hpp"
+
+namespace attention_hpc {
+
+using hipsup::check;
+
+KVBlockPool::KVBlockPool(size_t page_tokens, size_t heads, size_t head_dim, DataType dtype, size_t initial_pages,
+                         size_t growth, size_t max_bytes)
+    : page_tokens_(page_tokens), heads_(heads), head_dim_(head_dim), dtype_(dtype), growth_(growth), max_bytes_(max_bytes) {
+    if (page_tokens == 0 || heads == 0 || head_dim == 0)
+        throw AttentionException(AttentionError::INVALID_PARAMETERS, "KVBlockPool: page geometry must be positive");
+    slab_elems_per_page_ = page_tokens * heads * head_dim;
+    if (max_bytes_ == 0) {
+        ahpc_device_info info;
+        check(ahpc_hip_device_info(0, &info), "device query");
+        const uint64_t avail = info.free_memory_bytes ? info.free_memory_bytes : info.total_memory_bytes;
+        max_bytes_ = static_cast<size_t>(avail / 10 * 9);
+    }
+    std::lock_guard<std::mutex> lock(mutex_);
+    create_pages_locked(initial_pages);
+}
+
+KVBlockPool::~KVBlockPool() {
+    ahpc_hip_free(k_slab_);
+    ahpc_hip_free(v_slab_);
+}
+
+// Grows the slabs to hold at least `pages` pages: new allocation of twice the size (at least 64
+// pages), device-to-device copy of what exists, release of the old slabs.
+void KVBlockPool::reserve_locked(size_t pages) {
+    if (pages <= capacity_pages_) return;
+    const size_t page_bytes_one = slab_elems_per_page_ * hipsup::dtype_size(dtype_);
+    size_t want = std::max<size_t>(std::max<size_t>(capacity_pages_ * 2, pages), 64);
+    const size_t cap_by_budget = max_bytes_ / (2 * page_bytes_one);
+    if (want > cap_by_budget) want = cap_by_budget;
+    if (want < pages)
+        throw MemoryPoolException("KV block pool exhausted: " + std::to_string(pages) + " pages needed, device budget allows " +
+                                  std::to_string(cap_by_budget));
+    void* nk = nullptr;
+    void* nv = nullptr;
+    check(ahpc_hip_malloc(&nk, want * page_bytes_one), "KV slab allocation", true);
+    const int rc = ahpc_hip_malloc(&nv, want * page_bytes_one);
+    if (rc != 0) {
+        ahpc_hip_free(nk);
+        check(rc, "KV slab allocation", true);
+    }
+    if (capacity_pages_) {
+        check(ahpc_hip_memcpy_d2d(nk, k_slab_, capacity_pages_ * page_bytes_one, nullptr), "KV slab copy");
+        check(ahpc_hip_memcpy_d2d(nv, v_slab_, capacity_pages_ * page_bytes_one, nullptr), "KV slab copy");
+        check(ahpc_hip_stream_synchronize(nullptr), "KV slab copy");
+        ahpc_hip_free(k_slab_);
+        ahpc_hip_free(v_slab_);
+    }
+    k_slab_ = nk;
+    v_slab_ = nv;
+    capacity_pages_ = want;
+    ++generation_;
+}
+
+void KVBlockPool::create_pages_locked(size_t count) {
+    if (count == 0) return;
+    const size_t first = in_use_.size();
+    reserve_locked(first + count);
+    in_use_.resize(first + count, 0);
+    for (size_t i = 0; i < count; ++i) free_.push_back(static_cast<int32_t>(first + i));
+}
+
+int32_t KVBlockPool::allocate_page() {
+    std::lock_guard<std::mutex> lock(mutex_);
+    if (free_.empty()) {
+        if (growth_ == 0) throw MemoryPoolException("KV block pool exhausted (fixed-size pool)");
+        create_pages_locked(growth_);
+    }
+    const int32_t id = free_.front();
+    free_.pop_front();
+    in_use_[id] = 1;
+    ++allocated_;
+    peak_ = std::max(peak_, allocated_);
+    return id;
+}
+
+void KVBlockPool::deallocate_page(int32_t page) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    if (page < 0 || static_cast<size_t>(page) >= in_use_.size() || !in_use_[page]) return;
+    in_use_[page] = 0;
+    --allocated_;
+    free_.push_back(page);
+}
+
+void KVBlockPool::resize_pool(size_t new_total_pages) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    if (new_total_pages > in_use_.size()) create_pages_locked(new_total_pages - in_use_.size());
+}
+
+size_t KVBlockPool::get_pool_size() const {
+    std::lock_guard<std::mutex> lock(mutex_);
+    return in_use_.size();
+}
+size_t KVBlockPool::get_free_pages() const {
+    std::lock_guard<std::mutex> lock(mutex_);
+    return free_.size();
+}
+size_t KVBlockPool::get_allocated_pages() const {
+    std::lock_guard<std::mutex> lock(mutex_);
+    return allocated_;
+}
+
+KVBlockPoolStats KVBlockPool::stats() const {
+    std::lock_guard<std::mutex> lock(mutex_);
+    KVBlockPoolStats s;
+    s.total_pages = in_use_.size();
+    s.free_pages = free_.size();
+    s.allocated_pages = allocated_;
+    s.peak_allocated_pages = peak_;
+    s.page_bytes = 2 * slab_elems_per_page_ * hipsup::dtype_size(dtype_);
+    s.slab_capacity_pages = capacity_pages_;
+    s.slab_bytes = capacity_pages_ * s.page_bytes;
+    return s;
+}
+
+}  // namespace attention_hpc

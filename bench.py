@@ -1,0 +1,259 @@
+#!/usr/bin/env python3
+"""Benchmark of the two hot paths on one MI355X, through the C ABI (include/ahpc_hip.h).
+
+Headline (the JSON line's metric/value): FlashAttention forward, bf16, causal, B=4, N=4096, H=32,
+d=128, layout [B,N,H,d] - one "step" is one forward over that batch.  The same line carries the
+PagedAttention decode result (fp16, B=64, H=32, d=128, page 16, context lengths U[512,4096]) under
+"decode".  Inputs are synthetic and already resident in HBM when the timed region starts.
+
+  value            whole-job throughput: algorithmic FLOP (2*B*H*N^2*d for causal) / wall time of the
+                   K timed steps, bracketed by a device synchronize on both sides
+  roofline         algorithmic FLOP (or bytes) per launch / mean kernel duration measured with HIP
+                   events on the launch stream, against MI355X's dense bf16 MFMA peak (2.5 PFLOP/s)
+                   or HBM peak (8 TB/s)
+  cpu_baseline     the CPU oracle (oracle/, a restatement of the reference's algorithm) timed on this
+                   box's host cores over a bounded sample of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+
+FLASH = dict(B=4, N=4096, H=32, d=128, causal=True, dtype="bf16", seed=0xA77E0002)
+DECODE = dict(B=64, H=32, d=128, P=16, lo=512, hi=4096, dtype="fp16", seed=0xA77E0003)
+
+
+def lengths_and_table(cfg):
+    """Seeded context lengths and a shuffled block table (numpy only)."""
+    rng = np.random.default_rng(cfg["seed"])
+    lens = rng.integers(cfg["lo"], cfg["hi"] + 1, size=cfg["B"]).astype(np.int32)
+    P = cfg["P"]
+    pages_per = (lens + P - 1) // P
+    n_pages = int(pages_per.sum()) + 64
+    ids = rng.permutation(n_pages).astype(np.int32)
+    table = np.full((cfg["B"], int(pages_per.max())), -1, np.int32)
+    c = 0
+    for b in range(cfg["B"]):
+        table[b, :pages_per[b]] = ids[c:c + pages_per[b]]
+        c += pages_per[b]
+    return lens, table, n_pages
+
+
+def decode_bytes(lens, cfg):
+    """Algorithmic bytes of one decode step: K and V of every cached token once, q and o once, the
+    block-table entries and lengths once."""
+    H, d, P, B = cfg["H"], cfg["d"], cfg["P"], cfg["B"]
+    esz = 2
+    L = lens.astype(np.int64)
+    return int((2 * L * H * d * esz).sum() + 2 * B * H * d * esz + 4 * ((L + P - 1) // P).sum() + 4 * B)
+
+
+class Timer:
+    """HIP events on the launch stream (torch's events only see torch's own current stream)."""
+
+    def __init__(self, hip, stream, n):
+        import ctypes as C
+        self.hip, self.stream, self.C = hip, stream, C
+        self.lib = hip.load()
+        self.ev = []
+        for _ in range(2 * n):
+            e = C.c_void_p()
+            assert self.lib.ahpc_hip_event_create(C.byref(e)) == 0
+            self.ev.append(e)
+
+    def record(self, i):
+        assert self.lib.ahpc_hip_event_record(self.ev[i], self.stream) == 0
+
+    def elapsed_ms(self, i, j):
+        ms = self.C.c_float()
+        assert self.lib.ahpc_hip_event_synchronize(self.ev[j]) == 0
+        assert self.lib.ahpc_hip_event_elapsed_ms(self.ev[i], self.ev[j], self.C.byref(ms)) == 0
+        return ms.value
+
+    def close(self):
+        for e in self.ev:
+            self.lib.ahpc_hip_event_destroy(e)
+
+
+def timed_steps(hip, stream, launch, steps, warmup):
+    """W untimed launches, then exactly K timed ones: wall clock around all K (synchronised on both
+    sides) and an event pair around each launch."""
+    import torch
+    lib = hip.load()
+    for _ in range(warmup):
+        launch()
+    assert lib.ahpc_hip_stream_synchronize(stream) == 0
+    torch.cuda.synchronize()
+    t = Timer(hip, stream, steps)
+    t0 = time.perf_counter()
+    for i in range(steps):
+        t.record(2 * i)
+        launch()
+        t.record(2 * i + 1)
+    assert lib.ahpc_hip_stream_synchronize(stream) == 0
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per = [t.elapsed_ms(2 * i, 2 * i + 1) for i in range(steps)]
+    t.close()
+    return wall, per
+
+
+def bench_flash(hip, stream, steps, warmup, cpu):
+    import torch
+    c = FLASH
+    B, N, H, d = c["B"], c["N"], c["H"], c["d"]
+    g = torch.Generator(device="cuda").manual_seed(c["seed"])
+    q, k, v = (torch.randn((B, N, H, d), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16) for _ in range(3))
+    o = torch.empty_like(q)
+    torch.cuda.synchronize()
+    scale = 1.0 / np.sqrt(d)
+    strides = (N * H * d, H * d, d)
+
+    def launch():
+        hip.flash_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), hip.BF16, B, N, H, d, strides, scale, True, stream)
+
+    wall, per = timed_steps(hip, stream, launch, steps, warmup)
+    flops = 2.0 * B * H * N * N * d            # causal convention; exact count 4*B*H*d*N(N+1)/2 is 0.02% higher
+    value = flops * steps / wall / 1e12
+    kern_ms = float(np.mean(per))
+    achieved = flops / (kern_ms * 1e-3) / 1e12
+    res = {
+        "metric": "FlashAttn fwd TFLOP/s (bf16, N=4096, d=128)", "value": round(value, 2), "unit": "TFLOP/s",
+        "ms_per_step": round(wall / steps * 1e3, 4),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "flash_fwd_mfma_kernel<bf16,128,causal>", "kernel_ms_mean": round(kern_ms, 4),
+                     "kernel_ms_min": round(float(np.min(per)), 4), "flop_per_launch": flops},
+        "config": {"workload": "flash_fwd bf16 causal B=4 N=4096 H=32 d=128 layout [B,N,H,d], fp32 accumulate, bf16 out"},
+    }
+    if cpu:
+        from oracle import oracle as O
+        # bounded sample: batch entry 0 (all 32 heads), i.e. 1/4 of the step, on the box's host cores
+        qs, ks, vs = (t[0:1].float().cpu().numpy() for t in (q, k, v))
+        threads = O.cpu_threads()
+        t0 = time.perf_counter()
+        ref = O.attention(qs, ks, vs, 1, N, H, d, scale, True, threads=threads)
+        dt = time.perf_counter() - t0
+        err = float(np.abs(o[0:1].float().cpu().numpy() - ref).max())
+        res["cpu_baseline"] = {"value": round(2.0 * H * N * N * d / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads,
+                               "kind": "port", "sample": f"batch entry 0 of 4 (32 heads x 4096 rows), {dt:.1f} s",
+                               "max_abs_err_gpu_vs_cpu": err}
+    return res
+
+
+def bench_decode(hip, stream, steps, warmup, cpu):
+    import torch
+    c = DECODE
+    B, H, d, P = c["B"], c["H"], c["d"], c["P"]
+    lens, table, n_pages = lengths_and_table(c)
+    g = torch.Generator(device="cuda").manual_seed(c["seed"])
+    elems = n_pages * P * H * d
+    kpool = torch.randn(elems, generator=g, device="cuda", dtype=torch.float32).to(torch.float16)
+    vpool = torch.randn(elems, generator=g, device="cuda", dtype=torch.float32).to(torch.float16)
+    q = torch.randn((B, H, d), generator=g, device="cuda", dtype=torch.float32).to(torch.float16)
+    o = torch.empty_like(q)
+    dt_, dl = torch.from_numpy(table).cuda(), torch.from_numpy(lens).cuda()
+    max_len, max_pages = int(lens.max()), table.shape[1]
+    ws_bytes = hip.paged_decode_workspace_bytes(B, H, d, max_len, P, 0)
+    ws = torch.empty(max(ws_bytes, 4) // 4, dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    scale = 1.0 / np.sqrt(d)
+
+    def launch():
+        hip.paged_decode(q.data_ptr(), o.data_ptr(), hip.F16, kpool.data_ptr(), vpool.data_ptr(), hip.F16, dt_.data_ptr(),
+                         dl.data_ptr(), None, B, H, d, P, max_pages, max_len, scale, 0, ws.data_ptr(), ws_bytes, stream)
+
+    wall, per = timed_steps(hip, stream, launch, steps, warmup)
+    nbytes = decode_bytes(lens, c)
+    value = nbytes * steps / wall / 1e9
+    kern_ms = float(np.mean(per))
+    achieved = nbytes / (kern_ms * 1e-3) / 1e9
+    res = {
+        "metric": "paged decode HBM GB/s", "value": round(value, 1), "unit": "GB/s",
+        "ms_per_step": round(wall / steps * 1e3, 4),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "paged_decode_kernel<f16,128> + paged_merge_kernel", "kernel_ms_mean": round(kern_ms, 4),
+                     "kernel_ms_min": round(float(np.min(per)), 4), "bytes_per_launch": nbytes},
+        "config": {"workload": f"paged_decode fp16 B=64 H=32 d=128 page=16 context U[512,4096] (sum {int(lens.sum())} tokens), "
+                               f"shuffled block table, pool {n_pages} pages"},
+    }
+    if cpu:
+        from oracle import oracle as O
+        # bounded sample: the first 16 of the 64 sequences, their pages copied to the host
+        nb = 16
+        pages_per = (lens + P - 1) // P
+        sub_tables, kparts, vparts, c0 = [], [], [], 0
+        for b in range(nb):
+            pg = torch.from_numpy(table[b, :pages_per[b]].astype(np.int64)).cuda()
+            kparts.append(kpool.view(n_pages, -1)[pg].float().cpu().numpy().reshape(-1))
+            vparts.append(vpool.view(n_pages, -1)[pg].float().cpu().numpy().reshape(-1))
+            sub_tables.append(np.arange(c0, c0 + pages_per[b], dtype=np.int32))
+            c0 += int(pages_per[b])
+        st = np.full((nb, int(pages_per[:nb].max())), -1, np.int32)
+        for b in range(nb):
+            st[b, :pages_per[b]] = sub_tables[b]
+        kh, vh = np.concatenate(kparts), np.concatenate(vparts)
+        qh = q[:nb].float().cpu().numpy()
+        threads = O.cpu_threads()
+        t0 = time.perf_counter()
+        ref = O.paged_decode(qh, kh, vh, st, lens[:nb], None, nb, H, d, P, scale, threads=threads)
+        dt = time.perf_counter() - t0
+        sub = dict(c, B=nb)
+        err = float(np.abs(o[:nb].float().cpu().numpy() - ref).max())
+        res["cpu_baseline"] = {"value": round(decode_bytes(lens[:nb], sub) / dt / 1e9, 3), "unit": "GB/s", "cores": threads,
+                               "kind": "port", "sample": f"first 16 of 64 sequences ({int(lens[:nb].sum())} tokens), {dt:.1f} s; "
+                               "bytes counted at the GPU's 2-byte storage size", "max_abs_err_gpu_vs_cpu": err}
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", choices=["all", "flash", "decode"], default="all")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline (profiling runs)")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (both paths shard by head or sequence without communication); "
+                 f"--gpus {a.gpus} is not supported")
+    import torch
+    from attention_amd import hip
+    hip.load()
+    if not torch.cuda.is_available() or hip.device_count() < 1:
+        sys.exit("bench.py: no GPU visible")
+    import ctypes as C
+    s = C.c_void_p()
+    assert hip.load().ahpc_hip_stream_create(C.byref(s)) == 0
+    stream = s.value
+
+    out = {"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
+    flash = bench_flash(hip, stream, a.steps, a.warmup, not a.no_cpu) if a.workload in ("all", "flash") else None
+    decode = bench_decode(hip, stream, a.steps, a.warmup, not a.no_cpu) if a.workload in ("all", "decode") else None
+    head = flash or decode
+    out.update({k: head[k] for k in ("metric", "value", "unit", "ms_per_step", "config", "roofline")})
+    if "cpu_baseline" in head:
+        out["cpu_baseline"] = head["cpu_baseline"]
+    if flash is None:
+        out["dtype"] = "f16"
+    if flash and decode:
+        out["decode"] = decode
+    info = hip.device_info(0)
+    out["device"] = {"name": info.name.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units}
+    hip.load().ahpc_hip_stream_destroy(stream)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

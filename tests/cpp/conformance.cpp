@@ -1,0 +1,788 @@
+// Conformance suite for the C++ host classes, written after the reference's own gtest files
+// (tests/test_flash_attention.cpp, tests/test_backends.cpp) and its decode example
+// (examples/basic_usage.cpp:115-200): same fixtures, same tolerances, same expectations, with the CPU
+// oracle (oracle/oracle.h) as the expected value.  gtest is not available, so a few macros stand in.
+//
+//   ahpc_conformance            all cases (needs a GPU)
+//   ahpc_conformance --no-gpu   only the cases that never touch a device
+//   ahpc_conformance <filter>   cases whose name contains <filter>
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "algorithms/flash_attention.hpp"
+#include "algorithms/paged_attention.hpp"
+#include "api/backend_factory.hpp"
+#include "api/tensor.hpp"
+#include "oracle.h"
+
+using namespace attention_hpc;
+
+// ---- tiny harness --------------------------------------------------------------------------------
+struct Case {
+    const char* name;
+    bool needs_gpu;
+    std::function<void()> fn;
+};
+static std::vector<Case>& cases() {
+    static std::vector<Case> c;
+    return c;
+}
+static int g_failures = 0;
+struct Registrar {
+    Registrar(const char* n, bool gpu, std::function<void()> f) { cases().push_back({n, gpu, std::move(f)}); }
+};
+#define CASE(name, gpu)                                \
+    static void case_##name();                         \
+    static Registrar reg_##name(#name, gpu, case_##name); \
+    static void case_##name()
+#define EXPECT(cond)                                                              \
+    do {                                                                          \
+        if (!(cond)) {                                                            \
+            std::printf("    EXPECT failed %s:%d: %s\n", __FILE__, __LINE__, #cond); \
+            ++g_failures;                                                         \
+        }                                                                         \
+    } while (0)
+#define EXPECT_THROWS(stmt, code)                                                                  \
+    do {                                                                                           \
+        bool thrown = false;                                                                       \
+        try {                                                                                      \
+            stmt;                                                                                  \
+        } catch (const AttentionException& e) {                                                    \
+            thrown = true;                                                                         \
+            if (e.error_code() != (code)) {                                                        \
+                std::printf("    wrong error code %d at %s:%d\n", (int)e.error_code(), __FILE__, __LINE__); \
+                ++g_failures;                                                                      \
+            }                                                                                      \
+        }                                                                                          \
+        if (!thrown) {                                                                             \
+            std::printf("    expected AttentionException at %s:%d\n", __FILE__, __LINE__);         \
+            ++g_failures;                                                                          \
+        }                                                                                          \
+    } while (0)
+#define EXPECT_THROWS_ANY(stmt)                                                            \
+    do {                                                                                   \
+        bool thrown = false;                                                               \
+        try {                                                                              \
+            stmt;                                                                          \
+        } catch (const AttentionException&) {                                              \
+            thrown = true;                                                                 \
+        }                                                                                  \
+        if (!thrown) {                                                                     \
+            std::printf("    expected AttentionException at %s:%d\n", __FILE__, __LINE__); \
+            ++g_failures;                                                                  \
+        }                                                                                  \
+    } while (0)
+
+static std::vector<float> uniform(size_t n, uint64_t seed, uint64_t id, float lo = -1.0f, float hi = 1.0f) {
+    std::vector<float> v(n);
+    ahpc_oracle_fill_uniform(v.data(), n, seed, id, lo, hi);
+    return v;
+}
+static std::vector<float> normal(size_t n, uint64_t seed, uint64_t id, float sigma = 1.0f) {
+    std::vector<float> v(n);
+    ahpc_oracle_fill_normal(v.data(), n, seed, id, sigma);
+    return v;
+}
+static float max_abs_diff(const std::vector<float>& a, const std::vector<float>& b) {
+    float m = a.size() == b.size() ? 0.0f : INFINITY;
+    for (size_t i = 0; i < a.size() && i < b.size(); ++i) m = std::max(m, std::fabs(a[i] - b[i]));
+    return m;
+}
+static std::vector<float> oracle_bnhd(const std::vector<float>& q, const std::vector<float>& k, const std::vector<float>& v,
+                                      size_t B, size_t N, size_t H, size_t d, float scale, bool causal,
+                                      const float* mask = nullptr) {
+    std::vector<float> out(q.size(), 0.0f);
+    ahpc_oracle_attention(q.data(), k.data(), v.data(), out.data(), B, N, H, d, N * H * d, H * d, d, scale, causal, mask, 4);
+    return out;
+}
+static TensorShape shape4(size_t B, size_t N, size_t H, size_t d, DataType t = DataType::FLOAT32) {
+    return TensorShape({B, N, H, d}, t);
+}
+
+// fixture of tests/test_flash_attention.cpp:103-108
+static AttentionParams fixture_params() {
+    AttentionParams p{};
+    p.batch_size = 2;
+    p.sequence_length = 16;
+    p.num_heads = 4;
+    p.head_dimension = 64;
+    p.causal_mask = false;
+    p.scale_factor = 1.0f / std::sqrt(64.0f);
+    return p;
+}
+
+static float run_flash_and_compare(FlashAttention& fa, const AttentionParams& p, uint64_t seed) {
+    const size_t B = p.batch_size, N = p.sequence_length, H = p.num_heads, d = p.head_dimension, n = B * N * H * d;
+    auto q = uniform(n, seed, 1), k = uniform(n, seed, 2), v = uniform(n, seed, 3);
+    std::vector<float> out(n, 0.0f);
+    const TensorShape s = shape4(B, N, H, d);
+    fa.forward(s, q.data(), s, k.data(), s, v.data(), s, out.data());
+    return max_abs_diff(out, oracle_bnhd(q, k, v, B, N, H, d, p.scale_factor, p.causal_mask));
+}
+
+// ---- tests/test_flash_attention.cpp ---------------------------------------------------------------
+CASE(Flash_ForwardPassSmallInput, true) {  // :141-175, tolerance 1e-4
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    fa.configure(p);
+    EXPECT(run_flash_and_compare(fa, p, 1) <= 1e-4f);
+}
+
+CASE(Flash_CausalMaskTest, true) {  // :178-215: params.causal_mask = true must act
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    p.causal_mask = true;
+    fa.configure(p);
+    EXPECT(run_flash_and_compare(fa, p, 2) <= 1e-4f);
+}
+
+CASE(Flash_DifferentSequenceLengths, true) {  // :218-260
+    FlashAttention fa;
+    for (size_t N : {1u, 4u, 32u, 128u}) {
+        AttentionParams p = fixture_params();
+        p.sequence_length = N;
+        fa.configure(p);
+        EXPECT(run_flash_and_compare(fa, p, 3 + N) <= 1e-4f);
+    }
+}
+
+CASE(Flash_DifferentHeadDimensions, true) {  // :263-307, tolerance max(1e-4, 1e-5*sqrt(d))
+    FlashAttention fa;
+    for (size_t d : {16u, 32u, 64u, 128u}) {
+        AttentionParams p = fixture_params();
+        p.head_dimension = d;
+        p.scale_factor = 1.0f / std::sqrt((float)d);
+        fa.configure(p);
+        EXPECT(run_flash_and_compare(fa, p, 10 + d) <= std::max(1e-4f, 1e-5f * std::sqrt((float)d)));
+    }
+}
+
+CASE(Flash_InvalidInputs, true) {  // :310-357
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    fa.configure(p);
+    const size_t n = 2 * 16 * 4 * 64;
+    auto q = uniform(n, 5, 1), k = uniform(n, 5, 2), v = uniform(n, 5, 3);
+    std::vector<float> out(n);
+    const TensorShape ok = shape4(2, 16, 4, 64);
+    EXPECT_THROWS_ANY(fa.forward(shape4(2, 16, 4, 74), q.data(), ok, k.data(), ok, v.data(), ok, out.data()));
+    EXPECT_THROWS_ANY(fa.forward(shape4(3, 16, 4, 64), q.data(), ok, k.data(), ok, v.data(), ok, out.data()));
+    EXPECT_THROWS_ANY(fa.forward(ok, nullptr, ok, k.data(), ok, v.data(), ok, out.data()));
+    EXPECT(fa.validate_inputs(shape4(2, 16, 4, 74), ok, ok, ok, p) == AttentionError::INVALID_INPUT);
+    EXPECT(fa.validate_inputs(ok, ok, ok, ok, p) == AttentionError::SUCCESS);
+    EXPECT_THROWS_ANY(fa.safe_forward(ok, q.data(), ok, k.data(), shape4(2, 16, 5, 64), v.data(), ok, out.data()));
+}
+
+CASE(Flash_DifferentBlockSizes, true) {  // :360-402: result must not depend on the block sizes
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    FlashAttentionConfig c;
+    c.block_size_q = 32;
+    c.block_size_k = 32;
+    fa.configure(p);
+    fa.configure_flash_attention(c);
+    EXPECT(run_flash_and_compare(fa, p, 6) <= 1e-4f);
+}
+
+CASE(Flash_BackwardIsUnsupported, true) {  // :405-480 only checks "non-zero"; this backend has no backward
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    fa.configure(p);
+    const TensorShape s = shape4(2, 16, 4, 64);
+    std::vector<float> x(2 * 16 * 4 * 64, 0.1f);
+    EXPECT_THROWS(fa.backward(s, x.data(), s, x.data(), s, x.data(), s, x.data(), s, x.data(), s, x.data(), s, x.data()),
+                  AttentionError::UNSUPPORTED_OPERATION);
+}
+
+CASE(Flash_AttentionMask, true) {  // :483-582: mask [B,N,N] float, 0 = masked
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    fa.configure(p);
+    const size_t B = 2, N = 16, H = 4, d = 64, n = B * N * H * d;
+    auto q = uniform(n, 7, 1), k = uniform(n, 7, 2), v = uniform(n, 7, 3);
+    std::vector<float> mask(B * N * N, 1.0f);
+    for (size_t b = 0; b < B; ++b)
+        for (size_t i = 0; i < N; ++i)
+            for (size_t j = 0; j < N; ++j)
+                if ((i + 2 * j + b) % 3 == 0) mask[(b * N + i) * N + j] = 0.0f;
+    std::vector<float> out(n);
+    const TensorShape s = shape4(B, N, H, d);
+    fa.forward(s, q.data(), s, k.data(), s, v.data(), s, out.data(), mask.data());
+    EXPECT(max_abs_diff(out, oracle_bnhd(q, k, v, B, N, H, d, p.scale_factor, false, mask.data())) <= 1e-4f);
+}
+
+CASE(Flash_SingleToken, true) {  // :585-599: N = 1 => output = value
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    p.sequence_length = 1;
+    fa.configure(p);
+    const size_t n = 2 * 1 * 4 * 64;
+    auto q = uniform(n, 8, 1), k = uniform(n, 8, 2), v = uniform(n, 8, 3);
+    std::vector<float> out(n);
+    const TensorShape s = shape4(2, 1, 4, 64);
+    fa.forward(s, q.data(), s, k.data(), s, v.data(), s, out.data());
+    EXPECT(max_abs_diff(out, v) <= 1e-6f);
+}
+
+CASE(Flash_LayoutSwitchAndScaleOverride, true) {
+    // tensors indexed [B,H,N,d] as the reference oracle does (tests/test_flash_attention.cpp:46);
+    // FlashAttentionConfig::softmax_scale overrides AttentionParams::scale_factor
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    p.causal_mask = true;
+    fa.configure(p);
+    FlashAttentionConfig c;
+    c.tensor_layout_bhnd = true;
+    c.softmax_scale = 0.2f;
+    fa.configure_flash_attention(c);
+    const size_t B = 2, N = 16, H = 4, d = 64, n = B * N * H * d;
+    auto q = uniform(n, 9, 1), k = uniform(n, 9, 2), v = uniform(n, 9, 3);
+    std::vector<float> out(n), want(n);
+    const TensorShape s = shape4(B, N, H, d);
+    fa.forward(s, q.data(), s, k.data(), s, v.data(), s, out.data());
+    ahpc_oracle_attention(q.data(), k.data(), v.data(), want.data(), B, N, H, d, H * N * d, d, N * d, 0.2f, 1, nullptr, 1);
+    EXPECT(max_abs_diff(out, want) <= 1e-4f);
+}
+
+template <typename T> static std::vector<T> to_storage(const std::vector<float>& x) {
+    std::vector<T> y(x.size());
+    for (size_t i = 0; i < x.size(); ++i) y[i] = T(x[i]);
+    return y;
+}
+template <typename T> static std::vector<float> from_storage(const std::vector<T>& x) {
+    std::vector<float> y(x.size());
+    for (size_t i = 0; i < x.size(); ++i) y[i] = (float)x[i];
+    return y;
+}
+
+template <typename T> static void flash_16bit(size_t d, bool causal) {
+    FlashAttention fa;
+    AttentionParams p{};
+    p.batch_size = 2; p.sequence_length = 200; p.num_heads = 3; p.head_dimension = d; p.causal_mask = causal;
+    fa.configure(p);
+    const size_t n = 2 * 200 * 3 * d;
+    auto qs = to_storage<T>(normal(n, 11, 1)), ks = to_storage<T>(normal(n, 11, 2)), vs = to_storage<T>(normal(n, 11, 3));
+    std::vector<T> out(n);
+    const TensorShape s = shape4(2, 200, 3, d, DataTypeOf<T>::value);
+    fa.forward(s, qs.data(), s, ks.data(), s, vs.data(), s, out.data());
+    auto want = oracle_bnhd(from_storage(qs), from_storage(ks), from_storage(vs), 2, 200, 3, d, 1.0f / std::sqrt((float)d), causal);
+    EXPECT(max_abs_diff(from_storage(out), want) <= 2e-2f);
+}
+CASE(Flash_HalfAndBfloat16HostTensors, true) {
+    flash_16bit<half>(64, true);
+    flash_16bit<half>(128, false);
+    flash_16bit<bfloat16>(128, true);
+    flash_16bit<bfloat16>(64, false);
+}
+
+CASE(Flash_VarlenPackedBatch, true) {
+    FlashAttention fa;
+    AttentionParams p{};
+    p.batch_size = 4; p.sequence_length = 70; p.num_heads = 2; p.head_dimension = 64; p.causal_mask = true;
+    fa.configure(p);
+    const int32_t cu[5] = {0, 7, 77, 78, 130};
+    const size_t T = 130, H = 2, d = 64, n = T * H * d;
+    auto qs = to_storage<half>(normal(n, 12, 1, 0.5f)), ks = to_storage<half>(normal(n, 12, 2, 0.5f)), vs = to_storage<half>(normal(n, 12, 3, 0.5f));
+    std::vector<half> out(n);
+    fa.forward_varlen(TensorShape({T, H, d}, DataType::FLOAT16), qs.data(), ks.data(), vs.data(), out.data(), cu, 4);
+    std::vector<float> want(n);
+    auto qf = from_storage(qs), kf = from_storage(ks), vf = from_storage(vs);
+    ahpc_oracle_attention_varlen(qf.data(), kf.data(), vf.data(), want.data(), cu, 4, H, d, 0.125f, 1, 2);
+    EXPECT(max_abs_diff(from_storage(out), want) <= 2e-2f);
+    const int32_t bad[5] = {0, 7, 5, 78, 130};
+    EXPECT_THROWS(fa.forward_varlen(TensorShape({T, H, d}, DataType::FLOAT16), qs.data(), ks.data(), vs.data(), out.data(), bad, 4),
+                  AttentionError::INVALID_INPUT);
+}
+
+CASE(Flash_ProfilingResults, true) {  // enable_profiling / get_profiling_results / reset_profiling
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    fa.configure(p);
+    fa.enable_profiling(true);
+    run_flash_and_compare(fa, p, 13);
+    auto r = fa.get_profiling_results();
+    EXPECT(!r.empty() && r[0].first == "forward_pass" && r[0].second > 0.0);
+    fa.reset_profiling();
+    EXPECT(fa.get_profiling_results().empty());
+    fa.enable_profiling(false);
+    run_flash_and_compare(fa, p, 13);
+    EXPECT(fa.get_profiling_results().empty());
+}
+
+// ---- configuration errors (no device work) ------------------------------------------------------------
+CASE(Flash_UnconfiguredAndBadParameters, false) {  // src/algorithms/flash_attention.cpp:37-41, :74-77
+    FlashAttention fa;
+    const TensorShape s = shape4(2, 16, 4, 64);
+    std::vector<float> x(2 * 16 * 4 * 64);
+    EXPECT_THROWS(fa.forward(s, x.data(), s, x.data(), s, x.data(), s, x.data()), AttentionError::INVALID_PARAMETERS);
+    AttentionParams p = fixture_params();
+    p.num_heads = 0;
+    EXPECT_THROWS(fa.configure(p), AttentionError::INVALID_PARAMETERS);
+    p = fixture_params();
+    p.key_value_heads = 2;
+    EXPECT_THROWS(fa.configure(p), AttentionError::UNSUPPORTED_OPERATION);
+    EXPECT(fa.get_backend_name() == "HIP_FlashAttention");
+    EXPECT(fa.get_version() == "1.0.0");
+    EXPECT(fa.supports_data_type(DataType::FLOAT32) && fa.supports_data_type(DataType::BFLOAT16));
+    EXPECT(fa.supports_memory_layout(MemoryLayout::ROW_MAJOR) && !fa.supports_memory_layout(MemoryLayout::COLUMN_MAJOR));
+    PagedAttention pa;
+    EXPECT_THROWS(pa.create_sequence(16), AttentionError::INVALID_PARAMETERS);
+    EXPECT(pa.get_backend_name() == "HIP_PagedAttention");
+}
+
+CASE(Types_HalfAndBfloat16MatchOracleBitForBit, false) {
+    for (uint32_t i = 0; i < 65536; ++i) {
+        half h;
+        h.data = (uint16_t)i;
+        const float f = (float)h, g = ahpc_oracle_f16_to_f32((uint16_t)i);
+        EXPECT(std::memcmp(&f, &g, 4) == 0 || (std::isnan(f) && std::isnan(g)));
+        bfloat16 b;
+        b.data = (uint16_t)i;
+        const float fb = (float)b, gb = ahpc_oracle_bf16_to_f32((uint16_t)i);
+        EXPECT(std::memcmp(&fb, &gb, 4) == 0 || (std::isnan(fb) && std::isnan(gb)));
+        if (g_failures) return;
+    }
+    uint64_t z = 88172645463325252ull;
+    for (int i = 0; i < 400000; ++i) {
+        z ^= z << 13; z ^= z >> 7; z ^= z << 17;
+        uint32_t u = (uint32_t)z;
+        float f;
+        std::memcpy(&f, &u, 4);
+        EXPECT(half(f).data == ahpc_oracle_f32_to_f16(f) || std::isnan(f));
+        EXPECT(bfloat16(f).data == ahpc_oracle_f32_to_bf16(f) || std::isnan(f));
+        if (g_failures) return;
+    }
+    EXPECT(half(65520.0f).data == 0x7C00 && half(65519.0f).data == 0x7BFF && half(1e-8f).data == 0);
+    EXPECT(bfloat16(1.00390625f).data == 0x3F80 && bfloat16(1.01171875f).data == 0x3F82);  // ties to even
+}
+
+CASE(Merge_OnlineSoftmaxStateMatchesOracle, false) {  // src/algorithms/flash_attention.hpp:39-62
+    OnlineSoftmaxState s;
+    float m = -INFINITY, l = 0.0f;
+    const float ms[5] = {0.3f, 2.0f, -1.0f, 2.0f, 5.5f}, ls[5] = {1.5f, 0.2f, 7.0f, 1.0f, 0.01f};
+    for (int i = 0; i < 5; ++i) {
+        s.update(ms[i], ls[i]);
+        ahpc_oracle_softmax_merge(&m, &l, ms[i], ls[i]);
+        EXPECT(s.max_val == m && s.sum_exp == l);
+    }
+    EXPECT(OnlineSoftmaxState{}.get_normalizer() == 0.0f);
+}
+
+// ---- tests/test_backends.cpp --------------------------------------------------------------------------------
+CASE(Factory_NamesAndStrings, false) {
+    EXPECT(BackendFactory::backendTypeToString(BackendType::HIP) == "HIP");
+    EXPECT(BackendFactory::backendTypeToString(BackendType::CPU) == "CPU");
+    EXPECT(BackendFactory::stringToBackendType("hip") == BackendType::HIP);
+    EXPECT(BackendFactory::stringToBackendType("CUDA") == BackendType::CUDA);
+    bool threw = false;
+    try { BackendFactory::stringToBackendType("metal"); } catch (const std::invalid_argument&) { threw = true; }
+    EXPECT(threw);
+    EXPECT((int)BackendType::AUTO == 5 && (int)BackendType::HIP == 6);  // the reference's values are unchanged
+    EXPECT(!BackendFactory::isBackendAvailable(BackendType::CUDA));
+    EXPECT_THROWS(BackendFactory::createFlashAttention(BackendType::VULKAN), AttentionError::BACKEND_NOT_AVAILABLE);
+    try {
+        BackendFactory::createBackend(BackendType::OPENCL);
+        EXPECT(false);
+    } catch (const BackendException& e) {
+        EXPECT(e.backend_type() == BackendType::OPENCL);
+        EXPECT(std::string(e.what()).find("OpenCL") != std::string::npos);
+    }
+    BackendFactory::enableDebugMode(true);
+    EXPECT(BackendFactory::isDebugModeEnabled());
+    BackendFactory::enableDebugMode(false);
+    EXPECT(!BackendFactory::getSystemInfo().empty());
+}
+
+// A plug-in CPU backend made of the oracle: exercises registerBackend, and is the second backend of the
+// cross-backend consistency case.  It lives in the test, not in the library.
+class OracleCpuAttention : public AttentionInterface {
+public:
+    void configure(const AttentionParams& p, const PerformanceConfig& c = PerformanceConfig{}) override { current_params_ = p; current_perf_config_ = c; ok_ = true; }
+    void forward(const TensorShape& qs, const void* q, const TensorShape&, const void* k, const TensorShape&, const void* v,
+                 const TensorShape&, void* o, const void* mask = nullptr) override {
+        if (!ok_) throw AttentionException(AttentionError::INVALID_PARAMETERS, "not configured");
+        if (!q || !k || !v || !o) throw AttentionException(AttentionError::INVALID_INPUT, "null");
+        const size_t B = qs.dimensions[0], N = qs.dimensions[1], H = qs.dimensions[2], d = qs.dimensions[3];
+        const float scale = current_params_.scale_factor > 0 ? current_params_.scale_factor : 1.0f / std::sqrt((float)d);
+        ahpc_oracle_attention((const float*)q, (const float*)k, (const float*)v, (float*)o, B, N, H, d, N * H * d, H * d, d, scale,
+                              current_params_.causal_mask, (const float*)mask, 2);
+    }
+    void backward(const TensorShape&, const void*, const TensorShape&, const void*, const TensorShape&, const void*, const TensorShape&,
+                  const void*, const TensorShape&, void*, const TensorShape&, void*, const TensorShape&, void*, const void* = nullptr) override {
+        throw AttentionException(AttentionError::UNSUPPORTED_OPERATION, "no backward");
+    }
+    size_t get_workspace_size(const AttentionParams&) const override { return 0; }
+    void set_workspace(void*, size_t) override {}
+    bool supports_data_type(DataType t) const override { return t == DataType::FLOAT32; }
+    bool supports_memory_layout(MemoryLayout l) const override { return l == MemoryLayout::ROW_MAJOR; }
+    std::string get_backend_name() const override { return "CPU_OracleAttention"; }
+    std::string get_version() const override { return "test"; }
+    void enable_profiling(bool) override {}
+    std::vector<std::pair<std::string, double>> get_profiling_results() const override { return {}; }
+    void reset_profiling() override {}
+    AttentionError validate_inputs(const TensorShape&, const TensorShape&, const TensorShape&, const TensorShape&, const AttentionParams&) const override { return AttentionError::SUCCESS; }
+
+private:
+    bool ok_ = false;
+};
+
+CASE(Factory_PluginRegistration, false) {  // registerBackend / unregisterBackend, src/api/backend_factory.hpp:68-71
+    EXPECT(!BackendFactory::isBackendAvailable(BackendType::CPU));
+    BackendFactory::registerBackend(BackendType::CPU, "CPU", [] { return std::unique_ptr<AttentionInterface>(new OracleCpuAttention()); });
+    EXPECT(BackendFactory::isBackendAvailable(BackendType::CPU));
+    auto cpu = BackendFactory::createFlashAttention(BackendType::CPU);
+    EXPECT(cpu && cpu->get_backend_name().find(BackendFactory::backendTypeToString(BackendType::CPU)) == 0);
+    EXPECT_THROWS(BackendFactory::createPagedAttention(BackendType::CPU), AttentionError::BACKEND_NOT_AVAILABLE);
+    EXPECT(BackendFactory::selectBestBackend(std::vector<BackendType>{BackendType::CUDA, BackendType::CPU}) == BackendType::CPU);
+    BackendFactory::unregisterBackend(BackendType::CPU);
+    EXPECT(!BackendFactory::isBackendAvailable(BackendType::CPU));
+    EXPECT_THROWS(BackendFactory::createFlashAttention(BackendType::CPU), AttentionError::BACKEND_NOT_AVAILABLE);
+}
+
+CASE(Backends_AvailabilityAndCapability, true) {  // tests/test_backends.cpp:110-180
+    auto avail = BackendFactory::getAvailableBackends();
+    EXPECT(std::find(avail.begin(), avail.end(), BackendType::HIP) != avail.end());
+    const BackendCapability cap = BackendFactory::getBackendCapability(BackendType::HIP);
+    EXPECT(cap.available && !cap.version.empty() && !cap.device_name.empty());
+    EXPECT(!cap.supported_data_types.empty() && !cap.supported_layouts.empty());
+    EXPECT(cap.memory_size > (size_t)16 << 30 && cap.supports_tensor_cores);
+    EXPECT(cap.compute_capability_major == 9 && cap.compute_capability_minor == 50);
+    EXPECT(BackendFactory::selectBestBackend() == BackendType::HIP);
+    EXPECT(BackendFactory::isBackendAvailable(BackendType::AUTO));
+    AttentionParams p = fixture_params();
+    EXPECT(BackendFactory::validateBackendCompatibility(BackendType::HIP, p));
+    p.head_dimension = 1024;
+    EXPECT(!BackendFactory::validateBackendCompatibility(BackendType::HIP, p));
+}
+
+CASE(Backends_CreationAndConfiguration, true) {  // tests/test_backends.cpp:183-247
+    for (BackendType t : BackendFactory::getAvailableBackends()) {
+        auto fa = BackendFactory::createFlashAttention(t);
+        EXPECT(fa != nullptr);
+        EXPECT(fa->get_backend_name().find(BackendFactory::backendTypeToString(t)) == 0);
+        EXPECT(!fa->get_version().empty());
+        EXPECT(fa->supports_data_type(DataType::FLOAT32));
+        EXPECT(fa->supports_memory_layout(MemoryLayout::ROW_MAJOR));
+        auto pa = BackendFactory::createPagedAttention(t);
+        EXPECT(pa != nullptr && dynamic_cast<PagedAttention*>(pa.get()) != nullptr);
+        AttentionParams p = fixture_params();
+        fa->configure(p);
+        (void)fa->get_workspace_size(p);
+        fa->enable_profiling(true);
+        fa->enable_profiling(false);
+        const TensorShape s = shape4(2, 16, 4, 64);
+        EXPECT(fa->validate_inputs(s, s, s, s, p) == AttentionError::SUCCESS);
+    }
+    auto any = BackendFactory::createFlashAttention(BackendType::AUTO);  // README.md:150 of the reference
+    EXPECT(any && any->get_backend_name() == "HIP_FlashAttention");
+}
+
+CASE(Backends_CrossBackendConsistency, true) {  // tests/test_backends.cpp:252-324, tolerance 1e-3
+    BackendFactory::registerBackend(BackendType::CPU, "CPU", [] { return std::unique_ptr<AttentionInterface>(new OracleCpuAttention()); });
+    AttentionParams p = fixture_params();
+    p.sequence_length = 64;
+    const size_t n = 2 * 64 * 4 * 64;
+    auto q = uniform(n, 21, 1), k = uniform(n, 21, 2), v = uniform(n, 21, 3);
+    const TensorShape s = shape4(2, 64, 4, 64);
+    std::vector<std::vector<float>> outs;
+    for (BackendType t : BackendFactory::getAvailableBackends()) {
+        auto a = BackendFactory::createFlashAttention(t);
+        a->configure(p);
+        outs.emplace_back(n, 0.0f);
+        a->forward(s, q.data(), s, k.data(), s, v.data(), s, outs.back().data());
+    }
+    EXPECT(outs.size() >= 2);
+    for (size_t i = 1; i < outs.size(); ++i) EXPECT(max_abs_diff(outs[0], outs[i]) <= 1e-3f);
+    BackendFactory::unregisterBackend(BackendType::CPU);
+}
+
+CASE(Backends_ConcurrentInstancesAndLifecycles, true) {  // tests/test_backends.cpp:351-449
+    std::vector<std::thread> th;
+    std::vector<float> errs(4, 1.0f);
+    for (int i = 0; i < 4; ++i)
+        th.emplace_back([i, &errs] {
+            auto a = BackendFactory::createFlashAttention(BackendType::HIP);
+            AttentionParams p = fixture_params();
+            a->configure(p);
+            errs[i] = run_flash_and_compare(*static_cast<FlashAttention*>(a.get()), p, 30 + i);
+        });
+    for (auto& t : th) t.join();
+    for (float e : errs) EXPECT(e <= 1e-4f);
+    for (int cycle = 0; cycle < 3; ++cycle) {
+        auto a1 = BackendFactory::createFlashAttention(BackendType::HIP);
+        auto a2 = BackendFactory::createPagedAttention(BackendType::HIP);
+        AttentionParams p = fixture_params();
+        a1->configure(p);
+        a2->configure(p);
+    }
+}
+
+CASE(Backends_LargeInput, true) {  // tests/test_backends.cpp:474-516: B=8, N=256, H=8
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    p.batch_size = 8; p.sequence_length = 256; p.num_heads = 8;
+    fa.configure(p);
+    EXPECT(run_flash_and_compare(fa, p, 40) <= 1e-4f);
+}
+
+CASE(Backends_ErrorHandling, true) {  // tests/test_backends.cpp:631-680
+    auto a = BackendFactory::createFlashAttention(BackendType::HIP);
+    const TensorShape s = shape4(2, 16, 4, 64);
+    std::vector<float> x(2 * 16 * 4 * 64, 0.5f), o(x.size());
+    EXPECT_THROWS_ANY(a->forward(s, x.data(), s, x.data(), s, x.data(), s, o.data()));  // unconfigured
+    a->configure(fixture_params());
+    EXPECT_THROWS_ANY(a->forward(s, nullptr, s, x.data(), s, x.data(), s, o.data()));
+    EXPECT_THROWS_ANY(a->forward(shape4(2, 16, 4, 32), x.data(), s, x.data(), s, x.data(), s, o.data()));
+    TensorShape col = s;
+    col.layout = MemoryLayout::COLUMN_MAJOR;
+    EXPECT_THROWS(a->forward(col, x.data(), s, x.data(), s, x.data(), s, o.data()), AttentionError::UNSUPPORTED_OPERATION);
+}
+
+// ---- paged attention ------------------------------------------------------------------------------------------
+CASE(Paged_BasicUsageFlow, true) {  // examples/basic_usage.cpp:115-200
+    AttentionParams p{};
+    p.batch_size = 1; p.sequence_length = 1; p.num_heads = 4; p.head_dimension = 32; p.max_sequence_length = 128;
+    auto base = BackendFactory::createPagedAttention(BackendType::HIP);
+    auto* pa = dynamic_cast<PagedAttention*>(base.get());
+    EXPECT(pa != nullptr);
+    pa->configure(p);
+    const size_t id = pa->create_sequence(p.max_sequence_length);
+    EXPECT(id == 1);  // ids start at 1, src/algorithms/paged_attention.cpp:67, :336
+    const size_t L = 32, H = 4, d = 32;
+    auto k = uniform(L * H * d, 50, 2), v = uniform(L * H * d, 50, 3), q = uniform(H * d, 50, 1);
+    pa->append_kv_cache(id, k.data(), v.data(), L, DataType::FLOAT32);
+    EXPECT(pa->get_sequence_length(id) == L && pa->is_sequence_active(id));
+    std::vector<float> out(H * d, -1.0f);
+    const TensorShape qs = shape4(1, 1, H, d);
+    pa->forward_batch({id}, {qs}, {q.data()}, {qs}, {out.data()});
+    // expected: dense attention of the last row with the query at position L-1 == decode over all L keys
+    std::vector<float> want(H * d);
+    const int32_t table[2] = {0, 1};
+    const int32_t len = (int32_t)L;
+    ahpc_oracle_paged_decode(q.data(), want.data(), k.data(), v.data(), table, &len, nullptr, 1, H, d, 16, 2, 1.0f / std::sqrt((float)d), 1);
+    EXPECT(max_abs_diff(out, want) <= 1e-4f);
+    pa->destroy_sequence(id);
+    EXPECT(!pa->is_sequence_active(id) && pa->get_active_sequences_count() == 0);
+    pa->destroy_sequence(id);  // unknown ids are ignored
+}
+
+CASE(Paged_PoolOrderMatchesFifoModel, true) {  // src/algorithms/paged_attention.cpp:11-64
+    PagedAttention pa;
+    AttentionParams p{};
+    p.batch_size = 4; p.sequence_length = 1; p.num_heads = 2; p.head_dimension = 32; p.page_size = 4;
+    PagedAttentionConfig c;
+    c.initial_page_pool_size = 6;
+    c.page_pool_growth = 3;
+    pa.configure_paged_attention(c);
+    pa.configure(p);
+    ahpc_oracle_pool* model = ahpc_oracle_pool_create(6, 3);
+    const size_t H = 2, d = 32;
+    auto tok = [&](size_t n, uint64_t seed) { return uniform(n * H * d, seed, 2); };
+    std::vector<std::vector<int32_t>> want(3);
+    const size_t a = pa.create_sequence(64), b = pa.create_sequence(64), c3 = pa.create_sequence(64);
+    auto append = [&](size_t id, int slot, size_t have, size_t n) {
+        auto x = tok(n, id * 100 + have);
+        pa.append_kv_cache(id, x.data(), x.data(), n, DataType::FLOAT32);
+        for (size_t pg = (have + 3) / 4; pg < (have + n + 3) / 4; ++pg) want[slot].push_back(ahpc_oracle_pool_allocate(model));
+    };
+    append(a, 0, 0, 9);    // 3 pages
+    append(b, 1, 0, 4);    // 1 page
+    append(a, 0, 9, 3);    // fills page 3, no new page
+    append(c3, 2, 0, 10);  // 3 pages: pool (6) exhausted after 2 -> grows by 3
+    EXPECT(pa.get_sequence_pages(a) == want[0] && pa.get_sequence_pages(b) == want[1] && pa.get_sequence_pages(c3) == want[2]);
+    pa.truncate_sequence(a, 5);  // keeps 2 pages, frees the third
+    ahpc_oracle_pool_release(model, want[0].back());
+    want[0].pop_back();
+    pa.destroy_sequence(b);
+    ahpc_oracle_pool_release(model, want[1][0]);
+    append(c3, 2, 10, 9);  // 2 more pages: recycled FIFO
+    EXPECT(pa.get_sequence_pages(a) == want[0] && pa.get_sequence_pages(c3) == want[2]);
+    const KVBlockPoolStats st = pa.get_pool_stats();
+    EXPECT((int32_t)st.total_pages == ahpc_oracle_pool_total(model) && (int32_t)st.free_pages == ahpc_oracle_pool_free_count(model));
+    EXPECT(pa.get_total_memory_usage() == st.allocated_pages * st.page_bytes && pa.get_peak_memory_usage() >= pa.get_total_memory_usage());
+    EXPECT(pa.get_sequence_length(a) == 5 && pa.get_max_sequence_length(a) == 5);
+    ahpc_oracle_pool_destroy(model);
+}
+
+CASE(Paged_AppendThenGetRoundTrip, true) {
+    PagedAttention pa;
+    AttentionParams p{};
+    p.batch_size = 1; p.sequence_length = 1; p.num_heads = 4; p.head_dimension = 64;
+    pa.configure(p);
+    const size_t H = 4, d = 64, id = pa.create_sequence(256);
+    auto k1 = normal(21 * H * d, 60, 2), v1 = normal(21 * H * d, 60, 3), k2 = normal(40 * H * d, 61, 2), v2 = normal(40 * H * d, 61, 3);
+    pa.append_kv_cache(id, k1.data(), v1.data(), 21, DataType::FLOAT32);
+    pa.append_kv_cache(id, k2.data(), v2.data(), 40, DataType::FLOAT32);
+    std::vector<float> kg(61 * H * d), vg(61 * H * d);
+    pa.get_kv_cache(id, kg.data(), vg.data(), 0, 61, DataType::FLOAT32);
+    std::vector<float> kall = k1, vall = v1;
+    kall.insert(kall.end(), k2.begin(), k2.end());
+    vall.insert(vall.end(), v2.begin(), v2.end());
+    EXPECT(kg == kall && vg == vall);  // bit exact
+    std::vector<float> part(5 * H * d), partv(5 * H * d);
+    pa.get_kv_cache(id, part.data(), partv.data(), 19, 5, DataType::FLOAT32);
+    EXPECT(std::equal(part.begin(), part.end(), kall.begin() + 19 * H * d));
+    EXPECT_THROWS(pa.get_kv_cache(id, part.data(), partv.data(), 60, 5, DataType::FLOAT32), AttentionError::INVALID_INPUT);
+    EXPECT_THROWS(pa.append_kv_cache(999, k1.data(), v1.data(), 1, DataType::FLOAT32), AttentionError::INVALID_INPUT);
+    pa.clear_kv_cache(id);
+    EXPECT(pa.get_sequence_length(id) == 0 && pa.get_sequence_pages(id).empty());
+}
+
+template <typename T> static void paged_batch(DataType dt, float tol) {
+    PagedAttention pa;
+    AttentionParams p{};
+    p.batch_size = 5; p.sequence_length = 1; p.num_heads = 8; p.head_dimension = 128; p.max_sequence_length = 2048;
+    PagedAttentionConfig c;
+    c.split_chunk_tokens = 128;  // several chunks per sequence: exercises the merge
+    pa.configure_paged_attention(c);
+    pa.configure(p);
+    const size_t H = 8, d = 128, P = 16;
+    const size_t lens[5] = {700, 33, 0, 1500, 16};
+    std::vector<size_t> ids;
+    std::vector<std::vector<float>> ks, vs;
+    for (int i = 0; i < 5; ++i) {
+        ids.push_back(pa.create_sequence(2048));
+        auto k = from_storage(to_storage<T>(normal(lens[i] * H * d, 70 + i, 2)));
+        auto v = from_storage(to_storage<T>(normal(lens[i] * H * d, 70 + i, 3)));
+        auto kt = to_storage<T>(k), vt = to_storage<T>(v);
+        // interleave appends so that the sequences' pages interleave in the pool
+        size_t done = 0;
+        while (done < lens[i]) {
+            const size_t n = std::min<size_t>(lens[i] - done, 300);
+            pa.append_kv_cache(ids[i], kt.data() + done * H * d, vt.data() + done * H * d, n, dt);
+            done += n;
+        }
+        ks.push_back(k);
+        vs.push_back(v);
+    }
+    // decode in a different order than creation
+    const int order[5] = {3, 0, 4, 2, 1};
+    std::vector<size_t> bid;
+    std::vector<TensorShape> shp(5, TensorShape({1, 1, H, d}, dt));
+    std::vector<std::vector<T>> q(5), out(5);
+    std::vector<const void*> qp;
+    std::vector<void*> op;
+    for (int j = 0; j < 5; ++j) {
+        bid.push_back(ids[order[j]]);
+        q[j] = to_storage<T>(normal(H * d, 80 + j, 1));
+        out[j].assign(H * d, T(7.0f));
+        qp.push_back(q[j].data());
+        op.push_back(out[j].data());
+    }
+    pa.forward_batch(bid, shp, qp, shp, op);
+    for (int j = 0; j < 5; ++j) {
+        const size_t L = lens[order[j]];
+        std::vector<float> want(H * d, 0.0f);
+        if (L) {
+            std::vector<int32_t> table((L + P - 1) / P);
+            for (size_t i = 0; i < table.size(); ++i) table[i] = (int32_t)i;
+            std::vector<float> kp(table.size() * P * H * d, 0.0f), vp(kp.size(), 0.0f);
+            std::copy(ks[order[j]].begin(), ks[order[j]].end(), kp.begin());
+            std::copy(vs[order[j]].begin(), vs[order[j]].end(), vp.begin());
+            const int32_t len = (int32_t)L;
+            auto qf = from_storage(q[j]);
+            ahpc_oracle_paged_decode(qf.data(), want.data(), kp.data(), vp.data(), table.data(), &len, nullptr, 1, H, d, P, table.size(),
+                                     1.0f / std::sqrt((float)d), 2);
+        }
+        EXPECT(max_abs_diff(from_storage(out[j]), want) <= tol);
+    }
+    // vector size mismatch -> INVALID_INPUT (src/algorithms/paged_attention.cpp:511-516)
+    std::vector<const void*> short_q(qp.begin(), qp.begin() + 4);
+    EXPECT_THROWS(pa.forward_batch(bid, shp, short_q, shp, op), AttentionError::INVALID_INPUT);
+    EXPECT_THROWS(pa.forward_batch({12345}, {shp[0]}, {qp[0]}, {shp[0]}, {op[0]}), AttentionError::INVALID_INPUT);
+    EXPECT(pa.get_active_sequences_count() == 5);
+}
+CASE(Paged_ForwardBatchAgainstOracle, true) {
+    paged_batch<float>(DataType::FLOAT32, 1e-4f);
+    paged_batch<half>(DataType::FLOAT16, 2e-2f);
+    paged_batch<bfloat16>(DataType::BFLOAT16, 2e-2f);
+}
+
+CASE(Paged_ConvenienceForward, true) {  // src/algorithms/paged_attention.cpp:132-174
+    PagedAttention pa;
+    AttentionParams p{};
+    p.batch_size = 3; p.sequence_length = 50; p.num_heads = 4; p.head_dimension = 64;
+    pa.configure(p);
+    const size_t B = 3, N = 50, H = 4, d = 64;
+    auto q = normal(B * H * d, 90, 1), k = normal(B * N * H * d, 90, 2), v = normal(B * N * H * d, 90, 3);
+    std::vector<float> out(B * H * d);
+    pa.forward(shape4(B, 1, H, d), q.data(), shape4(B, N, H, d), k.data(), shape4(B, N, H, d), v.data(), shape4(B, 1, H, d), out.data());
+    // == last row of causal dense attention whose last query is q
+    for (size_t b = 0; b < B; ++b) {
+        std::vector<float> qq(N * H * d, 0.0f), want(N * H * d);
+        std::copy(q.begin() + b * H * d, q.begin() + (b + 1) * H * d, qq.begin() + (N - 1) * H * d);
+        ahpc_oracle_attention(qq.data(), k.data() + b * N * H * d, v.data() + b * N * H * d, want.data(), 1, N, H, d, N * H * d, H * d, d, 0.125f, 1, nullptr, 1);
+        float e = 0.0f;
+        for (size_t i = 0; i < H * d; ++i) e = std::max(e, std::fabs(out[b * H * d + i] - want[(N - 1) * H * d + i]));
+        EXPECT(e <= 1e-4f);
+    }
+    EXPECT(pa.get_active_sequences_count() == 0 && pa.get_total_memory_usage() == 0);
+    EXPECT_THROWS(pa.forward(shape4(B, N, H, d), k.data(), shape4(B, N, H, d), k.data(), shape4(B, N, H, d), v.data(), shape4(B, N, H, d), k.data()),
+                  AttentionError::UNSUPPORTED_OPERATION);
+}
+
+CASE(Paged_SequenceLifecycle, true) {  // extend / truncate / reset, src/algorithms/paged_attention.cpp:352-418
+    PagedAttention pa;
+    AttentionParams p{};
+    p.batch_size = 1; p.sequence_length = 1; p.num_heads = 2; p.head_dimension = 32;
+    pa.configure(p);
+    const size_t id = pa.create_sequence(20);
+    auto x = normal(20 * 2 * 32, 95, 2);
+    pa.append_kv_cache(id, x.data(), x.data(), 20, DataType::FLOAT32);
+    EXPECT(pa.get_sequence_pages(id).size() == 2 && pa.get_max_sequence_length(id) == 20);
+    pa.extend_sequence(id, 30);  // limit 50 -> 4 pages pre-allocated
+    EXPECT(pa.get_max_sequence_length(id) == 50 && pa.get_sequence_pages(id).size() == 4);
+    pa.truncate_sequence(id, 17);
+    EXPECT(pa.get_sequence_length(id) == 17 && pa.get_sequence_pages(id).size() == 2);
+    pa.reset_sequence(id);
+    EXPECT(pa.get_sequence_length(id) == 0 && pa.is_sequence_active(id) && pa.get_sequence_pages(id).empty());
+    // 40 sequences: more than the default 32 table rows
+    std::vector<size_t> ids;
+    for (int i = 0; i < 40; ++i) ids.push_back(pa.create_sequence(16));
+    EXPECT(pa.get_active_sequences_count() == 41);
+    for (size_t s : ids) pa.append_kv_cache(s, x.data(), x.data(), 3, DataType::FLOAT32);
+    std::vector<float> out(2 * 32), q = normal(2 * 32, 96, 1);
+    const TensorShape qs = shape4(1, 1, 2, 32);
+    pa.forward_batch({ids[39]}, {qs}, {q.data()}, {qs}, {out.data()});
+    EXPECT(std::isfinite(out[0]));
+}
+
+// ---- main ------------------------------------------------------------------------------------------------------
+int main(int argc, char** argv) {
+    bool no_gpu = false;
+    std::string filter;
+    for (int i = 1; i < argc; ++i) {
+        if (std::string(argv[i]) == "--no-gpu") no_gpu = true;
+        else filter = argv[i];
+    }
+    int ran = 0, failed = 0;
+    for (const Case& c : cases()) {
+        if (no_gpu && c.needs_gpu) continue;
+        if (!filter.empty() && std::string(c.name).find(filter) == std::string::npos) continue;
+        std::printf("[ RUN  ] %s\n", c.name);
+        std::fflush(stdout);
+        const int before = g_failures;
+        try {
+            c.fn();
+        } catch (const std::exception& e) {
+            std::printf("    unexpected exception: %s\n", e.what());
+            ++g_failures;
+        }
+        ++ran;
+        if (g_failures != before) {
+            ++failed;
+            std::printf("[ FAIL ] %s\n", c.name);
+        } else {
+            std::printf("[  OK  ] %s\n", c.name);
+        }
+        std::fflush(stdout);
+    }
+    std::printf("%d cases run, %d failed\n", ran, failed);
+    return failed == 0 ? 0 : 1;
+}

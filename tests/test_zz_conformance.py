@@ -1,0 +1,27 @@
+"""Runs the C++ conformance binary (tests/cpp/conformance.cpp): the reference's own gtest cases and
+decode example re-expressed against the C++ host classes, with the oracle as expected value."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "attention_amd", "lib", "ahpc_conformance")
+
+
+def run(args):
+    assert os.path.exists(BIN), f"{BIN} missing: run __graft_entry__.build()"
+    r = subprocess.run([BIN] + args, capture_output=True, text=True, timeout=600)
+    print(r.stdout[-6000:])
+    print(r.stderr[-2000:])
+    assert r.returncode == 0, "conformance failures:\n" + "\n".join(
+        l for l in r.stdout.splitlines() if "FAIL" in l or "EXPECT" in l or "exception" in l)
+
+
+def test_host_cases_without_gpu():
+    run(["--no-gpu"])
+
+
+@pytest.mark.gpu
+def test_all_cases_on_gpu():
+    run([])
