@@ -145,36 +145,23 @@ static int dispatch_simple(int dtype, const SimpleParams& p, int64_t B, hipStrea
 }
 
 // ---------------------------------------------------------------------------------------------
-// Queries per wavefront of the MFMA kernel, in blocks of 32.  Read once from AHPC_FLASH_QB
-// (1 or 2) so that both tilings can be timed; 0 / unset picks the default.
-static int flash_qb_override() {
-    static const int v = [] {
-        const char* e = std::getenv("AHPC_FLASH_QB");
-        return e ? std::atoi(e) : 0;
-    }();
-    return v;
-}
-
-template <typename T, int D, int QB, bool VARLEN>
+template <typename T, int D, bool VARLEN>
 static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
-    constexpr int BM = 128 * QB;
-    p.n_qtiles = (p.N + BM - 1) / BM;
+    p.n_qtiles = (p.N + kFlashRows - 1) / kFlashRows;
     const int64_t total = B * p.H * (int64_t)p.n_qtiles;
     if (total > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
     p.total_blocks = (int32_t)total;
     p.blocks_per_xcd = (int32_t)((total + 7) / 8);
     dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
-    if (causal) hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, QB, true, VARLEN>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, QB, false, VARLEN>), grid, block, 0, stream, p);
+    if (causal) hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, true, VARLEN>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, false, VARLEN>), grid, block, 0, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 
 template <typename T, bool VARLEN>
 static int dispatch_mfma(const FlashParams& p, int64_t B, int d, bool causal, hipStream_t stream) {
-    int qb = flash_qb_override();
-    if (qb != 1 && qb != 2) qb = 1;
-    if (d == 128) return qb == 2 ? launch_mfma<T, 128, 2, VARLEN>(p, B, causal, stream) : launch_mfma<T, 128, 1, VARLEN>(p, B, causal, stream);
-    if (d == 64) return qb == 2 ? launch_mfma<T, 64, 2, VARLEN>(p, B, causal, stream) : launch_mfma<T, 64, 1, VARLEN>(p, B, causal, stream);
+    if (d == 128) return launch_mfma<T, 128, VARLEN>(p, B, causal, stream);
+    if (d == 64) return launch_mfma<T, 64, VARLEN>(p, B, causal, stream);
     return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
 }
 

@@ -1,23 +1,27 @@
 // FlashAttention forward on the gfx950 matrix cores (fp16 / bf16 storage, fp32 accumulate).
 //
-// One workgroup = 4 wavefronts = 128*QB query rows of one (sequence, head); it walks the keys in
-// tiles of 64.  Per tile and wavefront:
+// One workgroup = 4 wavefronts = 128 query rows of one (sequence, head); it walks the keys in tiles
+// of 64.  Two workgroups share a CU (<= 256 registers per lane, 2 x 64 KiB of LDS), so that one
+// wavefront's softmax (VALU) overlaps the other's matrix work on the same SIMD.  Per tile and wave:
 //   S^T = K * Q^T      v_mfma_f32_32x32x16: A = K rows from LDS, B = Q^T held in registers for the
 //                      whole kernel.  In the 32x32 result a lane owns ONE query column (lane%32)
 //                      and 16 of the 32 key rows, so the softmax row reductions are in-lane plus
-//                      one exchange with lane^32.
+//                      one exchange between the wave halves (v_permlane32_swap).
 //   P^T = exp2(c*S^T - c*m)   online softmax in registers (c = scale*log2 e), fp32.
-//   O^T += V^T * P^T   A = V^T rows from LDS, B = P^T straight from the registers S^T was in: the
+//   O^T += V^T * P^T   A = V^T from LDS, B = P^T straight from the registers S^T was in: the
 //                      accumulator layout of the first product is the B-operand layout of the
 //                      second once the 16 keys of a k-step are taken in the order
-//                      key = 8*(e/4) + 4*(lane/32) + e%4 (e = 0..7); V^T is written to LDS in that
-//                      same order, so no data moves between the two products.
+//                      key = 8*(e/4) + 4*(lane/32) + e%4 (e = 0..7).  V stays row-major [key][d] in
+//                      LDS; ds_read_b64_tr_b16 (the gfx950 transposing LDS read) hands each lane
+//                      4 keys of one d, and two such reads fetch exactly the 8 keys above.
 // O^T keeps the query in the lane column, so the per-row rescale factors are per-lane scalars.
 //
-// LDS: K tile [64][D] with rows padded by 16 B (bank-conflict-free 16-B row reads); V^T tile
-// [D][64] built by a 4x8 in-register transpose (v_perm_b32) of what each thread loaded, XOR-swizzled
-// in 16-B columns so that both the 8-B transpose writes and the 16-B operand reads are conflict free.
-// The next tile's global loads are issued before the current tile's math and parked in registers.
+// Tiles reach LDS without touching registers: global_load_lds_dwordx4 writes 1 KiB per wave
+// instruction (lane i -> LDS base + 16*i).  Which global 16-byte chunk a lane fetches is free, so the
+// XOR swizzle that makes the later operand reads bank-conflict free is applied on the global side:
+// physical chunk = chunk ^ f(row), with f chosen per tile kind (16-byte row reads for K, 8-byte
+// transposing reads for V).  LDS is double buffered: tile t+1 streams in while tile t is consumed;
+// one barrier per tile.
 #pragma once
 
 #include "ahpc_device.hpp"
@@ -40,29 +44,79 @@ struct FlashParams {
 };
 
 constexpr int kFlashThreads = 256;
-constexpr int kFlashKeys = 64;  // keys per tile
+constexpr int kFlashRows = 128;  // query rows per workgroup
+constexpr int kFlashKeys = 64;   // keys per tile
 
-template <int D> struct FlashLds {
-    static constexpr int kRowBytes = D * 2 + 16;
-    static constexpr int kBytesK = kFlashKeys * kRowBytes;
-    static constexpr int kBytesV = D * 128;
-    static constexpr int kBytes = kBytesK + kBytesV;
+#define AHPC_LDS __attribute__((address_space(3)))
+#define AHPC_GLOBAL __attribute__((address_space(1)))
+
+template <typename T> struct TrRead;
+template <> struct TrRead<bf16_t> {
+    typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 vec;
+    __device__ static u32x2 load(const unsigned char* p) {
+        return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((AHPC_LDS vec*)p));
+    }
+};
+template <> struct TrRead<f16_t> {
+    typedef __attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16 vec;
+    __device__ static u32x2 load(const unsigned char* p) {
+        return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((AHPC_LDS vec*)p));
+    }
 };
 
-template <typename T, int D, int QB, bool CAUSAL, bool VARLEN>
-__global__ __launch_bounds__(kFlashThreads) void flash_fwd_mfma_kernel(const FlashParams p) {
-    constexpr int BM = 128 * QB;       // query rows per workgroup
-    constexpr int CPR = D / 8;         // 16-byte chunks per row
-    constexpr int KS = D / 16;         // k-steps of the first product
-    constexpr int MB = D / 32;         // 32-row blocks of O^T
-    constexpr int KROWS = kFlashThreads / CPR;            // K rows covered by one pass of the block
-    constexpr int KPASS = kFlashKeys / KROWS;             // passes to cover 64 keys
-    constexpr int KROW = FlashLds<D>::kRowBytes;
-    constexpr int VTHREADS = 16 * CPR;                    // threads that carry a 4-key x 8-lane V patch
+// max / sum of x over the two lanes that share a query column (lane and lane ^ 32).
+// v_permlane32_swap(a, b) exchanges the upper 32 lanes of a with the lower 32 lanes of b; with
+// a = b = x the two results hold x's lower half and x's upper half in every lane.
+__device__ inline float halves_max(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
+    return fmaxf(as_f32(r[0]), as_f32(r[1]));
+}
+__device__ inline float halves_sum(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
+    return as_f32(r[0]) + as_f32(r[1]);
+}
 
-    __shared__ __attribute__((aligned(16))) unsigned char lds[FlashLds<D>::kBytes];
-    unsigned char* const lds_k = lds;
-    unsigned char* const lds_v = lds + FlashLds<D>::kBytesK;
+template <int D> struct FlashTile {
+    static constexpr int kRowBytes = 2 * D;
+    static constexpr int kChunks = D / 8;                 // 16-byte chunks per row
+    static constexpr int kRowsPerInstr = 1024 / kRowBytes;  // rows one wave-wide DMA instruction covers
+    static constexpr int kInstrPerWave = kFlashKeys / (4 * kRowsPerInstr);
+    static constexpr int kBytes = kFlashKeys * kRowBytes;
+    // swizzles (XOR on the 16-byte chunk index)
+    __device__ static int fk(int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); }
+    __device__ static int fv(int row) { return D == 128 ? 4 * (row & 3) : 4 * ((row >> 1) & 1); }
+};
+
+// Streams one 64-key tile (K or V) from global memory into LDS.  Rows past the end of the sequence
+// re-read the last valid row (their scores are masked; V rows are zeroed afterwards by the caller).
+template <typename T, int D, bool IS_V>
+__device__ inline void dma_tile(const T* g, int64_t sn, int k0, int L, unsigned char* lds_tile, int wave, int lane) {
+    typedef FlashTile<D> TL;
+#pragma unroll
+    for (int i = 0; i < TL::kInstrPerWave; ++i) {
+        const int instr = wave * TL::kInstrPerWave + i;
+        const int r = instr * TL::kRowsPerInstr + lane / TL::kChunks;
+        const int pc = lane % TL::kChunks;
+        const int c = pc ^ (IS_V ? TL::fv(r) : TL::fk(r));
+        int key = k0 + r;
+        key = key < L ? key : L - 1;
+        const T* src = g + (int64_t)key * sn + c * 8;
+        __builtin_amdgcn_global_load_lds((const AHPC_GLOBAL void*)src, (AHPC_LDS void*)(lds_tile + instr * 1024), 16, 0, 0);
+    }
+}
+
+template <typename T, int D, bool CAUSAL, bool VARLEN>
+__global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const FlashParams p) {
+    typedef FlashTile<D> TL;
+    constexpr int KS = D / 16;  // k-steps of the first product
+    constexpr int MB = D / 32;  // 32-row blocks of O^T
+    constexpr int RB = TL::kRowBytes;
+
+    // two buffers, each its own array: the compiler can then tell a DMA into one from reads of the other
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[TL::kBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[TL::kBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_k1[TL::kBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[TL::kBytes];
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
@@ -90,7 +144,7 @@ __global__ __launch_bounds__(kFlashThreads) void flash_fwd_mfma_kernel(const Fla
         L = p.N;
         base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
     }
-    const int q_tile0 = qt * BM;
+    const int q_tile0 = qt * kFlashRows;
     if (q_tile0 >= L) return;
 
     const T* const gq = static_cast<const T*>(p.q) + base;
@@ -99,200 +153,180 @@ __global__ __launch_bounds__(kFlashThreads) void flash_fwd_mfma_kernel(const Fla
     T* const go = static_cast<T*>(p.o) + base;
     const int64_t sn = p.stride_n;
 
+    int k_end = L;
+    if (CAUSAL) k_end = (q_tile0 + kFlashRows) < L ? (q_tile0 + kFlashRows) : L;
+    const int n_tiles = (k_end + kFlashKeys - 1) / kFlashKeys;
+
+    // first tile on its way before anything else
+    dma_tile<T, D, false>(gk, sn, 0, L, lds_k0, wave, lane);
+    dma_tile<T, D, true>(gv, sn, 0, L, lds_v0, wave, lane);
+
     // ---- Q^T operands, kept for the whole kernel --------------------------------------------
-    const int qw = q_tile0 + wave * 32 * QB;  // first query row of this wavefront
-    u32x4 qreg[QB][KS];
-#pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-        int row = qw + 32 * qb + col;
-        row = row < L ? row : L - 1;
+    const int qw = q_tile0 + wave * 32;  // first query row of this wavefront
+    const int qrow = qw + col;
+    u32x4 qreg[KS];
+    {
+        const int row = qrow < L ? qrow : L - 1;
         const T* src = gq + (int64_t)row * sn + 8 * half;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qreg[qb][ks] = *reinterpret_cast<const u32x4*>(src + 16 * ks);
+        for (int ks = 0; ks < KS; ++ks) qreg[ks] = *reinterpret_cast<const u32x4*>(src + 16 * ks);
     }
 
-    // ---- per-thread tile-load geometry ----------------------------------------------------------
-    const int chunk = tid % CPR;          // 16-byte chunk of the row
-    const int krow0 = tid / CPR;          // first K row this thread carries
-    const int vquad = tid / CPR;          // V: keys 4*vquad .. 4*vquad+3 (threads < VTHREADS)
-    // V^T position of the quad: key 16g + 8a + 4hh + b  ->  position 16g + 8hh + 4a + b
-    const int vpos = 16 * (vquad >> 2) + 8 * (vquad & 1) + 4 * ((vquad >> 1) & 1);
-    const int vcx = (chunk & 7);          // (row/8)%8 of the rows 8*chunk + j this thread writes
-
-    u32x4 kreg[KPASS];
-    u32x4 vreg[4];
-
-    auto load_tile = [&](int k0) {
+    // ---- LDS operand addresses (byte offsets inside a tile) -------------------------------------
+    // K: lane reads row (32*kb + col), logical chunk 2*ks + half
+    int k_off[KS];
 #pragma unroll
-        for (int i = 0; i < KPASS; ++i) {
-            int key = k0 + krow0 + i * KROWS;
-            key = key < L ? key : L - 1;
-            kreg[i] = *reinterpret_cast<const u32x4*>(gk + (int64_t)key * sn + 8 * chunk);
-        }
-        if (tid < VTHREADS) {
+    for (int ks = 0; ks < KS; ++ks) k_off[ks] = col * RB + (((2 * ks + half) ^ TL::fk(col)) << 4);
+    // V (transposing read): source lane i = lane%16 points at key (4*half + i/4) of the 16g+8a group,
+    // d-quad 32*mb + 16*((lane/16)%2) + 4*(i%4)
+    const int vi = lane & 15;
+    const int vkey = 4 * half + (vi >> 2);
+    int v_off[MB];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int key = k0 + 4 * vquad + r;
-                const int ck = key < L ? key : L - 1;
-                u32x4 t = *reinterpret_cast<const u32x4*>(gv + (int64_t)ck * sn + 8 * chunk);
-                if (key >= L) t = u32x4{0u, 0u, 0u, 0u};
-                vreg[r] = t;
-            }
-        }
-    };
-
-    auto store_tile = [&]() {
-#pragma unroll
-        for (int i = 0; i < KPASS; ++i)
-            *reinterpret_cast<u32x4*>(lds_k + (krow0 + i * KROWS) * KROW + chunk * 16) = kreg[i];
-        if (tid < VTHREADS) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                // dword i of each key row holds lanes 2i (low) and 2i+1 (high)
-                const uint32_t lo01 = __builtin_amdgcn_perm(vreg[1][i], vreg[0][i], 0x05040100u);
-                const uint32_t lo23 = __builtin_amdgcn_perm(vreg[3][i], vreg[2][i], 0x05040100u);
-                const uint32_t hi01 = __builtin_amdgcn_perm(vreg[1][i], vreg[0][i], 0x07060302u);
-                const uint32_t hi23 = __builtin_amdgcn_perm(vreg[3][i], vreg[2][i], 0x07060302u);
-                const int row_lo = 8 * chunk + 2 * i;
-                const int row_hi = row_lo + 1;
-                const int x_lo = ((2 * i) ^ vcx) << 4;
-                const int x_hi = ((2 * i + 1) ^ vcx) << 4;
-                *reinterpret_cast<u32x2*>(lds_v + row_lo * 128 + ((2 * vpos) ^ x_lo)) = u32x2{lo01, lo23};
-                *reinterpret_cast<u32x2*>(lds_v + row_hi * 128 + ((2 * vpos) ^ x_hi)) = u32x2{hi01, hi23};
-            }
-        }
-    };
+    for (int mb = 0; mb < MB; ++mb) {
+        const int c = 4 * mb + 2 * ((lane >> 4) & 1) + ((vi & 3) >> 1);
+        v_off[mb] = vkey * RB + ((c ^ TL::fv(vkey)) << 4) + 8 * (vi & 1);
+    }
 
     // ---- running state ----------------------------------------------------------------------------
-    f32x16 oacc[MB][QB];
-    float m_run[QB], l_run[QB];
+    f32x16 oacc[MB];
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-        m_run[qb] = -INFINITY;
-        l_run[qb] = 0.0f;
+    for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[mb][qb][r] = 0.0f;
-    }
-
-    int k_end = L;
-    if (CAUSAL) k_end = (q_tile0 + BM) < L ? (q_tile0 + BM) : L;
-    const int n_tiles = (k_end + kFlashKeys - 1) / kFlashKeys;
+        for (int r = 0; r < 16; ++r) oacc[mb][r] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
     const float c = p.scale_log2;
 
-    load_tile(0);
-    for (int t = 0; t < n_tiles; ++t) {
-        const int k0 = t * kFlashKeys;
-        __syncthreads();  // every wavefront is done reading the previous tile
-        store_tile();
-        __syncthreads();
-        if (t + 1 < n_tiles) load_tile(k0 + kFlashKeys);
-
-        // a wavefront whose queries all precede this tile has nothing to add
-        if (CAUSAL && k0 > qw + 32 * QB - 1) continue;
-
+    auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int k0) {
         // ---- S^T = K Q^T ---------------------------------------------------------------------------
-        f32x16 s[2][QB];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) s[kb][qb][r] = 0.0f;
+        f32x16 s[2];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
-            const unsigned char* arow = lds_k + (32 * kb + col) * KROW + 16 * half;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const u32x4 a = *reinterpret_cast<const u32x4*>(arow + 32 * ks);
+            for (int r = 0; r < 16; ++r) s[kb][r] = 0.0f;
+            u32x4 a[KS];
 #pragma unroll
-                for (int qb = 0; qb < QB; ++qb) s[kb][qb] = mfma_32x32x16<T>(a, qreg[qb][ks], s[kb][qb]);
-            }
+            for (int ks = 0; ks < KS; ++ks) a[ks] = *reinterpret_cast<const u32x4*>(tile_k + kb * 32 * RB + k_off[ks]);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) s[kb] = mfma_32x32x16<T>(a[ks], qreg[ks], s[kb]);
         }
 
-        // ---- online softmax, P^T packed as the B operand of the second product ---------------
+        // ---- online softmax --------------------------------------------------------------------------
         const bool need_mask = (k0 + kFlashKeys > L) || (CAUSAL && (k0 + kFlashKeys - 1 > qw));
-        u32x4 pb[QB][4];
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) {
-            const int qrow = qw + 32 * qb + col;
-            if (need_mask) {
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int key = k0 + 32 * kb + 8 * (r >> 2) + 4 * half + (r & 3);
-                        const bool ok = key < L && (!CAUSAL || key <= qrow);
-                        s[kb][qb][r] = ok ? s[kb][qb][r] : -INFINITY;
-                    }
-            }
-            float mx = s[0][qb][0];
-#pragma unroll
-            for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[0][qb][r]);
-#pragma unroll
-            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[1][qb][r]);
-            mx = fmaxf(mx, swap_halves(mx));
-            const float m_new = fmaxf(m_run[qb], mx);
-            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-            const float alpha = fast_exp2((m_run[qb] - m_use) * c);
-            const float neg = -m_use * c;
-            float sum = 0.0f;
+        if (need_mask) {
+            // key = k0 + 4*half + off(kb, r); visible iff key <= min(qrow, L-1)  <=>  off <= lim
+            int lim = L - 1;
+            if (CAUSAL) lim = qrow < lim ? qrow : lim;
+            lim -= k0 + 4 * half;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const float pv = fast_exp2(__builtin_fmaf(s[kb][qb][r], c, neg));
-                    s[kb][qb][r] = pv;
-                    sum += pv;
+                    const int off = 32 * kb + 8 * (r >> 2) + (r & 3);
+                    s[kb][r] = off <= lim ? s[kb][r] : -INFINITY;
                 }
-            l_run[qb] = l_run[qb] * alpha + sum;
-            m_run[qb] = m_new;
+        }
+        float mx = fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
+        mx = halves_max(mx);
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+        const float neg = -m_use * c;
+        float sum = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float pv = fast_exp2(__builtin_fmaf(s[kb][r], c, neg));
+                s[kb][r] = pv;
+                sum += pv;
+            }
+        // the accumulators only need rescaling when some row's maximum moved
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+            const float alpha = fast_exp2((m_run - m_use) * c);
+            l_run *= alpha;
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) oacc[mb][qb][r] *= alpha;
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int kb = g >> 1, r0 = 8 * (g & 1);
-                pb[qb][g] = u32x4{pack2<T>(s[kb][qb][r0 + 0], s[kb][qb][r0 + 1]), pack2<T>(s[kb][qb][r0 + 2], s[kb][qb][r0 + 3]),
-                                  pack2<T>(s[kb][qb][r0 + 4], s[kb][qb][r0 + 5]), pack2<T>(s[kb][qb][r0 + 6], s[kb][qb][r0 + 7])};
-            }
+                for (int r = 0; r < 16; ++r) oacc[mb][r] *= alpha;
+            m_run = m_new;
         }
+        l_run += sum;
 
-        // ---- O^T += V^T P^T ------------------------------------------------------------------------
+        // ---- P^T packed as B operands, O^T += V^T P^T ------------------------------------------------
+        u32x4 pb[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int kb = g >> 1, r0 = 8 * (g & 1);
+            pb[g] = u32x4{pack2<T>(s[kb][r0 + 0], s[kb][r0 + 1]), pack2<T>(s[kb][r0 + 2], s[kb][r0 + 3]),
+                          pack2<T>(s[kb][r0 + 4], s[kb][r0 + 5]), pack2<T>(s[kb][r0 + 6], s[kb][r0 + 7])};
+        }
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-            const int row = 32 * mb + col;
-            const int x = (row & 7) ^ ((row >> 3) & 7);
-            const unsigned char* vrow = lds_v + row * 128;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const u32x4 a = *reinterpret_cast<const u32x4*>(vrow + (((2 * g + half) ^ x) << 4));
-#pragma unroll
-                for (int qb = 0; qb < QB; ++qb) oacc[mb][qb] = mfma_32x32x16<T>(a, pb[qb][g], oacc[mb][qb]);
+                const u32x2 lo = TrRead<T>::load(tile_v + v_off[mb] + (16 * g) * RB);
+                const u32x2 hi = TrRead<T>::load(tile_v + v_off[mb] + (16 * g + 8) * RB);
+                oacc[mb] = mfma_32x32x16<T>(u32x4{lo[0], lo[1], hi[0], hi[1]}, pb[g], oacc[mb]);
             }
         }
+    };
+
+    // Zeroes the V rows of a tile that lie past the end of the sequence (they hold copies of the last
+    // row, and 0 * inf would poison the accumulators).
+    auto clear_v_tail = [&](unsigned char* tile_v, int k0) {
+        const int first = L - k0;  // first invalid row, 1..63
+        for (int i = tid; i < (kFlashKeys - first) * (RB / 16); i += kFlashThreads) {
+            const int r = first + i / (RB / 16);
+            *reinterpret_cast<u32x4*>(tile_v + r * RB + (i % (RB / 16)) * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
+    };
+
+    auto step = [&](unsigned char* cur_k, unsigned char* cur_v, unsigned char* nxt_k, unsigned char* nxt_v, int t) {
+        const int k0 = t * kFlashKeys;
+        const bool more = t + 1 < n_tiles;
+        if (more) {
+            dma_tile<T, D, false>(gk, sn, k0 + kFlashKeys, L, nxt_k, wave, lane);
+            dma_tile<T, D, true>(gv, sn, k0 + kFlashKeys, L, nxt_v, wave, lane);
+        }
+        // a wavefront whose queries all precede this tile has nothing to add
+        if (!(CAUSAL && k0 > qw + 31)) compute_tile(cur_k, cur_v, k0);
+        if (more) {
+            __builtin_amdgcn_s_waitcnt(0);  // this wave's part of the next tile has landed
+            __syncthreads();                // everyone's has, and everyone is done with the current one
+            if (k0 + 2 * kFlashKeys > L) {
+                clear_v_tail(nxt_v, k0 + kFlashKeys);
+                __syncthreads();
+            }
+        }
+    };
+
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (kFlashKeys > L) {
+        clear_v_tail(lds_v0, 0);
+        __syncthreads();
+    }
+    for (int t = 0; t < n_tiles; t += 2) {
+        step(lds_k0, lds_v0, lds_k1, lds_v1, t);
+        if (t + 1 < n_tiles) step(lds_k1, lds_v1, lds_k0, lds_v0, t + 1);
     }
 
     // ---- normalise and store: lane holds, per 32-row block, 4 runs of 4 consecutive lanes of d -----
+    const float l = halves_sum(l_run);
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    if (qrow < L) {
+        T* dst = go + (int64_t)qrow * sn + 4 * half;
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-        const float l = l_run[qb] + swap_halves(l_run[qb]);
-        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-        const int qrow = qw + 32 * qb + col;
-        if (qrow < L) {
-            T* dst = go + (int64_t)qrow * sn + 4 * half;
+        for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                for (int g4 = 0; g4 < 4; ++g4) {
-                    const f32x16& a = oacc[mb][qb];
-                    const u32x2 w = u32x2{pack2<T>(a[4 * g4 + 0] * inv, a[4 * g4 + 1] * inv),
-                                          pack2<T>(a[4 * g4 + 2] * inv, a[4 * g4 + 3] * inv)};
-                    *reinterpret_cast<u32x2*>(dst + 32 * mb + 8 * g4) = w;
-                }
-        }
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const f32x16& a = oacc[mb];
+                const u32x2 w = u32x2{pack2<T>(a[4 * g4 + 0] * inv, a[4 * g4 + 1] * inv),
+                                      pack2<T>(a[4 * g4 + 2] * inv, a[4 * g4 + 3] * inv)};
+                *reinterpret_cast<u32x2*>(dst + 32 * mb + 8 * g4) = w;
+            }
     }
 }
 
