@@ -7,7 +7,12 @@
 //                      whole kernel.  In the 32x32 result a lane owns ONE query column (lane%32)
 //                      and 16 of the 32 key rows, so the softmax row reductions are in-lane plus
 //                      one exchange between the wave halves (v_permlane32_swap).
-//   P^T = exp2(c*S^T - c*m)   online softmax in registers (c = scale*log2 e), fp32.
+//   P^T = exp2(S^T)    online softmax in registers, fp32.  Q is pre-multiplied by c = scale*log2(e) and
+//                      the product starts from an accumulator holding -c*m (m = the row's reference
+//                      maximum), so the matrix core delivers c*s - c*m and the VALU only has to apply
+//                      exp2.  m is a stabiliser, not necessarily the exact running maximum: it is
+//                      raised only when a tile's scores exceed it by more than 2^8, which keeps every
+//                      p in (0, 256], leaves O/l unchanged, and makes the accumulator rescale rare.
 //   O^T += V^T * P^T   A = V^T from LDS, B = P^T straight from the registers S^T was in: the
 //                      accumulator layout of the first product is the B-operand layout of the
 //                      second once the 16 keys of a k-step are taken in the order
@@ -105,6 +110,19 @@ __device__ inline void dma_tile(const T* g, int64_t sn, int k0, int L, unsigned 
     }
 }
 
+// Full tiles: every lane's byte offset from the tile's first row is fixed for the whole kernel
+// (`off[i]`, computed once); per tile only the uniform row base moves.
+template <typename T, int D>
+__device__ inline void dma_tile_fast(const T* tile_base, const int* off, unsigned char* lds_tile, int wave) {
+    typedef FlashTile<D> TL;
+    const char* b = reinterpret_cast<const char*>(tile_base);
+#pragma unroll
+    for (int i = 0; i < TL::kInstrPerWave; ++i) {
+        const int instr = wave * TL::kInstrPerWave + i;
+        __builtin_amdgcn_global_load_lds((const AHPC_GLOBAL void*)(b + (unsigned)off[i]), (AHPC_LDS void*)(lds_tile + instr * 1024), 16, 0, 0);
+    }
+}
+
 template <typename T, int D, bool CAUSAL, bool VARLEN>
 __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const FlashParams p) {
     typedef FlashTile<D> TL;
@@ -157,19 +175,44 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
     if (CAUSAL) k_end = (q_tile0 + kFlashRows) < L ? (q_tile0 + kFlashRows) : L;
     const int n_tiles = (k_end + kFlashKeys - 1) / kFlashKeys;
 
-    // first tile on its way before anything else
-    dma_tile<T, D, false>(gk, sn, 0, L, lds_k0, wave, lane);
-    dma_tile<T, D, true>(gv, sn, 0, L, lds_v0, wave, lane);
+    // ---- per-lane DMA offsets (bytes from the first row of a tile), fixed for the whole kernel ------
+    int dma_off_k[TL::kInstrPerWave], dma_off_v[TL::kInstrPerWave];
+#pragma unroll
+    for (int i = 0; i < TL::kInstrPerWave; ++i) {
+        const int r = (wave * TL::kInstrPerWave + i) * TL::kRowsPerInstr + lane / TL::kChunks;
+        const int pc = lane % TL::kChunks;
+        dma_off_k[i] = (int)(r * sn * 2) + ((pc ^ TL::fk(r)) << 4);
+        dma_off_v[i] = (int)(r * sn * 2) + ((pc ^ TL::fv(r)) << 4);
+    }
+    auto dma_both = [&](int k0, unsigned char* dst_k, unsigned char* dst_v) {
+        if (k0 + kFlashKeys <= L) {
+            dma_tile_fast<T, D>(gk + (int64_t)k0 * sn, dma_off_k, dst_k, wave);
+            dma_tile_fast<T, D>(gv + (int64_t)k0 * sn, dma_off_v, dst_v, wave);
+        } else {  // ragged last tile: rows are clamped lane by lane
+            dma_tile<T, D, false>(gk, sn, k0, L, dst_k, wave, lane);
+            dma_tile<T, D, true>(gv, sn, k0, L, dst_v, wave, lane);
+        }
+    };
 
-    // ---- Q^T operands, kept for the whole kernel --------------------------------------------
+    // first tile on its way before anything else
+    dma_both(0, lds_k0, lds_v0);
+
+    // ---- Q^T operands, pre-multiplied by c = scale*log2(e), kept for the whole kernel -------------
     const int qw = q_tile0 + wave * 32;  // first query row of this wavefront
     const int qrow = qw + col;
     u32x4 qreg[KS];
     {
         const int row = qrow < L ? qrow : L - 1;
         const T* src = gq + (int64_t)row * sn + 8 * half;
+        const float c = p.scale_log2;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qreg[ks] = *reinterpret_cast<const u32x4*>(src + 16 * ks);
+        for (int ks = 0; ks < KS; ++ks) {
+            const u32x4 raw = *reinterpret_cast<const u32x4*>(src + 16 * ks);
+            u32x4 sc;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) sc[w] = pack2<T>(lo_f32<T>(raw[w]) * c, hi_f32<T>(raw[w]) * c);
+            qreg[ks] = sc;
+        }
     }
 
     // ---- LDS operand addresses (byte offsets inside a tile) -------------------------------------
@@ -184,34 +227,39 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
     int v_off[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-        const int c = 4 * mb + 2 * ((lane >> 4) & 1) + ((vi & 3) >> 1);
-        v_off[mb] = vkey * RB + ((c ^ TL::fv(vkey)) << 4) + 8 * (vi & 1);
+        const int cch = 4 * mb + 2 * ((lane >> 4) & 1) + ((vi & 3) >> 1);
+        v_off[mb] = vkey * RB + ((cch ^ TL::fv(vkey)) << 4) + 8 * (vi & 1);
     }
 
     // ---- running state ----------------------------------------------------------------------------
+    // All score arithmetic is in log2 units (c is folded into Q).  `neg_m` = -(reference maximum) of the
+    // lane's query row, as a 16-wide vector because it is the C operand of the first k-step.
     f32x16 oacc[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[mb][r] = 0.0f;
-    float m_run = -INFINITY, l_run = 0.0f;
-    const float c = p.scale_log2;
+    f32x16 neg_m;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) neg_m[r] = 0.0f;
+    float l_run = 0.0f;
+    bool first = true;
+    constexpr float kRaise = 8.0f;  // raise the reference maximum only when exceeded by 2^8
+    const uint32_t ones = pack2<T>(1.0f, 1.0f);
 
     auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int k0) {
-        // ---- S^T = K Q^T ---------------------------------------------------------------------------
+        // ---- S^T = c*K Q^T - m  (log2 units) -------------------------------------------------------
         f32x16 s[2];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s[kb][r] = 0.0f;
             u32x4 a[KS];
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) a[ks] = *reinterpret_cast<const u32x4*>(tile_k + kb * 32 * RB + k_off[ks]);
+            s[kb] = mfma_32x32x16<T>(a[0], qreg[0], neg_m);
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) s[kb] = mfma_32x32x16<T>(a[ks], qreg[ks], s[kb]);
+            for (int ks = 1; ks < KS; ++ks) s[kb] = mfma_32x32x16<T>(a[ks], qreg[ks], s[kb]);
         }
 
-        // ---- online softmax --------------------------------------------------------------------------
         const bool need_mask = (k0 + kFlashKeys > L) || (CAUSAL && (k0 + kFlashKeys - 1 > qw));
         if (need_mask) {
             // key = k0 + 4*half + off(kb, r); visible iff key <= min(qrow, L-1)  <=>  off <= lim
@@ -226,42 +274,46 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
                     s[kb][r] = off <= lim ? s[kb][r] : -INFINITY;
                 }
         }
+        // ---- reference maximum: exact on the first tile, afterwards raised only when a score tops it
+        //      by more than kRaise (rare, and the only time the accumulators are rescaled) ---------------
         float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
         for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
-        mx = halves_max(mx);
-        const float m_new = fmaxf(m_run, mx);
-        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-        const float neg = -m_use * c;
-        float sum = 0.0f;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float pv = fast_exp2(__builtin_fmaf(s[kb][r], c, neg));
-                s[kb][r] = pv;
-                sum += pv;
-            }
-        // the accumulators only need rescaling when some row's maximum moved
-        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
-            const float alpha = fast_exp2((m_run - m_use) * c);
+        if (first || __builtin_amdgcn_ballot_w64(mx > kRaise) != 0) {
+            mx = halves_max(mx);                       // both lanes of a query agree
+            const float delta = first ? mx : fmaxf(mx, 0.0f);
+            const float alpha = fast_exp2(-delta);
             l_run *= alpha;
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) oacc[mb][r] *= alpha;
-            m_run = m_new;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[kb][r] -= delta;
+            const float nm = neg_m[0] - delta;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) neg_m[r] = nm;
+            first = false;
         }
-        l_run += sum;
 
-        // ---- P^T packed as B operands, O^T += V^T P^T ------------------------------------------------
+        // ---- P^T = exp2(S^T), packed as B operands; row sums from the packed (rounded) values ----------
         u32x4 pb[4];
+        float sum = 0.0f;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const int kb = g >> 1, r0 = 8 * (g & 1);
-            pb[g] = u32x4{pack2<T>(s[kb][r0 + 0], s[kb][r0 + 1]), pack2<T>(s[kb][r0 + 2], s[kb][r0 + 3]),
-                          pack2<T>(s[kb][r0 + 4], s[kb][r0 + 5]), pack2<T>(s[kb][r0 + 6], s[kb][r0 + 7])};
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t pk = pack2<T>(fast_exp2(s[kb][r0 + 2 * w]), fast_exp2(s[kb][r0 + 2 * w + 1]));
+                pb[g][w] = pk;
+                sum = dot2<T>(pk, ones, sum);
+            }
         }
+        l_run += sum;
+
+        // ---- O^T += V^T P^T ------------------------------------------------------------------------------
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
@@ -276,9 +328,9 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
     // Zeroes the V rows of a tile that lie past the end of the sequence (they hold copies of the last
     // row, and 0 * inf would poison the accumulators).
     auto clear_v_tail = [&](unsigned char* tile_v, int k0) {
-        const int first = L - k0;  // first invalid row, 1..63
-        for (int i = tid; i < (kFlashKeys - first) * (RB / 16); i += kFlashThreads) {
-            const int r = first + i / (RB / 16);
+        const int first_bad = L - k0;  // first invalid row, 1..63
+        for (int i = tid; i < (kFlashKeys - first_bad) * (RB / 16); i += kFlashThreads) {
+            const int r = first_bad + i / (RB / 16);
             *reinterpret_cast<u32x4*>(tile_v + r * RB + (i % (RB / 16)) * 16) = u32x4{0u, 0u, 0u, 0u};
         }
     };
@@ -286,10 +338,7 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
     auto step = [&](unsigned char* cur_k, unsigned char* cur_v, unsigned char* nxt_k, unsigned char* nxt_v, int t) {
         const int k0 = t * kFlashKeys;
         const bool more = t + 1 < n_tiles;
-        if (more) {
-            dma_tile<T, D, false>(gk, sn, k0 + kFlashKeys, L, nxt_k, wave, lane);
-            dma_tile<T, D, true>(gv, sn, k0 + kFlashKeys, L, nxt_v, wave, lane);
-        }
+        if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
         // a wavefront whose queries all precede this tile has nothing to add
         if (!(CAUSAL && k0 > qw + 31)) compute_tile(cur_k, cur_v, k0);
         if (more) {
