@@ -97,16 +97,57 @@ struct DecodeParams {
     float scale_log2;
 };
 
-__device__ __forceinline__ float load_qo(const void* base, int dtype, int64_t i) {
-    if (dtype == AHPC_F32) return static_cast<const float*>(base)[i];
-    if (dtype == AHPC_F16) return (float)static_cast<const f16_t*>(base)[i];
-    return (float)static_cast<const bf16_t*>(base)[i];
-}
-
 __device__ __forceinline__ void store_qo(void* base, int dtype, int64_t i, float x) {
     if (dtype == AHPC_F32) static_cast<float*>(base)[i] = x;
     else if (dtype == AHPC_F16) static_cast<f16_t*>(base)[i] = (f16_t)x;
     else static_cast<bf16_t*>(base)[i] = (bf16_t)x;
+}
+
+// N (4 or 8) consecutive q/o elements starting at element index i (a multiple of N; the tensors are
+// 16-byte aligned), moved with one or two vector accesses whatever the element type.
+template <int N> __device__ __forceinline__ void load_qo_vec(const void* base, int dtype, int64_t i, float (&out)[N]) {
+    if (dtype == AHPC_F32) {
+        const f32x4* src = reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + i);
+#pragma unroll
+        for (int v = 0; v < N / 4; ++v) {
+            const f32x4 x = src[v];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) out[4 * v + e] = x[e];
+        }
+    } else {
+        uint32_t w[N / 2];
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(base) + i);
+        if (N == 8) {
+            const u32x4 x = *reinterpret_cast<const u32x4*>(src);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e % (N / 2)] = x[e];
+        } else {
+            const u32x2 x = *reinterpret_cast<const u32x2*>(src);
+            w[0] = x[0];
+            w[1] = x[1];
+        }
+#pragma unroll
+        for (int e = 0; e < N / 2; ++e) {
+            out[2 * e] = dtype == AHPC_F16 ? lo_f32<f16_t>(w[e]) : lo_f32<bf16_t>(w[e]);
+            out[2 * e + 1] = dtype == AHPC_F16 ? hi_f32<f16_t>(w[e]) : hi_f32<bf16_t>(w[e]);
+        }
+    }
+}
+
+template <int N> __device__ __forceinline__ void store_qo_vec(void* base, int dtype, int64_t i, const float (&x)[N]) {
+    if (dtype == AHPC_F32) {
+        f32x4* dst = reinterpret_cast<f32x4*>(static_cast<float*>(base) + i);
+#pragma unroll
+        for (int v = 0; v < N / 4; ++v) dst[v] = f32x4{x[4 * v], x[4 * v + 1], x[4 * v + 2], x[4 * v + 3]};
+    } else {
+        uint32_t w[N / 2];
+#pragma unroll
+        for (int e = 0; e < N / 2; ++e)
+            w[e] = dtype == AHPC_F16 ? pack2<f16_t>(x[2 * e], x[2 * e + 1]) : pack2<bf16_t>(x[2 * e], x[2 * e + 1]);
+        uint32_t* dst = reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(base) + i);
+        if (N == 8) *reinterpret_cast<u32x4*>(dst) = u32x4{w[0], w[1], w[2 % (N / 2)], w[3 % (N / 2)]};
+        else *reinterpret_cast<u32x2*>(dst) = u32x2{w[0], w[1]};
+    }
 }
 
 // Sum over the LPH lanes that share a head; every one of them gets the total.
@@ -120,13 +161,20 @@ template <int LPH> __device__ __forceinline__ float head_allreduce(float x) {
     return x;
 }
 
-constexpr int kDecodeBatch = 8;  // tokens whose K and V rows are in flight together, per lane
+#ifndef AHPC_DECODE_BATCH
+#define AHPC_DECODE_BATCH 8
+#endif
+constexpr int kDecodeBatch = AHPC_DECODE_BATCH;  // tokens whose K and V rows are in flight together, per lane
 
-// T: pool element type.  D: head dimension.  A lane owns EPL = 16/sizeof(T) consecutive lanes of
-// one head.  Grid: (chunk, batch entry, head group); every wavefront works on its own heads and
-// needs no LDS and no barrier.
-template <typename T, int D>
-__global__ __launch_bounds__(256) void paged_decode_kernel(const DecodeParams p) {
+// T: pool element type.  D: head dimension.  PT: tokens per page when known at compile time (16), or 0
+// for any page size.  A lane owns EPL = 16/sizeof(T) consecutive elements of one head.  Grid: (chunk,
+// batch entry, head group); every wavefront works on its own heads and needs no LDS and no barrier.
+//
+// A chunk starts on a page boundary.  Its page ids are fetched once (one table entry per lane) and
+// handed out with v_readlane, so the only per-token address work is a uniform add; K and V rows of
+// the next 8 tokens are requested before the current 8 are consumed.
+template <typename T, int D, int PT>
+__global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p) {
     constexpr int EPL = 16 / (int)sizeof(T);
     constexpr int LPH = D / EPL;
     constexpr int HPW = kWave / LPH;
@@ -136,22 +184,32 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(const DecodeParams p)
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int waves = blockDim.x >> 6;
-    const int chunk = blockIdx.x;
-    const int b = blockIdx.y;
-    const int h_raw = (blockIdx.z * waves + wave) * HPW + lane / LPH;
+    // head group is the fastest grid dimension: the workgroups that together cover the 2*H*D bytes of a
+    // token row are dispatched side by side and stream whole pages between them
+    const int chunk = blockIdx.y;
+    const int b = blockIdx.z;
+    const int h_raw = (blockIdx.x * waves + wave) * HPW + lane / LPH;
     const bool head_ok = h_raw < p.H;
     const int h = head_ok ? h_raw : p.H - 1;
     const int e0 = (lane % LPH) * EPL;
+    const int P = PT ? PT : p.P;
 
     const int64_t row = p.batch_rows ? p.batch_rows[b] : b;
-    const int L = p.seq_lens[row] < p.max_len ? p.seq_lens[row] : p.max_len;
     const int t0 = chunk * p.chunk_tokens;
+    // page ids of the chunk (at most 64: the host caps chunk_tokens at 64 pages): lane i holds the id of
+    // page (first_page + i).  Requested before the sequence length is known (any entry of the row may
+    // be read), so that this load and the length load are in flight together.
+    const int first_page = t0 / P;
+    int my_page = 0;
+    if (first_page + lane < p.max_pages) my_page = p.table[row * p.max_pages + first_page + lane];
+    const int L = p.seq_lens[row] < p.max_len ? p.seq_lens[row] : p.max_len;
     if (t0 >= L) {
         // an empty sequence still owns an output row: zeros (with several chunks the merge writes it)
         if (chunk == 0 && p.n_chunks == 1 && head_ok) {
-            const int64_t oi = ((int64_t)b * p.H + h) * D + e0;
+            float zero[EPL];
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) store_qo(p.o, p.qo_dtype, oi + e, 0.0f);
+            for (int e = 0; e < EPL; ++e) zero[e] = 0.0f;
+            store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + h) * D + e0, zero);
         }
         return;
     }
@@ -161,33 +219,52 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(const DecodeParams p)
     float qf[EPL];
     uint32_t qp[4];
     {
-        const int64_t qi = ((int64_t)b * p.H + h) * D + e0;
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) qf[e] = load_qo(p.q, p.qo_dtype, qi + e);
+        load_qo_vec<EPL>(p.q, p.qo_dtype, ((int64_t)b * p.H + h) * D + e0, qf);
         if (kPacked) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) qp[i] = pack2<TP>(qf[2 * i], qf[2 * i + 1]);
         }
     }
 
-    const T* const kp = static_cast<const T*>(p.k_pool) + (int64_t)h * D + e0;
-    const T* const vp = static_cast<const T*>(p.v_pool) + (int64_t)h * D + e0;
+    // byte offset of this lane's piece inside a token row; token rows are tok_bytes apart
+    const uint32_t lane_off = (uint32_t)((h * D + e0) * (int)sizeof(T));
+    const int64_t tok_bytes = (int64_t)p.H * D * (int64_t)sizeof(T);
+    const char* const kbase = static_cast<const char*>(p.k_pool);
+    const char* const vbase = static_cast<const char*>(p.v_pool);
 
-    auto token_offset = [&](int t) -> int64_t {
-        // tokens past the chunk end re-read the last valid token (their score is masked below);
-        // a missing page reads page 0 (the host never hands out such a table)
-        const int tc = t < t1 ? t : t1 - 1;
-        const int64_t off = kv_token_offset(p.table, p.max_pages, row, tc, p.P, p.H, D);
-        return off < 0 ? 0 : off;
-    };
+    my_page = my_page < 0 ? 0 : my_page;  // a missing page reads page 0 (the host never hands out such a table)
 
-    u32x4 kreg[kDecodeBatch], vreg[kDecodeBatch];
-    auto load_batch = [&](int tb) {
+    const int n_tok = t1 - t0;
+    const int n_batches = (n_tok + kDecodeBatch - 1) / kDecodeBatch;
+
+    // Requests the K and V rows of batch `bi` (tokens 8*bi .. 8*bi+7 of the chunk).  Tokens past the
+    // end of the chunk re-read the last valid one; their scores are masked when the batch is consumed.
+    // The loads are non-temporal: every K/V byte is used exactly once, and keeping the stream out of
+    // the caches is worth about 10% of bandwidth here.
+    auto issue = [&](u32x4 (&kr)[kDecodeBatch], u32x4 (&vr)[kDecodeBatch], int bi) {
+        const int ti0 = bi * kDecodeBatch;
+        const int last = n_tok - 1 - ti0;  // index of the last valid token of this batch (>= 0)
+        if (PT == 16) {
+            // 8 consecutive slots of one page: one page id, rows tok_bytes apart
+            const int page_id = __builtin_amdgcn_readlane(my_page, ti0 >> 4);
+            const int64_t base = ((int64_t)page_id * 16 + (ti0 & 15)) * tok_bytes;
 #pragma unroll
-        for (int i = 0; i < kDecodeBatch; ++i) {
-            const int64_t off = token_offset(tb + i);
-            kreg[i] = *reinterpret_cast<const u32x4*>(kp + off);
-            vreg[i] = *reinterpret_cast<const u32x4*>(vp + off);
+            for (int i = 0; i < kDecodeBatch; ++i) {
+                const int ic = i < last ? i : last;
+                const int64_t off = base + ic * tok_bytes;
+                kr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + off + lane_off));
+                vr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + off + lane_off));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kDecodeBatch; ++i) {
+                const int tc = ti0 + (i < last ? i : last);
+                const int pg = tc / P;
+                const int page_id = __builtin_amdgcn_readlane(my_page, pg);
+                const int64_t off = ((int64_t)page_id * P + (tc - pg * P)) * tok_bytes;
+                kr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + off + lane_off));
+                vr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + off + lane_off));
+            }
         }
     };
 
@@ -197,16 +274,8 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(const DecodeParams p)
     float m = -INFINITY, l = 0.0f;
     const float c = p.scale_log2;
 
-    load_batch(t0);
-    for (int tb = t0; tb < t1; tb += kDecodeBatch) {
-        u32x4 kc[kDecodeBatch], vc[kDecodeBatch];
-#pragma unroll
-        for (int i = 0; i < kDecodeBatch; ++i) {
-            kc[i] = kreg[i];
-            vc[i] = vreg[i];
-        }
-        if (tb + kDecodeBatch < t1) load_batch(tb + kDecodeBatch);
-
+    auto consume = [&](const u32x4 (&kc)[kDecodeBatch], const u32x4 (&vc)[kDecodeBatch], int bi) {
+        const int valid = n_tok - bi * kDecodeBatch;  // >= 1; >= 8 for all but the last batch
         float s[kDecodeBatch];
         float mx = -INFINITY;
 #pragma unroll
@@ -220,7 +289,7 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(const DecodeParams p)
                 for (int w = 0; w < 4; ++w) part = __builtin_fmaf(qf[w % EPL], as_f32(kc[i][w]), part);
             }
             part = head_allreduce<LPH>(part);
-            s[i] = (tb + i < t1) ? part * c : -INFINITY;
+            s[i] = (i < valid) ? part * c : -INFINITY;
             mx = fmaxf(mx, s[i]);
         }
         const float m_new = fmaxf(m, mx);              // finite: the batch holds at least one token
@@ -245,14 +314,27 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(const DecodeParams p)
         }
         l = l * alpha + sum;
         m = m_new;
+    };
+
+    // two register sets in ping-pong: while one batch is consumed the next is in flight
+    u32x4 ka[kDecodeBatch], va[kDecodeBatch], kb2[kDecodeBatch], vb2[kDecodeBatch];
+    issue(ka, va, 0);
+    for (int bi = 0; bi < n_batches; bi += 2) {
+        if (bi + 1 < n_batches) issue(kb2, vb2, bi + 1);
+        consume(ka, va, bi);
+        if (bi + 1 < n_batches) {
+            if (bi + 2 < n_batches) issue(ka, va, bi + 2);
+            consume(kb2, vb2, bi + 1);
+        }
     }
 
     if (!head_ok) return;
     if (p.n_chunks == 1) {
         const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-        const int64_t oi = ((int64_t)b * p.H + h) * D + e0;
+        float res[EPL];
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) store_qo(p.o, p.qo_dtype, oi + e, acc[e] * inv);
+        for (int e = 0; e < EPL; ++e) res[e] = acc[e] * inv;
+        store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + h) * D + e0, res);
     } else {
         const int64_t slot = ((int64_t)b * p.n_chunks + chunk) * p.H + h;
         f32x4* dst = reinterpret_cast<f32x4*>(p.part_o + slot * D + e0);
@@ -265,30 +347,31 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(const DecodeParams p)
     }
 }
 
-// One thread per output element: folds the chunk partials of its (batch entry, head) with
-// m' = max(m, m2), l' = l*2^(m-m') + l2*2^(m2-m') and the same factors on the accumulators.
-__global__ void paged_merge_kernel(const DecodeParams p) {
+// One thread per output element: folds the chunk partials of its (batch entry, head) with the rule
+// m' = max(m, m2), l' = l*2^(m-m') + l2*2^(m2-m'), accumulators scaled by the same factors.  Done in
+// two passes (global maximum first) so that the loads of the second pass do not wait on one another.
+__global__ __launch_bounds__(256) void paged_merge_kernel(const DecodeParams p) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t hd = (int64_t)p.H * p.d;
     if (idx >= p.B * hd) return;
     const int64_t b = idx / hd;
     const int64_t he = idx - b * hd;
     const int h = (int)(he / p.d);
+    const int e = (int)(he - (int64_t)h * p.d);
     const int64_t row = p.batch_rows ? p.batch_rows[b] : b;
     const int L = p.seq_lens[row] < p.max_len ? p.seq_lens[row] : p.max_len;
     const int n = (L + p.chunk_tokens - 1) / p.chunk_tokens;
-    float m = -INFINITY, l = 0.0f, acc = 0.0f;
+    const float* ml = p.part_ml + ((b * p.n_chunks) * p.H + h) * 2;
+    const float* po = p.part_o + ((b * p.n_chunks) * p.H + h) * p.d + e;
+    const int64_t ml_step = (int64_t)p.H * 2, po_step = (int64_t)p.H * p.d;
+    float m = -INFINITY;
+    for (int ci = 0; ci < n; ++ci) m = fmaxf(m, ml[ci * ml_step]);
+    float l = 0.0f, acc = 0.0f;
+#pragma unroll 4
     for (int ci = 0; ci < n; ++ci) {
-        const int64_t slot = (b * p.n_chunks + ci) * p.H + h;
-        const float m2 = p.part_ml[slot * 2];
-        const float l2 = p.part_ml[slot * 2 + 1];
-        const float o2 = p.part_o[slot * p.d + (he - (int64_t)h * p.d)];
-        const float m_new = fmaxf(m, m2);
-        const float f1 = fast_exp2(m - m_new);
-        const float f2 = fast_exp2(m2 - m_new);
-        l = l * f1 + l2 * f2;
-        acc = acc * f1 + o2 * f2;
-        m = m_new;
+        const float f = fast_exp2(ml[ci * ml_step] - m);
+        l = __builtin_fmaf(ml[ci * ml_step + 1], f, l);
+        acc = __builtin_fmaf(po[ci * po_step], f, acc);
     }
     store_qo(p.o, p.qo_dtype, idx, l > 0.0f ? acc / l : 0.0f);
 }
@@ -299,13 +382,11 @@ static int env_int(const char* name, int dflt) {
 }
 
 // Waves per decode workgroup (each wave works alone; this only sets how many heads travel together).
-static int decode_waves() {
-    static const int v = env_int("AHPC_DECODE_WAVES", 0);
-    return v;
-}
+static int decode_waves() { return env_int("AHPC_DECODE_WAVES", 0); }
 
 static int64_t pick_chunk_tokens(int64_t B, int64_t H, int64_t max_len, int64_t P, int64_t requested) {
     int64_t chunk = requested;
+    if (chunk <= 0) chunk = env_int("AHPC_DECODE_CHUNK", 0);
     if (chunk <= 0) {
         // enough workgroups to keep every CU busy several times over, while the fp32 partials stay
         // below ~1% of the K/V bytes of a chunk
@@ -314,19 +395,25 @@ static int64_t pick_chunk_tokens(int64_t B, int64_t H, int64_t max_len, int64_t 
     }
     chunk = ((chunk + P - 1) / P) * P;
     if (chunk < P) chunk = P;
+    if (chunk > 64 * P) chunk = 64 * P;  // the decode kernel keeps one page id per lane
     return chunk;
+}
+
+template <typename T, int PT>
+static int launch_decode_dp(const DecodeParams& p, dim3 grid, dim3 block, hipStream_t st) {
+    switch (p.d) {
+        case 32: hipLaunchKernelGGL((paged_decode_kernel<T, 32, PT>), grid, block, 0, st, p); break;
+        case 64: hipLaunchKernelGGL((paged_decode_kernel<T, 64, PT>), grid, block, 0, st, p); break;
+        case 128: hipLaunchKernelGGL((paged_decode_kernel<T, 128, PT>), grid, block, 0, st, p); break;
+        case 256: hipLaunchKernelGGL((paged_decode_kernel<T, 256, PT>), grid, block, 0, st, p); break;
+        default: return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+    }
+    return static_cast<int>(hipGetLastError());
 }
 
 template <typename T>
 static int launch_decode_d(const DecodeParams& p, dim3 grid, dim3 block, hipStream_t st) {
-    switch (p.d) {
-        case 32: hipLaunchKernelGGL((paged_decode_kernel<T, 32>), grid, block, 0, st, p); break;
-        case 64: hipLaunchKernelGGL((paged_decode_kernel<T, 64>), grid, block, 0, st, p); break;
-        case 128: hipLaunchKernelGGL((paged_decode_kernel<T, 128>), grid, block, 0, st, p); break;
-        case 256: hipLaunchKernelGGL((paged_decode_kernel<T, 256>), grid, block, 0, st, p); break;
-        default: return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
-    }
-    return static_cast<int>(hipGetLastError());
+    return p.P == 16 ? launch_decode_dp<T, 16>(p, grid, block, st) : launch_decode_dp<T, 0>(p, grid, block, st);
 }
 
 }  // namespace ahpc
@@ -432,7 +519,9 @@ int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype, const void* k_po
     if (B <= 0 || B > 65535 || max_len <= 0 || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;
     if ((max_len + P - 1) / P > max_pages) return AHPC_ERR_BAD_SHAPE;
     if (d != 32 && d != 64 && d != 128 && d != 256) return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
-    if ((reinterpret_cast<uintptr_t>(k_pool) & 15u) || (reinterpret_cast<uintptr_t>(v_pool) & 15u)) return AHPC_ERR_BAD_ALIGNMENT;
+    if ((reinterpret_cast<uintptr_t>(k_pool) & 15u) || (reinterpret_cast<uintptr_t>(v_pool) & 15u) ||
+        (reinterpret_cast<uintptr_t>(q) & 15u) || (reinterpret_cast<uintptr_t>(o) & 15u))
+        return AHPC_ERR_BAD_ALIGNMENT;
     if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
 
     const int64_t chunk = pick_chunk_tokens(B, H, max_len, P, chunk_tokens);
@@ -459,7 +548,7 @@ int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype, const void* k_po
     if (lph < 1 || lph > 64) return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
     const int hpw = 64 / lph;
     int waves = decode_waves();
-    if (waves < 1 || waves > 4) waves = 1;
+    if (waves < 1 || waves > 8) waves = 2;
     const int64_t heads_per_wg = (int64_t)hpw * waves;
     const int64_t head_groups = (H + heads_per_wg - 1) / heads_per_wg;
     if (head_groups > 65535) return AHPC_ERR_BAD_SHAPE;
@@ -467,7 +556,7 @@ int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype, const void* k_po
     const int64_t total = B * H * d;
     dim3 eblock(256), egrid((unsigned)((total + 255) / 256));
 
-    dim3 grid((unsigned)n_chunks, (unsigned)B, (unsigned)head_groups), block(64 * waves);
+    dim3 grid((unsigned)head_groups, (unsigned)n_chunks, (unsigned)B), block(64 * waves);
     int rc;
     switch (pool_dtype) {
         case AHPC_F32: rc = launch_decode_d<float>(p, grid, block, st); break;

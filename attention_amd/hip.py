@@ -9,7 +9,8 @@ import os
 F32, F16, BF16 = 0, 1, 2
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libahpc_hip.so")
+# AHPC_HIP_LIB points at another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("AHPC_HIP_LIB") or os.path.join(_HERE, "lib", "libahpc_hip.so")
 
 
 class HipError(RuntimeError):
