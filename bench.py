@@ -28,6 +28,11 @@ sys.path.insert(0, ROOT)
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on exactly these workloads,
+# each counter scaled by its reading for a 1 GiB device copy (profiles/*.txt hold the runs).
+FLASH_TRAFFIC_BYTES = 542_200_000     # 408.0 MB fetched + 134.2 MB written (algorithmic: 536.9 MB)
+DECODE_TRAFFIC_BYTES = 2_364_900_000  # decode 2343.7 + 9.8 MB, merge 10.9 + 0.5 MB (algorithmic: 2342.9 MB)
+
 FLASH = dict(B=4, N=4096, H=32, d=128, causal=True, dtype="bf16", seed=0xA77E0002)
 DECODE = dict(B=64, H=32, d=128, P=16, lo=512, hi=4096, dtype="fp16", seed=0xA77E0003)
 
@@ -130,23 +135,24 @@ def bench_flash(hip, stream, steps, warmup, cpu):
         "metric": "FlashAttn fwd TFLOP/s (bf16, N=4096, d=128)", "value": round(value, 2), "unit": "TFLOP/s",
         "ms_per_step": round(wall / steps * 1e3, 4),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": FLASH_TRAFFIC_BYTES,
                      "kernel": "flash_fwd_mfma_kernel<bf16,128,causal>", "kernel_ms_mean": round(kern_ms, 4),
                      "kernel_ms_min": round(float(np.min(per)), 4), "flop_per_launch": flops},
         "config": {"workload": "flash_fwd bf16 causal B=4 N=4096 H=32 d=128 layout [B,N,H,d], fp32 accumulate, bf16 out"},
     }
     if cpu:
         from oracle import oracle as O
-        # bounded sample: batch entry 0 (all 32 heads), i.e. 1/4 of the step, on the box's host cores
-        qs, ks, vs = (t[0:1].float().cpu().numpy() for t in (q, k, v))
+        # bounded sample: the first `nb` batch entries (all 32 heads each) on the box's host cores
+        nb = 2
+        qs, ks, vs = (t[0:nb].float().cpu().numpy() for t in (q, k, v))
         threads = O.cpu_threads()
         t0 = time.perf_counter()
-        ref = O.attention(qs, ks, vs, 1, N, H, d, scale, True, threads=threads)
+        ref = O.attention(qs, ks, vs, nb, N, H, d, scale, True, threads=threads)
         dt = time.perf_counter() - t0
-        err = float(np.abs(o[0:1].float().cpu().numpy() - ref).max())
-        res["cpu_baseline"] = {"value": round(2.0 * H * N * N * d / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads,
-                               "kind": "port", "sample": f"batch entry 0 of 4 (32 heads x 4096 rows), {dt:.1f} s",
-                               "max_abs_err_gpu_vs_cpu": err}
+        err = float(np.abs(o[0:nb].float().cpu().numpy() - ref).max())
+        res["cpu_baseline"] = {"value": round(2.0 * nb * H * N * N * d / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads,
+                               "kind": "port", "sample": f"batch entries 0-{nb - 1} of 4 ({nb}x32 heads x 4096 rows), "
+                               f"{dt:.1f} s wall on {threads} threads", "max_abs_err_gpu_vs_cpu": err}
     return res
 
 
@@ -181,7 +187,7 @@ def bench_decode(hip, stream, steps, warmup, cpu):
         "metric": "paged decode HBM GB/s", "value": round(value, 1), "unit": "GB/s",
         "ms_per_step": round(wall / steps * 1e3, 4),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": DECODE_TRAFFIC_BYTES,
                      "kernel": "paged_decode_kernel<f16,128> + paged_merge_kernel", "kernel_ms_mean": round(kern_ms, 4),
                      "kernel_ms_min": round(float(np.min(per)), 4), "bytes_per_launch": nbytes},
         "config": {"workload": f"paged_decode fp16 B=64 H=32 d=128 page=16 context U[512,4096] (sum {int(lens.sum())} tokens), "
@@ -189,8 +195,8 @@ def bench_decode(hip, stream, steps, warmup, cpu):
     }
     if cpu:
         from oracle import oracle as O
-        # bounded sample: the first 16 of the 64 sequences, their pages copied to the host
-        nb = 16
+        # bounded sample: the first 32 of the 64 sequences, their pages copied to the host; 8 passes
+        nb = 32
         pages_per = (lens + P - 1) // P
         sub_tables, kparts, vparts, c0 = [], [], [], 0
         for b in range(nb):
@@ -205,15 +211,35 @@ def bench_decode(hip, stream, steps, warmup, cpu):
         kh, vh = np.concatenate(kparts), np.concatenate(vparts)
         qh = q[:nb].float().cpu().numpy()
         threads = O.cpu_threads()
+        reps = 8
         t0 = time.perf_counter()
-        ref = O.paged_decode(qh, kh, vh, st, lens[:nb], None, nb, H, d, P, scale, threads=threads)
-        dt = time.perf_counter() - t0
+        for _ in range(reps):
+            ref = O.paged_decode(qh, kh, vh, st, lens[:nb], None, nb, H, d, P, scale, threads=threads)
+        dt = (time.perf_counter() - t0) / reps
         sub = dict(c, B=nb)
         err = float(np.abs(o[:nb].float().cpu().numpy() - ref).max())
         res["cpu_baseline"] = {"value": round(decode_bytes(lens[:nb], sub) / dt / 1e9, 3), "unit": "GB/s", "cores": threads,
-                               "kind": "port", "sample": f"first 16 of 64 sequences ({int(lens[:nb].sum())} tokens), {dt:.1f} s; "
-                               "bytes counted at the GPU's 2-byte storage size", "max_abs_err_gpu_vs_cpu": err}
+                               "kind": "port", "sample": f"first {nb} of 64 sequences ({int(lens[:nb].sum())} tokens), mean of "
+                               f"{reps} passes of {dt:.2f} s on {threads} threads; bytes counted at the GPU's 2-byte storage size "
+                               "(the CPU path streams fp32 copies, twice as many bytes)", "max_abs_err_gpu_vs_cpu": err}
     return res
+
+
+def run_calibration(steps):
+    """A plain device-to-device copy of known size (1 GiB read + 1 GiB written per launch): what the
+    FETCH_SIZE / WRITE_SIZE counters read for it is the scale for the same counters on our kernels."""
+    import torch
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    print(json.dumps({"workload": "calibration copy", "bytes_read": n, "bytes_written": n, "launches": steps,
+                      "ms_per_launch": round(dt * 1e3, 4), "GBps_read_plus_write": round(2 * n / dt / 1e9, 1)}))
 
 
 def main():
@@ -221,7 +247,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", choices=["all", "flash", "decode"], default="all")
+    ap.add_argument("--workload", choices=["all", "flash", "decode", "calib"], default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline (profiling runs)")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -232,6 +258,9 @@ def main():
     hip.load()
     if not torch.cuda.is_available() or hip.device_count() < 1:
         sys.exit("bench.py: no GPU visible")
+    if a.workload == "calib":
+        run_calibration(a.steps)
+        return
     import ctypes as C
     s = C.c_void_p()
     assert hip.load().ahpc_hip_stream_create(C.byref(s)) == 0
