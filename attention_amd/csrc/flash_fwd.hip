@@ -148,8 +148,12 @@ static int dispatch_simple(int dtype, const SimpleParams& p, int64_t B, hipStrea
 template <typename T, int D, bool VARLEN>
 static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
     p.n_qtiles = (p.N + kFlashRows - 1) / kFlashRows;
-    const int64_t total = B * p.H * (int64_t)p.n_qtiles;
+    int64_t total = B * p.H * (int64_t)p.n_qtiles;
     if (total > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
+    // Causal launches with enough workgroups to fill the chip twice over pair a late query tile with an
+    // early one, so that every workgroup walks the same number of key tiles.
+    p.paired = (causal && p.n_qtiles >= 2 && total >= 1024) ? 1 : 0;
+    if (p.paired) total = B * p.H * (int64_t)((p.n_qtiles + 1) / 2);
     p.total_blocks = (int32_t)total;
     p.blocks_per_xcd = (int32_t)((total + 7) / 8);
     dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
@@ -172,7 +176,9 @@ static bool mfma_eligible(int dtype, int64_t d, const void* q, const void* k, co
     if (dtype != AHPC_F16 && dtype != AHPC_BF16) return false;
     if (d != 64 && d != 128) return false;
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return false;
-    return (s0 % 8 == 0) && (s1 % 8 == 0) && (s2 % 8 == 0);
+    if ((s0 % 8) || (s1 % 8) || (s2 % 8)) return false;
+    // a key tile is addressed with 32-bit byte offsets from its first row, and rows must not overlap
+    return s1 >= d && s1 < (int64_t(1) << 24);
 }
 
 static int check_dense(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N, int64_t H,

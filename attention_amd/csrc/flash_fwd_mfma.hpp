@@ -21,12 +21,22 @@
 //                      4 keys of one d, and two such reads fetch exactly the 8 keys above.
 // O^T keeps the query in the lane column, so the per-row rescale factors are per-lane scalars.
 //
-// Tiles reach LDS without touching registers: global_load_lds_dwordx4 writes 1 KiB per wave
-// instruction (lane i -> LDS base + 16*i).  Which global 16-byte chunk a lane fetches is free, so the
-// XOR swizzle that makes the later operand reads bank-conflict free is applied on the global side:
+// Tiles reach LDS without touching registers: buffer_load_dwordx4 ... lds writes 1 KiB per wave
+// instruction (lane i -> LDS base + 16*i).  The address is a uniform buffer descriptor (first row of the
+// tile, bytes valid from there) plus a per-lane 32-bit offset that never changes, so a tile costs eight
+// back-to-back loads and no vector arithmetic, and rows past the end of a sequence are out of range for
+// the descriptor and arrive as zeros.  Which global 16-byte chunk a lane fetches is free, so the XOR
+// swizzle that makes the later operand reads bank-conflict free is applied on the global side:
 // physical chunk = chunk ^ f(row), with f chosen per tile kind (16-byte row reads for K, 8-byte
 // transposing reads for V).  LDS is double buffered: tile t+1 streams in while tile t is consumed;
 // one barrier per tile.
+//
+// A wavefront gets ~29 B/clk out of LDS, about what its matrix instructions consume, so operand reads
+// are issued ahead of their use: the first product keeps four K operand pairs in flight, and the first
+// V operands of the second product are requested before the softmax arithmetic starts.
+//
+// With `paired` set a workgroup handles query tile (last - i) and then tile i of a head: under a causal
+// mask all workgroups then walk the same number of key tiles, which evens out the end of the launch.
 #pragma once
 
 #include "ahpc_device.hpp"
@@ -43,7 +53,8 @@ struct FlashParams {
     int32_t N;                  // sequence length (dense) / longest sequence (ragged)
     int32_t H;
     int32_t n_qtiles;           // query tiles per sequence (of the longest one)
-    int32_t total_blocks;       // B * H * n_qtiles
+    int32_t paired;             // 1: a workgroup takes two query tiles of a head (see above)
+    int32_t total_blocks;       // B * H * n_qtiles, or B * H * ceil(n_qtiles / 2) when paired
     int32_t blocks_per_xcd;     // ceil(total_blocks / 8)
     float scale_log2;           // scale * log2(e)
 };
@@ -53,7 +64,6 @@ constexpr int kFlashRows = 128;  // query rows per workgroup
 constexpr int kFlashKeys = 64;   // keys per tile
 
 #define AHPC_LDS __attribute__((address_space(3)))
-#define AHPC_GLOBAL __attribute__((address_space(1)))
 
 template <typename T> struct TrRead;
 template <> struct TrRead<bf16_t> {
@@ -92,35 +102,19 @@ template <int D> struct FlashTile {
     __device__ static int fv(int row) { return D == 128 ? 4 * (row & 3) : 4 * ((row >> 1) & 1); }
 };
 
-// Streams one 64-key tile (K or V) from global memory into LDS.  Rows past the end of the sequence
-// re-read the last valid row (their scores are masked; V rows are zeroed afterwards by the caller).
-template <typename T, int D, bool IS_V>
-__device__ inline void dma_tile(const T* g, int64_t sn, int k0, int L, unsigned char* lds_tile, int wave, int lane) {
+// Streams one 64-key tile (K or V) from global memory into LDS through a buffer descriptor.
+// `base` = first row of the tile, `nrec` = bytes that may be read from there on (anything beyond reads
+// as zero), off[i] = this lane's byte offset for its i-th instruction, wave_u = wavefront index (uniform).
+template <int D>
+__device__ inline void dma_tile(const void* base, unsigned nrec, const int* off, unsigned char* lds_tile, int wave_u) {
     typedef FlashTile<D> TL;
+#if defined(__HIP_DEVICE_COMPILE__)  // the descriptor type exists only in the device pass
+    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, nrec, 0x00020000);
 #pragma unroll
-    for (int i = 0; i < TL::kInstrPerWave; ++i) {
-        const int instr = wave * TL::kInstrPerWave + i;
-        const int r = instr * TL::kRowsPerInstr + lane / TL::kChunks;
-        const int pc = lane % TL::kChunks;
-        const int c = pc ^ (IS_V ? TL::fv(r) : TL::fk(r));
-        int key = k0 + r;
-        key = key < L ? key : L - 1;
-        const T* src = g + (int64_t)key * sn + c * 8;
-        __builtin_amdgcn_global_load_lds((const AHPC_GLOBAL void*)src, (AHPC_LDS void*)(lds_tile + instr * 1024), 16, 0, 0);
-    }
-}
-
-// Full tiles: every lane's byte offset from the tile's first row is fixed for the whole kernel
-// (`off[i]`, computed once); per tile only the uniform row base moves.
-template <typename T, int D>
-__device__ inline void dma_tile_fast(const T* tile_base, const int* off, unsigned char* lds_tile, int wave) {
-    typedef FlashTile<D> TL;
-    const char* b = reinterpret_cast<const char*>(tile_base);
-#pragma unroll
-    for (int i = 0; i < TL::kInstrPerWave; ++i) {
-        const int instr = wave * TL::kInstrPerWave + i;
-        __builtin_amdgcn_global_load_lds((const AHPC_GLOBAL void*)(b + (unsigned)off[i]), (AHPC_LDS void*)(lds_tile + instr * 1024), 16, 0, 0);
-    }
+    for (int i = 0; i < TL::kInstrPerWave; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (AHPC_LDS void*)(lds_tile + (wave_u * TL::kInstrPerWave + i) * 1024), 16,
+                                                 off[i], 0, 0, 0);
+#endif
 }
 
 template <typename T, int D, bool CAUSAL, bool VARLEN>
@@ -142,13 +136,15 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
     const int col = lane & 31;   // query column / operand row owned by this lane
     const int half = lane >> 5;
 
-    // Workgroup id -> (sequence*head, query tile).  Consecutive logical ids run on the same XCD so
-    // that the tiles of one head share that XCD's L2; within a head the long (late) tiles go first.
+    // Workgroup id -> (sequence*head, query tile or pair of tiles).  Consecutive logical ids run on the
+    // same XCD so that the tiles of one head share that XCD's L2; within a head the long (late) tiles
+    // go first.
     const int xcd = blockIdx.x & 7;
     const int logical = xcd * p.blocks_per_xcd + (blockIdx.x >> 3);
     if (logical >= p.total_blocks) return;
-    const int bh = logical / p.n_qtiles;
-    const int qt = p.n_qtiles - 1 - (logical - bh * p.n_qtiles);
+    const int per_head = p.paired ? (p.n_qtiles + 1) >> 1 : p.n_qtiles;
+    const int bh = logical / per_head;
+    const int slot = logical - bh * per_head;
     const int b = bh / p.H;
     const int h = bh - b * p.H;
 
@@ -162,18 +158,12 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
         L = p.N;
         base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
     }
-    const int q_tile0 = qt * kFlashRows;
-    if (q_tile0 >= L) return;
-
     const T* const gq = static_cast<const T*>(p.q) + base;
     const T* const gk = static_cast<const T*>(p.k) + base;
     const T* const gv = static_cast<const T*>(p.v) + base;
     T* const go = static_cast<T*>(p.o) + base;
     const int64_t sn = p.stride_n;
-
-    int k_end = L;
-    if (CAUSAL) k_end = (q_tile0 + kFlashRows) < L ? (q_tile0 + kFlashRows) : L;
-    const int n_tiles = (k_end + kFlashKeys - 1) / kFlashKeys;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
 
     // ---- per-lane DMA offsets (bytes from the first row of a tile), fixed for the whole kernel ------
     int dma_off_k[TL::kInstrPerWave], dma_off_v[TL::kInstrPerWave];
@@ -184,36 +174,15 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
         dma_off_k[i] = (int)(r * sn * 2) + ((pc ^ TL::fk(r)) << 4);
         dma_off_v[i] = (int)(r * sn * 2) + ((pc ^ TL::fv(r)) << 4);
     }
+    // Keys k0.. of this head into a buffer pair.  Bytes from the tile's first row to the end of the
+    // sequence's last row bound the descriptor, so the rows of a ragged last tile that do not exist
+    // read as zeros (their scores are masked; zero V rows keep 0 * x finite).
     auto dma_both = [&](int k0, unsigned char* dst_k, unsigned char* dst_v) {
-        if (k0 + kFlashKeys <= L) {
-            dma_tile_fast<T, D>(gk + (int64_t)k0 * sn, dma_off_k, dst_k, wave);
-            dma_tile_fast<T, D>(gv + (int64_t)k0 * sn, dma_off_v, dst_v, wave);
-        } else {  // ragged last tile: rows are clamped lane by lane
-            dma_tile<T, D, false>(gk, sn, k0, L, dst_k, wave, lane);
-            dma_tile<T, D, true>(gv, sn, k0, L, dst_v, wave, lane);
-        }
+        const int64_t rem = (int64_t)(L - k0 - 1) * sn * 2 + 2 * D;
+        const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
+        dma_tile<D>(gk + (int64_t)k0 * sn, nrec, dma_off_k, dst_k, wave_u);
+        dma_tile<D>(gv + (int64_t)k0 * sn, nrec, dma_off_v, dst_v, wave_u);
     };
-
-    // first tile on its way before anything else
-    dma_both(0, lds_k0, lds_v0);
-
-    // ---- Q^T operands, pre-multiplied by c = scale*log2(e), kept for the whole kernel -------------
-    const int qw = q_tile0 + wave * 32;  // first query row of this wavefront
-    const int qrow = qw + col;
-    u32x4 qreg[KS];
-    {
-        const int row = qrow < L ? qrow : L - 1;
-        const T* src = gq + (int64_t)row * sn + 8 * half;
-        const float c = p.scale_log2;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            const u32x4 raw = *reinterpret_cast<const u32x4*>(src + 16 * ks);
-            u32x4 sc;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) sc[w] = pack2<T>(lo_f32<T>(raw[w]) * c, hi_f32<T>(raw[w]) * c);
-            qreg[ks] = sc;
-        }
-    }
 
     // ---- LDS operand addresses (byte offsets inside a tile) -------------------------------------
     // K: lane reads row (32*kb + col), logical chunk 2*ks + half
@@ -231,150 +200,202 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
         v_off[mb] = vkey * RB + ((cch ^ TL::fv(vkey)) << 4) + 8 * (vi & 1);
     }
 
-    // ---- running state ----------------------------------------------------------------------------
-    // All score arithmetic is in log2 units (c is folded into Q).  `neg_m` = -(reference maximum) of the
-    // lane's query row, as a 16-wide vector because it is the C operand of the first k-step.
-    f32x16 oacc[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[mb][r] = 0.0f;
-    f32x16 neg_m;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) neg_m[r] = 0.0f;
-    float l_run = 0.0f;
-    bool first = true;
-    constexpr float kRaise = 8.0f;  // raise the reference maximum only when exceeded by 2^8
-
-    auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int k0) {
-        // ---- S^T = c*K Q^T - m  (log2 units) -------------------------------------------------------
-        f32x16 s[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-            u32x4 a[KS];
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) a[ks] = *reinterpret_cast<const u32x4*>(tile_k + kb * 32 * RB + k_off[ks]);
-            s[kb] = mfma_32x32x16<T>(a[0], qreg[0], neg_m);
-#pragma unroll
-            for (int ks = 1; ks < KS; ++ks) s[kb] = mfma_32x32x16<T>(a[ks], qreg[ks], s[kb]);
+    for (int part = 0; part < 2; ++part) {
+        int qt;
+        if (p.paired) {
+            if (part == 1 && 2 * slot == p.n_qtiles - 1) break;  // odd count: the middle tile has no partner
+            qt = part == 0 ? p.n_qtiles - 1 - slot : slot;
+        } else {
+            if (part == 1) break;
+            qt = p.n_qtiles - 1 - slot;
         }
+        const int q_tile0 = qt * kFlashRows;
+        if (q_tile0 >= L) continue;
 
-        const bool need_mask = (k0 + kFlashKeys > L) || (CAUSAL && (k0 + kFlashKeys - 1 > qw));
-        if (need_mask) {
-            // key = k0 + 4*half + off(kb, r); visible iff key <= min(qrow, L-1)  <=>  off <= lim
-            int lim = L - 1;
-            if (CAUSAL) lim = qrow < lim ? qrow : lim;
-            lim -= k0 + 4 * half;
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int off = 32 * kb + 8 * (r >> 2) + (r & 3);
-                    s[kb][r] = off <= lim ? s[kb][r] : -INFINITY;
-                }
-        }
-        // ---- reference maximum: exact on the first tile, afterwards raised only when a score tops it
-        //      by more than kRaise (rare, and the only time the accumulators are rescaled) ---------------
-        float mx = fmaxf(s[0][0], s[1][0]);
-#pragma unroll
-        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
-        if (first || __builtin_amdgcn_ballot_w64(mx > kRaise) != 0) {
-            mx = halves_max(mx);                       // both lanes of a query agree
-            const float delta = first ? mx : fmaxf(mx, 0.0f);
-            const float alpha = fast_exp2(-delta);
-            l_run *= alpha;
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) oacc[mb][r] *= alpha;
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) s[kb][r] -= delta;
-            const float nm = neg_m[0] - delta;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) neg_m[r] = nm;
-            first = false;
-        }
+        int k_end = L;
+        if (CAUSAL) k_end = (q_tile0 + kFlashRows) < L ? (q_tile0 + kFlashRows) : L;
+        const int n_tiles = (k_end + kFlashKeys - 1) / kFlashKeys;
 
-        // ---- P^T = exp2(S^T), packed as B operands; row sums in fp32 ------------------------------------
-        u32x4 pb[4];
-        float sum = 0.0f;
+        // first tile on its way before anything else
+        dma_both(0, lds_k0, lds_v0);
+
+        // ---- Q^T operands, pre-multiplied by c = scale*log2(e), kept for the whole query tile --------
+        const int qw = q_tile0 + wave * 32;  // first query row of this wavefront
+        const int qrow = qw + col;
+        u32x4 qreg[KS];
+        {
+            const int row = qrow < L ? qrow : L - 1;
+            const T* src = gq + (int64_t)row * sn + 8 * half;
+            const float c = p.scale_log2;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int kb = g >> 1, r0 = 8 * (g & 1);
+            for (int ks = 0; ks < KS; ++ks) {
+                const u32x4 raw = *reinterpret_cast<const u32x4*>(src + 16 * ks);
+                u32x4 sc;
 #pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const float p0 = fast_exp2(s[kb][r0 + 2 * w]), p1 = fast_exp2(s[kb][r0 + 2 * w + 1]);
-                pb[g][w] = pack2<T>(p0, p1);
-                sum += p0 + p1;  // plain adds co-issue with the matrix pipe; v_dot2 does not
+                for (int w = 0; w < 4; ++w) sc[w] = pack2<T>(lo_f32<T>(raw[w]) * c, hi_f32<T>(raw[w]) * c);
+                qreg[ks] = sc;
             }
         }
-        l_run += sum;
 
-        // ---- O^T += V^T P^T ------------------------------------------------------------------------------
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const u32x2 lo = TrRead<T>::load(tile_v + v_off[mb] + (16 * g) * RB);
-                const u32x2 hi = TrRead<T>::load(tile_v + v_off[mb] + (16 * g + 8) * RB);
-                oacc[mb] = mfma_32x32x16<T>(u32x4{lo[0], lo[1], hi[0], hi[1]}, pb[g], oacc[mb]);
-            }
-        }
-    };
-
-    // Zeroes the V rows of a tile that lie past the end of the sequence (they hold copies of the last
-    // row, and 0 * inf would poison the accumulators).
-    auto clear_v_tail = [&](unsigned char* tile_v, int k0) {
-        const int first_bad = L - k0;  // first invalid row, 1..63
-        for (int i = tid; i < (kFlashKeys - first_bad) * (RB / 16); i += kFlashThreads) {
-            const int r = first_bad + i / (RB / 16);
-            *reinterpret_cast<u32x4*>(tile_v + r * RB + (i % (RB / 16)) * 16) = u32x4{0u, 0u, 0u, 0u};
-        }
-    };
-
-    auto step = [&](unsigned char* cur_k, unsigned char* cur_v, unsigned char* nxt_k, unsigned char* nxt_v, int t) {
-        const int k0 = t * kFlashKeys;
-        const bool more = t + 1 < n_tiles;
-        if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
-        // a wavefront whose queries all precede this tile has nothing to add
-        if (!(CAUSAL && k0 > qw + 31)) compute_tile(cur_k, cur_v, k0);
-        if (more) {
-            __builtin_amdgcn_s_waitcnt(0);  // this wave's part of the next tile has landed
-            __syncthreads();                // everyone's has, and everyone is done with the current one
-            if (k0 + 2 * kFlashKeys > L) {
-                clear_v_tail(nxt_v, k0 + kFlashKeys);
-                __syncthreads();
-            }
-        }
-    };
-
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    if (kFlashKeys > L) {
-        clear_v_tail(lds_v0, 0);
-        __syncthreads();
-    }
-    for (int t = 0; t < n_tiles; t += 2) {
-        step(lds_k0, lds_v0, lds_k1, lds_v1, t);
-        if (t + 1 < n_tiles) step(lds_k1, lds_v1, lds_k0, lds_v0, t + 1);
-    }
-
-    // ---- normalise and store: lane holds, per 32-row block, 4 runs of 4 consecutive lanes of d -----
-    const float l = halves_sum(l_run);
-    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    if (qrow < L) {
-        T* dst = go + (int64_t)qrow * sn + 4 * half;
+        // ---- running state ------------------------------------------------------------------------
+        // All score arithmetic is in log2 units (c is folded into Q).  `neg_m` = -(reference maximum) of
+        // the lane's query row, as a 16-wide vector because it is the C operand of the first k-step.
+        f32x16 oacc[MB];
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const f32x16& a = oacc[mb];
-                const u32x2 w = u32x2{pack2<T>(a[4 * g4 + 0] * inv, a[4 * g4 + 1] * inv),
-                                      pack2<T>(a[4 * g4 + 2] * inv, a[4 * g4 + 3] * inv)};
-                *reinterpret_cast<u32x2*>(dst + 32 * mb + 8 * g4) = w;
+            for (int r = 0; r < 16; ++r) oacc[mb][r] = 0.0f;
+        f32x16 neg_m;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) neg_m[r] = 0.0f;
+        float l_run = 0.0f;
+        bool first = true;
+        constexpr float kRaise = 8.0f;  // raise the reference maximum only when exceeded by 2^8
+
+        auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int k0) {
+            // ---- S^T = c*K Q^T - m  (log2 units).  The two 32-key blocks alternate, kAhead operand
+            //      pairs are requested before the first product and one more after every two products.
+            f32x16 s[2];
+            {
+                u32x4 a0[KS], a1[KS];
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    a0[ks] = *reinterpret_cast<const u32x4*>(tile_k + k_off[ks]);
+                    a1[ks] = *reinterpret_cast<const u32x4*>(tile_k + 32 * RB + k_off[ks]);
+                }
+                s[0] = mfma_32x32x16<T>(a0[0], qreg[0], neg_m);
+                s[1] = mfma_32x32x16<T>(a1[0], qreg[0], neg_m);
+#pragma unroll
+                for (int ks = 1; ks < KS; ++ks) {
+                    s[0] = mfma_32x32x16<T>(a0[ks], qreg[ks], s[0]);
+                    s[1] = mfma_32x32x16<T>(a1[ks], qreg[ks], s[1]);
+                }
+                constexpr int kAhead = KS < 4 ? KS : 4;
+                __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);  // LDS reads
+#pragma unroll
+                for (int i = 0; i < KS - kAhead; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // matrix instructions
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < kAhead; ++i) __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
             }
+            // V operands of the first 16 keys: requested now, used after the softmax arithmetic
+            u32x2 vf[4][MB][2];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                vf[0][mb][0] = TrRead<T>::load(tile_v + v_off[mb]);
+                vf[0][mb][1] = TrRead<T>::load(tile_v + v_off[mb] + 8 * RB);
+            }
+
+            const bool need_mask = (k0 + kFlashKeys > L) || (CAUSAL && (k0 + kFlashKeys - 1 > qw));
+            if (need_mask) {
+                // key = k0 + 4*half + off(kb, r); visible iff key <= min(qrow, L-1)  <=>  off <= lim
+                int lim = L - 1;
+                if (CAUSAL) lim = qrow < lim ? qrow : lim;
+                lim -= k0 + 4 * half;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int off = 32 * kb + 8 * (r >> 2) + (r & 3);
+                        s[kb][r] = off <= lim ? s[kb][r] : -INFINITY;
+                    }
+            }
+            // ---- reference maximum: exact on the first tile, afterwards raised only when a score tops
+            //      it by more than kRaise (rare, and the only time the accumulators are rescaled) ------
+            float mx = fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+            for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
+            if (first || __builtin_amdgcn_ballot_w64(mx > kRaise) != 0) {
+                mx = halves_max(mx);                       // both lanes of a query agree
+                const float delta = first ? mx : fmaxf(mx, 0.0f);
+                const float alpha = fast_exp2(-delta);
+                l_run *= alpha;
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[mb][r] *= alpha;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) s[kb][r] -= delta;
+                const float nm = neg_m[0] - delta;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) neg_m[r] = nm;
+                first = false;
+            }
+
+            // ---- P^T = exp2(S^T) packed as B operands (row sums in fp32), and O^T += V^T P^T, 16 keys
+            //      at a time: while the matrix core works on group g the VALU prepares group g+1 and LDS
+            //      delivers its V operands.  The scheduling fences keep the groups apart.
+            u32x4 pb[4];
+            float sum = 0.0f;
+            auto make_pb = [&](int g) {
+                const int kb = g >> 1, r0 = 8 * (g & 1);
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const float p0 = fast_exp2(s[kb][r0 + 2 * w]), p1 = fast_exp2(s[kb][r0 + 2 * w + 1]);
+                    pb[g][w] = pack2<T>(p0, p1);
+                    sum += p0 + p1;  // plain adds co-issue with the matrix pipe; v_dot2 does not
+                }
+            };
+            make_pb(0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+                    oacc[mb] = mfma_32x32x16<T>(u32x4{vf[g][mb][0][0], vf[g][mb][0][1], vf[g][mb][1][0], vf[g][mb][1][1]},
+                                                pb[g], oacc[mb]);
+                if (g < 3) {
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) {
+                        vf[g + 1][mb][0] = TrRead<T>::load(tile_v + v_off[mb] + (16 * (g + 1)) * RB);
+                        vf[g + 1][mb][1] = TrRead<T>::load(tile_v + v_off[mb] + (16 * (g + 1) + 8) * RB);
+                    }
+                    make_pb(g + 1);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            l_run += sum;
+        };
+
+        auto step = [&](unsigned char* cur_k, unsigned char* cur_v, unsigned char* nxt_k, unsigned char* nxt_v, int t) {
+            const int k0 = t * kFlashKeys;
+            const bool more = t + 1 < n_tiles;
+            if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
+            // a wavefront whose queries all precede this tile has nothing to add
+            if (!(CAUSAL && k0 > qw + 31)) compute_tile(cur_k, cur_v, k0);
+            if (more) {
+                __builtin_amdgcn_s_waitcnt(0);  // this wave's part of the next tile has landed
+                __syncthreads();                // everyone's has, and everyone is done with the current one
+            }
+        };
+
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        for (int t = 0; t < n_tiles; t += 2) {
+            step(lds_k0, lds_v0, lds_k1, lds_v1, t);
+            if (t + 1 < n_tiles) step(lds_k1, lds_v1, lds_k0, lds_v0, t + 1);
+        }
+
+        // ---- normalise and store: lane holds, per 32-row block, 4 runs of 4 consecutive lanes of d ---
+        const float l = halves_sum(l_run);
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+        if (qrow < L) {
+            T* dst = go + (int64_t)qrow * sn + 4 * half;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const f32x16& a = oacc[mb];
+                    const u32x2 w = u32x2{pack2<T>(a[4 * g4 + 0] * inv, a[4 * g4 + 1] * inv),
+                                          pack2<T>(a[4 * g4 + 2] * inv, a[4 * g4 + 3] * inv)};
+                    *reinterpret_cast<u32x2*>(dst + 32 * mb + 8 * g4) = w;
+                }
+        }
+        __syncthreads();  // the next query tile's first DMA reuses the buffers
     }
 }
 
