@@ -22,8 +22,10 @@ struct SimpleParams {
     void* o;
     const int32_t* cu_seqlens;
     const float* mask;          // [B,N,N] or null
-    int64_t stride_b, stride_n, stride_h;
+    int64_t stride_b, stride_n, stride_h;           // Q and O
+    int64_t kv_stride_b, kv_stride_n, kv_stride_h;  // K and V
     int32_t N, H, d;
+    int32_t kv_group;           // query heads per key/value head
     float scale;
     int32_t causal;
 };
@@ -39,14 +41,17 @@ __global__ __launch_bounds__(kSimpleRows) void flash_fwd_simple_kernel(const Sim
     const int tid = threadIdx.x;
     const int h = blockIdx.y, b = blockIdx.z;
     int L;
-    int64_t base;
+    int64_t base, kv_base;
+    const int hk = h / p.kv_group;
     if (VARLEN) {
         const int s0 = p.cu_seqlens[b];
         L = p.cu_seqlens[b + 1] - s0;
         base = (int64_t)s0 * p.stride_n + (int64_t)h * p.stride_h;
+        kv_base = (int64_t)s0 * p.kv_stride_n + (int64_t)hk * p.kv_stride_h;
     } else {
         L = p.N;
         base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+        kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
     }
     const int row0 = blockIdx.x * kSimpleRows;
     if (row0 >= L) return;
@@ -55,8 +60,8 @@ __global__ __launch_bounds__(kSimpleRows) void flash_fwd_simple_kernel(const Sim
     const int d = p.d;
 
     const T* gq = static_cast<const T*>(p.q) + base;
-    const T* gk = static_cast<const T*>(p.k) + base;
-    const T* gv = static_cast<const T*>(p.v) + base;
+    const T* gk = static_cast<const T*>(p.k) + kv_base;
+    const T* gv = static_cast<const T*>(p.v) + kv_base;
 
     float qv[DP], acc[DP];
 #pragma unroll
@@ -82,8 +87,8 @@ __global__ __launch_bounds__(kSimpleRows) void flash_fwd_simple_kernel(const Sim
             const int key = k0 + kr;
             float kx = 0.0f, vx = 0.0f;
             if (key < L) {
-                kx = Storage<T>::load(gk + (int64_t)key * p.stride_n + e);
-                vx = Storage<T>::load(gv + (int64_t)key * p.stride_n + e);
+                kx = Storage<T>::load(gk + (int64_t)key * p.kv_stride_n + e);
+                vx = Storage<T>::load(gv + (int64_t)key * p.kv_stride_n + e);
             }
             sk[kr][e] = kx;
             sv[kr][e] = vx;
@@ -171,24 +176,29 @@ static int dispatch_mfma(const FlashParams& p, int64_t B, int d, bool causal, hi
 
 static bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 
+struct Strides {
+    int64_t b, n, h;
+};
+
 static bool mfma_eligible(int dtype, int64_t d, const void* q, const void* k, const void* v, const void* o,
-                          int64_t s0, int64_t s1, int64_t s2) {
+                          const Strides& sq, const Strides& skv) {
     if (dtype != AHPC_F16 && dtype != AHPC_BF16) return false;
     if (d != 64 && d != 128) return false;
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return false;
-    if ((s0 % 8) || (s1 % 8) || (s2 % 8)) return false;
+    if ((sq.b % 8) || (sq.n % 8) || (sq.h % 8) || (skv.b % 8) || (skv.n % 8) || (skv.h % 8)) return false;
     // a key tile is addressed with 32-bit byte offsets from its first row, and rows must not overlap
-    return s1 >= d && s1 < (int64_t(1) << 24);
+    return sq.n >= d && skv.n >= d && skv.n < (int64_t(1) << 24);
 }
 
 static int check_dense(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N, int64_t H,
-                       int64_t d, int64_t sb, int64_t sn, int64_t sh) {
+                       int64_t H_kv, int64_t d, const Strides& sq, const Strides& skv) {
     if (!q || !k || !v || !o) return AHPC_ERR_NULL_POINTER;
     if (dtype < AHPC_F32 || dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
-    if (B <= 0 || N <= 0 || H <= 0 || d <= 0) return AHPC_ERR_BAD_SHAPE;
+    if (B <= 0 || N <= 0 || H <= 0 || d <= 0 || H_kv <= 0) return AHPC_ERR_BAD_SHAPE;
+    if (H % H_kv) return AHPC_ERR_BAD_SHAPE;  // every K/V head serves the same number of query heads
     if (B > 65535 || H > 65535 || N > 0x7FFFFF00ll) return AHPC_ERR_BAD_SHAPE;
     if (d > 256) return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
-    if (sn < d || sh < d || sb < 0) return AHPC_ERR_BAD_SHAPE;
+    if (sq.n < d || sq.h < d || sq.b < 0 || skv.n < d || skv.h < d || skv.b < 0) return AHPC_ERR_BAD_SHAPE;
     return AHPC_OK;
 }
 
@@ -198,53 +208,81 @@ using namespace ahpc;
 
 extern "C" {
 
+int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N, int64_t H,
+                           int64_t H_kv, int64_t d, int64_t stride_b, int64_t stride_n, int64_t stride_h,
+                           int64_t kv_stride_b, int64_t kv_stride_n, int64_t kv_stride_h, float scale, int causal,
+                           const float* mask, void* stream) {
+    const Strides sq{stride_b, stride_n, stride_h}, skv{kv_stride_b, kv_stride_n, kv_stride_h};
+    if (int rc = check_dense(q, k, v, o, dtype, B, N, H, H_kv, d, sq, skv)) return rc;
+    if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int32_t group = (int32_t)(H / H_kv);
+    if (!mask && mfma_eligible(dtype, d, q, k, v, o, sq, skv)) {
+        FlashParams p{};
+        p.q = q; p.k = k; p.v = v; p.o = o;
+        p.stride_b = sq.b; p.stride_n = sq.n; p.stride_h = sq.h;
+        p.kv_stride_b = skv.b; p.kv_stride_n = skv.n; p.kv_stride_h = skv.h;
+        p.N = (int32_t)N; p.H = (int32_t)H; p.kv_group = group;
+        p.scale_log2 = scale * kLog2e;
+        return dtype == AHPC_F16 ? dispatch_mfma<f16_t, false>(p, B, (int)d, causal != 0, st)
+                                 : dispatch_mfma<bf16_t, false>(p, B, (int)d, causal != 0, st);
+    }
+    SimpleParams p{q, k, v, o, nullptr, mask, sq.b, sq.n, sq.h, skv.b, skv.n, skv.h, (int32_t)N, (int32_t)H, (int32_t)d, group, scale, causal ? 1 : 0};
+    return dispatch_simple<false>(dtype, p, B, st);
+}
+
 int ahpc_hip_flash_fwd_masked(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N,
                               int64_t H, int64_t d, int64_t stride_b, int64_t stride_n, int64_t stride_h, float scale,
                               int causal, const float* mask, void* stream) {
-    if (int rc = check_dense(q, k, v, o, dtype, B, N, H, d, stride_b, stride_n, stride_h)) return rc;
-    if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
-    SimpleParams p{q, k, v, o, nullptr, mask, stride_b, stride_n, stride_h, (int32_t)N, (int32_t)H, (int32_t)d, scale, causal ? 1 : 0};
-    return dispatch_simple<false>(dtype, p, B, static_cast<hipStream_t>(stream));
+    if (!mask) {
+        // no mask: still the fp32-FMA kernel, as documented for this entry point
+        const Strides s{stride_b, stride_n, stride_h};
+        if (int rc = check_dense(q, k, v, o, dtype, B, N, H, H, d, s, s)) return rc;
+        if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
+        SimpleParams p{q, k, v, o, nullptr, nullptr, s.b, s.n, s.h, s.b, s.n, s.h, (int32_t)N, (int32_t)H, (int32_t)d, 1, scale, causal ? 1 : 0};
+        return dispatch_simple<false>(dtype, p, B, static_cast<hipStream_t>(stream));
+    }
+    return ahpc_hip_flash_fwd_gqa(q, k, v, o, dtype, B, N, H, H, d, stride_b, stride_n, stride_h, stride_b, stride_n,
+                                  stride_h, scale, causal, mask, stream);
 }
 
 int ahpc_hip_flash_fwd(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N, int64_t H,
                        int64_t d, int64_t stride_b, int64_t stride_n, int64_t stride_h, float scale, int causal,
                        void* stream) {
-    if (int rc = check_dense(q, k, v, o, dtype, B, N, H, d, stride_b, stride_n, stride_h)) return rc;
+    return ahpc_hip_flash_fwd_gqa(q, k, v, o, dtype, B, N, H, H, d, stride_b, stride_n, stride_h, stride_b, stride_n,
+                                  stride_h, scale, causal, nullptr, stream);
+}
+
+int ahpc_hip_flash_fwd_varlen_gqa(const void* q, const void* k, const void* v, void* o, int dtype,
+                                  const int32_t* cu_seqlens, int64_t n_seqs, int64_t max_len, int64_t H, int64_t H_kv,
+                                  int64_t d, int64_t stride_t, int64_t stride_h, int64_t kv_stride_t, int64_t kv_stride_h,
+                                  float scale, int causal, void* stream) {
+    if (!cu_seqlens) return AHPC_ERR_NULL_POINTER;
+    const Strides sq{0, stride_t, stride_h}, skv{0, kv_stride_t, kv_stride_h};
+    if (int rc = check_dense(q, k, v, o, dtype, n_seqs, max_len, H, H_kv, d, sq, skv)) return rc;
     if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (mfma_eligible(dtype, d, q, k, v, o, stride_b, stride_n, stride_h)) {
+    const int32_t group = (int32_t)(H / H_kv);
+    if (mfma_eligible(dtype, d, q, k, v, o, sq, skv)) {
         FlashParams p{};
         p.q = q; p.k = k; p.v = v; p.o = o;
-        p.stride_b = stride_b; p.stride_n = stride_n; p.stride_h = stride_h;
-        p.N = (int32_t)N; p.H = (int32_t)H;
+        p.cu_seqlens = cu_seqlens;
+        p.stride_b = 0; p.stride_n = sq.n; p.stride_h = sq.h;
+        p.kv_stride_b = 0; p.kv_stride_n = skv.n; p.kv_stride_h = skv.h;
+        p.N = (int32_t)max_len; p.H = (int32_t)H; p.kv_group = group;
         p.scale_log2 = scale * kLog2e;
-        return dtype == AHPC_F16 ? dispatch_mfma<f16_t, false>(p, B, (int)d, causal != 0, st)
-                                 : dispatch_mfma<bf16_t, false>(p, B, (int)d, causal != 0, st);
+        return dtype == AHPC_F16 ? dispatch_mfma<f16_t, true>(p, n_seqs, (int)d, causal != 0, st)
+                                 : dispatch_mfma<bf16_t, true>(p, n_seqs, (int)d, causal != 0, st);
     }
-    SimpleParams p{q, k, v, o, nullptr, nullptr, stride_b, stride_n, stride_h, (int32_t)N, (int32_t)H, (int32_t)d, scale, causal ? 1 : 0};
-    return dispatch_simple<false>(dtype, p, B, st);
+    SimpleParams p{q, k, v, o, cu_seqlens, nullptr, 0, sq.n, sq.h, 0, skv.n, skv.h, (int32_t)max_len, (int32_t)H, (int32_t)d, group, scale, causal ? 1 : 0};
+    return dispatch_simple<true>(dtype, p, n_seqs, st);
 }
 
 int ahpc_hip_flash_fwd_varlen(const void* q, const void* k, const void* v, void* o, int dtype, const int32_t* cu_seqlens,
                               int64_t n_seqs, int64_t max_len, int64_t H, int64_t d, int64_t stride_t, int64_t stride_h,
                               float scale, int causal, void* stream) {
-    if (!cu_seqlens) return AHPC_ERR_NULL_POINTER;
-    if (int rc = check_dense(q, k, v, o, dtype, n_seqs, max_len, H, d, 0, stride_t, stride_h)) return rc;
-    if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    if (mfma_eligible(dtype, d, q, k, v, o, 0, stride_t, stride_h)) {
-        FlashParams p{};
-        p.q = q; p.k = k; p.v = v; p.o = o;
-        p.cu_seqlens = cu_seqlens;
-        p.stride_b = 0; p.stride_n = stride_t; p.stride_h = stride_h;
-        p.N = (int32_t)max_len; p.H = (int32_t)H;
-        p.scale_log2 = scale * kLog2e;
-        return dtype == AHPC_F16 ? dispatch_mfma<f16_t, true>(p, n_seqs, (int)d, causal != 0, st)
-                                 : dispatch_mfma<bf16_t, true>(p, n_seqs, (int)d, causal != 0, st);
-    }
-    SimpleParams p{q, k, v, o, cu_seqlens, nullptr, 0, stride_t, stride_h, (int32_t)max_len, (int32_t)H, (int32_t)d, scale, causal ? 1 : 0};
-    return dispatch_simple<true>(dtype, p, n_seqs, st);
+    return ahpc_hip_flash_fwd_varlen_gqa(q, k, v, o, dtype, cu_seqlens, n_seqs, max_len, H, H, d, stride_t, stride_h,
+                                         stride_t, stride_h, scale, causal, stream);
 }
 
 }  // extern "C"

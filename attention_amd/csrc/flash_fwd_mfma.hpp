@@ -49,9 +49,11 @@ struct FlashParams {
     const void* v;
     void* o;
     const int32_t* cu_seqlens;  // ragged batches only
-    int64_t stride_b, stride_n, stride_h;
+    int64_t stride_b, stride_n, stride_h;           // Q and O
+    int64_t kv_stride_b, kv_stride_n, kv_stride_h;  // K and V
     int32_t N;                  // sequence length (dense) / longest sequence (ragged)
-    int32_t H;
+    int32_t H;                  // query heads
+    int32_t kv_group;           // query heads per key/value head (1 = every head has its own K/V)
     int32_t n_qtiles;           // query tiles per sequence (of the longest one)
     int32_t paired;             // 1: a workgroup takes two query tiles of a head (see above)
     int32_t total_blocks;       // B * H * n_qtiles, or B * H * ceil(n_qtiles / 2) when paired
@@ -149,20 +151,24 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
     const int h = bh - b * p.H;
 
     int L;
-    int64_t base;
+    int64_t base, kv_base;
+    const int hk = h / p.kv_group;  // grouped-query attention: consecutive query heads share a K/V head
     if (VARLEN) {
         const int s0 = p.cu_seqlens[b];
         L = p.cu_seqlens[b + 1] - s0;
         base = (int64_t)s0 * p.stride_n + (int64_t)h * p.stride_h;
+        kv_base = (int64_t)s0 * p.kv_stride_n + (int64_t)hk * p.kv_stride_h;
     } else {
         L = p.N;
         base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+        kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
     }
     const T* const gq = static_cast<const T*>(p.q) + base;
-    const T* const gk = static_cast<const T*>(p.k) + base;
-    const T* const gv = static_cast<const T*>(p.v) + base;
+    const T* const gk = static_cast<const T*>(p.k) + kv_base;
+    const T* const gv = static_cast<const T*>(p.v) + kv_base;
     T* const go = static_cast<T*>(p.o) + base;
     const int64_t sn = p.stride_n;
+    const int64_t skv = p.kv_stride_n;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
 
     // ---- per-lane DMA offsets (bytes from the first row of a tile), fixed for the whole kernel ------
@@ -171,17 +177,17 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
     for (int i = 0; i < TL::kInstrPerWave; ++i) {
         const int r = (wave * TL::kInstrPerWave + i) * TL::kRowsPerInstr + lane / TL::kChunks;
         const int pc = lane % TL::kChunks;
-        dma_off_k[i] = (int)(r * sn * 2) + ((pc ^ TL::fk(r)) << 4);
-        dma_off_v[i] = (int)(r * sn * 2) + ((pc ^ TL::fv(r)) << 4);
+        dma_off_k[i] = (int)(r * skv * 2) + ((pc ^ TL::fk(r)) << 4);
+        dma_off_v[i] = (int)(r * skv * 2) + ((pc ^ TL::fv(r)) << 4);
     }
     // Keys k0.. of this head into a buffer pair.  Bytes from the tile's first row to the end of the
     // sequence's last row bound the descriptor, so the rows of a ragged last tile that do not exist
     // read as zeros (their scores are masked; zero V rows keep 0 * x finite).
     auto dma_both = [&](int k0, unsigned char* dst_k, unsigned char* dst_v) {
-        const int64_t rem = (int64_t)(L - k0 - 1) * sn * 2 + 2 * D;
+        const int64_t rem = (int64_t)(L - k0 - 1) * skv * 2 + 2 * D;
         const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
-        dma_tile<D>(gk + (int64_t)k0 * sn, nrec, dma_off_k, dst_k, wave_u);
-        dma_tile<D>(gv + (int64_t)k0 * sn, nrec, dma_off_v, dst_v, wave_u);
+        dma_tile<D>(gk + (int64_t)k0 * skv, nrec, dma_off_k, dst_k, wave_u);
+        dma_tile<D>(gv + (int64_t)k0 * skv, nrec, dma_off_v, dst_v, wave_u);
     };
 
     // ---- LDS operand addresses (byte offsets inside a tile) -------------------------------------

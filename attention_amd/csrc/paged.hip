@@ -90,7 +90,8 @@ struct DecodeParams {
     float* part_o;    // [B][n_chunks][H][d]
     float* part_ml;   // [B][n_chunks][H][2]  (m in log2 units, l)
     int64_t max_pages;
-    int32_t B, H, d, P;
+    int32_t B, H, d, P;       // H = query heads
+    int32_t H_kv;             // heads in the pool; H / H_kv consecutive query heads share one
     int32_t chunk_tokens, n_chunks;
     int32_t max_len;
     int32_t qo_dtype;
@@ -161,20 +162,18 @@ template <int LPH> __device__ __forceinline__ float head_allreduce(float x) {
     return x;
 }
 
-#ifndef AHPC_DECODE_BATCH
-#define AHPC_DECODE_BATCH 8
-#endif
-constexpr int kDecodeBatch = AHPC_DECODE_BATCH;  // tokens whose K and V rows are in flight together, per lane
-
 // T: pool element type.  D: head dimension.  PT: tokens per page when known at compile time (16), or 0
-// for any page size.  A lane owns EPL = 16/sizeof(T) consecutive elements of one head.  Grid: (chunk,
-// batch entry, head group); every wavefront works on its own heads and needs no LDS and no barrier.
+// for any page size.  G: query heads per pool head (grouped-query attention; 1 = one each).  A lane owns
+// EPL = 16/sizeof(T) consecutive elements of one pool head and serves the G query heads of that head
+// from the same K and V registers.  Grid: (head group, chunk, batch entry); every wavefront works on
+// its own heads and needs no LDS and no barrier.
 //
 // A chunk starts on a page boundary.  Its page ids are fetched once (one table entry per lane) and
 // handed out with v_readlane, so the only per-token address work is a uniform add; K and V rows of
-// the next 8 tokens are requested before the current 8 are consumed.
-template <typename T, int D, int PT>
+// the next kDecodeBatch tokens are requested before the current ones are consumed.
+template <typename T, int D, int PT, int G>
 __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p) {
+    constexpr int kDecodeBatch = G >= 4 ? 4 : 8;  // tokens whose K and V rows are in flight together, per lane
     constexpr int EPL = 16 / (int)sizeof(T);
     constexpr int LPH = D / EPL;
     constexpr int HPW = kWave / LPH;
@@ -188,9 +187,9 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     // token row are dispatched side by side and stream whole pages between them
     const int chunk = blockIdx.y;
     const int b = blockIdx.z;
-    const int h_raw = (blockIdx.x * waves + wave) * HPW + lane / LPH;
-    const bool head_ok = h_raw < p.H;
-    const int h = head_ok ? h_raw : p.H - 1;
+    const int h_raw = (blockIdx.x * waves + wave) * HPW + lane / LPH;  // pool head
+    const bool head_ok = h_raw < p.H_kv;
+    const int h = head_ok ? h_raw : p.H_kv - 1;
     const int e0 = (lane % LPH) * EPL;
     const int P = PT ? PT : p.P;
 
@@ -209,26 +208,28 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
             float zero[EPL];
 #pragma unroll
             for (int e = 0; e < EPL; ++e) zero[e] = 0.0f;
-            store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + h) * D + e0, zero);
+#pragma unroll
+            for (int g = 0; g < G; ++g) store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + h * G + g) * D + e0, zero);
         }
         return;
     }
     const int t1 = (t0 + p.chunk_tokens) < L ? (t0 + p.chunk_tokens) : L;
 
-    // query piece of this lane
-    float qf[EPL];
-    uint32_t qp[4];
-    {
-        load_qo_vec<EPL>(p.q, p.qo_dtype, ((int64_t)b * p.H + h) * D + e0, qf);
+    // query pieces of this lane, one per query head of the group
+    float qf[G][EPL];
+    uint32_t qp[G][4];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        load_qo_vec<EPL>(p.q, p.qo_dtype, ((int64_t)b * p.H + h * G + g) * D + e0, qf[g]);
         if (kPacked) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) qp[i] = pack2<TP>(qf[2 * i], qf[2 * i + 1]);
+            for (int i = 0; i < 4; ++i) qp[g][i] = pack2<TP>(qf[g][2 * i], qf[g][2 * i + 1]);
         }
     }
 
     // byte offset of this lane's piece inside a token row; token rows are tok_bytes apart
     const uint32_t lane_off = (uint32_t)((h * D + e0) * (int)sizeof(T));
-    const int64_t tok_bytes = (int64_t)p.H * D * (int64_t)sizeof(T);
+    const int64_t tok_bytes = (int64_t)p.H_kv * D * (int64_t)sizeof(T);
     const char* const kbase = static_cast<const char*>(p.k_pool);
     const char* const vbase = static_cast<const char*>(p.v_pool);
 
@@ -245,7 +246,7 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
         const int ti0 = bi * kDecodeBatch;
         const int last = n_tok - 1 - ti0;  // index of the last valid token of this batch (>= 0)
         if (PT == 16) {
-            // 8 consecutive slots of one page: one page id, rows tok_bytes apart
+            // consecutive slots of one page (the batch size divides 16): one page id, rows tok_bytes apart
             const int page_id = __builtin_amdgcn_readlane(my_page, ti0 >> 4);
             const int64_t base = ((int64_t)page_id * 16 + (ti0 & 15)) * tok_bytes;
 #pragma unroll
@@ -268,52 +269,60 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
         }
     };
 
-    float acc[EPL];
+    float acc[G][EPL];
+    float m[G], l[G];
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) acc[e] = 0.0f;
-    float m = -INFINITY, l = 0.0f;
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) acc[g][e] = 0.0f;
+        m[g] = -INFINITY;
+        l[g] = 0.0f;
+    }
     const float c = p.scale_log2;
 
     auto consume = [&](const u32x4 (&kc)[kDecodeBatch], const u32x4 (&vc)[kDecodeBatch], int bi) {
-        const int valid = n_tok - bi * kDecodeBatch;  // >= 1; >= 8 for all but the last batch
-        float s[kDecodeBatch];
-        float mx = -INFINITY;
+        const int valid = n_tok - bi * kDecodeBatch;  // >= 1; >= kDecodeBatch for all but the last batch
 #pragma unroll
-        for (int i = 0; i < kDecodeBatch; ++i) {
-            float part = 0.0f;
-            if (kPacked) {
+        for (int g = 0; g < G; ++g) {
+            float s[kDecodeBatch];
+            float mx = -INFINITY;
 #pragma unroll
-                for (int w = 0; w < 4; ++w) part = dot2<TP>(qp[w], kc[i][w], part);
-            } else {
+            for (int i = 0; i < kDecodeBatch; ++i) {
+                float part = 0.0f;
+                if (kPacked) {
 #pragma unroll
-                for (int w = 0; w < 4; ++w) part = __builtin_fmaf(qf[w % EPL], as_f32(kc[i][w]), part);
-            }
-            part = head_allreduce<LPH>(part);
-            s[i] = (i < valid) ? part * c : -INFINITY;
-            mx = fmaxf(mx, s[i]);
-        }
-        const float m_new = fmaxf(m, mx);              // finite: the batch holds at least one token
-        const float alpha = fast_exp2(m - m_new);      // first batch: exp2(-inf) = 0
-        float sum = 0.0f;
+                    for (int w = 0; w < 4; ++w) part = dot2<TP>(qp[g][w], kc[i][w], part);
+                } else {
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) acc[e] *= alpha;
-#pragma unroll
-        for (int i = 0; i < kDecodeBatch; ++i) {
-            const float w = fast_exp2(s[i] - m_new);
-            sum += w;
-            if (kPacked) {
-#pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    acc[(2 * x) % EPL] = __builtin_fmaf(w, lo_f32<TP>(vc[i][x]), acc[(2 * x) % EPL]);
-                    acc[(2 * x + 1) % EPL] = __builtin_fmaf(w, hi_f32<TP>(vc[i][x]), acc[(2 * x + 1) % EPL]);
+                    for (int w = 0; w < 4; ++w) part = __builtin_fmaf(qf[g][w % EPL], as_f32(kc[i][w]), part);
                 }
-            } else {
-#pragma unroll
-                for (int x = 0; x < 4; ++x) acc[x % EPL] = __builtin_fmaf(w, as_f32(vc[i][x]), acc[x % EPL]);
+                part = head_allreduce<LPH>(part);
+                s[i] = (i < valid) ? part * c : -INFINITY;
+                mx = fmaxf(mx, s[i]);
             }
+            const float m_new = fmaxf(m[g], mx);            // finite: the batch holds at least one token
+            const float alpha = fast_exp2(m[g] - m_new);    // first batch: exp2(-inf) = 0
+            float sum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) acc[g][e] *= alpha;
+#pragma unroll
+            for (int i = 0; i < kDecodeBatch; ++i) {
+                const float w = fast_exp2(s[i] - m_new);
+                sum += w;
+                if (kPacked) {
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        acc[g][(2 * x) % EPL] = __builtin_fmaf(w, lo_f32<TP>(vc[i][x]), acc[g][(2 * x) % EPL]);
+                        acc[g][(2 * x + 1) % EPL] = __builtin_fmaf(w, hi_f32<TP>(vc[i][x]), acc[g][(2 * x + 1) % EPL]);
+                    }
+                } else {
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) acc[g][x % EPL] = __builtin_fmaf(w, as_f32(vc[i][x]), acc[g][x % EPL]);
+                }
+            }
+            l[g] = l[g] * alpha + sum;
+            m[g] = m_new;
         }
-        l = l * alpha + sum;
-        m = m_new;
     };
 
     // two register sets in ping-pong: while one batch is consumed the next is in flight
@@ -329,20 +338,24 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     }
 
     if (!head_ok) return;
-    if (p.n_chunks == 1) {
-        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-        float res[EPL];
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) res[e] = acc[e] * inv;
-        store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + h) * D + e0, res);
-    } else {
-        const int64_t slot = ((int64_t)b * p.n_chunks + chunk) * p.H + h;
-        f32x4* dst = reinterpret_cast<f32x4*>(p.part_o + slot * D + e0);
+    for (int g = 0; g < G; ++g) {
+        const int hq = h * G + g;
+        if (p.n_chunks == 1) {
+            const float inv = l[g] > 0.0f ? 1.0f / l[g] : 0.0f;
+            float res[EPL];
 #pragma unroll
-        for (int e = 0; e < EPL; e += 4) dst[e / 4] = f32x4{acc[e], acc[e + 1], acc[e + 2], acc[e + 3]};
-        if (lane % LPH == 0) {
-            p.part_ml[slot * 2] = m;
-            p.part_ml[slot * 2 + 1] = l;
+            for (int e = 0; e < EPL; ++e) res[e] = acc[g][e] * inv;
+            store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + hq) * D + e0, res);
+        } else {
+            const int64_t slot = ((int64_t)b * p.n_chunks + chunk) * p.H + hq;
+            f32x4* dst = reinterpret_cast<f32x4*>(p.part_o + slot * D + e0);
+#pragma unroll
+            for (int e = 0; e < EPL; e += 4) dst[e / 4] = f32x4{acc[g][e], acc[g][e + 1], acc[g][e + 2], acc[g][e + 3]};
+            if (lane % LPH == 0) {
+                p.part_ml[slot * 2] = m[g];
+                p.part_ml[slot * 2 + 1] = l[g];
+            }
         }
     }
 }
@@ -399,16 +412,27 @@ static int64_t pick_chunk_tokens(int64_t B, int64_t H, int64_t max_len, int64_t 
     return chunk;
 }
 
-template <typename T, int PT>
-static int launch_decode_dp(const DecodeParams& p, dim3 grid, dim3 block, hipStream_t st) {
+template <typename T, int PT, int G>
+static int launch_decode_dpg(const DecodeParams& p, dim3 grid, dim3 block, hipStream_t st) {
     switch (p.d) {
-        case 32: hipLaunchKernelGGL((paged_decode_kernel<T, 32, PT>), grid, block, 0, st, p); break;
-        case 64: hipLaunchKernelGGL((paged_decode_kernel<T, 64, PT>), grid, block, 0, st, p); break;
-        case 128: hipLaunchKernelGGL((paged_decode_kernel<T, 128, PT>), grid, block, 0, st, p); break;
-        case 256: hipLaunchKernelGGL((paged_decode_kernel<T, 256, PT>), grid, block, 0, st, p); break;
+        case 32: hipLaunchKernelGGL((paged_decode_kernel<T, 32, PT, G>), grid, block, 0, st, p); break;
+        case 64: hipLaunchKernelGGL((paged_decode_kernel<T, 64, PT, G>), grid, block, 0, st, p); break;
+        case 128: hipLaunchKernelGGL((paged_decode_kernel<T, 128, PT, G>), grid, block, 0, st, p); break;
+        case 256: hipLaunchKernelGGL((paged_decode_kernel<T, 256, PT, G>), grid, block, 0, st, p); break;
         default: return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
     }
     return static_cast<int>(hipGetLastError());
+}
+
+template <typename T, int PT>
+static int launch_decode_dp(const DecodeParams& p, dim3 grid, dim3 block, hipStream_t st) {
+    switch (p.H / p.H_kv) {
+        case 1: return launch_decode_dpg<T, PT, 1>(p, grid, block, st);
+        case 2: return launch_decode_dpg<T, PT, 2>(p, grid, block, st);
+        case 4: return launch_decode_dpg<T, PT, 4>(p, grid, block, st);
+        case 8: return launch_decode_dpg<T, PT, 8>(p, grid, block, st);
+        default: return AHPC_ERR_UNSUPPORTED_GROUP;
+    }
 }
 
 template <typename T>
@@ -510,11 +534,13 @@ size_t ahpc_hip_paged_decode_workspace_bytes(int64_t B, int64_t H, int64_t d, in
     return (size_t)(B * n_chunks * H * (d + 2)) * sizeof(float);
 }
 
-int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype, const void* k_pool, const void* v_pool, int pool_dtype,
-                          const int32_t* block_table, const int32_t* seq_lens, const int32_t* batch_rows, int64_t B,
-                          int64_t H, int64_t d, int64_t P, int64_t max_pages, int64_t max_len, float scale,
-                          int64_t chunk_tokens, void* workspace, size_t workspace_bytes, void* stream) {
+int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* k_pool, const void* v_pool, int pool_dtype,
+                              const int32_t* block_table, const int32_t* seq_lens, const int32_t* batch_rows, int64_t B,
+                              int64_t H, int64_t H_kv, int64_t d, int64_t P, int64_t max_pages, int64_t max_len,
+                              float scale, int64_t chunk_tokens, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !o || !k_pool || !v_pool || !block_table || !seq_lens) return AHPC_ERR_NULL_POINTER;
+    if (H_kv <= 0 || H <= 0 || H % H_kv) return AHPC_ERR_BAD_SHAPE;
+    { const int64_t g = H / H_kv; if (g != 1 && g != 2 && g != 4 && g != 8) return AHPC_ERR_UNSUPPORTED_GROUP; }
     if (qo_dtype < AHPC_F32 || qo_dtype > AHPC_BF16 || pool_dtype < AHPC_F32 || pool_dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
     if (B <= 0 || B > 65535 || max_len <= 0 || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;
     if ((max_len + P - 1) / P > max_pages) return AHPC_ERR_BAD_SHAPE;
@@ -537,6 +563,7 @@ int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype, const void* k_po
     p.part_ml = p.part_o ? p.part_o + B * n_chunks * H * d : nullptr;
     p.max_pages = max_pages;
     p.B = (int32_t)B; p.H = (int32_t)H; p.d = (int32_t)d; p.P = (int32_t)P;
+    p.H_kv = (int32_t)H_kv;
     p.chunk_tokens = (int32_t)chunk; p.n_chunks = (int32_t)n_chunks;
     p.max_len = (int32_t)max_len;
     p.qo_dtype = qo_dtype;
@@ -549,8 +576,8 @@ int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype, const void* k_po
     const int hpw = 64 / lph;
     int waves = decode_waves();
     if (waves < 1 || waves > 8) waves = 2;
-    const int64_t heads_per_wg = (int64_t)hpw * waves;
-    const int64_t head_groups = (H + heads_per_wg - 1) / heads_per_wg;
+    const int64_t heads_per_wg = (int64_t)hpw * waves;  // pool heads
+    const int64_t head_groups = (H_kv + heads_per_wg - 1) / heads_per_wg;
     if (head_groups > 65535) return AHPC_ERR_BAD_SHAPE;
 
     const int64_t total = B * H * d;
@@ -569,6 +596,14 @@ int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype, const void* k_po
         return static_cast<int>(hipGetLastError());
     }
     return AHPC_OK;
+}
+
+int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype, const void* k_pool, const void* v_pool, int pool_dtype,
+                          const int32_t* block_table, const int32_t* seq_lens, const int32_t* batch_rows, int64_t B,
+                          int64_t H, int64_t d, int64_t P, int64_t max_pages, int64_t max_len, float scale,
+                          int64_t chunk_tokens, void* workspace, size_t workspace_bytes, void* stream) {
+    return ahpc_hip_paged_decode_gqa(q, o, qo_dtype, k_pool, v_pool, pool_dtype, block_table, seq_lens, batch_rows, B, H, H,
+                                     d, P, max_pages, max_len, scale, chunk_tokens, workspace, workspace_bytes, stream);
 }
 
 int ahpc_hip_paged_gather_indices(const int32_t* block_table, const int32_t* seq_lens, const int32_t* batch_rows, int64_t B,

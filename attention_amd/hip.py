@@ -59,12 +59,15 @@ SIGNATURES = {
     "ahpc_hip_event_synchronize": (_ci, [_vp]),
     "ahpc_hip_event_elapsed_ms": (_ci, [_vp, _vp, C.POINTER(_f32)]),
     "ahpc_hip_flash_fwd": (_ci, [_vp, _vp, _vp, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp]),
+    "ahpc_hip_flash_fwd_gqa": (_ci, [_vp, _vp, _vp, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp, _vp]),
     "ahpc_hip_flash_fwd_masked": (_ci, [_vp, _vp, _vp, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp, _vp]),
     "ahpc_hip_flash_fwd_varlen": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp]),
+    "ahpc_hip_flash_fwd_varlen_gqa": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp]),
     "ahpc_hip_kv_scatter": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
     "ahpc_hip_kv_gather": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
     "ahpc_hip_paged_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64]),
     "ahpc_hip_paged_decode": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp, _sz, _vp]),
+    "ahpc_hip_paged_decode_gqa": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp, _sz, _vp]),
     "ahpc_hip_paged_gather_indices": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp]),
 }
 
@@ -117,6 +120,20 @@ def flash_fwd(q, k, v, o, dtype, B, N, H, d, strides, scale, causal, stream=None
     _check(rc, "flash_fwd")
 
 
+def flash_fwd_gqa(q, k, v, o, dtype, B, N, H, H_kv, d, strides, kv_strides, scale, causal, stream=None, mask=None):
+    sb, sn, sh = strides
+    kb, kn, kh = kv_strides
+    _check(load().ahpc_hip_flash_fwd_gqa(q, k, v, o, dtype, B, N, H, H_kv, d, sb, sn, sh, kb, kn, kh, scale, int(causal),
+                                        mask, stream), "flash_fwd_gqa")
+
+
+def flash_fwd_varlen_gqa(q, k, v, o, dtype, cu_seqlens, n_seqs, max_len, H, H_kv, d, stride_t, stride_h, kv_stride_t,
+                         kv_stride_h, scale, causal, stream=None):
+    _check(load().ahpc_hip_flash_fwd_varlen_gqa(q, k, v, o, dtype, cu_seqlens, n_seqs, max_len, H, H_kv, d, stride_t,
+                                               stride_h, kv_stride_t, kv_stride_h, scale, int(causal), stream),
+           "flash_fwd_varlen_gqa")
+
+
 def flash_fwd_varlen(q, k, v, o, dtype, cu_seqlens, n_seqs, max_len, H, d, stride_t, stride_h, scale, causal, stream=None):
     _check(load().ahpc_hip_flash_fwd_varlen(q, k, v, o, dtype, cu_seqlens, n_seqs, max_len, H, d, stride_t, stride_h,
                                            scale, int(causal), stream), "flash_fwd_varlen")
@@ -142,6 +159,13 @@ def paged_decode(q, o, qo_dtype, k_pool, v_pool, pool_dtype, table, seq_lens, ba
     _check(load().ahpc_hip_paged_decode(q, o, qo_dtype, k_pool, v_pool, pool_dtype, table, seq_lens, batch_rows, B, H, d,
                                        P, max_pages, max_len, scale, chunk_tokens, workspace, workspace_bytes, stream),
            "paged_decode")
+
+
+def paged_decode_gqa(q, o, qo_dtype, k_pool, v_pool, pool_dtype, table, seq_lens, batch_rows, B, H, H_kv, d, P, max_pages,
+                     max_len, scale, chunk_tokens=0, workspace=None, workspace_bytes=0, stream=None):
+    _check(load().ahpc_hip_paged_decode_gqa(q, o, qo_dtype, k_pool, v_pool, pool_dtype, table, seq_lens, batch_rows, B, H,
+                                           H_kv, d, P, max_pages, max_len, scale, chunk_tokens, workspace,
+                                           workspace_bytes, stream), "paged_decode_gqa")
 
 
 def paged_gather_indices(table, seq_lens, batch_rows, B, H, d, P, max_pages, max_len, offsets, stream=None):

@@ -289,7 +289,7 @@ bool BackendFactory::validateBackendCompatibility(BackendType type, const Attent
     if (p.batch_size == 0 || p.sequence_length == 0 || p.num_heads == 0 || p.head_dimension == 0) return false;
     if (type != BackendType::HIP) return true;
     if (p.head_dimension > 256) return false;
-    if (p.key_value_heads != 0 && p.key_value_heads != p.num_heads) return false;
+    if (p.key_value_heads != 0 && (p.key_value_heads > p.num_heads || p.num_heads % p.key_value_heads)) return false;
     const auto& cap = f.capabilities_.at(key(type));
     const double bytes = 4.0 * 4.0 * (double)p.batch_size * (double)p.sequence_length * (double)p.num_heads * (double)p.head_dimension;
     return bytes < (double)cap.memory_size;

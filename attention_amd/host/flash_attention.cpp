@@ -28,8 +28,10 @@ FlashAttention::~FlashAttention() { delete impl_; }
 void FlashAttention::configure(const AttentionParams& params, const PerformanceConfig& perf_config) {
     if (params.batch_size == 0 || params.sequence_length == 0 || params.num_heads == 0 || params.head_dimension == 0)
         throw AttentionException(AttentionError::INVALID_PARAMETERS, "Invalid attention parameters: dimensions must be positive");
-    if (params.key_value_heads != 0 && params.key_value_heads != params.num_heads)
-        throw AttentionException(AttentionError::UNSUPPORTED_OPERATION, "key_value_heads must be 0 or equal to num_heads");
+    // Grouped key/value heads (AttentionParams::key_value_heads, src/api/attention_interface.hpp:61; the
+    // reference reads the field nowhere): consecutive query heads share a K/V head, so the counts must divide.
+    if (params.key_value_heads != 0 && (params.key_value_heads > params.num_heads || params.num_heads % params.key_value_heads))
+        throw AttentionException(AttentionError::INVALID_PARAMETERS, "key_value_heads must divide num_heads");
     if (params.apply_rotary_embedding)
         throw AttentionException(AttentionError::UNSUPPORTED_OPERATION, "rotary embedding is not applied by this backend");
     if (params.head_dimension > 256)
@@ -49,16 +51,19 @@ void FlashAttention::configure_flash_attention(const FlashAttentionConfig& flash
     impl_->cfg = flash_config;
 }
 
-static bool shape_ok(const TensorShape& s, const AttentionParams& p) {
+static size_t kv_heads(const AttentionParams& p) { return p.key_value_heads ? p.key_value_heads : p.num_heads; }
+
+static bool shape_ok(const TensorShape& s, const AttentionParams& p, size_t heads) {
     return s.dimensions.size() == 4 && s.dimensions[0] == p.batch_size && s.dimensions[1] > 0 &&
-           s.dimensions[2] == p.num_heads && s.dimensions[3] == p.head_dimension;
+           s.dimensions[2] == heads && s.dimensions[3] == p.head_dimension;
 }
 
 // Reference: FlashAttention::validate_inputs, src/algorithms/flash_attention.cpp:238-275 (4-D, batch,
 // heads and head_dim must match the configured parameters; the sequence dimension is free).
 AttentionError FlashAttention::validate_inputs(const TensorShape& q, const TensorShape& k, const TensorShape& v,
                                                const TensorShape& o, const AttentionParams& params) const {
-    if (!shape_ok(q, params) || !shape_ok(k, params) || !shape_ok(v, params) || !shape_ok(o, params))
+    if (!shape_ok(q, params, params.num_heads) || !shape_ok(k, params, kv_heads(params)) ||
+        !shape_ok(v, params, kv_heads(params)) || !shape_ok(o, params, params.num_heads))
         return AttentionError::INVALID_INPUT;
     return AttentionError::SUCCESS;
 }
@@ -94,14 +99,15 @@ void FlashAttention::forward(const TensorShape& qs, const void* q, const TensorS
             throw AttentionException(AttentionError::UNSUPPORTED_OPERATION, "only ROW_MAJOR tensors are supported");
 
     const size_t B = current_params_.batch_size, H = current_params_.num_heads, d = current_params_.head_dimension;
-    const size_t bytes = qs.total_bytes();
+    const size_t Hkv = kv_heads(current_params_);
+    const size_t bytes = qs.total_bytes(), kv_bytes = ks.total_bytes();
     void* st = impl_->stream.get();
     hipsup::EventTimer timer;
     const auto wall0 = std::chrono::steady_clock::now();
 
     const void* dq = stage_in(q, bytes, impl_->dq, st);
-    const void* dk = stage_in(k, bytes, impl_->dk, st);
-    const void* dv = stage_in(v, bytes, impl_->dv, st);
+    const void* dk = stage_in(k, kv_bytes, impl_->dk, st);
+    const void* dv = stage_in(v, kv_bytes, impl_->dv, st);
     const bool out_on_device = hipsup::is_device_pointer(o);
     void* dout = out_on_device ? o : impl_->dout.reserve(bytes);
     const float* dmask = nullptr;
@@ -110,20 +116,18 @@ void FlashAttention::forward(const TensorShape& qs, const void* q, const TensorS
     float scale = impl_->cfg.softmax_scale > 0.0f ? impl_->cfg.softmax_scale : current_params_.scale_factor;
     if (!(scale > 0.0f)) scale = 1.0f / std::sqrt(static_cast<float>(d));
     const int causal = (current_params_.causal_mask || impl_->cfg.use_causal_mask) ? 1 : 0;
-    int64_t sb, sn, sh;
+    int64_t sb, sn, sh, kb, kn, kh;
     if (impl_->cfg.tensor_layout_bhnd) {
         sb = (int64_t)(H * N * d); sh = (int64_t)(N * d); sn = (int64_t)d;
+        kb = (int64_t)(Hkv * N * d); kh = sh; kn = sn;
     } else {
         sb = (int64_t)(N * H * d); sn = (int64_t)(H * d); sh = (int64_t)d;
+        kb = (int64_t)(N * Hkv * d); kn = (int64_t)(Hkv * d); kh = sh;
     }
     const int dt = hipsup::dtype_code(qs.data_type);
     if (profiling_enabled_) timer.start(st);
-    if (dmask)
-        check(ahpc_hip_flash_fwd_masked(dq, dk, dv, dout, dt, (int64_t)B, (int64_t)N, (int64_t)H, (int64_t)d, sb, sn, sh,
-                                        scale, causal, dmask, st), "flash forward (masked)");
-    else
-        check(ahpc_hip_flash_fwd(dq, dk, dv, dout, dt, (int64_t)B, (int64_t)N, (int64_t)H, (int64_t)d, sb, sn, sh, scale,
-                                 causal, st), "flash forward");
+    check(ahpc_hip_flash_fwd_gqa(dq, dk, dv, dout, dt, (int64_t)B, (int64_t)N, (int64_t)H, (int64_t)Hkv, (int64_t)d, sb, sn,
+                                 sh, kb, kn, kh, scale, causal, dmask, st), "flash forward");
     if (profiling_enabled_) timer.stop(st);
     if (!out_on_device) check(ahpc_hip_memcpy_d2h(o, dout, bytes, st), "copy from device");
     impl_->stream.sync();
@@ -140,6 +144,8 @@ void FlashAttention::forward(const TensorShape& qs, const void* q, const TensorS
     }
 }
 
+// `shape` is the packed shape of Q and O, [total_tokens, num_heads, head_dim]; K and V are
+// [total_tokens, key_value_heads, head_dim].
 void FlashAttention::forward_varlen(const TensorShape& shape, const void* q, const void* k, const void* v, void* o,
                                     const int32_t* cu_seqlens, size_t n_seqs) {
     if (!impl_->configured)
@@ -159,10 +165,11 @@ void FlashAttention::forward_varlen(const TensorShape& shape, const void* q, con
         throw AttentionException(AttentionError::INVALID_INPUT, "cu_seqlens must end at total_tokens");
     if (max_len == 0) return;
     void* st = impl_->stream.get();
-    const size_t bytes = shape.total_bytes();
+    const size_t Hkv = kv_heads(current_params_);
+    const size_t bytes = shape.total_bytes(), kv_bytes = bytes / H * Hkv;
     const void* dq = stage_in(q, bytes, impl_->dq, st);
-    const void* dk = stage_in(k, bytes, impl_->dk, st);
-    const void* dv = stage_in(v, bytes, impl_->dv, st);
+    const void* dk = stage_in(k, kv_bytes, impl_->dk, st);
+    const void* dv = stage_in(v, kv_bytes, impl_->dv, st);
     const bool out_on_device = hipsup::is_device_pointer(o);
     void* dout = out_on_device ? o : impl_->dout.reserve(bytes);
     if (!out_on_device) check(ahpc_hip_memset(dout, 0, bytes, st), "clear output");
@@ -171,9 +178,10 @@ void FlashAttention::forward_varlen(const TensorShape& shape, const void* q, con
     float scale = impl_->cfg.softmax_scale > 0.0f ? impl_->cfg.softmax_scale : current_params_.scale_factor;
     if (!(scale > 0.0f)) scale = 1.0f / std::sqrt(static_cast<float>(d));
     const int causal = (current_params_.causal_mask || impl_->cfg.use_causal_mask) ? 1 : 0;
-    check(ahpc_hip_flash_fwd_varlen(dq, dk, dv, dout, hipsup::dtype_code(shape.data_type), static_cast<const int32_t*>(dcu),
-                                    (int64_t)n_seqs, max_len, (int64_t)H, (int64_t)d, (int64_t)(H * d), (int64_t)d, scale,
-                                    causal, st), "flash forward (ragged)");
+    check(ahpc_hip_flash_fwd_varlen_gqa(dq, dk, dv, dout, hipsup::dtype_code(shape.data_type),
+                                        static_cast<const int32_t*>(dcu), (int64_t)n_seqs, max_len, (int64_t)H, (int64_t)Hkv,
+                                        (int64_t)d, (int64_t)(H * d), (int64_t)d, (int64_t)(Hkv * d), (int64_t)d, scale, causal,
+                                        st), "flash forward (ragged)");
     if (!out_on_device) check(ahpc_hip_memcpy_d2h(o, dout, bytes, st), "copy from device");
     impl_->stream.sync();
 }

@@ -29,7 +29,8 @@ struct Sequence {
 struct PagedAttention::Impl {
     PagedAttentionConfig cfg;
     bool configured = false;
-    size_t H = 0, d = 0, P = 16;
+    size_t H = 0, d = 0, P = 16;  // H = query heads
+    size_t Hkv = 0;               // heads stored in the pool (AttentionParams::key_value_heads, 0 = H)
     size_t max_pages = 0;             // columns of the block table
     size_t n_rows = 0;                // rows of the block table
 
@@ -71,7 +72,7 @@ struct PagedAttention::Impl {
     void ensure_pool_locked(DataType dtype) {
         if (pool) return;
         const DataType dt = cfg.kv_cache_dtype >= 0 ? static_cast<DataType>(cfg.kv_cache_dtype) : dtype;
-        pool.reset(new KVBlockPool(P, H, d, dt, cfg.initial_page_pool_size, cfg.page_pool_growth, cfg.device_pool_max_bytes));
+        pool.reset(new KVBlockPool(P, Hkv, d, dt, cfg.initial_page_pool_size, cfg.page_pool_growth, cfg.device_pool_max_bytes));
     }
 
     void release_pages_locked(Sequence& s, size_t keep_pages) {
@@ -121,8 +122,15 @@ PagedAttention::~PagedAttention() { delete impl_; }
 void PagedAttention::configure(const AttentionParams& params, const PerformanceConfig& perf_config) {
     if (params.batch_size == 0 || params.sequence_length == 0 || params.num_heads == 0 || params.head_dimension == 0)
         throw AttentionException(AttentionError::INVALID_PARAMETERS, "Invalid attention parameters: dimensions must be positive");
-    if (params.key_value_heads != 0 && params.key_value_heads != params.num_heads)
-        throw AttentionException(AttentionError::UNSUPPORTED_OPERATION, "key_value_heads must be 0 or equal to num_heads");
+    // Grouped key/value heads: the pool stores key_value_heads heads per token and every one of them serves
+    // num_heads / key_value_heads consecutive query heads (the decode kernel takes groups of 1, 2, 4, 8).
+    if (params.key_value_heads != 0) {
+        if (params.key_value_heads > params.num_heads || params.num_heads % params.key_value_heads)
+            throw AttentionException(AttentionError::INVALID_PARAMETERS, "key_value_heads must divide num_heads");
+        const size_t g = params.num_heads / params.key_value_heads;
+        if (g != 1 && g != 2 && g != 4 && g != 8)
+            throw AttentionException(AttentionError::UNSUPPORTED_OPERATION, "paged decode supports 1, 2, 4 or 8 query heads per key/value head");
+    }
     if (params.page_size == 0) throw AttentionException(AttentionError::INVALID_PARAMETERS, "page_size must be positive");
     const size_t d = params.head_dimension;
     if (d != 32 && d != 64 && d != 128 && d != 256)
@@ -145,6 +153,7 @@ void PagedAttention::configure(const AttentionParams& params, const PerformanceC
     m.n_rows = m.max_pages = 0;
     m.next_id = 1;
     m.H = params.num_heads;
+    m.Hkv = params.key_value_heads ? params.key_value_heads : params.num_heads;
     m.d = d;
     m.P = params.page_size;
     m.cfg.page_size = m.P;
@@ -278,7 +287,7 @@ void PagedAttention::append_kv_cache(size_t sequence_id, const void* key_data, c
         m.sync_table_locked();
     }
     void* st = m.stream.get();
-    const size_t bytes = num_tokens * m.H * m.d * hipsup::dtype_size(data_type);
+    const size_t bytes = num_tokens * m.Hkv * m.d * hipsup::dtype_size(data_type);
     const void* dk = key_data;
     const void* dv = value_data;
     if (!hipsup::is_device_pointer(key_data)) {
@@ -291,7 +300,7 @@ void PagedAttention::append_kv_cache(size_t sequence_id, const void* key_data, c
     }
     check(ahpc_hip_kv_scatter(dk, dv, hipsup::dtype_code(data_type), m.pool->k_slab(), m.pool->v_slab(),
                               hipsup::dtype_code(m.pool->dtype()), static_cast<const int32_t*>(m.d_table.get()),
-                              (int64_t)m.max_pages, nullptr, nullptr, row, (int64_t)start, (int64_t)num_tokens, (int64_t)m.H,
+                              (int64_t)m.max_pages, nullptr, nullptr, row, (int64_t)start, (int64_t)num_tokens, (int64_t)m.Hkv,
                               (int64_t)m.d, (int64_t)m.P, st), "KV scatter");
     m.stream.sync();
     {
@@ -321,13 +330,13 @@ void PagedAttention::get_kv_cache(size_t sequence_id, void* key_data, void* valu
         m.sync_table_locked();
     }
     void* st = m.stream.get();
-    const size_t bytes = num_tokens * m.H * m.d * hipsup::dtype_size(data_type);
+    const size_t bytes = num_tokens * m.Hkv * m.d * hipsup::dtype_size(data_type);
     const bool kdev = hipsup::is_device_pointer(key_data), vdev = hipsup::is_device_pointer(value_data);
     void* dk = kdev ? key_data : m.d_tmp_k.reserve(bytes);
     void* dv = vdev ? value_data : m.d_tmp_v.reserve(bytes);
     check(ahpc_hip_kv_gather(dk, dv, hipsup::dtype_code(data_type), m.pool->k_slab(), m.pool->v_slab(),
                              hipsup::dtype_code(m.pool->dtype()), static_cast<const int32_t*>(m.d_table.get()),
-                             (int64_t)m.max_pages, row, (int64_t)start_token, (int64_t)num_tokens, (int64_t)m.H, (int64_t)m.d,
+                             (int64_t)m.max_pages, row, (int64_t)start_token, (int64_t)num_tokens, (int64_t)m.Hkv, (int64_t)m.d,
                              (int64_t)m.P, st), "KV gather");
     if (!kdev) check(ahpc_hip_memcpy_d2h(key_data, dk, bytes, st), "copy keys from device");
     if (!vdev) check(ahpc_hip_memcpy_d2h(value_data, dv, bytes, st), "copy values from device");
@@ -422,11 +431,11 @@ void PagedAttention::forward_batch(const std::vector<size_t>& ids, const std::ve
         float scale = current_params_.scale_factor > 0.0f ? current_params_.scale_factor : 1.0f / std::sqrt(static_cast<float>(m.d));
         hipsup::EventTimer timer;
         if (profiling_enabled_) timer.start(st);
-        check(ahpc_hip_paged_decode(dq, dout, hipsup::dtype_code(qdt), m.pool->k_slab(), m.pool->v_slab(),
-                                    hipsup::dtype_code(m.pool->dtype()), static_cast<const int32_t*>(m.d_table.get()),
-                                    static_cast<const int32_t*>(m.d_lens.get()), static_cast<const int32_t*>(drows), (int64_t)B,
-                                    (int64_t)m.H, (int64_t)m.d, (int64_t)m.P, (int64_t)m.max_pages, (int64_t)max_len, scale, chunk,
-                                    ws, ws_bytes, st), "paged decode");
+        check(ahpc_hip_paged_decode_gqa(dq, dout, hipsup::dtype_code(qdt), m.pool->k_slab(), m.pool->v_slab(),
+                                        hipsup::dtype_code(m.pool->dtype()), static_cast<const int32_t*>(m.d_table.get()),
+                                        static_cast<const int32_t*>(m.d_lens.get()), static_cast<const int32_t*>(drows),
+                                        (int64_t)B, (int64_t)m.H, (int64_t)m.Hkv, (int64_t)m.d, (int64_t)m.P,
+                                        (int64_t)m.max_pages, (int64_t)max_len, scale, chunk, ws, ws_bytes, st), "paged decode");
         if (profiling_enabled_) {
             timer.stop(st);
             m.profile.emplace_back("decode_kernel_ms", timer.elapsed_ms());
@@ -467,7 +476,7 @@ void PagedAttention::forward(const TensorShape& qs, const void* q, const TensorS
     std::vector<TensorShape> qsh(B, TensorShape({1, 1, H, d}, qs.data_type)), osh(B, TensorShape({1, 1, H, d}, os.data_type));
     std::vector<const void*> qp(B);
     std::vector<void*> op(B);
-    const size_t kv_stride = N * H * d * ks.element_size();
+    const size_t kv_stride = N * impl_->Hkv * d * ks.element_size();
     const size_t q_stride = H * d * qs.element_size();
     try {
         for (size_t b = 0; b < B; ++b) {

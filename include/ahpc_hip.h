@@ -42,7 +42,8 @@ typedef enum ahpc_status {
     AHPC_ERR_UNSUPPORTED_HEAD_DIM = -4,
     AHPC_ERR_WORKSPACE_TOO_SMALL = -5,
     AHPC_ERR_NO_DEVICE = -6,
-    AHPC_ERR_BAD_ALIGNMENT = -7    /* pointers/strides must allow 16-byte vector access */
+    AHPC_ERR_BAD_ALIGNMENT = -7,   /* pointers/strides must allow 16-byte vector access */
+    AHPC_ERR_UNSUPPORTED_GROUP = -8 /* query heads per K/V head: decode takes 1, 2, 4 or 8 */
 } ahpc_status;
 
 const char* ahpc_hip_error_string(int code);
@@ -107,6 +108,19 @@ int ahpc_hip_flash_fwd(const void* q, const void* k, const void* v, void* o, int
                        int64_t stride_b, int64_t stride_n, int64_t stride_h,
                        float scale, int causal, void* stream);
 
+/* Grouped-query attention: H query heads over H_kv <= H key/value heads (H % H_kv == 0); query
+ * head h reads K/V head h / (H / H_kv), i.e. consecutive query heads share one.  This is what
+ * AttentionParams::key_value_heads announces (src/api/attention_interface.hpp:61; 0 = H) and the
+ * reference never implements (the field is read nowhere; README.md:367-368 lists it as planned).
+ * Q and O use (stride_b, stride_n, stride_h), K and V their own strides; with H_kv == H and equal
+ * strides this is ahpc_hip_flash_fwd.  mask: NULL, or fp32 [B,N,N] as in the masked entry point
+ * (then the fp32-FMA kernel runs). */
+int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o, int dtype,
+                           int64_t B, int64_t N, int64_t H, int64_t H_kv, int64_t d,
+                           int64_t stride_b, int64_t stride_n, int64_t stride_h,
+                           int64_t kv_stride_b, int64_t kv_stride_n, int64_t kv_stride_h,
+                           float scale, int causal, const float* mask, void* stream);
+
 /* Same with a dense fp32 mask [B,N,N] shared by all heads, 0.0f removes the key
  * (FlashAttention::apply_attention_mask, src/algorithms/flash_attention.cpp:596-607;
  * indexing :432-435).  mask may be NULL.  Always runs on the fp32-FMA kernel. */
@@ -125,6 +139,13 @@ int ahpc_hip_flash_fwd_varlen(const void* q, const void* k, const void* v, void*
                               const int32_t* cu_seqlens, int64_t n_seqs, int64_t max_len,
                               int64_t H, int64_t d, int64_t stride_t, int64_t stride_h,
                               float scale, int causal, void* stream);
+
+/* Ragged batch with grouped K/V heads: Q, O packed [T,H,d], K, V packed [T,H_kv,d]. */
+int ahpc_hip_flash_fwd_varlen_gqa(const void* q, const void* k, const void* v, void* o, int dtype,
+                                  const int32_t* cu_seqlens, int64_t n_seqs, int64_t max_len,
+                                  int64_t H, int64_t H_kv, int64_t d,
+                                  int64_t stride_t, int64_t stride_h, int64_t kv_stride_t, int64_t kv_stride_h,
+                                  float scale, int causal, void* stream);
 
 /* ---- paged KV pool ---------------------------------------------------------------------------
  * Pool layout: K and V are separate slabs  [page][slot 0..P-1][head][d]  (the layout
@@ -181,6 +202,17 @@ int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype,
                           int64_t B, int64_t H, int64_t d, int64_t P, int64_t max_pages, int64_t max_len,
                           float scale, int64_t chunk_tokens,
                           void* workspace, size_t workspace_bytes, void* stream);
+
+/* Decode with grouped K/V heads: the pool holds H_kv heads per token (its kv_scatter / kv_gather /
+ * gather_indices calls take H = H_kv), q and o hold H = g * H_kv heads, g in {1, 2, 4, 8}; query
+ * head h reads pool head h / g.  Every K/V byte is still read once and serves g query heads.
+ * Workspace size: ahpc_hip_paged_decode_workspace_bytes with the QUERY head count. */
+int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype,
+                              const void* k_pool, const void* v_pool, int pool_dtype,
+                              const int32_t* block_table, const int32_t* seq_lens, const int32_t* batch_rows,
+                              int64_t B, int64_t H, int64_t H_kv, int64_t d, int64_t P, int64_t max_pages,
+                              int64_t max_len, float scale, int64_t chunk_tokens,
+                              void* workspace, size_t workspace_bytes, void* stream);
 
 /* Debug twin of the decode kernel's addressing: offsets[b*max_len + t] = the element offset
  * of (token t, head 0, lane 0) of batch entry b, computed by the same device function the

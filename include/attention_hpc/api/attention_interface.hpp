@@ -72,7 +72,7 @@ struct AttentionParams {
     size_t sequence_length;
     size_t num_heads;
     size_t head_dimension;
-    size_t key_value_heads = 0;          // 0 = num_heads; other values are rejected (no GQA/MQA yet)
+    size_t key_value_heads = 0;          // 0 = num_heads; else a divisor of it (grouped / multi-query K and V)
     float scale_factor = 0.0f;           // 0 = 1/sqrt(head_dimension)
     bool causal_mask = false;
     bool apply_rotary_embedding = false; // must stay false

@@ -325,8 +325,8 @@ CASE(Flash_UnconfiguredAndBadParameters, false) {  // src/algorithms/flash_atten
     p.num_heads = 0;
     EXPECT_THROWS(fa.configure(p), AttentionError::INVALID_PARAMETERS);
     p = fixture_params();
-    p.key_value_heads = 2;
-    EXPECT_THROWS(fa.configure(p), AttentionError::UNSUPPORTED_OPERATION);
+    p.key_value_heads = 3;  // does not divide the four query heads
+    EXPECT_THROWS(fa.configure(p), AttentionError::INVALID_PARAMETERS);
     EXPECT(fa.get_backend_name() == "HIP_FlashAttention");
     EXPECT(fa.get_version() == "1.0.0");
     EXPECT(fa.supports_data_type(DataType::FLOAT32) && fa.supports_data_type(DataType::BFLOAT16));
@@ -725,6 +725,63 @@ CASE(Paged_ConvenienceForward, true) {  // src/algorithms/paged_attention.cpp:13
     EXPECT(pa.get_active_sequences_count() == 0 && pa.get_total_memory_usage() == 0);
     EXPECT_THROWS(pa.forward(shape4(B, N, H, d), k.data(), shape4(B, N, H, d), k.data(), shape4(B, N, H, d), v.data(), shape4(B, N, H, d), k.data()),
                   AttentionError::UNSUPPORTED_OPERATION);
+}
+
+// Grouped key/value heads (AttentionParams::key_value_heads; read nowhere in the reference, so the only
+// yardstick is the definition: query head h uses K/V head h / (H / H_kv)).  The grouped call must equal the
+// oracle fed K and V with every head repeated.
+static std::vector<float> repeat_heads(const std::vector<float>& x, size_t rows, size_t Hkv, size_t g, size_t d) {
+    std::vector<float> y(rows * Hkv * g * d);
+    for (size_t r = 0; r < rows; ++r)
+        for (size_t h = 0; h < Hkv * g; ++h)
+            std::copy(x.begin() + (r * Hkv + h / g) * d, x.begin() + (r * Hkv + h / g + 1) * d, y.begin() + (r * Hkv * g + h) * d);
+    return y;
+}
+CASE(Gqa_FlashForwardEqualsRepeatedHeads, true) {
+    const size_t B = 2, N = 96, H = 8, Hkv = 2, d = 64, g = H / Hkv;
+    AttentionParams p{};
+    p.batch_size = B; p.sequence_length = N; p.num_heads = H; p.key_value_heads = Hkv; p.head_dimension = d; p.causal_mask = true;
+    FlashAttention fa;
+    fa.configure(p);
+    auto q = uniform(B * N * H * d, 95, 1), k = uniform(B * N * Hkv * d, 95, 2), v = uniform(B * N * Hkv * d, 95, 3);
+    std::vector<float> out(q.size(), 0.0f);
+    fa.forward(shape4(B, N, H, d), q.data(), shape4(B, N, Hkv, d), k.data(), shape4(B, N, Hkv, d), v.data(), shape4(B, N, H, d), out.data());
+    auto want = oracle_bnhd(q, repeat_heads(k, B * N, Hkv, g, d), repeat_heads(v, B * N, Hkv, g, d), B, N, H, d, 0.125f, true);
+    EXPECT(max_abs_diff(out, want) <= 1e-4f);
+    // K/V shaped like Q is now a shape error, and a head count that does not divide is refused at configure
+    EXPECT_THROWS(fa.forward(shape4(B, N, H, d), q.data(), shape4(B, N, H, d), q.data(), shape4(B, N, H, d), q.data(), shape4(B, N, H, d), out.data()),
+                  AttentionError::INVALID_INPUT);
+    p.key_value_heads = 3;
+    EXPECT_THROWS(fa.configure(p), AttentionError::INVALID_PARAMETERS);
+}
+CASE(Gqa_PagedDecodeEqualsRepeatedHeads, true) {
+    const size_t H = 8, Hkv = 2, d = 128, P = 16, g = H / Hkv, L = 300;
+    AttentionParams p{};
+    p.batch_size = 1; p.sequence_length = 1; p.num_heads = H; p.key_value_heads = Hkv; p.head_dimension = d; p.max_sequence_length = 512;
+    PagedAttention pa;
+    pa.configure(p);
+    const size_t id = pa.create_sequence(512);
+    auto k = normal(L * Hkv * d, 96, 2), v = normal(L * Hkv * d, 96, 3), q = normal(H * d, 96, 1);
+    pa.append_kv_cache(id, k.data(), v.data(), L, DataType::FLOAT32);   // [n, key_value_heads, d]
+    std::vector<float> out(H * d, 7.0f);
+    const TensorShape s({1, 1, H, d}, DataType::FLOAT32);
+    pa.forward_batch({id}, {s}, {q.data()}, {s}, {out.data()});
+    std::vector<int32_t> table((L + P - 1) / P);
+    for (size_t i = 0; i < table.size(); ++i) table[i] = (int32_t)i;
+    auto kx = repeat_heads(k, L, Hkv, g, d), vx = repeat_heads(v, L, Hkv, g, d);
+    kx.resize(table.size() * P * H * d, 0.0f);
+    vx.resize(kx.size(), 0.0f);
+    std::vector<float> want(H * d, 0.0f);
+    const int32_t len = (int32_t)L;
+    ahpc_oracle_paged_decode(q.data(), want.data(), kx.data(), vx.data(), table.data(), &len, nullptr, 1, H, d, P, table.size(),
+                             1.0f / std::sqrt((float)d), 1);
+    EXPECT(max_abs_diff(out, want) <= 1e-4f);
+    // read-back returns what was appended, in the pool's own head count
+    std::vector<float> kb(L * Hkv * d), vb(L * Hkv * d);
+    pa.get_kv_cache(id, kb.data(), vb.data(), 0, L, DataType::FLOAT32);
+    EXPECT(kb == k && vb == v);
+    p.key_value_heads = 1; p.num_heads = 3;  // three query heads per K/V head: refused by the decode kernel
+    EXPECT_THROWS(pa.configure(p), AttentionError::UNSUPPORTED_OPERATION);
 }
 
 CASE(Paged_SequenceLifecycle, true) {  // extend / truncate / reset, src/algorithms/paged_attention.cpp:352-418
