@@ -1,0 +1,39 @@
+"""The sweep benchmark (attention_amd/host/bench_report.cpp) writes a results file with the field names of the
+reference's SaveResultsToJSON, benchmarks/benchmark_attention.cpp:625-669, and its derived figures follow
+the reference's formulas (:241-246)."""
+import json
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "attention_amd", "lib", "ahpc_bench_report")
+
+pytestmark = pytest.mark.gpu
+
+REFERENCE_FIELDS = ["backend", "batch_size", "sequence_length", "num_heads", "head_dimension", "total_elements", "success",
+                    "forward_time_ms", "backward_time_ms", "total_time_ms", "memory_usage_bytes", "peak_memory_bytes", "gflops",
+                    "throughput_tokens_per_sec", "theoretical_flops"]
+
+
+@pytest.mark.parametrize("args", [["--device", "--dtype", "bf16", "--causal"], []])
+def test_quick_sweep_writes_reference_shaped_results(tmp_path, args):
+    assert os.path.exists(BIN), f"{BIN} missing: run __graft_entry__.build()"
+    out = tmp_path / "benchmark_results.json"
+    r = subprocess.run([BIN, "--quick", "--json", str(out)] + args, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "=== Performance Report ===" in r.stdout and "Best GFLOPS" in r.stdout
+    rows = json.loads(out.read_text())["benchmark_results"]
+    assert len(rows) == 2 * 3 * 2 * 2
+    for row in rows:
+        for f in REFERENCE_FIELDS:
+            assert f in row, f
+        assert row["success"] is True and row["backend"] == "HIP"
+        B, N, H, d = (row[k] for k in ("batch_size", "sequence_length", "num_heads", "head_dimension"))
+        assert row["total_elements"] == B * N * H * d
+        assert row["backward_time_ms"] == 0 and row["total_time_ms"] == pytest.approx(row["forward_time_ms"])
+        assert row["gflops"] == pytest.approx(B * H * N * N * d * 2 / 1e9 / (row["total_time_ms"] / 1e3), rel=1e-3)
+        assert row["throughput_tokens_per_sec"] == pytest.approx(B * N / (row["forward_time_ms"] / 1e3), rel=1e-3)
+        assert row["theoretical_flops"] == pytest.approx(B * H * N * N * (2 * d + 4), rel=1e-5)
+        assert row["tensors_resident_on_device"] is ("--device" in args)
