@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on exactly these workloads,
 # each counter scaled by its reading for a 1 GiB device copy (profiles/*.txt hold the runs).
-FLASH_TRAFFIC_BYTES = 542_200_000     # 408.0 MB fetched + 134.2 MB written (algorithmic: 536.9 MB)
+FLASH_TRAFFIC_BYTES = 672_100_000     # 537.9 MB fetched + 134.2 MB written (algorithmic: 536.9 MB)
 DECODE_TRAFFIC_BYTES = 2_364_900_000  # decode 2343.7 + 9.8 MB, merge 10.9 + 0.5 MB (algorithmic: 2342.9 MB)
 
 FLASH = dict(B=4, N=4096, H=32, d=128, causal=True, dtype="bf16", seed=0xA77E0002)
