@@ -66,6 +66,71 @@ __global__ void kv_gather_kernel(TO* __restrict__ k_out, TO* __restrict__ v_out,
     Storage<TO>::store(v_out + idx, vx);
 }
 
+// Batched append: the K and V rows of many sequences in one launch, straight from the tensors a prefill
+// just attended over.  One wavefront per (sequence, token) moves that token's two H*d rows; when source
+// and pool share a type and everything is 16-byte aligned the rows go as 16-byte pieces (a pure copy at
+// HBM speed), otherwise element by element with conversion.
+struct ScatterBatchParams {
+    const void* k_src;
+    const void* v_src;
+    void* k_pool;
+    void* v_pool;
+    const int32_t* table;
+    const int32_t* seq_rows;    // [B] table row of sequence b
+    const int32_t* seq_start;   // [B] position of its first new token, or null = 0
+    const int32_t* seq_tokens;  // [B] number of new tokens, or null = N
+    const int32_t* cu_seqlens;  // [B+1] packed source: sequence b owns source rows cu[b] .. cu[b+1]-1, or null
+    int64_t max_pages;
+    int64_t stride_b, stride_n;  // source strides in elements (stride_b unused with cu_seqlens)
+    int32_t B, N, H, d, P;
+};
+
+template <typename TI, typename TO, bool VEC>
+__global__ __launch_bounds__(256) void kv_scatter_batch_kernel(const ScatterBatchParams p) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int b = blockIdx.y;
+    const int t = blockIdx.x * 4 + wave;
+    int n_new = p.N;
+    int64_t src_row0 = 0;
+    if (p.cu_seqlens) {
+        n_new = p.cu_seqlens[b + 1] - p.cu_seqlens[b];
+        src_row0 = (int64_t)p.cu_seqlens[b] * p.stride_n;
+    } else {
+        if (p.seq_tokens) n_new = p.seq_tokens[b];
+        src_row0 = (int64_t)b * p.stride_b;
+    }
+    if (t >= n_new) return;
+    const int64_t row = p.seq_rows[b];
+    if (row < 0) return;
+    const int pos = (p.seq_start ? p.seq_start[b] : 0) + t;
+    const int64_t dst = kv_token_offset(p.table, p.max_pages, row, pos, p.P, p.H, p.d);
+    if (dst < 0) return;
+    const int64_t src = src_row0 + (int64_t)t * p.stride_n;
+    const int hd = p.H * p.d;
+    if (VEC) {
+        constexpr int EPV = 16 / (int)sizeof(TO);
+        const u32x4* ks = reinterpret_cast<const u32x4*>(static_cast<const TI*>(p.k_src) + src);
+        const u32x4* vs = reinterpret_cast<const u32x4*>(static_cast<const TI*>(p.v_src) + src);
+        u32x4* kd = reinterpret_cast<u32x4*>(static_cast<TO*>(p.k_pool) + dst);
+        u32x4* vd = reinterpret_cast<u32x4*>(static_cast<TO*>(p.v_pool) + dst);
+        for (int i = lane; i < hd / EPV; i += kWave) {
+            const u32x4 kx = ks[i], vx = vs[i];
+            kd[i] = kx;
+            vd[i] = vx;
+        }
+    } else {
+        const TI* ks = static_cast<const TI*>(p.k_src) + src;
+        const TI* vs = static_cast<const TI*>(p.v_src) + src;
+        TO* kd = static_cast<TO*>(p.k_pool) + dst;
+        TO* vd = static_cast<TO*>(p.v_pool) + dst;
+        for (int i = lane; i < hd; i += kWave) {
+            Storage<TO>::store(kd + i, Storage<TI>::load(ks + i));
+            Storage<TO>::store(vd + i, Storage<TI>::load(vs + i));
+        }
+    }
+}
+
 __global__ void gather_indices_kernel(const int32_t* __restrict__ table, const int32_t* __restrict__ seq_lens,
                                       const int32_t* __restrict__ batch_rows, int64_t B, int H, int d, int P,
                                       int64_t max_pages, int64_t max_len, int64_t* __restrict__ offsets) {
@@ -507,6 +572,44 @@ int ahpc_hip_kv_scatter(const void* k_new, const void* v_new, int in_dtype, void
         case AHPC_BF16: return scatter_out<bf16_t>(pool_dtype, k_new, v_new, k_pool, v_pool, block_table, max_pages, token_row, token_pos, row0, pos0, n_tokens, (int)H, (int)d, (int)P, st);
         default: return AHPC_ERR_BAD_DTYPE;
     }
+}
+
+int ahpc_hip_kv_scatter_batch(const void* k_src, const void* v_src, int in_dtype, int64_t stride_b, int64_t stride_n,
+                              void* k_pool, void* v_pool, int pool_dtype, const int32_t* block_table, int64_t max_pages,
+                              const int32_t* seq_rows, const int32_t* seq_start, const int32_t* seq_tokens,
+                              const int32_t* cu_seqlens, int64_t B, int64_t N, int64_t H, int64_t d, int64_t P, void* stream) {
+    if (B == 0 || N == 0) return AHPC_OK;
+    if (!k_src || !v_src || !k_pool || !v_pool || !block_table || !seq_rows) return AHPC_ERR_NULL_POINTER;
+    if (B < 0 || B > 65535 || N < 0 || N > 0x7FFFFFF0ll || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;
+    if (stride_n < H * d || (!cu_seqlens && stride_b < 0)) return AHPC_ERR_BAD_SHAPE;
+    if (in_dtype < AHPC_F32 || in_dtype > AHPC_BF16 || pool_dtype < AHPC_F32 || pool_dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
+    ScatterBatchParams p{k_src, v_src, k_pool, v_pool, block_table, seq_rows, seq_start, seq_tokens, cu_seqlens, max_pages,
+                         stride_b, stride_n, (int32_t)B, (int32_t)N, (int32_t)H, (int32_t)d, (int32_t)P};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    dim3 block(256), grid((unsigned)((N + 3) / 4), (unsigned)B);
+    const int esz = in_dtype == AHPC_F32 ? 4 : 2;
+    auto aligned = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    const bool vec = in_dtype == pool_dtype && aligned(k_src) && aligned(v_src) && aligned(k_pool) && aligned(v_pool) &&
+                     (H * d * esz) % 16 == 0 && (stride_n * esz) % 16 == 0 && (stride_b * esz) % 16 == 0;
+#define AHPC_SB(TI, TO, V) hipLaunchKernelGGL((kv_scatter_batch_kernel<TI, TO, V>), grid, block, 0, st, p)
+    if (vec) {
+        if (in_dtype == AHPC_F32) AHPC_SB(float, float, true);
+        else AHPC_SB(f16_t, f16_t, true);  // 16-bit rows are moved as bits: fp16 and bf16 alike
+    } else {
+        switch (in_dtype * 3 + pool_dtype) {
+            case 0: AHPC_SB(float, float, false); break;
+            case 1: AHPC_SB(float, f16_t, false); break;
+            case 2: AHPC_SB(float, bf16_t, false); break;
+            case 3: AHPC_SB(f16_t, float, false); break;
+            case 4: AHPC_SB(f16_t, f16_t, false); break;
+            case 5: AHPC_SB(f16_t, bf16_t, false); break;
+            case 6: AHPC_SB(bf16_t, float, false); break;
+            case 7: AHPC_SB(bf16_t, f16_t, false); break;
+            default: AHPC_SB(bf16_t, bf16_t, false); break;
+        }
+    }
+#undef AHPC_SB
+    return static_cast<int>(hipGetLastError());
 }
 
 int ahpc_hip_kv_gather(void* k_out, void* v_out, int out_dtype, const void* k_pool, const void* v_pool, int pool_dtype,

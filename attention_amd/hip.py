@@ -64,6 +64,7 @@ SIGNATURES = {
     "ahpc_hip_flash_fwd_varlen": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp]),
     "ahpc_hip_flash_fwd_varlen_gqa": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp]),
     "ahpc_hip_kv_scatter": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
+    "ahpc_hip_kv_scatter_batch": (_ci, [_vp, _vp, _ci, _i64, _i64, _vp, _vp, _ci, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "ahpc_hip_kv_gather": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
     "ahpc_hip_paged_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64]),
     "ahpc_hip_paged_decode": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp, _sz, _vp]),
@@ -143,6 +144,13 @@ def kv_scatter(k_new, v_new, in_dtype, k_pool, v_pool, pool_dtype, table, max_pa
                token_row=None, token_pos=None, row0=0, pos0=0, stream=None):
     _check(load().ahpc_hip_kv_scatter(k_new, v_new, in_dtype, k_pool, v_pool, pool_dtype, table, max_pages, token_row,
                                      token_pos, row0, pos0, n_tokens, H, d, P, stream), "kv_scatter")
+
+
+def kv_scatter_batch(k_src, v_src, in_dtype, stride_b, stride_n, k_pool, v_pool, pool_dtype, table, max_pages, seq_rows, B, N,
+                     H, d, P, seq_start=None, seq_tokens=None, cu_seqlens=None, stream=None):
+    _check(load().ahpc_hip_kv_scatter_batch(k_src, v_src, in_dtype, stride_b, stride_n, k_pool, v_pool, pool_dtype, table,
+                                           max_pages, seq_rows, seq_start, seq_tokens, cu_seqlens, B, N, H, d, P, stream),
+           "kv_scatter_batch")
 
 
 def kv_gather(k_out, v_out, out_dtype, k_pool, v_pool, pool_dtype, table, max_pages, row, start, n, H, d, P, stream=None):

@@ -106,6 +106,10 @@ struct PagedAttention::Impl {
         table_dirty = false;
     }
 
+    void append_many(const std::vector<size_t>& ids, const std::vector<size_t>& counts, const void* key_data,
+                     const void* value_data, size_t total_rows, DataType dt, int64_t stride_b, int64_t stride_n,
+                     const int32_t* cu_seqlens, size_t n_max);
+
     Sequence& find_locked(size_t id) {
         auto it = seqs.find(id);
         if (it == seqs.end()) throw AttentionException(AttentionError::INVALID_INPUT, "Sequence not found");
@@ -311,6 +315,117 @@ void PagedAttention::append_kv_cache(size_t sequence_id, const void* key_data, c
             m.lens[row] = static_cast<int32_t>(start + num_tokens);
             m.table_dirty = true;
         }
+    }
+}
+
+namespace {
+struct BatchAppend {
+    std::vector<int32_t> rows, start, count;
+};
+}  // namespace
+
+void PagedAttention::append_kv_cache_batch(const std::vector<size_t>& sequence_ids, const TensorShape& kv_shape,
+                                           const void* key_data, const void* value_data, const std::vector<size_t>& num_tokens) {
+    Impl& m = *impl_;
+    if (!m.configured) throw AttentionException(AttentionError::INVALID_PARAMETERS, "PagedAttention not configured. Call configure() first.");
+    if (!key_data || !value_data) throw AttentionException(AttentionError::INVALID_INPUT, "null key/value pointer");
+    const auto& dm = kv_shape.dimensions;
+    if (dm.size() != 4 || dm[0] != sequence_ids.size() || dm[2] != m.Hkv || dm[3] != m.d || (!num_tokens.empty() && num_tokens.size() != dm[0]))
+        throw AttentionException(AttentionError::INVALID_INPUT, "expected [sequences, tokens, key_value_heads, head_dim] and one count per sequence");
+    const size_t B = dm[0], N = dm[1];
+    std::vector<size_t> counts(B, N);
+    for (size_t b = 0; b < num_tokens.size(); ++b) {
+        if (num_tokens[b] > N) throw AttentionException(AttentionError::INVALID_INPUT, "num_tokens exceeds the tensor's sequence dimension");
+        counts[b] = num_tokens[b];
+    }
+    if (B == 0 || N == 0) return;
+    m.append_many(sequence_ids, counts, key_data, value_data, B * N, kv_shape.data_type, (int64_t)(N * m.Hkv * m.d),
+                (int64_t)(m.Hkv * m.d), nullptr, N);
+}
+
+void PagedAttention::append_kv_cache_packed(const std::vector<size_t>& sequence_ids, const TensorShape& kv_shape,
+                                            const void* key_data, const void* value_data, const int32_t* cu_seqlens) {
+    Impl& m = *impl_;
+    if (!m.configured) throw AttentionException(AttentionError::INVALID_PARAMETERS, "PagedAttention not configured. Call configure() first.");
+    if (!key_data || !value_data || !cu_seqlens) throw AttentionException(AttentionError::INVALID_INPUT, "null pointer");
+    const auto& dm = kv_shape.dimensions;
+    const size_t B = sequence_ids.size();
+    if (dm.size() != 3 || dm[1] != m.Hkv || dm[2] != m.d)
+        throw AttentionException(AttentionError::INVALID_INPUT, "packed tensors must be [total_tokens, key_value_heads, head_dim]");
+    if (B == 0) return;
+    if (cu_seqlens[0] != 0 || (size_t)cu_seqlens[B] != dm[0]) throw AttentionException(AttentionError::INVALID_INPUT, "cu_seqlens must run from 0 to total_tokens");
+    std::vector<size_t> counts(B);
+    size_t n_max = 0;
+    for (size_t b = 0; b < B; ++b) {
+        if (cu_seqlens[b + 1] < cu_seqlens[b]) throw AttentionException(AttentionError::INVALID_INPUT, "cu_seqlens must not decrease");
+        counts[b] = (size_t)(cu_seqlens[b + 1] - cu_seqlens[b]);
+        n_max = std::max(n_max, counts[b]);
+    }
+    if (n_max == 0) return;
+    m.append_many(sequence_ids, counts, key_data, value_data, dm[0], kv_shape.data_type, 0, (int64_t)(m.Hkv * m.d), cu_seqlens, n_max);
+}
+
+// Shared by the dense and the packed hand-off: reserves pages for every sequence, uploads the table and the
+// index arrays, scatters with one launch, then publishes the new lengths.
+void PagedAttention::Impl::append_many(const std::vector<size_t>& ids, const std::vector<size_t>& counts, const void* key_data,
+                                       const void* value_data, size_t total_rows, DataType dt, int64_t stride_b,
+                                       int64_t stride_n, const int32_t* cu_seqlens, size_t n_max) {
+    Impl& m = *this;
+    std::lock_guard<std::mutex> run(m.run_mutex);
+    const size_t B = ids.size();
+    BatchAppend ba;
+    {
+        std::lock_guard<std::mutex> lock(m.seq_mutex);
+        for (size_t b = 0; b < B; ++b)  // every id must exist before anything is changed
+            m.find_locked(ids[b]);
+        for (size_t b = 0; b < B; ++b)
+            for (size_t c = b + 1; c < B; ++c)
+                if (ids[b] == ids[c]) throw AttentionException(AttentionError::INVALID_INPUT, "a sequence may appear only once in a batched append");
+        m.ensure_pool_locked(dt);
+        for (size_t b = 0; b < B; ++b) {
+            Sequence& s = m.find_locked(ids[b]);
+            m.grow_pages_locked(s, (s.total_tokens + counts[b] + m.P - 1) / m.P);
+            ba.rows.push_back(s.row);
+            ba.start.push_back((int32_t)s.total_tokens);
+            ba.count.push_back((int32_t)counts[b]);
+        }
+        m.sync_table_locked();
+    }
+    void* st = m.stream.get();
+    const size_t bytes = total_rows * m.Hkv * m.d * hipsup::dtype_size(dt);
+    const void* dk = key_data;
+    const void* dv = value_data;
+    if (!hipsup::is_device_pointer(key_data)) {
+        check(ahpc_hip_memcpy_h2d(m.d_in_k.reserve(bytes), key_data, bytes, st), "copy keys to device");
+        dk = m.d_in_k.get();
+    }
+    if (!hipsup::is_device_pointer(value_data)) {
+        check(ahpc_hip_memcpy_h2d(m.d_in_v.reserve(bytes), value_data, bytes, st), "copy values to device");
+        dv = m.d_in_v.get();
+    }
+    // index arrays: rows | start | count | cu_seqlens, one upload
+    std::vector<int32_t> idx;
+    idx.insert(idx.end(), ba.rows.begin(), ba.rows.end());
+    idx.insert(idx.end(), ba.start.begin(), ba.start.end());
+    idx.insert(idx.end(), ba.count.begin(), ba.count.end());
+    if (cu_seqlens) idx.insert(idx.end(), cu_seqlens, cu_seqlens + B + 1);
+    int32_t* didx = static_cast<int32_t*>(m.d_rows.reserve(idx.size() * sizeof(int32_t)));
+    check(ahpc_hip_memcpy_h2d(didx, idx.data(), idx.size() * sizeof(int32_t), st), "copy index arrays");
+    check(ahpc_hip_kv_scatter_batch(dk, dv, hipsup::dtype_code(dt), stride_b, stride_n, m.pool->k_slab(), m.pool->v_slab(),
+                                    hipsup::dtype_code(m.pool->dtype()), static_cast<const int32_t*>(m.d_table.get()),
+                                    (int64_t)m.max_pages, didx, didx + B, cu_seqlens ? nullptr : didx + 2 * B,
+                                    cu_seqlens ? didx + 3 * B : nullptr, (int64_t)B, (int64_t)n_max, (int64_t)m.Hkv, (int64_t)m.d,
+                                    (int64_t)m.P, st), "batched KV scatter");
+    m.stream.sync();
+    {
+        std::lock_guard<std::mutex> lock(m.seq_mutex);
+        for (size_t b = 0; b < B; ++b) {
+            auto it = m.seqs.find(ids[b]);
+            if (it == m.seqs.end()) continue;
+            it->second.total_tokens = (size_t)ba.start[b] + counts[b];
+            m.lens[ba.rows[b]] = (int32_t)it->second.total_tokens;
+        }
+        m.table_dirty = true;
     }
 }
 

@@ -226,6 +226,102 @@ def bench_decode(hip, stream, steps, warmup, cpu):
     return res
 
 
+def bench_extras(hip, stream, steps, warmup):
+    """The other BASELINE configurations and the widened paths, one row each (not the headline)."""
+    import torch
+    rows = []
+    g = torch.Generator(device="cuda").manual_seed(0xA77E0009)
+
+    def randn(shape, dtype):
+        return torch.randn(shape, generator=g, device="cuda", dtype=torch.float32).to(dtype)
+
+    def run(name, launch, flops=None, nbytes=None):
+        wall, per = timed_steps(hip, stream, launch, steps, warmup)
+        ms = float(np.mean(per))
+        row = {"workload": name, "kernel_ms_mean": round(ms, 4), "kernel_ms_min": round(float(np.min(per)), 4)}
+        if flops:
+            row["TFLOP/s"] = round(flops / (ms * 1e-3) / 1e12, 1)
+            row["frac_of_2.5_PFLOP/s"] = round(flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)
+        if nbytes:
+            row["GB/s"] = round(nbytes / (ms * 1e-3) / 1e9, 1)
+            row["frac_of_8_TB/s"] = round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        rows.append(row)
+
+    # flash forward, same shape as the headline: non-causal, fp16, grouped K/V heads
+    B, N, H, d = 4, 4096, 32, 128
+    q = randn((B, N, H, d), torch.bfloat16); k = randn((B, N, H, d), torch.bfloat16); v = randn((B, N, H, d), torch.bfloat16)
+    o = torch.empty_like(q)
+    sc = 1.0 / np.sqrt(d)
+    st = (N * H * d, H * d, d)
+    run("flash_fwd bf16 non-causal B=4 N=4096 H=32 d=128",
+        lambda: hip.flash_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), hip.BF16, B, N, H, d, st, sc, False, stream),
+        flops=4.0 * B * H * N * N * d)
+    qh, kh, vh = q.to(torch.float16), k.to(torch.float16), v.to(torch.float16)
+    run("flash_fwd fp16 causal B=4 N=4096 H=32 d=128",
+        lambda: hip.flash_fwd(qh.data_ptr(), kh.data_ptr(), vh.data_ptr(), o.data_ptr(), hip.F16, B, N, H, d, st, sc, True, stream),
+        flops=2.0 * B * H * N * N * d)
+    Hkv = 8
+    kg, vg = randn((B, N, Hkv, d), torch.bfloat16), randn((B, N, Hkv, d), torch.bfloat16)
+    run("flash_fwd bf16 causal B=4 N=4096 H=32 (8 K/V heads) d=128",
+        lambda: hip.flash_fwd_gqa(q.data_ptr(), kg.data_ptr(), vg.data_ptr(), o.data_ptr(), hip.BF16, B, N, H, Hkv, d, st,
+                                  (N * Hkv * d, Hkv * d, d), sc, True, stream),
+        flops=2.0 * B * H * N * N * d)
+
+    # ragged fp16 causal batch: 16 sequences, lengths U[128,8192], H=32, d=64 (sigma 0.5)
+    rng = np.random.default_rng(0xA77E0005)
+    lens = rng.integers(128, 8193, size=16).astype(np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T, Hv, dv_ = int(cu[-1]), 32, 64
+    qv = (randn((T, Hv, dv_), torch.float32) * 0.5).to(torch.float16)
+    kv = (randn((T, Hv, dv_), torch.float32) * 0.5).to(torch.float16)
+    vv = (randn((T, Hv, dv_), torch.float32) * 0.5).to(torch.float16)
+    ov = torch.empty_like(qv)
+    dcu = torch.from_numpy(cu).cuda()
+    L = lens.astype(np.float64)
+    run(f"flash_fwd_varlen fp16 causal 16 seqs U[128,8192] ({T} tokens) H=32 d=64",
+        lambda: hip.flash_fwd_varlen(qv.data_ptr(), kv.data_ptr(), vv.data_ptr(), ov.data_ptr(), hip.F16, dcu.data_ptr(), 16,
+                                     int(lens.max()), Hv, dv_, Hv * dv_, dv_, 1.0 / np.sqrt(dv_), True, stream),
+        flops=float((4.0 * Hv * dv_ * L * (L + 1) / 2).sum()))
+
+    # decode: long contexts (bf16, B=8, U[16384,32768]) and grouped heads (H=32 over 8 pool heads)
+    def decode_case(name, cfg, Hq, Hp, dtype_code, tdtype):
+        lens, table, n_pages = lengths_and_table(cfg)
+        P = cfg["P"]
+        elems = n_pages * P * Hp * cfg["d"]
+        kp, vp = randn(elems, tdtype), randn(elems, tdtype)
+        qd = randn((cfg["B"], Hq, cfg["d"]), tdtype)
+        od = torch.empty_like(qd)
+        dt_, dl = torch.from_numpy(table).cuda(), torch.from_numpy(lens).cuda()
+        max_len = int(lens.max())
+        wsb = hip.paged_decode_workspace_bytes(cfg["B"], Hq, cfg["d"], max_len, P, 0)
+        ws = torch.empty(max(wsb, 4) // 4, dtype=torch.float32, device="cuda")
+        scl = 1.0 / np.sqrt(cfg["d"])
+        nb = decode_bytes(lens, dict(cfg, H=Hp)) + 2 * cfg["B"] * (Hq - Hp) * cfg["d"] * 2
+        run(name + f" (sum {int(lens.sum())} tokens)",
+            lambda: hip.paged_decode_gqa(qd.data_ptr(), od.data_ptr(), dtype_code, kp.data_ptr(), vp.data_ptr(), dtype_code,
+                                         dt_.data_ptr(), dl.data_ptr(), None, cfg["B"], Hq, Hp, cfg["d"], P, table.shape[1],
+                                         max_len, scl, 0, ws.data_ptr(), wsb, stream),
+            nbytes=nb)
+
+    decode_case("paged_decode bf16 B=8 H=32 d=128 page=16 context U[16384,32768]",
+                dict(B=8, H=32, d=128, P=16, lo=16384, hi=32768, seed=0xA77E0004), 32, 32, hip.BF16, torch.bfloat16)
+    decode_case("paged_decode fp16 B=64 H=32 over 8 pool heads d=128 page=16 context U[512,4096]",
+                dict(DECODE), 32, 8, hip.F16, torch.float16)
+
+    # prefill -> cache hand-off: K and V of the headline prefill into the pool, one launch
+    P = 16
+    pages_per = N // P
+    table = torch.randperm(B * pages_per, generator=torch.Generator().manual_seed(5)).to(torch.int32).reshape(B, pages_per).cuda()
+    kpool = torch.empty(B * pages_per * P * H * d, dtype=torch.bfloat16, device="cuda")
+    vpool = torch.empty_like(kpool)
+    rows_ = torch.arange(B, dtype=torch.int32, device="cuda")
+    run("kv_scatter_batch bf16 B=4 N=4096 H=32 d=128 -> pool (page 16)",
+        lambda: hip.kv_scatter_batch(k.data_ptr(), v.data_ptr(), hip.BF16, N * H * d, H * d, kpool.data_ptr(), vpool.data_ptr(),
+                                     hip.BF16, table.data_ptr(), pages_per, rows_.data_ptr(), B, N, H, d, P, stream=stream),
+        nbytes=4 * B * N * H * d * 2)
+    return rows
+
+
 def run_calibration(steps):
     """A plain device-to-device copy of known size (1 GiB read + 1 GiB written per launch): what the
     FETCH_SIZE / WRITE_SIZE counters read for it is the scale for the same counters on our kernels."""
@@ -248,7 +344,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", choices=["all", "flash", "decode", "calib"], default="all")
+    ap.add_argument("--workload", choices=["all", "flash", "decode", "calib", "extras"], default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline (profiling runs)")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -267,6 +363,10 @@ def main():
     assert hip.load().ahpc_hip_stream_create(C.byref(s)) == 0
     stream = s.value
 
+    if a.workload == "extras":
+        print(json.dumps({"extras": bench_extras(hip, stream, a.steps, a.warmup)}))
+        hip.load().ahpc_hip_stream_destroy(stream)
+        return
     out = {"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "higher_is_better": True, "scaling": "weak",
            "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
     flash = bench_flash(hip, stream, a.steps, a.warmup, not a.no_cpu) if a.workload in ("all", "flash") else None

@@ -169,6 +169,23 @@ int ahpc_hip_kv_scatter(const void* k_new, const void* v_new, int in_dtype,
                         int64_t row0, int64_t pos0, int64_t n_tokens,
                         int64_t H, int64_t d, int64_t P, void* stream);
 
+/* Batched append, one launch for B sequences: the hand-off from a prefill to the cache.  Sequence b
+ * receives seq_tokens[b] new tokens (NULL = N each) at positions seq_start[b].. (NULL = 0..) of table
+ * row seq_rows[b]; its source rows are k_src/v_src + b*stride_b + t*stride_n (elements; each row is
+ * H*d contiguous elements), i.e. the [B,N,H,d] K and V tensors a FlashAttention forward just read, or -
+ * with cu_seqlens (int32[B+1], device) - rows cu_seqlens[b].. of a packed [T,H,d] batch (lengths from
+ * cu_seqlens, stride_b ignored).  N bounds the tokens per sequence (it sizes the grid).  All index
+ * arrays live on the device.  Same layout, conversion and skipping rules as ahpc_hip_kv_scatter; the
+ * reference appends one sequence at a time (PagedAttention::append_kv_cache,
+ * src/algorithms/paged_attention.cpp:434-462). */
+int ahpc_hip_kv_scatter_batch(const void* k_src, const void* v_src, int in_dtype,
+                              int64_t stride_b, int64_t stride_n,
+                              void* k_pool, void* v_pool, int pool_dtype,
+                              const int32_t* block_table, int64_t max_pages,
+                              const int32_t* seq_rows, const int32_t* seq_start, const int32_t* seq_tokens,
+                              const int32_t* cu_seqlens,
+                              int64_t B, int64_t N, int64_t H, int64_t d, int64_t P, void* stream);
+
 /* Read tokens [start, start+n) of table row `row` back as [n,H,d] in out_dtype.  Replaces
  * PagedAttention::get_kv_cache -> gather_keys_values,
  * src/algorithms/paged_attention.cpp:464-490. */

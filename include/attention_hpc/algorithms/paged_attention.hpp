@@ -87,6 +87,16 @@ public:
     // taken from the pool as needed.  Unknown sequence -> INVALID_INPUT.
     void append_kv_cache(size_t sequence_id, const void* key_data, const void* value_data, size_t num_tokens,
                          DataType data_type);
+    // The prefill -> cache hand-off: the K and V tensors a FlashAttention forward just attended over go into
+    // the caches of `sequence_ids` in ONE launch.  Dense: kv_shape = {B, N, key_value_heads, head_dim}, batch
+    // entry b feeds sequence_ids[b] with its first num_tokens[b] tokens (empty vector = all N).  Packed:
+    // kv_shape = {total_tokens, key_value_heads, head_dim} with cu_seqlens[0..B] as in forward_varlen.
+    // Host or device memory; same errors as append_kv_cache.  (The reference appends one sequence per call,
+    // src/algorithms/paged_attention.cpp:434-462.)
+    void append_kv_cache_batch(const std::vector<size_t>& sequence_ids, const TensorShape& kv_shape, const void* key_data,
+                               const void* value_data, const std::vector<size_t>& num_tokens = {});
+    void append_kv_cache_packed(const std::vector<size_t>& sequence_ids, const TensorShape& kv_shape, const void* key_data,
+                                const void* value_data, const int32_t* cu_seqlens);
     void get_kv_cache(size_t sequence_id, void* key_data, void* value_data, size_t start_token, size_t num_tokens,
                       DataType data_type);
     void clear_kv_cache(size_t sequence_id);

@@ -784,6 +784,66 @@ CASE(Gqa_PagedDecodeEqualsRepeatedHeads, true) {
     EXPECT_THROWS(pa.configure(p), AttentionError::UNSUPPORTED_OPERATION);
 }
 
+CASE(Paged_PrefillHandOffBatchAndPacked, true) {
+    // K/V of a prefill batch go into the caches of several sequences in one call; reading them back and
+    // decoding must give what appending sequence by sequence gives.
+    const size_t B = 3, N = 40, H = 4, d = 64;
+    AttentionParams p{};
+    p.batch_size = B; p.sequence_length = 1; p.num_heads = H; p.head_dimension = d; p.max_sequence_length = 256;
+    PagedAttention a, b;
+    a.configure(p);
+    b.configure(p);
+    auto k = normal(B * N * H * d, 97, 2), v = normal(B * N * H * d, 97, 3);
+    const std::vector<size_t> counts = {40, 7, 33};
+    std::vector<size_t> ia, ib;
+    for (size_t i = 0; i < B; ++i) {
+        ia.push_back(a.create_sequence(256));
+        ib.push_back(b.create_sequence(256));
+    }
+    // both start with a few tokens already cached, so that the new ones land mid-page
+    auto k0 = normal(5 * H * d, 98, 2), v0 = normal(5 * H * d, 98, 3);
+    for (size_t i = 0; i < B; ++i) {
+        a.append_kv_cache(ia[i], k0.data(), v0.data(), 5, DataType::FLOAT32);
+        b.append_kv_cache(ib[i], k0.data(), v0.data(), 5, DataType::FLOAT32);
+    }
+    a.append_kv_cache_batch(ia, shape4(B, N, H, d), k.data(), v.data(), counts);
+    for (size_t i = 0; i < B; ++i) b.append_kv_cache(ib[i], k.data() + i * N * H * d, v.data() + i * N * H * d, counts[i], DataType::FLOAT32);
+    for (size_t i = 0; i < B; ++i) {
+        EXPECT(a.get_sequence_length(ia[i]) == 5 + counts[i]);
+        EXPECT(a.get_sequence_pages(ia[i]) == b.get_sequence_pages(ib[i]));
+        const size_t L = 5 + counts[i];
+        std::vector<float> ka(L * H * d), va(L * H * d), kb(L * H * d), vb(L * H * d);
+        a.get_kv_cache(ia[i], ka.data(), va.data(), 0, L, DataType::FLOAT32);
+        b.get_kv_cache(ib[i], kb.data(), vb.data(), 0, L, DataType::FLOAT32);
+        EXPECT(ka == kb && va == vb);
+    }
+    // packed: three more chunks of lengths 9, 0, 20 out of one [29,H,d] tensor
+    const int32_t cu[4] = {0, 9, 9, 29};
+    auto kp = normal(29 * H * d, 99, 2), vp = normal(29 * H * d, 99, 3);
+    a.append_kv_cache_packed(ia, TensorShape({29, H, d}, DataType::FLOAT32), kp.data(), vp.data(), cu);
+    for (size_t i = 0; i < B; ++i) {
+        const size_t n = (size_t)(cu[i + 1] - cu[i]);
+        if (n) b.append_kv_cache(ib[i], kp.data() + (size_t)cu[i] * H * d, vp.data() + (size_t)cu[i] * H * d, n, DataType::FLOAT32);
+    }
+    std::vector<TensorShape> shp(B, TensorShape({1, 1, H, d}, DataType::FLOAT32));
+    auto q = normal(B * H * d, 97, 1);
+    std::vector<float> oa(B * H * d, 1.0f), ob(B * H * d, 2.0f);
+    std::vector<const void*> qp;
+    std::vector<void*> pa, pb;
+    for (size_t i = 0; i < B; ++i) {
+        qp.push_back(q.data() + i * H * d);
+        pa.push_back(oa.data() + i * H * d);
+        pb.push_back(ob.data() + i * H * d);
+    }
+    a.forward_batch(ia, shp, qp, shp, pa);
+    b.forward_batch(ib, shp, qp, shp, pb);
+    EXPECT(oa == ob);
+    EXPECT_THROWS(a.append_kv_cache_batch({ia[0], 4242, ia[2]}, shape4(B, N, H, d), k.data(), v.data()), AttentionError::INVALID_INPUT);
+    EXPECT_THROWS(a.append_kv_cache_batch({ia[0], ia[0], ia[2]}, shape4(B, N, H, d), k.data(), v.data()), AttentionError::INVALID_INPUT);
+    EXPECT_THROWS(a.append_kv_cache_batch(ia, shape4(B, N, H + 1, d), k.data(), v.data()), AttentionError::INVALID_INPUT);
+    EXPECT(a.get_sequence_length(ia[0]) == 5 + 40 + 9);  // failed calls changed nothing
+}
+
 CASE(Paged_SequenceLifecycle, true) {  // extend / truncate / reset, src/algorithms/paged_attention.cpp:352-418
     PagedAttention pa;
     AttentionParams p{};

@@ -234,3 +234,79 @@ def test_bad_arguments_are_rejected_without_launch(gpu):
     with pytest.raises(gpu.HipError):
         gpu.paged_decode(p, p, O.F32, p, p, O.F32, p, p, None, 1, 4, 64, 16, 64, 1024, 0.1, chunk_tokens=16, workspace=None, workspace_bytes=0)
     torch.cuda.synchronize()
+
+
+# ---- batched append: the prefill -> cache hand-off ---------------------------------------------------
+def _tables_for(lens_total, P, seed, extra=3):
+    lens_total = np.asarray(lens_total, np.int32)
+    pages_per = (lens_total + P - 1) // P
+    n_pages = int(pages_per.sum()) + extra
+    ids = O.permutation(n_pages, seed, 5)
+    table = np.full((len(lens_total), max(1, int(pages_per.max()))), -1, np.int32)
+    c = 0
+    for b in range(len(lens_total)):
+        table[b, :pages_per[b]] = ids[c:c + pages_per[b]]
+        c += pages_per[b]
+    return table, n_pages
+
+
+@pytest.mark.parametrize("in_dtype,pool_dtype", [(O.F16, O.F16), (O.BF16, O.BF16), (O.F32, O.F32), (O.F32, O.F16), (O.BF16, O.F32)])
+def test_scatter_batch_dense_prefill_matches_oracle_bit_for_bit(gpu, in_dtype, pool_dtype):
+    import torch
+    from gpu_util import to_dev, to_host, stream_ptr, dev_i32
+    B, N, H, d, P = 4, 70, 3, 64, 16
+    start = np.array([0, 5, 16, 33], np.int32)       # tokens already cached per sequence
+    n_new = np.array([70, 1, 0, 37], np.int32)       # new tokens taken from the [B,N,H,d] prefill tensors
+    rows = np.array([2, 0, 3, 1], np.int32)          # batch entry -> table row
+    lens_total = np.zeros(4, np.int32)
+    lens_total[rows] = start + n_new
+    table, n_pages = _tables_for(lens_total, P, 61)
+    k = O.round_to(O.fill_normal((B, N, H, d), 61, 2), in_dtype)
+    v = O.round_to(O.fill_normal((B, N, H, d), 61, 3), in_dtype)
+    kp = np.zeros(n_pages * P * H * d, np.float32)
+    vp = np.zeros_like(kp)
+    for b in range(B):
+        if n_new[b]:
+            O.kv_scatter(O.round_to(k[b, :n_new[b]], pool_dtype), O.round_to(v[b, :n_new[b]], pool_dtype), kp, vp, table,
+                         int(rows[b]), int(start[b]), P, H, d)
+    dk, dv = to_dev(k, in_dtype), to_dev(v, in_dtype)
+    dkp, dvp = to_dev(np.zeros_like(kp), pool_dtype), to_dev(np.zeros_like(vp), pool_dtype)
+    # the index arrays must stay alive until the launch has run: keep the tensors, not just their addresses
+    dtab, drows, dstart, dnew = dev_i32(table), dev_i32(rows), dev_i32(start), dev_i32(n_new)
+    gpu.kv_scatter_batch(dk.data_ptr(), dv.data_ptr(), in_dtype, N * H * d, H * d, dkp.data_ptr(), dvp.data_ptr(), pool_dtype,
+                         dtab.data_ptr(), table.shape[1], drows.data_ptr(), B, N, H, d, P,
+                         seq_start=dstart.data_ptr(), seq_tokens=dnew.data_ptr(), stream=stream_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host(dkp), kp) and np.array_equal(to_host(dvp), vp)
+
+
+def test_scatter_batch_packed_prefill_then_decode(gpu):
+    """Ragged prefill tensors [T,H,d] + cu_seqlens -> pool in one launch; a decode over the pool then
+    matches the oracle's decode over the oracle-filled pool."""
+    import torch
+    from gpu_util import to_dev, to_host, stream_ptr, dev_i32
+    H, d, P = 8, 128, 16
+    lens = np.array([130, 16, 1, 255], np.int32)
+    B = len(lens)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    table, n_pages = _tables_for(lens, P, 62)
+    k = O.round_to(O.fill_normal((T, H, d), 62, 2), O.F16)
+    v = O.round_to(O.fill_normal((T, H, d), 62, 3), O.F16)
+    kp = np.zeros(n_pages * P * H * d, np.float32)
+    vp = np.zeros_like(kp)
+    for b in range(B):
+        O.kv_scatter(k[cu[b]:cu[b + 1]], v[cu[b]:cu[b + 1]], kp, vp, table, b, 0, P, H, d)
+    dk, dv = to_dev(k, O.F16), to_dev(v, O.F16)
+    dkp, dvp = to_dev(np.zeros_like(kp), O.F16), to_dev(np.zeros_like(vp), O.F16)
+    dtab, drows, dcu = dev_i32(table), dev_i32(np.arange(B, dtype=np.int32)), dev_i32(cu)
+    gpu.kv_scatter_batch(dk.data_ptr(), dv.data_ptr(), O.F16, 0, H * d, dkp.data_ptr(), dvp.data_ptr(), O.F16,
+                         dtab.data_ptr(), table.shape[1], drows.data_ptr(), B, int(lens.max()), H, d, P,
+                         cu_seqlens=dcu.data_ptr(), stream=stream_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host(dkp), kp) and np.array_equal(to_host(dvp), vp)
+    q = O.round_to(O.fill_normal((B, H, d), 62, 1), O.F16)
+    scale = 1.0 / np.sqrt(d)
+    got = gpu_decode(gpu, q, dkp, dvp, table, lens, None, B, H, d, P, O.F16, O.F16, scale)
+    want = O.paged_decode(q, kp, vp, table, lens, None, B, H, d, P, scale)
+    assert np.abs(got - want).max() <= 2e-2
