@@ -109,8 +109,8 @@ template <int D> struct FlashTile {
 // as zero), off[i] = this lane's byte offset for its i-th instruction, wave_u = wavefront index (uniform).
 template <int D>
 __device__ inline void dma_tile(const void* base, unsigned nrec, const int* off, unsigned char* lds_tile, int wave_u) {
-    typedef FlashTile<D> TL;
 #if defined(__HIP_DEVICE_COMPILE__)  // the descriptor type exists only in the device pass
+    typedef FlashTile<D> TL;
     const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, nrec, 0x00020000);
 #pragma unroll
     for (int i = 0; i < TL::kInstrPerWave; ++i)
