@@ -150,8 +150,10 @@ static int dispatch_simple(int dtype, const SimpleParams& p, int64_t B, hipStrea
 }
 
 // ---------------------------------------------------------------------------------------------
-template <typename T, int D, bool VARLEN>
-static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
+// Fills the launch geometry of the MFMA kernel (query tiles, pairing, workgroup count, interleaving of
+// heads) from N, H and the batch size already in `p`.  Shared by the launcher and by the host-side dump
+// of the workgroup map.
+static int plan_mfma(FlashParams& p, int64_t B, bool causal) {
     p.n_qtiles = (p.N + kFlashRows - 1) / kFlashRows;
     int64_t total = B * p.H * (int64_t)p.n_qtiles;
     if (total > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
@@ -161,6 +163,22 @@ static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream
     if (p.paired) total = B * p.H * (int64_t)((p.n_qtiles + 1) / 2);
     p.total_blocks = (int32_t)total;
     p.blocks_per_xcd = (int32_t)((total + 7) / 8);
+    // AHPC_FLASH_HEADS_TOGETHER = n lets n heads advance side by side on an XCD (default: one after the
+    // other); AHPC_FLASH_ROUND_SLOTS sets how many workgroups a head contributes per round (default 64 / n:
+    // an XCD holds 64 workgroups of this kernel).  Tuning knobs; every setting computes the same result.
+    int ht = 1, rs = 0;
+    if (const char* e = std::getenv("AHPC_FLASH_HEADS_TOGETHER")) ht = std::atoi(e);
+    if (const char* e = std::getenv("AHPC_FLASH_ROUND_SLOTS")) rs = std::atoi(e);
+    if (ht < 1 || ht > 64) ht = 1;
+    if (rs < 1) rs = 64 / ht;
+    p.heads_together = ht;
+    p.round_slots = rs;
+    return AHPC_OK;
+}
+
+template <typename T, int D, bool VARLEN>
+static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
+    if (int rc = plan_mfma(p, B, causal)) return rc;
     dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
     if (causal) hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, true, VARLEN>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, false, VARLEN>), grid, block, 0, stream, p);
@@ -229,6 +247,26 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
     }
     SimpleParams p{q, k, v, o, nullptr, mask, sq.b, sq.n, sq.h, skv.b, skv.n, skv.h, (int32_t)N, (int32_t)H, (int32_t)d, group, scale, causal ? 1 : 0};
     return dispatch_simple<false>(dtype, p, B, st);
+}
+
+int ahpc_hip_flash_block_map(int64_t B, int64_t N, int64_t H, int causal, int64_t capacity, int64_t* n_blocks,
+                             int32_t* seq_head, int32_t* first_tile, int32_t* second_tile) {
+    if (!n_blocks) return AHPC_ERR_NULL_POINTER;
+    if (B <= 0 || N <= 0 || H <= 0 || B > 65535 || H > 65535 || N > 0x7FFFFF00ll) return AHPC_ERR_BAD_SHAPE;
+    FlashParams p{};
+    p.N = (int32_t)N; p.H = (int32_t)H; p.kv_group = 1;
+    if (int rc = plan_mfma(p, B, causal != 0)) return rc;
+    const int64_t grid = (int64_t)p.blocks_per_xcd * 8;
+    *n_blocks = grid;
+    if (!seq_head && !first_tile && !second_tile) return AHPC_OK;
+    if (!seq_head || !first_tile || !second_tile || capacity < grid) return AHPC_ERR_BAD_SHAPE;
+    for (int64_t i = 0; i < grid; ++i) {
+        const FlashWork w = flash_work_of_block((unsigned)i, p);
+        seq_head[i] = w.valid ? w.bh : -1;
+        first_tile[i] = w.valid ? flash_qtile_of_part(p, w.slot, 0) : -1;
+        second_tile[i] = w.valid ? flash_qtile_of_part(p, w.slot, 1) : -1;
+    }
+    return AHPC_OK;
 }
 
 int ahpc_hip_flash_fwd_masked(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N,

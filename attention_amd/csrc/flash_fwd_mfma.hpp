@@ -58,6 +58,8 @@ struct FlashParams {
     int32_t paired;             // 1: a workgroup takes two query tiles of a head (see above)
     int32_t total_blocks;       // B * H * n_qtiles, or B * H * ceil(n_qtiles / 2) when paired
     int32_t blocks_per_xcd;     // ceil(total_blocks / 8)
+    int32_t heads_together;     // <= 1: a head's workgroups are consecutive; n: n heads advance side by side
+    int32_t round_slots;        // with heads_together > 1: workgroups one head contributes per round
     float scale_log2;           // scale * log2(e)
 };
 
@@ -119,6 +121,53 @@ __device__ inline void dma_tile(const void* base, unsigned nrec, const int* off,
 #endif
 }
 
+// Workgroup id -> work.  Hardware deals consecutive workgroup ids to the 8 XCDs in turn; `logical` undoes
+// that, so that consecutive logical ids run on the same XCD and share its L2.  A head owns `per_head`
+// consecutive logical ids (its query tiles, or pairs of them), late (long) tiles first.  With
+// heads_together = n > 1 the ids of n heads are interleaved instead, round_slots of each head per round,
+// so that n heads stream their K/V side by side (more L2 channels busy, less reuse per head).
+// Host and device evaluate the same code: a host-side dump of this function is what the tests check.
+struct FlashWork {
+    int bh;     // sequence * H + head
+    int slot;   // 0 .. per_head-1
+    bool valid;
+};
+__host__ __device__ inline int flash_per_head(const FlashParams& p) { return p.paired ? (p.n_qtiles + 1) >> 1 : p.n_qtiles; }
+__host__ __device__ inline FlashWork flash_work_of_block(unsigned block_id, const FlashParams& p) {
+    const int xcd = (int)(block_id & 7u);
+    const int logical = xcd * p.blocks_per_xcd + (int)(block_id >> 3);
+    if (logical >= p.total_blocks) return FlashWork{0, 0, false};
+    const int per_head = flash_per_head(p);
+    if (p.heads_together <= 1) {
+        const int bh = logical / per_head;
+        return FlashWork{bh, logical - bh * per_head, true};
+    }
+    const int n_heads = p.total_blocks / per_head;
+    const int group = logical / (p.heads_together * per_head);
+    const int first = group * p.heads_together;
+    const int ch = (n_heads - first) < p.heads_together ? (n_heads - first) : p.heads_together;  // heads in this group
+    const int r = logical - first * per_head;                 // 0 .. ch*per_head-1
+    const int sl = p.round_slots > 0 ? p.round_slots : 1;
+    const int full_rounds = per_head / sl;
+    const int full_items = full_rounds * ch * sl;
+    if (r < full_items) {
+        const int round = r / (ch * sl);
+        const int rr = r - round * (ch * sl);
+        return FlashWork{first + rr / sl, round * sl + rr % sl, true};
+    }
+    const int rem = per_head - full_rounds * sl;               // slots of the last, partial round (> 0 here)
+    const int rr = r - full_items;
+    return FlashWork{first + rr / rem, full_rounds * sl + rr % rem, true};
+}
+// Query tile a workgroup handles in its first (part 0) and second (part 1) pass; -1 = none.
+__host__ __device__ inline int flash_qtile_of_part(const FlashParams& p, int slot, int part) {
+    if (p.paired) {
+        if (part == 1 && 2 * slot == p.n_qtiles - 1) return -1;  // odd count: the middle tile has no partner
+        return part == 0 ? p.n_qtiles - 1 - slot : slot;
+    }
+    return part == 0 ? p.n_qtiles - 1 - slot : -1;
+}
+
 template <typename T, int D, bool CAUSAL, bool VARLEN>
 __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const FlashParams p) {
     typedef FlashTile<D> TL;
@@ -138,15 +187,10 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
     const int col = lane & 31;   // query column / operand row owned by this lane
     const int half = lane >> 5;
 
-    // Workgroup id -> (sequence*head, query tile or pair of tiles).  Consecutive logical ids run on the
-    // same XCD so that the tiles of one head share that XCD's L2; within a head the long (late) tiles
-    // go first.
-    const int xcd = blockIdx.x & 7;
-    const int logical = xcd * p.blocks_per_xcd + (blockIdx.x >> 3);
-    if (logical >= p.total_blocks) return;
-    const int per_head = p.paired ? (p.n_qtiles + 1) >> 1 : p.n_qtiles;
-    const int bh = logical / per_head;
-    const int slot = logical - bh * per_head;
+    const FlashWork work = flash_work_of_block(blockIdx.x, p);
+    if (!work.valid) return;
+    const int bh = work.bh;
+    const int slot = work.slot;
     const int b = bh / p.H;
     const int h = bh - b * p.H;
 
@@ -207,14 +251,8 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
     }
 
     for (int part = 0; part < 2; ++part) {
-        int qt;
-        if (p.paired) {
-            if (part == 1 && 2 * slot == p.n_qtiles - 1) break;  // odd count: the middle tile has no partner
-            qt = part == 0 ? p.n_qtiles - 1 - slot : slot;
-        } else {
-            if (part == 1) break;
-            qt = p.n_qtiles - 1 - slot;
-        }
+        const int qt = flash_qtile_of_part(p, slot, part);
+        if (qt < 0) break;
         const int q_tile0 = qt * kFlashRows;
         if (q_tile0 >= L) continue;
 

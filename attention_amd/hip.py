@@ -60,6 +60,7 @@ SIGNATURES = {
     "ahpc_hip_event_elapsed_ms": (_ci, [_vp, _vp, C.POINTER(_f32)]),
     "ahpc_hip_flash_fwd": (_ci, [_vp, _vp, _vp, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp]),
     "ahpc_hip_flash_fwd_gqa": (_ci, [_vp, _vp, _vp, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp, _vp]),
+    "ahpc_hip_flash_block_map": (_ci, [_i64, _i64, _i64, _ci, _i64, C.POINTER(_i64), _vp, _vp, _vp]),
     "ahpc_hip_flash_fwd_masked": (_ci, [_vp, _vp, _vp, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp, _vp]),
     "ahpc_hip_flash_fwd_varlen": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp]),
     "ahpc_hip_flash_fwd_varlen_gqa": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp]),
@@ -119,6 +120,17 @@ def flash_fwd(q, k, v, o, dtype, B, N, H, d, strides, scale, causal, stream=None
     else:
         rc = load().ahpc_hip_flash_fwd_masked(q, k, v, o, dtype, B, N, H, d, sb, sn, sh, scale, int(causal), mask, stream)
     _check(rc, "flash_fwd")
+
+
+def flash_block_map(B, N, H, causal):
+    """Host-side dump of the MFMA kernel's workgroup -> (sequence*head, first tile, second tile) map (numpy)."""
+    import numpy as np
+    n = _i64(0)
+    _check(load().ahpc_hip_flash_block_map(B, N, H, int(causal), 0, C.byref(n), None, None, None), "flash_block_map")
+    bh, t0, t1 = (np.empty(n.value, np.int32) for _ in range(3))
+    _check(load().ahpc_hip_flash_block_map(B, N, H, int(causal), n.value, C.byref(n), bh.ctypes.data, t0.ctypes.data,
+                                          t1.ctypes.data), "flash_block_map")
+    return bh, t0, t1
 
 
 def flash_fwd_gqa(q, k, v, o, dtype, B, N, H, H_kv, d, strides, kv_strides, scale, causal, stream=None, mask=None):

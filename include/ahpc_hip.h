@@ -147,6 +147,16 @@ int ahpc_hip_flash_fwd_varlen_gqa(const void* q, const void* k, const void* v, v
                                   int64_t stride_t, int64_t stride_h, int64_t kv_stride_t, int64_t kv_stride_h,
                                   float scale, int causal, void* stream);
 
+/* Debug twin of the MFMA kernel's launch geometry, evaluated on the HOST by the very function the kernel
+ * uses (no GPU needed): for a dense fp16/bf16 launch of B sequences, N tokens, H heads it reports the grid
+ * size in *n_blocks and, when the three arrays (capacity entries each) are given, for every workgroup id
+ * its (sequence * H + head), the query tile (of 128 rows) it handles first and the one it handles second
+ * (-1 = none; all -1 for padding workgroups).  Lets a test check that every query tile of every head is
+ * handled exactly once, whatever the pairing and interleaving in force.  No counterpart in the reference
+ * (its kernels are launched one tile per block, src/backends/cuda/cuda_kernels.cu:125-127). */
+int ahpc_hip_flash_block_map(int64_t B, int64_t N, int64_t H, int causal, int64_t capacity, int64_t* n_blocks,
+                             int32_t* seq_head, int32_t* first_tile, int32_t* second_tile);
+
 /* ---- paged KV pool ---------------------------------------------------------------------------
  * Pool layout: K and V are separate slabs  [page][slot 0..P-1][head][d]  (the layout
  * update_kv_cache_kernel writes, src/backends/cuda/cuda_kernels.cu:547-556).
