@@ -67,7 +67,9 @@ constexpr int kFlashThreads = 256;
 constexpr int kFlashRows = 128;  // query rows per workgroup
 constexpr int kFlashKeys = 64;   // keys per tile
 
+#ifndef AHPC_LDS
 #define AHPC_LDS __attribute__((address_space(3)))
+#endif
 
 template <typename T> struct TrRead;
 template <> struct TrRead<bf16_t> {

@@ -1,0 +1,100 @@
+// Test infrastructure: small kernels that exist only to check the lane-by-lane executor itself.  Most of
+// them are wrong on purpose (a barrier only part of a wavefront reaches, lanes at different cross-lane
+// operations, a direct-to-LDS load consumed before its wait); they are compiled for the CPU executor
+// only, never for a GPU.  The others are known-answer checks of the cross-lane operations.
+#include <hip/hip_runtime.h>
+
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+__global__ void half_wave_at_barrier(float* out) {
+    float x = (float)threadIdx.x;
+    if (threadIdx.x & 1) __syncthreads();
+    else x = __shfl_xor(x, 1, 64);
+    out[threadIdx.x] = x;
+}
+
+__global__ void lanes_at_different_operations(float* out) {
+    float x = (float)threadIdx.x;
+    if (threadIdx.x & 1) x = __shfl_xor(x, 2, 64);
+    else x = (float)__builtin_amdgcn_ballot_w64(x > 3.0f);
+    out[threadIdx.x] = x;
+}
+
+__global__ void reads_a_finished_lane(int* out) {
+    if (threadIdx.x >= 32) return;
+    out[threadIdx.x] = __builtin_amdgcn_readlane((int)threadIdx.x, 40);
+}
+
+// every lane copies 16 bytes global -> LDS with the direct load and reads them back; `wait` says whether
+// the wait that makes the data visible is executed
+__global__ void dma_round_trip(const unsigned char* src, unsigned char* dst, int wait) {
+    __shared__ __attribute__((aligned(1024))) unsigned char tile[1024];
+    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(src), 0, 1000, 0x00020000);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, tile, 16, (int)threadIdx.x * 16, 0, 0, 0);
+    if (wait) __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    for (int i = 0; i < 16; ++i) dst[threadIdx.x * 16 + i] = tile[threadIdx.x * 16 + i];
+}
+
+// D = A * B + C with A[i][k] = a[i*16+k], B[k][j] = b[k*32+j], operands and result laid out as documented
+// for v_mfma_f32_32x32x16_bf16
+__global__ void matrix_instruction(const float* a, const float* b, const float* c, float* d) {
+    const int lane = threadIdx.x, col = lane & 31, half = lane >> 5;
+    bf16x8 av, bv;
+    for (int e = 0; e < 8; ++e) {
+        av[e] = (__bf16)a[col * 16 + 8 * half + e];
+        bv[e] = (__bf16)b[(8 * half + e) * 32 + col];
+    }
+    f32x16 acc;
+    for (int r = 0; r < 16; ++r) acc[r] = c[(8 * (r / 4) + 4 * half + r % 4) * 32 + col];
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc, 0, 0, 0);
+    for (int r = 0; r < 16; ++r) d[(8 * (r / 4) + 4 * half + r % 4) * 32 + col] = acc[r];
+}
+
+// butterfly sums over 2, 4, 8 and 16 neighbouring lanes with the DPP controls the decode kernel uses
+__global__ void dpp_sums(const float* in, float* out) {
+    float x = in[threadIdx.x];
+    auto dpp = [](float v, int ctrl) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xF, 0xF, true));
+    };
+    x += dpp(x, 0xB1);
+    out[threadIdx.x] = x;
+    x += dpp(x, 0x4E);
+    out[64 + threadIdx.x] = x;
+    x += dpp(x, 0x141);
+    out[128 + threadIdx.x] = x;
+    x += dpp(x, 0x140);
+    out[192 + threadIdx.x] = x;
+}
+
+}  // namespace
+
+extern "C" {
+int simt_selftest_half_wave_at_barrier(float* out) {
+    hipLaunchKernelGGL(half_wave_at_barrier, dim3(1), dim3(64), 0, nullptr, out);
+    return hipGetLastError();
+}
+int simt_selftest_lanes_at_different_operations(float* out) {
+    hipLaunchKernelGGL(lanes_at_different_operations, dim3(1), dim3(64), 0, nullptr, out);
+    return hipGetLastError();
+}
+int simt_selftest_reads_a_finished_lane(int* out) {
+    hipLaunchKernelGGL(reads_a_finished_lane, dim3(1), dim3(64), 0, nullptr, out);
+    return hipGetLastError();
+}
+int simt_selftest_dma_round_trip(const unsigned char* src, unsigned char* dst, int wait) {
+    hipLaunchKernelGGL(dma_round_trip, dim3(1), dim3(64), 0, nullptr, src, dst, wait);
+    return hipGetLastError();
+}
+int simt_selftest_matrix_instruction(const float* a, const float* b, const float* c, float* d) {
+    hipLaunchKernelGGL(matrix_instruction, dim3(1), dim3(64), 0, nullptr, a, b, c, d);
+    return hipGetLastError();
+}
+int simt_selftest_dpp_sums(const float* in, float* out) {
+    hipLaunchKernelGGL(dpp_sums, dim3(1), dim3(64), 0, nullptr, in, out);
+    return hipGetLastError();
+}
+}

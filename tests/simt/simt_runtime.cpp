@@ -1,0 +1,491 @@
+// Test infrastructure: executes kernels compiled against shim/hip/hip_runtime.h on the CPU.
+// One operating-system thread; every work-item of the workgroup being executed is a ucontext fiber.
+// A fiber runs until it needs the other lanes (cross-lane operation, barrier) and then yields; the
+// scheduler resumes fibers whose condition has become true, visiting wavefronts in a seeded random
+// order so that different interleavings of the wavefronts of a workgroup are exercised.
+#include <hip/hip_runtime.h>
+#include <ucontext.h>
+
+#include <cstdio>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#if defined(__has_feature)
+#if __has_feature(address_sanitizer)
+#define SIMT_ASAN 1
+extern "C" void __sanitizer_start_switch_fiber(void** fake_stack_save, const void* bottom, size_t size);
+extern "C" void __sanitizer_finish_switch_fiber(void* fake_stack_save, const void** bottom_old, size_t* size_old);
+#endif
+#endif
+
+dim3 threadIdx, blockIdx, blockDim, gridDim;
+
+extern "C" unsigned char __start_simt_lds[];
+extern "C" unsigned char __stop_simt_lds[];
+
+namespace simt {
+namespace {
+
+constexpr int kWaveSize = 64;
+constexpr int kPayload = 64;          // bytes a lane can publish per cross-lane operation
+constexpr size_t kStackBytes = 512 * 1024;
+
+enum Kind : int { K_NONE = 0, K_MFMA, K_TR, K_SWAP, K_BALLOT, K_RFL, K_RL, K_DPP, K_SHFL };
+
+struct PendingDma {
+    unsigned char* dst;
+    const unsigned char* src;  // null: zeros
+};
+
+struct Wave {
+    int live = 0;
+    int arrived[2] = {0, 0};
+    long gen_of[2] = {-1, -1};
+    int kind[2] = {K_NONE, K_NONE};
+    bool present[2][kWaveSize];
+    alignas(16) unsigned char slot[2][kWaveSize][kPayload];
+};
+
+struct Fiber {
+    ucontext_t ctx;
+    unsigned char* stack = nullptr;
+    dim3 tid;
+    int wave = 0, lane = 0;
+    bool done = false;
+    const int* wait_counter = nullptr;  // resume when *wait_counter >= *wait_target
+    const int* wait_target = nullptr;
+    long coll_gen = 0, bar_gen = 0;
+    std::vector<PendingDma> dma;
+    void* asan_fake = nullptr;
+};
+
+struct Block {
+    std::vector<Fiber> fibers;
+    std::vector<Wave> waves;
+    int live = 0;
+    int bar_arrived[2] = {0, 0};
+    long bar_gen_of[2] = {-1, -1};
+};
+
+Block g_block;
+Fiber* g_cur = nullptr;
+ucontext_t g_main;
+void* g_main_fake = nullptr;
+const void* g_main_bottom = nullptr;  // the scheduler's stack, as AddressSanitizer reports it
+size_t g_main_size = 0;
+const std::function<void()>* g_body = nullptr;
+std::string g_error;
+thread_local hipError_t g_status = hipSuccess;  // what hipGetLastError reports to the launching thread
+std::mutex g_launch_mutex;                      // one launch at a time: the executor's state is global
+bool g_dma_late = false;
+uint64_t g_rng = 0x9E3779B97F4A7C15ull;
+std::vector<unsigned char*> g_stacks;  // reused between launches
+long g_switches = 0;
+
+uint64_t next_rand() {
+    g_rng ^= g_rng << 13;
+    g_rng ^= g_rng >> 7;
+    g_rng ^= g_rng << 17;
+    return g_rng;
+}
+
+void enter_fiber(Fiber* f) {
+    g_cur = f;
+    threadIdx = f->tid;
+    ++g_switches;
+#ifdef SIMT_ASAN
+    __sanitizer_start_switch_fiber(&g_main_fake, f->stack, kStackBytes);
+#endif
+    swapcontext(&g_main, &f->ctx);
+#ifdef SIMT_ASAN
+    __sanitizer_finish_switch_fiber(g_main_fake, nullptr, nullptr);
+#endif
+    g_cur = nullptr;
+}
+
+void yield_to_scheduler() {
+    Fiber* f = g_cur;
+#ifdef SIMT_ASAN
+    __sanitizer_start_switch_fiber(&f->asan_fake, g_main_bottom, g_main_size);
+#endif
+    swapcontext(&f->ctx, &g_main);
+#ifdef SIMT_ASAN
+    __sanitizer_finish_switch_fiber(f->asan_fake, &g_main_bottom, &g_main_size);
+#endif
+    threadIdx = f->tid;
+}
+
+[[noreturn]] void leave_for_good() {
+    // Used on errors and at the end of a fiber: never comes back to this fiber.
+    Fiber* f = g_cur;
+#ifdef SIMT_ASAN
+    __sanitizer_start_switch_fiber(nullptr, g_main_bottom, g_main_size);
+#endif
+    swapcontext(&f->ctx, &g_main);
+    std::abort();
+}
+
+void fail(const std::string& what) {
+    if (g_error.empty()) {
+        char where[160];
+        if (g_cur)
+            std::snprintf(where, sizeof where, " [block (%u,%u,%u) thread %u wave %d lane %d]", blockIdx.x, blockIdx.y,
+                          blockIdx.z, g_cur->tid.x, g_cur->wave, g_cur->lane);
+        else
+            where[0] = 0;
+        g_error = what + where;
+        std::fprintf(stderr, "simt: %s\n", g_error.c_str());
+    }
+    g_status = hipErrorLaunchFailure;
+    if (g_cur) {
+        g_cur->done = true;  // the scheduler stops at the first error
+        leave_for_good();
+    }
+}
+
+void flush_dma(Fiber* f) {
+    for (const PendingDma& d : f->dma) {
+        if (d.src) std::memcpy(d.dst, d.src, 16);
+        else std::memset(d.dst, 0, 16);
+    }
+    f->dma.clear();
+}
+
+void wait_until(const int* counter, const int* target) {
+    Fiber* f = g_cur;
+    while (*counter < *target) {
+        f->wait_counter = counter;
+        f->wait_target = target;
+        yield_to_scheduler();
+        if (g_status != hipSuccess) {
+            f->done = true;
+            leave_for_good();
+        }
+    }
+    f->wait_counter = f->wait_target = nullptr;
+}
+
+void trampoline() {
+#ifdef SIMT_ASAN
+    __sanitizer_finish_switch_fiber(nullptr, &g_main_bottom, &g_main_size);
+#endif
+    Fiber* f = g_cur;
+    threadIdx = f->tid;
+    (*g_body)();
+    flush_dma(f);  // the hardware completes outstanding loads of a finished wave as well
+    f->done = true;
+    g_block.waves[f->wave].live--;
+    g_block.live--;
+    leave_for_good();
+}
+
+// Publishes `n` bytes for the other lanes of the wavefront and waits until every live lane of the
+// wavefront has published for the same operation.  Returns the generation's slot table.
+struct View {
+    const Wave* w;
+    int g;
+    const unsigned char* of(int lane) const {
+        if (!w->present[g][lane]) fail("cross-lane operation reads a lane that is not executing it");
+        return w->slot[g][lane];
+    }
+    bool has(int lane) const { return w->present[g][lane]; }
+};
+
+View exchange(int kind, const void* payload, size_t n) {
+    Fiber* f = g_cur;
+    if (!f) {
+        std::fprintf(stderr, "simt: cross-lane operation outside a kernel\n");
+        std::abort();
+    }
+    Wave& w = g_block.waves[f->wave];
+    const long gen = f->coll_gen++;
+    const int g = (int)(gen & 1);
+    if (w.gen_of[g] != gen) {
+        w.gen_of[g] = gen;
+        w.arrived[g] = 0;
+        w.kind[g] = kind;
+        std::memset(w.present[g], 0, sizeof w.present[g]);
+    }
+    if (w.kind[g] != kind) fail("lanes of one wavefront are at different cross-lane operations (divergent control flow)");
+    if (n > (size_t)kPayload) fail("internal: payload too large");
+    std::memcpy(w.slot[g][f->lane], payload, n);
+    w.present[g][f->lane] = true;
+    w.arrived[g]++;
+    wait_until(&w.arrived[g], &w.live);
+    return View{&w, g};
+}
+
+bool in_lds(const void* p, size_t n) {
+    const unsigned char* q = static_cast<const unsigned char*>(p);
+    return q >= __start_simt_lds && q + n <= __stop_simt_lds;
+}
+
+template <typename T> float to_f32(T x) { return (float)x; }
+
+template <typename V> f32x16 mfma_impl(V a, V b, f32x16 c) {
+    struct Ops {
+        V a, b;
+    } mine{a, b};
+    const View v = exchange(K_MFMA, &mine, sizeof mine);
+    const Fiber* f = g_cur;
+    const int col = f->lane & 31, half = f->lane >> 5;
+    f32x16 d = c;
+    for (int r = 0; r < 16; ++r) {
+        const int row = 8 * (r / 4) + 4 * half + (r % 4);
+        double acc = 0.0;
+        for (int kh = 0; kh < 2; ++kh) {
+            Ops oa, ob;
+            std::memcpy(&oa, v.of(row + 32 * kh), sizeof oa);  // A[row][8*kh ..]
+            std::memcpy(&ob, v.of(col + 32 * kh), sizeof ob);  // B[8*kh ..][col]
+            for (int e = 0; e < 8; ++e) acc += (double)to_f32(oa.a[e]) * (double)to_f32(ob.b[e]);
+        }
+        d[r] = (float)((double)c[r] + acc);
+    }
+    return d;
+}
+
+}  // namespace
+
+// ---- what the shim header declares --------------------------------------------------------------
+hipError_t last_error() {
+    const hipError_t s = g_status;
+    g_status = hipSuccess;
+    return s;
+}
+
+int lane_id() { return g_cur ? g_cur->lane : 0; }
+
+void syncthreads() {
+    Fiber* f = g_cur;
+    Block& b = g_block;
+    const long gen = f->bar_gen++;
+    const int g = (int)(gen & 1);
+    if (b.bar_gen_of[g] != gen) {
+        b.bar_gen_of[g] = gen;
+        b.bar_arrived[g] = 0;
+    }
+    b.bar_arrived[g]++;
+    wait_until(&b.bar_arrived[g], &b.live);
+}
+
+f32x16 mfma_32x32x16_f16(f16x8 a, f16x8 b, f32x16 c) { return mfma_impl(a, b, c); }
+f32x16 mfma_32x32x16_bf16(bf16x8 a, bf16x8 b, f32x16 c) { return mfma_impl(a, b, c); }
+
+// ds_read_b64_tr_b16: the 16 lanes of a row each address four 16-bit elements; lane j of the row
+// receives element (j % 4) of the lanes 4*r + j/4, r = 0..3 (a 16x4 block handed out transposed).
+uint64_t ds_read_tr16_b64(const void* lds_ptr) {
+    uint64_t mine = 0;
+    if (!in_lds(lds_ptr, 8)) fail("transposing LDS read outside the workgroup's LDS");
+    if ((reinterpret_cast<uintptr_t>(lds_ptr) & 7) != 0) fail("transposing LDS read not 8-byte aligned");
+    std::memcpy(&mine, lds_ptr, 8);
+    const View v = exchange(K_TR, &mine, 8);
+    const int lane = g_cur->lane, row0 = lane & ~15, j = lane & 15;
+    uint16_t out[4];
+    for (int r = 0; r < 4; ++r) {
+        uint16_t src[4];
+        std::memcpy(src, v.of(row0 + 4 * r + j / 4), 8);
+        out[r] = src[j % 4];
+    }
+    uint64_t res;
+    std::memcpy(&res, out, 8);
+    return res;
+}
+
+// v_permlane32_swap a, b: the upper 32 lanes of a and the lower 32 lanes of b change places.
+u32x2 permlane32_swap(unsigned a, unsigned b) {
+    unsigned mine[2] = {a, b};
+    const View v = exchange(K_SWAP, mine, 8);
+    const int lane = g_cur->lane;
+    unsigned other[2];
+    std::memcpy(other, v.of(lane ^ 32), 8);
+    u32x2 r;
+    if (lane < 32) {
+        r[0] = a;
+        r[1] = other[0];  // a of lane + 32
+    } else {
+        r[0] = other[1];  // b of lane - 32
+        r[1] = b;
+    }
+    return r;
+}
+
+uint64_t ballot(bool pred) {
+    const unsigned char mine = pred ? 1 : 0;
+    const View v = exchange(K_BALLOT, &mine, 1);
+    uint64_t m = 0;
+    for (int l = 0; l < kWaveSize; ++l)
+        if (v.has(l) && *v.of(l)) m |= 1ull << l;
+    return m;
+}
+
+int readfirstlane(int x) {
+    const View v = exchange(K_RFL, &x, 4);
+    for (int l = 0; l < kWaveSize; ++l)
+        if (v.has(l)) {
+            int r;
+            std::memcpy(&r, v.of(l), 4);
+            return r;
+        }
+    return x;
+}
+
+int readlane(int x, int lane) {
+    if (lane < 0 || lane >= kWaveSize) fail("readlane: lane index out of range");
+    const View v = exchange(K_RL, &x, 4);
+    int r;
+    std::memcpy(&r, v.of(lane), 4);
+    return r;
+}
+
+int update_dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl) {
+    (void)old;
+    (void)bound_ctrl;
+    if (row_mask != 0xF || bank_mask != 0xF) fail("update_dpp: only full row and bank masks are modelled");
+    const View v = exchange(K_DPP, &src, 4);
+    const int lane = g_cur->lane;
+    int from;
+    if (ctrl >= 0 && ctrl <= 0xFF) from = (lane & ~3) | ((ctrl >> (2 * (lane & 3))) & 3);  // quad_perm
+    else if (ctrl == 0x140) from = (lane & ~15) | (15 - (lane & 15));                       // row_mirror
+    else if (ctrl == 0x141) from = (lane & ~7) | (7 - (lane & 7));                          // row_half_mirror
+    else {
+        fail("update_dpp: control value not modelled");
+        return 0;
+    }
+    int r;
+    std::memcpy(&r, v.of(from), 4);
+    return r;
+}
+
+int shfl_xor_bits(int x, int mask, int width) {
+    if (width != kWaveSize) fail("shuffle width other than 64 is not modelled");
+    const View v = exchange(K_SHFL, &x, 4);
+    const int from = g_cur->lane ^ mask;
+    if (from < 0 || from >= kWaveSize) return x;
+    int r;
+    std::memcpy(&r, v.of(from), 4);
+    return r;
+}
+
+// buffer_load_dwordx4 ... lds: lane i's 16 bytes go to lds_base + imm + 16*i; a source range that is
+// not completely inside the descriptor reads as zeros.
+void buffer_load_lds(BufferRsrc r, void* lds_base, int size, int voffset, int soffset, int imm, int aux) {
+    (void)aux;
+    if (size != 16) fail("buffer_load_lds: only 16-byte loads are modelled");
+    Fiber* f = g_cur;
+    unsigned char* dst = static_cast<unsigned char*>(lds_base) + imm + 16 * f->lane;
+    if (!in_lds(dst, 16)) fail("buffer_load_lds writes outside the workgroup's LDS");
+    const uint64_t off = (uint64_t)(uint32_t)voffset + (uint64_t)(uint32_t)soffset + (uint64_t)(uint32_t)imm;
+    if (voffset < 0) fail("buffer_load_lds: negative lane offset");
+    const bool inside = off + 16 <= (uint64_t)r.num_records;
+    PendingDma d{dst, inside ? r.base + off : nullptr};
+    if (g_dma_late) f->dma.push_back(d);
+    else {
+        f->dma.push_back(d);
+        flush_dma(f);
+    }
+}
+
+void waitcnt(int imm) {
+    if (imm != 0) fail("s_waitcnt: only the wait-for-everything form is modelled");
+    if (g_cur) flush_dma(g_cur);
+}
+
+void launch(dim3 grid, dim3 block, const std::function<void()>& body) {
+    if (g_status != hipSuccess) return;
+    std::lock_guard<std::mutex> guard(g_launch_mutex);
+    const int n = (int)(block.x * block.y * block.z);
+    if (n <= 0 || n > 1024) {
+        g_status = hipErrorLaunchFailure;
+        g_error = "launch: bad workgroup size";
+        return;
+    }
+    if (grid.x == 0 || grid.y == 0 || grid.z == 0) {
+        g_status = hipErrorLaunchFailure;
+        g_error = "launch: empty grid";
+        return;
+    }
+    while ((int)g_stacks.size() < n) g_stacks.push_back(static_cast<unsigned char*>(std::malloc(kStackBytes)));
+    const int n_waves = (n + kWaveSize - 1) / kWaveSize;
+    gridDim = grid;
+    blockDim = block;
+    g_body = &body;
+    std::vector<int> order(n_waves);
+    for (unsigned bz = 0; bz < grid.z && g_status == hipSuccess; ++bz)
+        for (unsigned by = 0; by < grid.y && g_status == hipSuccess; ++by)
+            for (unsigned bx = 0; bx < grid.x && g_status == hipSuccess; ++bx) {
+                blockIdx = dim3(bx, by, bz);
+                std::memset(__start_simt_lds, 0xFF, (size_t)(__stop_simt_lds - __start_simt_lds));
+                Block& b = g_block;
+                b.fibers.assign(n, Fiber());
+                b.waves.assign(n_waves, Wave());
+                b.live = n;
+                b.bar_arrived[0] = b.bar_arrived[1] = 0;
+                b.bar_gen_of[0] = b.bar_gen_of[1] = -1;
+                for (int i = 0; i < n; ++i) {
+                    Fiber& f = b.fibers[i];
+                    f.stack = g_stacks[i];
+                    f.tid = dim3(i % block.x, (i / block.x) % block.y, i / (block.x * block.y));
+                    f.wave = i / kWaveSize;
+                    f.lane = i % kWaveSize;
+                    b.waves[f.wave].live++;
+                    getcontext(&f.ctx);
+                    f.ctx.uc_stack.ss_sp = f.stack;
+                    f.ctx.uc_stack.ss_size = kStackBytes;
+                    f.ctx.uc_link = nullptr;
+                    makecontext(&f.ctx, trampoline, 0);
+                }
+                while (b.live > 0 && g_status == hipSuccess) {
+                    for (int w = 0; w < n_waves; ++w) order[w] = w;
+                    for (int w = n_waves - 1; w > 0; --w) std::swap(order[w], order[next_rand() % (uint64_t)(w + 1)]);
+                    bool progressed = false;
+                    for (int wi = 0; wi < n_waves && g_status == hipSuccess; ++wi) {
+                        const int w = order[wi];
+                        const int lo = w * kWaveSize, hi = std::min(n, lo + kWaveSize);
+                        for (int i = lo; i < hi && g_status == hipSuccess; ++i) {
+                            Fiber& f = b.fibers[i];
+                            if (f.done) continue;
+                            if (f.wait_counter && *f.wait_counter < *f.wait_target) continue;
+                            progressed = true;
+                            enter_fiber(&f);
+                        }
+                    }
+                    if (!progressed && b.live > 0 && g_status == hipSuccess) {
+                        int at_barrier = 0, at_cross = 0;
+                        for (const Fiber& f : b.fibers)
+                            if (!f.done) {
+                                if (f.wait_target == &b.live) ++at_barrier;
+                                else ++at_cross;
+                            }
+                        char msg[200];
+                        std::snprintf(msg, sizeof msg,
+                                      "workgroup (%u,%u,%u) cannot make progress: %d work-items wait at a barrier, %d at a "
+                                      "cross-lane operation",
+                                      bx, by, bz, at_barrier, at_cross);
+                        g_error = msg;
+                        std::fprintf(stderr, "simt: %s\n", msg);
+                        g_status = hipErrorLaunchFailure;
+                    }
+                }
+            }
+    g_body = nullptr;
+}
+
+}  // namespace simt
+
+// ---- control from the tests (ctypes) ---------------------------------------------------------------
+extern "C" {
+// dma_late != 0: direct-to-LDS loads land at the issuing lane's next s_waitcnt instead of at issue.
+// seed: order in which the wavefronts of a workgroup are advanced.
+void simt_configure(int dma_late, uint64_t seed) {
+    simt::g_dma_late = dma_late != 0;
+    simt::g_rng = seed * 0x9E3779B97F4A7C15ull + 0x2545F4914F6CDD1Dull;
+    if (simt::g_rng == 0) simt::g_rng = 1;
+}
+const char* simt_last_error_text() { return simt::g_error.c_str(); }
+void simt_clear_error() {
+    simt::g_error.clear();
+    simt::g_status = hipSuccess;
+}
+long simt_switch_count() { return simt::g_switches; }
+}

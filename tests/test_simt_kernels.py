@@ -1,0 +1,284 @@
+"""The library's kernels, compiled as host C++ and executed lane by lane on the CPU (tests/simt), against
+the CPU oracle: same entry points, same bars as the GPU parity tests, at sizes that run in seconds.
+
+What this covers that the GPU tests cannot show: every buffer sits directly against an inaccessible page,
+so an access past either end of a tensor faults here instead of on a GPU; cross-lane operations in
+divergent control flow, barriers some wavefronts skip, direct-to-LDS loads that are consumed before the
+wait that covers them, and LDS that is read before it is written all fail the run.  What it cannot show:
+timing, and instruction-level behaviour of the real compiler's code."""
+import os
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from simt import simt as S
+
+TOL = {O.F32: 1e-4, O.F16: 2e-2, O.BF16: 2e-2}
+
+
+@pytest.fixture(scope="module")
+def emu():
+    S.load()
+    S.configure(False, 1)
+    return S.EmulatedHip()
+
+
+def qkv(shape, seed, dtype, sigma=1.0):
+    return tuple(O.round_to(O.fill_normal(shape, seed, t, sigma), dtype) for t in (1, 2, 3))
+
+
+def dev(x, dtype, front=False):
+    return S.guarded(S.to_storage(x, dtype), front)
+
+
+def flash(emu, q, k, v, dtype, B, N, H, d, scale, causal, H_kv=None, mask=None, front=False):
+    H_kv = H_kv or H
+    dq, dk, dv = dev(q, dtype, front), dev(k, dtype, front), dev(v, dtype, front)
+    do = S.guarded(S.empty_storage((B, N, H, d), dtype), front)
+    dm = None if mask is None else S.guarded(mask, front)
+    emu.flash_fwd_gqa(S.ptr(dq), S.ptr(dk), S.ptr(dv), S.ptr(do), dtype, B, N, H, H_kv, d, (N * H * d, H * d, d),
+                      (N * H_kv * d, H_kv * d, d), scale, causal, None, None if dm is None else S.ptr(dm))
+    return S.from_storage(do, dtype)
+
+
+# ---- FlashAttention forward -----------------------------------------------------------------------------
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("N,d", [(16, 64), (129, 64), (40, 80), (1, 32)])
+def test_fp32_kernel(emu, N, d, causal):
+    B, H = 2, 3
+    q, k, v = qkv((B, N, H, d), 11, O.F32)
+    scale = 1.0 / np.sqrt(d)
+    got = flash(emu, q, k, v, O.F32, B, N, H, d, scale, causal)
+    assert np.abs(got - O.attention(q, k, v, B, N, H, d, scale, causal)).max() <= 1e-4
+
+
+def test_fp32_kernel_dense_mask(emu):
+    B, N, H, d = 2, 37, 2, 64
+    q, k, v = qkv((B, N, H, d), 12, O.F32)
+    mask = (O.fill_uniform((B, N, N), 12, 6) > 0.3).astype(np.float32)
+    mask[0, 5, :] = 0.0  # a row that sees nothing: output 0
+    got = flash(emu, q, k, v, O.F32, B, N, H, d, 0.125, False, mask=mask)
+    want = O.attention(q, k, v, B, N, H, d, 0.125, False, mask=mask)
+    assert np.all(got[0, 5] == 0.0)
+    assert np.abs(got - want).max() <= 1e-4
+
+
+@pytest.mark.parametrize("dma_late", [False, True])
+@pytest.mark.parametrize("dtype", [O.BF16, O.F16])
+@pytest.mark.parametrize("N,d,causal", [(64, 128, False), (129, 128, True), (300, 64, True), (200, 64, False), (1, 128, True)])
+def test_matrix_core_kernel(emu, dtype, N, d, causal, dma_late):
+    B, H = 2, 2
+    q, k, v = qkv((B, N, H, d), 13, dtype)
+    scale = 1.0 / np.sqrt(d)
+    S.configure(dma_late, seed=N + d)
+    try:
+        got = flash(emu, q, k, v, dtype, B, N, H, d, scale, causal, front=dma_late)
+    finally:
+        S.configure(False, 1)
+    assert np.isfinite(got).all()
+    assert np.abs(got - O.attention(q, k, v, B, N, H, d, scale, causal)).max() <= TOL[dtype]
+
+
+@pytest.mark.parametrize("H,H_kv,dtype,d", [(4, 2, O.BF16, 128), (4, 1, O.F16, 64), (6, 3, O.F32, 32)])
+def test_grouped_heads_equal_repeated_heads(emu, H, H_kv, dtype, d):
+    B, N = 1, 150
+    q = O.round_to(O.fill_normal((B, N, H, d), 14, 1), dtype)
+    k = O.round_to(O.fill_normal((B, N, H_kv, d), 14, 2), dtype)
+    v = O.round_to(O.fill_normal((B, N, H_kv, d), 14, 3), dtype)
+    got = flash(emu, q, k, v, dtype, B, N, H, d, 0.1, True, H_kv=H_kv)
+    g = H // H_kv
+    want = O.attention(q, np.repeat(k, g, axis=2), np.repeat(v, g, axis=2), B, N, H, d, 0.1, True)
+    assert np.abs(got - want).max() <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype,d", [(O.F16, 64), (O.BF16, 128), (O.F32, 64)])
+def test_ragged_batch(emu, dtype, d):
+    H = 2
+    lens = np.array([1, 130, 64, 257], np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    q, k, v = qkv((T, H, d), 15, dtype)
+    dq, dk, dv = dev(q, dtype), dev(k, dtype), dev(v, dtype)
+    do = S.guarded(S.empty_storage((T, H, d), dtype))
+    dcu = S.guarded(cu)
+    scale = 1.0 / np.sqrt(d)
+    emu.flash_fwd_varlen(S.ptr(dq), S.ptr(dk), S.ptr(dv), S.ptr(do), dtype, S.ptr(dcu), len(lens), int(lens.max()), H, d,
+                         H * d, d, scale, True)
+    want = O.attention_varlen(q, k, v, cu, H, d, scale, True)
+    assert np.abs(S.from_storage(do, dtype) - want).max() <= TOL[dtype]
+
+
+def test_head_major_strides(emu):
+    # the same tensors laid out [B,H,N,d]: only the strides change
+    B, N, H, d = 1, 140, 3, 128
+    q, k, v = qkv((B, N, H, d), 16, O.BF16)
+    t = lambda x: np.ascontiguousarray(x.transpose(0, 2, 1, 3))
+    dq, dk, dv = dev(t(q), O.BF16), dev(t(k), O.BF16), dev(t(v), O.BF16)
+    do = S.guarded(S.empty_storage((B, H, N, d), O.BF16))
+    emu.flash_fwd(S.ptr(dq), S.ptr(dk), S.ptr(dv), S.ptr(do), O.BF16, B, N, H, d, (H * N * d, d, N * d), 0.09, True)
+    got = S.from_storage(do, O.BF16).transpose(0, 2, 1, 3)
+    assert np.abs(got - O.attention(q, k, v, B, N, H, d, 0.09, True)).max() <= 2e-2
+
+
+@pytest.mark.parametrize("together,slots", [(2, 0), (4, 1), (3, 2), (64, 0)])
+def test_interleaved_workgroup_map_computes_the_same(emu, together, slots, monkeypatch):
+    B, N, H, d = 1, 520, 5, 64   # 5 query tiles per head, 5 heads: partial groups and partial rounds
+    q, k, v = qkv((B, N, H, d), 17, O.F16)
+    plain = flash(emu, q, k, v, O.F16, B, N, H, d, 0.125, True)
+    monkeypatch.setenv("AHPC_FLASH_HEADS_TOGETHER", str(together))
+    if slots:
+        monkeypatch.setenv("AHPC_FLASH_ROUND_SLOTS", str(slots))
+    mixed = flash(emu, q, k, v, O.F16, B, N, H, d, 0.125, True)
+    assert np.array_equal(plain, mixed)
+    assert np.abs(plain - O.attention(q, k, v, B, N, H, d, 0.125, True)).max() <= 2e-2
+
+
+# ---- paged KV pool and decode -----------------------------------------------------------------------------
+from test_gpu_paged import build_problem, _tables_for  # problem builders only (pure numpy + oracle)
+
+
+def decode(emu, q, kp, vp, table, lens, rows, B, H, H_kv, d, P, dtype, qo_dtype, scale, chunk=0):
+    dq = dev(q, qo_dtype)
+    do = S.guarded(S.empty_storage((B, H, d), qo_dtype))
+    dk, dv = dev(kp, dtype), dev(vp, dtype)
+    dt, dl = S.guarded(table), S.guarded(np.asarray(lens, np.int32))
+    dr = None if rows is None else S.guarded(np.asarray(rows, np.int32))
+    max_len = int(max(1, np.max(lens)))
+    ws_bytes = emu.paged_decode_workspace_bytes(B, H, d, max_len, P, chunk)
+    ws = S.guarded(np.full(max(ws_bytes, 4) // 4, np.nan, np.float32))
+    emu.paged_decode_gqa(S.ptr(dq), S.ptr(do), qo_dtype, S.ptr(dk), S.ptr(dv), dtype, S.ptr(dt), S.ptr(dl),
+                         None if dr is None else S.ptr(dr), B, H, H_kv, d, P, table.shape[1], max_len, scale, chunk,
+                         S.ptr(ws), ws_bytes)
+    return S.from_storage(do, qo_dtype)
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.F16, O.BF16])
+@pytest.mark.parametrize("H,d,P", [(4, 32, 16), (8, 128, 16), (6, 64, 4), (3, 128, 16), (2, 256, 8)])
+def test_decode(emu, dtype, H, d, P):
+    B = 4
+    q, kp, vp, table, lens, _, _ = build_problem(B, H, d, P, [33, 1, 16, 150], 21, dtype)
+    scale = 1.0 / np.sqrt(d)
+    want = O.paged_decode(q, kp, vp, table, lens, None, B, H, d, P, scale)
+    for chunk in (0, P, 4 * P):
+        got = decode(emu, q, kp, vp, table, lens, None, B, H, H, d, P, dtype, dtype, scale, chunk)
+        assert np.isfinite(got).all()
+        assert np.abs(got - want).max() <= TOL[dtype], f"chunk={chunk}"
+
+
+@pytest.mark.parametrize("G", [2, 4, 8])
+def test_decode_grouped_heads(emu, G):
+    B, H_kv, d, P = 3, 2, 128, 16
+    H = G * H_kv
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [70, 5, 129], 22, O.F16)
+    q = O.round_to(O.fill_normal((B, H, d), 22, 1), O.F16)
+    scale = 1.0 / np.sqrt(d)
+    # the ordinary oracle on a pool whose heads are repeated G times
+    rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
+    want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    for chunk in (0, 32):
+        got = decode(emu, q, kp, vp, table, lens, None, B, H, H_kv, d, P, O.F16, O.F16, scale, chunk)
+        assert np.abs(got - want).max() <= 2e-2
+
+
+def test_decode_empty_sequence_and_batch_rows(emu):
+    B, H, d, P = 4, 4, 64, 16
+    q, kp, vp, table, lens, _, _ = build_problem(B, H, d, P, [40, 7, 90, 16], 41, O.BF16)
+    lens = lens.copy()
+    lens[1] = 0
+    rows = np.array([2, 1, 0, 3], np.int32)
+    want = O.paged_decode(q, kp, vp, table, lens, rows, B, H, d, P, 0.125)
+    got = decode(emu, q, kp, vp, table, lens, rows, B, H, H, d, P, O.BF16, O.BF16, 0.125, 32)
+    assert np.all(got[1] == 0.0)
+    assert np.abs(got - want).max() <= 2e-2
+
+
+def test_gather_indices_bit_exact(emu):
+    B, H, d, P = 6, 32, 128, 16
+    lens = O.fill_lengths(B, 51, 4, 1, 300)
+    _, _, _, table, lens, _, _ = build_problem(B, 1, 1, P, lens, 51, O.F32)
+    max_len = int(lens.max())
+    rows = np.array([5, 0, 3, 1, 2, 4], np.int32)
+    out = S.guarded(np.full((B, max_len), -7, np.int64))
+    dt, dl, dr = S.guarded(table), S.guarded(lens), S.guarded(rows)
+    emu.paged_gather_indices(S.ptr(dt), S.ptr(dl), S.ptr(dr), B, H, d, P, table.shape[1], max_len, S.ptr(out))
+    assert np.array_equal(out, O.gather_offsets(table, lens, rows, B, max_len, P, H, d))
+
+
+@pytest.mark.parametrize("in_dtype,pool_dtype", [(O.F32, O.F32), (O.F32, O.F16), (O.F16, O.F16), (O.BF16, O.BF16)])
+def test_scatter_then_gather_roundtrip(emu, in_dtype, pool_dtype):
+    H, d, P, n_pages = 4, 32, 16, 12
+    table = np.array([[7, 2, 9, 0, -1], [3, 11, 5, -1, -1]], np.int32)
+    store = O.F16 if O.F16 in (in_dtype, pool_dtype) else (O.BF16 if O.BF16 in (in_dtype, pool_dtype) else O.F32)
+    k1, v1 = (O.round_to(O.fill_normal((21, H, d), 1, t), store) for t in (2, 3))
+    k2, v2 = (O.round_to(O.fill_normal((30, H, d), 2, t), store) for t in (2, 3))
+    dt = S.guarded(table)
+    kpool = S.guarded(S.to_storage(np.zeros(n_pages * P * H * d, np.float32), pool_dtype))
+    vpool = S.guarded(S.to_storage(np.zeros(n_pages * P * H * d, np.float32), pool_dtype))
+    a, b, c, e = dev(k1, in_dtype), dev(v1, in_dtype), dev(k2, in_dtype), dev(v2, in_dtype)
+    emu.kv_scatter(S.ptr(a), S.ptr(b), in_dtype, S.ptr(kpool), S.ptr(vpool), pool_dtype, S.ptr(dt), 5, 21, H, d, P, row0=0, pos0=0)
+    emu.kv_scatter(S.ptr(c), S.ptr(e), in_dtype, S.ptr(kpool), S.ptr(vpool), pool_dtype, S.ptr(dt), 5, 30, H, d, P, row0=0, pos0=21)
+    trow, tpos = S.guarded(np.full(21, 1, np.int32)), S.guarded(np.arange(21, dtype=np.int32)[::-1].copy())
+    emu.kv_scatter(S.ptr(a), S.ptr(b), in_dtype, S.ptr(kpool), S.ptr(vpool), pool_dtype, S.ptr(dt), 5, 21, H, d, P,
+                   token_row=S.ptr(trow), token_pos=S.ptr(tpos))
+    ko, vo = S.guarded(np.empty(51 * H * d, np.float32)), S.guarded(np.empty(51 * H * d, np.float32))
+    emu.kv_gather(S.ptr(ko), S.ptr(vo), O.F32, S.ptr(kpool), S.ptr(vpool), pool_dtype, S.ptr(dt), 5, 0, 0, 51, H, d, P)
+    assert np.array_equal(ko.reshape(51, H, d), np.concatenate([k1, k2]))
+    assert np.array_equal(vo.reshape(51, H, d), np.concatenate([v1, v2]))
+    kp, vp = np.zeros(n_pages * P * H * d, np.float32), np.zeros(n_pages * P * H * d, np.float32)
+    O.kv_scatter(k1, v1, kp, vp, table, 0, 0, P, H, d)
+    O.kv_scatter(k2, v2, kp, vp, table, 0, 21, P, H, d)
+    O.kv_scatter(np.ascontiguousarray(k1[::-1]), np.ascontiguousarray(v1[::-1]), kp, vp, table, 1, 0, P, H, d)
+    assert np.array_equal(S.from_storage(kpool, pool_dtype), kp) and np.array_equal(S.from_storage(vpool, pool_dtype), vp)
+
+
+@pytest.mark.parametrize("in_dtype,pool_dtype", [(O.F16, O.F16), (O.F32, O.F16), (O.BF16, O.F32)])
+def test_scatter_batch_dense(emu, in_dtype, pool_dtype):
+    B, N, H, d, P = 4, 70, 3, 64, 16
+    start = np.array([0, 5, 16, 33], np.int32)
+    n_new = np.array([70, 1, 0, 37], np.int32)
+    rows = np.array([2, 0, 3, 1], np.int32)
+    lens_total = np.zeros(4, np.int32)
+    lens_total[rows] = start + n_new
+    table, n_pages = _tables_for(lens_total, P, 61)
+    k, v = (O.round_to(O.fill_normal((B, N, H, d), 61, t), in_dtype) for t in (2, 3))
+    kp, vp = np.zeros(n_pages * P * H * d, np.float32), np.zeros(n_pages * P * H * d, np.float32)
+    for b in range(B):
+        if n_new[b]:
+            O.kv_scatter(O.round_to(k[b, :n_new[b]], pool_dtype), O.round_to(v[b, :n_new[b]], pool_dtype), kp, vp, table,
+                         int(rows[b]), int(start[b]), P, H, d)
+    dk, dv = dev(k, in_dtype), dev(v, in_dtype)
+    dkp, dvp = dev(np.zeros_like(kp), pool_dtype), dev(np.zeros_like(vp), pool_dtype)
+    dtab, drows, dstart, dnew = S.guarded(table), S.guarded(rows), S.guarded(start), S.guarded(n_new)
+    emu.kv_scatter_batch(S.ptr(dk), S.ptr(dv), in_dtype, N * H * d, H * d, S.ptr(dkp), S.ptr(dvp), pool_dtype, S.ptr(dtab),
+                         table.shape[1], S.ptr(drows), B, N, H, d, P, seq_start=S.ptr(dstart), seq_tokens=S.ptr(dnew))
+    assert np.array_equal(S.from_storage(dkp, pool_dtype), kp) and np.array_equal(S.from_storage(dvp, pool_dtype), vp)
+
+
+def test_scatter_batch_packed(emu):
+    H, d, P = 2, 128, 16
+    lens = np.array([130, 16, 1, 55], np.int32)
+    B = len(lens)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    table, n_pages = _tables_for(lens, P, 62)
+    k, v = (O.round_to(O.fill_normal((T, H, d), 62, t), O.F16) for t in (2, 3))
+    kp, vp = np.zeros(n_pages * P * H * d, np.float32), np.zeros(n_pages * P * H * d, np.float32)
+    for b in range(B):
+        O.kv_scatter(k[cu[b]:cu[b + 1]], v[cu[b]:cu[b + 1]], kp, vp, table, b, 0, P, H, d)
+    dk, dv = dev(k, O.F16), dev(v, O.F16)
+    dkp, dvp = dev(np.zeros_like(kp), O.F16), dev(np.zeros_like(vp), O.F16)
+    dtab, drows, dcu = S.guarded(table), S.guarded(np.arange(B, dtype=np.int32)), S.guarded(cu)
+    emu.kv_scatter_batch(S.ptr(dk), S.ptr(dv), O.F16, 0, H * d, S.ptr(dkp), S.ptr(dvp), O.F16, S.ptr(dtab), table.shape[1],
+                         S.ptr(drows), B, int(lens.max()), H, d, P, cu_seqlens=S.ptr(dcu))
+    assert np.array_equal(S.from_storage(dkp, O.F16), kp) and np.array_equal(S.from_storage(dvp, O.F16), vp)
+
+
+def test_paired_query_tiles(emu):
+    """Causal launches with at least 1024 query tiles hand each workgroup a late tile and then an early one."""
+    B, N, H, d = 1, 256, 512, 64
+    _, _, second = emu.flash_block_map(B, N, H, True)
+    assert (second >= 0).any()
+    q, k, v = qkv((B, N, H, d), 18, O.F16)
+    got = flash(emu, q, k, v, O.F16, B, N, H, d, 0.125, True)
+    assert np.abs(got - O.attention(q, k, v, B, N, H, d, 0.125, True)).max() <= 2e-2
