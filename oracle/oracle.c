@@ -7,6 +7,12 @@
  *        shape B=2,N=16,H=4,d=64 and others; closed forms: V constant => O constant,
  *        Q = 0 => mean of V (prefix mean when causal), N = 1 => O = V, one dominant logit =>
  *        that V row, key-permutation invariance, fully masked row => 0; committed fixtures.
+ *   ahpc_oracle_attention_backward          central differences of an independent float64 forward (numpy)
+ *        in sampled entries of q, k and v; torch autograd in float64 on whole tensors; closed forms:
+ *        N = 1 => dV = dO and dQ = dK = 0; V with equal rows => dQ = dK = 0; K with equal rows =>
+ *        dQ = 0 and dV_j = mean_i dO_i; sum_j dV_j = sum_i dO_i; sum_i q_i.dQ_i = sum_j k_j.dK_j;
+ *        grouped heads = repeated heads with the group's dK, dV summed.  The reference has no
+ *        backward to compare with (placeholder): parity unpinned by the reference.
  *   ahpc_oracle_softmax_merge / _row_split  equals direct softmax for any split count;
  *        commutative/associative up to rounding.
  *   ahpc_oracle_kv_offset / gather_offsets  brute-force enumeration on a tiny pool.
@@ -211,6 +217,85 @@ void ahpc_oracle_attention_rows(const float* q, const float* k, const float* v, 
             dense_row(q, k, v, out + i * d, b, h, n, N, d, sb, sn, sh, scale, causal, NULL, scores, acc);
         }
         free(scores);
+    }
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* backward: the derivative of the function above.  The reference's backward is a placeholder
+ * (src/algorithms/flash_attention.cpp:496-580 sums products that ignore the attention weights, and its
+ * test only asks for non-zero gradients, tests/test_flash_attention.cpp:447-479), so there is nothing to
+ * follow line by line: this differentiates compute_reference_attention (tests/test_flash_attention.cpp:30-97)
+ *   P = softmax(scale * Q K^T + mask),  O = P V
+ *   dV = P^T dO,  dP = dO V^T,  dS = P o (dP - rowsum(P o dP)),  dQ = scale * dS K,  dK = scale * dS^T Q
+ * in double precision, rounding once at the end.  q, d_out, d_q are [B,N,H,d]; k, v, d_k, d_v are
+ * [B,N,H_kv,d] and query head h uses key/value head h / (H / H_kv), whose gradient sums over its group. */
+void ahpc_oracle_attention_backward(const float* q, const float* k, const float* v, const float* d_out,
+                                    float* d_q, float* d_k, float* d_v,
+                                    int64_t B, int64_t N, int64_t H, int64_t H_kv, int64_t d,
+                                    float scale, int causal, const float* mask, int n_threads) {
+    const int64_t G = H / H_kv;
+    const int64_t sq = H * d, skv = H_kv * d;
+    if (n_threads < 1) n_threads = 1;
+#pragma omp parallel num_threads(n_threads)
+    {
+        double* p = (double*)malloc(sizeof(double) * (size_t)(2 * N + d + 2 * N * d));
+        double* dp = p + N;
+        double* dq_row = dp + N;
+        double* dk_acc = dq_row + d;
+        double* dv_acc = dk_acc + N * d;
+#pragma omp for schedule(dynamic, 1)
+        for (int64_t bh = 0; bh < B * H_kv; ++bh) {
+            const int64_t b = bh / H_kv, hk = bh % H_kv;
+            const float* kb = k + b * N * skv + hk * d;
+            const float* vb = v + b * N * skv + hk * d;
+            for (int64_t x = 0; x < 2 * N * d; ++x) dk_acc[x] = 0.0;
+            for (int64_t g = 0; g < G; ++g) {
+                const int64_t h = hk * G + g;
+                for (int64_t i = 0; i < N; ++i) {
+                    const float* qi = q + (b * N + i) * sq + h * d;
+                    const float* doi = d_out + (b * N + i) * sq + h * d;
+                    float* dqi = d_q + (b * N + i) * sq + h * d;
+                    const float* keep = mask ? mask + (b * N + i) * N : NULL;
+                    const int64_t n_keys = causal ? i + 1 : N;
+                    double top = -INFINITY;
+                    for (int64_t j = 0; j < n_keys; ++j) {
+                        if (keep && keep[j] == 0.0f) { p[j] = -INFINITY; continue; }
+                        double s = 0.0;
+                        for (int64_t e = 0; e < d; ++e) s += (double)qi[e] * (double)kb[j * skv + e];
+                        p[j] = s * (double)scale;
+                        if (p[j] > top) top = p[j];
+                    }
+                    for (int64_t e = 0; e < d; ++e) dq_row[e] = 0.0;
+                    if (top != -INFINITY) {
+                        double total = 0.0, delta = 0.0;
+                        for (int64_t j = 0; j < n_keys; ++j) { p[j] = exp(p[j] - top); total += p[j]; }
+                        for (int64_t j = 0; j < n_keys; ++j) {
+                            p[j] /= total;
+                            double t = 0.0;
+                            for (int64_t e = 0; e < d; ++e) t += (double)doi[e] * (double)vb[j * skv + e];
+                            dp[j] = t;
+                            delta += p[j] * t;
+                        }
+                        for (int64_t j = 0; j < n_keys; ++j) {
+                            if (p[j] == 0.0) continue;
+                            const double ds = p[j] * (dp[j] - delta) * (double)scale;
+                            for (int64_t e = 0; e < d; ++e) {
+                                dq_row[e] += ds * (double)kb[j * skv + e];
+                                dk_acc[j * d + e] += ds * (double)qi[e];
+                                dv_acc[j * d + e] += p[j] * (double)doi[e];
+                            }
+                        }
+                    }
+                    for (int64_t e = 0; e < d; ++e) dqi[e] = (float)dq_row[e];
+                }
+            }
+            for (int64_t j = 0; j < N; ++j)
+                for (int64_t e = 0; e < d; ++e) {
+                    d_k[(b * N + j) * skv + hk * d + e] = (float)dk_acc[j * d + e];
+                    d_v[(b * N + j) * skv + hk * d + e] = (float)dv_acc[j * d + e];
+                }
+        }
+        free(p);
     }
 }
 

@@ -90,6 +90,14 @@ void ahpc_oracle_attention_varlen_rows(const float* q, const float* k, const flo
                                        float scale, int causal,
                                        const int64_t* rows, int64_t n_rows, int n_threads);
 
+/* Gradients of ahpc_oracle_attention with respect to q, k and v for a given d_out, in double precision
+ * (the reference's own backward, src/algorithms/flash_attention.cpp:496-580, is a placeholder).
+ * q, d_out, d_q: contiguous [B,N,H,d]; k, v, d_k, d_v: contiguous [B,N,H_kv,d], H_kv divides H. */
+void ahpc_oracle_attention_backward(const float* q, const float* k, const float* v, const float* d_out,
+                                    float* d_q, float* d_k, float* d_v,
+                                    int64_t B, int64_t N, int64_t H, int64_t H_kv, int64_t d,
+                                    float scale, int causal, const float* mask, int n_threads);
+
 /* ---- online-softmax merge --------------------------------------------------------- */
 /* (m, l) <- merge((m, l), (m2, l2)): restates OnlineSoftmaxState::update,
  * src/algorithms/flash_attention.hpp:50-57. */

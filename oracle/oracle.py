@@ -44,6 +44,7 @@ def _load():
         "ahpc_oracle_attention_rows": (None, [fp, fp, fp, fp, i64, i64, i64, i64, i64, i64, i64, f32, ci, lp, i64, ci]),
         "ahpc_oracle_attention_varlen": (None, [fp, fp, fp, fp, ip, i64, i64, i64, f32, ci, ci]),
         "ahpc_oracle_attention_varlen_rows": (None, [fp, fp, fp, fp, ip, i64, i64, i64, f32, ci, lp, i64, ci]),
+        "ahpc_oracle_attention_backward": (None, [fp, fp, fp, fp, fp, fp, fp, i64, i64, i64, i64, i64, f32, ci, fp, ci]),
         "ahpc_oracle_softmax_merge": (None, [fp, fp, f32, f32]),
         "ahpc_oracle_attention_row_split": (None, [fp, fp, fp, fp, i64, i64, i64, f32, ci]),
         "ahpc_oracle_kv_offset": (i64, [ip, i64, i64, i64, i64, i64, i64, i64]),
@@ -154,6 +155,19 @@ def attention(q, k, v, B, N, H, d, scale, causal=False, mask=None, layout="BNHD"
     lib.ahpc_oracle_attention(_f(q), _f(k), _f(v), _f(out), B, N, H, d, sb, sn, sh, scale, int(causal), m,
                               threads or cpu_threads())
     return out.reshape((B, N, H, d) if layout == "BNHD" else (B, H, N, d))
+
+
+def attention_backward(q, k, v, d_out, B, N, H, d, scale, causal=False, H_kv=None, mask=None, threads=None):
+    """Gradients (d_q [B,N,H,d], d_k and d_v [B,N,H_kv,d]) of attention() for the given d_out."""
+    H_kv = H_kv or H
+    q, k, v, d_out = (np.ascontiguousarray(a, np.float32).reshape(-1) for a in (q, k, v, d_out))
+    dq = np.zeros(B * N * H * d, np.float32)
+    dk = np.zeros(B * N * H_kv * d, np.float32)
+    dv = np.zeros(B * N * H_kv * d, np.float32)
+    m = None if mask is None else _f(np.ascontiguousarray(mask, np.float32).reshape(-1))
+    lib.ahpc_oracle_attention_backward(_f(q), _f(k), _f(v), _f(d_out), _f(dq), _f(dk), _f(dv), B, N, H, H_kv, d, scale,
+                                       int(causal), m, threads or cpu_threads())
+    return dq.reshape(B, N, H, d), dk.reshape(B, N, H_kv, d), dv.reshape(B, N, H_kv, d)
 
 
 def attention_rows(q, k, v, B, N, H, d, scale, rows, causal=False, layout="BNHD", threads=None):
