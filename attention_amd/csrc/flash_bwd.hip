@@ -1,0 +1,405 @@
+// FlashAttention backward entry points: argument checks, kernel choice, launches.
+//
+// The interface hands over Q, K, V and dO only (no forward output, no softmax statistics), so a backward
+// is three launches:
+//   1. statistics  per query row i: lse_i = log sum_j exp(scale q_i.k_j) and delta_i = dO_i . O_i
+//                  (a forward pass that keeps its output in registers),
+//   2. dQ          a workgroup owns query rows and walks the keys:  dS_ij = P_ij (dO_i.v_j - delta_i),
+//                  dQ_i = scale * sum_j dS_ij k_j,
+//   3. dK, dV      a workgroup owns key rows and walks the queries: dV_j = sum_i P_ij dO_i,
+//                  dK_j = scale * sum_i dS_ij q_i  (summed over the query heads of a K/V head).
+// with P_ij = exp(scale q_i.k_j - lse_i).  Nothing is accumulated through atomics, so results do not depend
+// on launch order.  The statistics live in the caller's workspace: two floats per (sequence, head, row).
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdlib>
+
+#include "ahpc_device.hpp"
+#include "flash_bwd_mfma.hpp"
+
+namespace ahpc {
+
+struct BwdParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* d_out;
+    void* d_q;
+    void* d_k;
+    void* d_v;
+    const float* mask;          // [B,N,N] or null
+    float* lse;                 // [B*H][rows_padded]
+    float* delta;               // [B*H][rows_padded]
+    int64_t rows_padded;
+    int64_t stride_b, stride_n, stride_h;           // Q, dO, dQ
+    int64_t kv_stride_b, kv_stride_n, kv_stride_h;  // K, V, dK, dV
+    int32_t N, H, d;
+    int32_t kv_group;           // query heads per key/value head
+    float scale;
+    int32_t causal;
+};
+
+// ---------------------------------------------------------------------------------------------
+// fp32-FMA kernels: any dtype, head dimension up to 256, optional dense mask.  One thread owns one row
+// (query row in the first two kernels, key row in the third) and keeps it in registers; the rows it walks
+// over are staged in LDS as fp32, 16 at a time, by the 128 threads of the workgroup.  This is the accuracy
+// path (fp32 tensors, 1e-4 tolerance) and the fallback for what the matrix-core kernels do not take.
+constexpr int kBwdRows = 128;
+constexpr int kBwdTile = 16;
+
+// Stages rows [r0, r0+16) of a [rows][d] tensor (row stride `stride`) into dst[16][DP] as fp32; rows at or
+// beyond `n_rows` and columns at or beyond d become zero.
+template <typename T, int DP>
+__device__ inline void stage_rows(float (*dst)[DP], const T* src, int64_t stride, int r0, int n_rows, int d, int tid) {
+    for (int i = tid; i < kBwdTile * DP; i += kBwdRows) {
+        const int r = i / DP, e = i - r * DP;
+        const int row = r0 + r;
+        dst[r][e] = (row < n_rows && e < d) ? Storage<T>::load(src + (int64_t)row * stride + e) : 0.0f;
+    }
+}
+
+template <typename T, int DP>
+__global__ __launch_bounds__(kBwdRows) void flash_bwd_stats_simple_kernel(const BwdParams p) {
+    __shared__ float sk[kBwdTile][DP];
+    __shared__ float sv[kBwdTile][DP];
+    const int tid = threadIdx.x;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int hk = h / p.kv_group;
+    const int L = p.N, d = p.d;
+    const int row0 = blockIdx.x * kBwdRows;
+    if (row0 >= L) return;
+    const int n = row0 + tid;
+    const bool active = n < L;
+    const int64_t base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+    const int64_t kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
+    const T* gq = static_cast<const T*>(p.q) + base;
+    const T* gdo = static_cast<const T*>(p.d_out) + base;
+    const T* gk = static_cast<const T*>(p.k) + kv_base;
+    const T* gv = static_cast<const T*>(p.v) + kv_base;
+
+    float qv[DP], acc[DP];
+#pragma unroll
+    for (int e = 0; e < DP; ++e) {
+        qv[e] = (active && e < d) ? Storage<T>::load(gq + (int64_t)n * p.stride_n + e) : 0.0f;
+        acc[e] = 0.0f;
+    }
+    float m = -INFINITY, l = 0.0f;
+    int k_end = L;
+    if (p.causal) k_end = (row0 + kBwdRows) < L ? (row0 + kBwdRows) : L;
+    const float* mrow = (p.mask && active) ? p.mask + ((int64_t)b * p.N + n) * p.N : nullptr;
+
+    for (int k0 = 0; k0 < k_end; k0 += kBwdTile) {
+        __syncthreads();
+        stage_rows<T, DP>(sk, gk, p.kv_stride_n, k0, L, d, tid);
+        stage_rows<T, DP>(sv, gv, p.kv_stride_n, k0, L, d, tid);
+        __syncthreads();
+        if (!active) continue;
+        for (int kr = 0; kr < kBwdTile; ++kr) {
+            const int key = k0 + kr;
+            if (key >= L) break;
+            if (p.causal && key > n) break;
+            if (mrow && mrow[key] == 0.0f) continue;
+            float dot = 0.0f;
+#pragma unroll
+            for (int e = 0; e < DP; ++e) dot = __builtin_fmaf(qv[e], sk[kr][e], dot);
+            const float s = dot * p.scale;
+            if (s > m) {
+                const float a = __expf(m - s);  // first key: exp(-inf) = 0
+                l = l * a + 1.0f;
+#pragma unroll
+                for (int e = 0; e < DP; ++e) acc[e] = __builtin_fmaf(acc[e], a, sv[kr][e]);
+                m = s;
+            } else {
+                const float w = __expf(s - m);
+                l += w;
+#pragma unroll
+                for (int e = 0; e < DP; ++e) acc[e] = __builtin_fmaf(w, sv[kr][e], acc[e]);
+            }
+        }
+    }
+    if (!active) return;
+    // a row that sees no key: every weight is exp(s - inf) = 0 later on, and nothing flows through it
+    float lse = INFINITY, delta = 0.0f;
+    if (l > 0.0f) {
+        lse = m + logf(l);
+        float dot = 0.0f;
+#pragma unroll
+        for (int e = 0; e < DP; ++e)
+            if (e < d) dot = __builtin_fmaf(acc[e], Storage<T>::load(gdo + (int64_t)n * p.stride_n + e), dot);
+        delta = dot / l;
+    }
+    const int64_t row = ((int64_t)b * p.H + h) * p.rows_padded + n;
+    p.lse[row] = lse;
+    p.delta[row] = delta;
+}
+
+template <typename T, int DP>
+__global__ __launch_bounds__(kBwdRows) void flash_bwd_dq_simple_kernel(const BwdParams p) {
+    __shared__ float sk[kBwdTile][DP];
+    __shared__ float sv[kBwdTile][DP];
+    const int tid = threadIdx.x;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int hk = h / p.kv_group;
+    const int L = p.N, d = p.d;
+    const int row0 = blockIdx.x * kBwdRows;
+    if (row0 >= L) return;
+    const int n = row0 + tid;
+    const bool active = n < L;
+    const int64_t base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+    const int64_t kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
+    const T* gq = static_cast<const T*>(p.q) + base;
+    const T* gdo = static_cast<const T*>(p.d_out) + base;
+    const T* gk = static_cast<const T*>(p.k) + kv_base;
+    const T* gv = static_cast<const T*>(p.v) + kv_base;
+
+    float qv[DP], dov[DP], dq[DP];
+#pragma unroll
+    for (int e = 0; e < DP; ++e) {
+        const bool in = active && e < d;
+        qv[e] = in ? Storage<T>::load(gq + (int64_t)n * p.stride_n + e) : 0.0f;
+        dov[e] = in ? Storage<T>::load(gdo + (int64_t)n * p.stride_n + e) : 0.0f;
+        dq[e] = 0.0f;
+    }
+    const int64_t row = ((int64_t)b * p.H + h) * p.rows_padded + (active ? n : 0);
+    const float lse = p.lse[row], delta = p.delta[row];
+    int k_end = L;
+    if (p.causal) k_end = (row0 + kBwdRows) < L ? (row0 + kBwdRows) : L;
+    const float* mrow = (p.mask && active) ? p.mask + ((int64_t)b * p.N + n) * p.N : nullptr;
+
+    for (int k0 = 0; k0 < k_end; k0 += kBwdTile) {
+        __syncthreads();
+        stage_rows<T, DP>(sk, gk, p.kv_stride_n, k0, L, d, tid);
+        stage_rows<T, DP>(sv, gv, p.kv_stride_n, k0, L, d, tid);
+        __syncthreads();
+        if (!active) continue;
+        for (int kr = 0; kr < kBwdTile; ++kr) {
+            const int key = k0 + kr;
+            if (key >= L) break;
+            if (p.causal && key > n) break;
+            if (mrow && mrow[key] == 0.0f) continue;
+            float dot = 0.0f, dp = 0.0f;
+#pragma unroll
+            for (int e = 0; e < DP; ++e) {
+                dot = __builtin_fmaf(qv[e], sk[kr][e], dot);
+                dp = __builtin_fmaf(dov[e], sv[kr][e], dp);
+            }
+            const float ds = __expf(dot * p.scale - lse) * (dp - delta);
+#pragma unroll
+            for (int e = 0; e < DP; ++e) dq[e] = __builtin_fmaf(ds, sk[kr][e], dq[e]);
+        }
+    }
+    if (!active) return;
+    T* out = static_cast<T*>(p.d_q) + base + (int64_t)n * p.stride_n;
+#pragma unroll
+    for (int e = 0; e < DP; ++e)
+        if (e < d) Storage<T>::store(out + e, dq[e] * p.scale);
+}
+
+// grid.y = key/value heads: the query heads of a group are walked one after the other
+template <typename T, int DP>
+__global__ __launch_bounds__(kBwdRows) void flash_bwd_dkv_simple_kernel(const BwdParams p) {
+    __shared__ float sq[kBwdTile][DP];
+    __shared__ float sdo[kBwdTile][DP];
+    __shared__ float s_lse[kBwdTile];
+    __shared__ float s_delta[kBwdTile];
+    const int tid = threadIdx.x;
+    const int hk = blockIdx.y, b = blockIdx.z;
+    const int L = p.N, d = p.d;
+    const int row0 = blockIdx.x * kBwdRows;
+    if (row0 >= L) return;
+    const int j = row0 + tid;
+    const bool active = j < L;
+    const int64_t kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
+    const T* gk = static_cast<const T*>(p.k) + kv_base;
+    const T* gv = static_cast<const T*>(p.v) + kv_base;
+
+    float kv[DP], vv[DP], dk[DP], dv[DP];
+#pragma unroll
+    for (int e = 0; e < DP; ++e) {
+        const bool in = active && e < d;
+        kv[e] = in ? Storage<T>::load(gk + (int64_t)j * p.kv_stride_n + e) : 0.0f;
+        vv[e] = in ? Storage<T>::load(gv + (int64_t)j * p.kv_stride_n + e) : 0.0f;
+        dk[e] = 0.0f;
+        dv[e] = 0.0f;
+    }
+    // under a causal mask only queries at or after the first key of this workgroup contribute
+    const int i_begin = p.causal ? (row0 / kBwdTile) * kBwdTile : 0;
+
+    for (int g = 0; g < p.kv_group; ++g) {
+        const int h = hk * p.kv_group + g;
+        const int64_t base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+        const T* gq = static_cast<const T*>(p.q) + base;
+        const T* gdo = static_cast<const T*>(p.d_out) + base;
+        const int64_t stat0 = ((int64_t)b * p.H + h) * p.rows_padded;
+        for (int i0 = i_begin; i0 < L; i0 += kBwdTile) {
+            __syncthreads();
+            stage_rows<T, DP>(sq, gq, p.stride_n, i0, L, d, tid);
+            stage_rows<T, DP>(sdo, gdo, p.stride_n, i0, L, d, tid);
+            if (tid < kBwdTile) {
+                const int i = i0 + tid;
+                s_lse[tid] = i < L ? p.lse[stat0 + i] : INFINITY;
+                s_delta[tid] = i < L ? p.delta[stat0 + i] : 0.0f;
+            }
+            __syncthreads();
+            if (!active) continue;
+            for (int r = 0; r < kBwdTile; ++r) {
+                const int i = i0 + r;
+                if (i >= L) break;
+                if (p.causal && i < j) continue;
+                if (p.mask && p.mask[((int64_t)b * p.N + i) * p.N + j] == 0.0f) continue;
+                float dot = 0.0f, dp = 0.0f;
+#pragma unroll
+                for (int e = 0; e < DP; ++e) {
+                    dot = __builtin_fmaf(sq[r][e], kv[e], dot);
+                    dp = __builtin_fmaf(sdo[r][e], vv[e], dp);
+                }
+                const float pw = __expf(dot * p.scale - s_lse[r]);
+                const float ds = pw * (dp - s_delta[r]);
+#pragma unroll
+                for (int e = 0; e < DP; ++e) {
+                    dv[e] = __builtin_fmaf(pw, sdo[r][e], dv[e]);
+                    dk[e] = __builtin_fmaf(ds, sq[r][e], dk[e]);
+                }
+            }
+        }
+    }
+    if (!active) return;
+    T* out_k = static_cast<T*>(p.d_k) + kv_base + (int64_t)j * p.kv_stride_n;
+    T* out_v = static_cast<T*>(p.d_v) + kv_base + (int64_t)j * p.kv_stride_n;
+#pragma unroll
+    for (int e = 0; e < DP; ++e)
+        if (e < d) {
+            Storage<T>::store(out_k + e, dk[e] * p.scale);
+            Storage<T>::store(out_v + e, dv[e]);
+        }
+}
+
+template <typename T, int DP>
+static int launch_simple_dp(const BwdParams& p, int64_t B, int64_t H_kv, hipStream_t stream) {
+    const unsigned tiles = (unsigned)((p.N + kBwdRows - 1) / kBwdRows);
+    dim3 block(kBwdRows);
+    hipLaunchKernelGGL((flash_bwd_stats_simple_kernel<T, DP>), dim3(tiles, (unsigned)p.H, (unsigned)B), block, 0, stream, p);
+    hipLaunchKernelGGL((flash_bwd_dq_simple_kernel<T, DP>), dim3(tiles, (unsigned)p.H, (unsigned)B), block, 0, stream, p);
+    hipLaunchKernelGGL((flash_bwd_dkv_simple_kernel<T, DP>), dim3(tiles, (unsigned)H_kv, (unsigned)B), block, 0, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
+template <typename T>
+static int launch_simple(const BwdParams& p, int64_t B, int64_t H_kv, hipStream_t stream) {
+    if (p.d <= 32) return launch_simple_dp<T, 32>(p, B, H_kv, stream);
+    if (p.d <= 64) return launch_simple_dp<T, 64>(p, B, H_kv, stream);
+    if (p.d <= 128) return launch_simple_dp<T, 128>(p, B, H_kv, stream);
+    if (p.d <= 256) return launch_simple_dp<T, 256>(p, B, H_kv, stream);
+    return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+}
+
+// ---------------------------------------------------------------------------------------------
+static bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+static int64_t padded_rows(int64_t N) { return (N + kFlashRows - 1) / kFlashRows * kFlashRows; }
+
+template <typename T, int D>
+static int launch_mfma_d(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool causal, float* lse2, float* delta,
+                         hipStream_t stream) {
+    // 1. statistics: the forward kernel with its output kept in registers
+    FlashParams f{};
+    f.q = p.q; f.k = p.k; f.v = p.v; f.o = nullptr;
+    f.stride_b = p.stride_b; f.stride_n = p.stride_n; f.stride_h = p.stride_h;
+    f.kv_stride_b = p.kv_stride_b; f.kv_stride_n = p.kv_stride_n; f.kv_stride_h = p.kv_stride_h;
+    f.N = p.N; f.H = p.H; f.kv_group = p.kv_group;
+    f.scale_log2 = p.scale_log2;
+    if (int rc = flash_plan_launch(f, B, causal)) return rc;
+    const FlashStatsOut st{p.d_out, lse2, delta, p.rows_padded};
+    const dim3 block(kFlashThreads);
+    const dim3 grid_stats((unsigned)(f.blocks_per_xcd * 8));
+    const unsigned tiles = (unsigned)((p.N + kFlashRows - 1) / kFlashRows);
+    const dim3 grid_q(tiles, (unsigned)p.H, (unsigned)B), grid_kv(tiles, (unsigned)H_kv, (unsigned)B);
+    if (causal) {
+        hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, true>), grid_stats, block, 0, stream, f, st);
+        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, true>), grid_q, block, 0, stream, p);
+        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, true>), grid_kv, block, 0, stream, p);
+    } else {
+        hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, false>), grid_stats, block, 0, stream, f, st);
+        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, false>), grid_q, block, 0, stream, p);
+        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, false>), grid_kv, block, 0, stream, p);
+    }
+    return static_cast<int>(hipGetLastError());
+}
+
+template <typename T>
+static int launch_mfma(const FlashBwdParams& p, int64_t B, int64_t H_kv, int d, bool causal, float* lse2, float* delta,
+                       hipStream_t stream) {
+    if (d == 128) return launch_mfma_d<T, 128>(p, B, H_kv, causal, lse2, delta, stream);
+    if (d == 64) return launch_mfma_d<T, 64>(p, B, H_kv, causal, lse2, delta, stream);
+    return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+}
+
+}  // namespace ahpc
+
+using namespace ahpc;
+
+extern "C" {
+
+size_t ahpc_hip_flash_bwd_workspace_bytes(int64_t B, int64_t N, int64_t H) {
+    if (B <= 0 || N <= 0 || H <= 0) return 0;
+    // two floats per (sequence, head, row), rows padded to whole query tiles of the matrix-core kernels
+    return (size_t)B * (size_t)H * (size_t)padded_rows(N) * 2 * sizeof(float);
+}
+
+int ahpc_hip_flash_bwd(const void* d_out, const void* q, const void* k, const void* v, void* d_q, void* d_k, void* d_v,
+                       int dtype, int64_t B, int64_t N, int64_t H, int64_t H_kv, int64_t d, int64_t stride_b, int64_t stride_n,
+                       int64_t stride_h, int64_t kv_stride_b, int64_t kv_stride_n, int64_t kv_stride_h, float scale, int causal,
+                       const float* mask, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!d_out || !q || !k || !v || !d_q || !d_k || !d_v) return AHPC_ERR_NULL_POINTER;
+    if (dtype < AHPC_F32 || dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
+    if (B <= 0 || N <= 0 || H <= 0 || d <= 0 || H_kv <= 0) return AHPC_ERR_BAD_SHAPE;
+    if (H % H_kv) return AHPC_ERR_BAD_SHAPE;
+    if (B > 65535 || H > 65535 || N > 0x7FFFFF00ll) return AHPC_ERR_BAD_SHAPE;
+    if (d > 256) return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+    if (stride_n < d || stride_h < d || stride_b < 0 || kv_stride_n < d || kv_stride_h < d || kv_stride_b < 0)
+        return AHPC_ERR_BAD_SHAPE;
+    if (!workspace) return AHPC_ERR_NULL_POINTER;
+    if (workspace_bytes < ahpc_hip_flash_bwd_workspace_bytes(B, N, H)) return AHPC_ERR_WORKSPACE_TOO_SMALL;
+    if (!aligned16(workspace)) return AHPC_ERR_BAD_ALIGNMENT;
+    if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+
+    BwdParams p{};
+    p.q = q; p.k = k; p.v = v; p.d_out = d_out;
+    p.d_q = d_q; p.d_k = d_k; p.d_v = d_v;
+    p.mask = mask;
+    p.lse = static_cast<float*>(workspace);
+    p.rows_padded = padded_rows(N);
+    p.delta = p.lse + (size_t)B * (size_t)H * (size_t)p.rows_padded;
+    p.stride_b = stride_b; p.stride_n = stride_n; p.stride_h = stride_h;
+    p.kv_stride_b = kv_stride_b; p.kv_stride_n = kv_stride_n; p.kv_stride_h = kv_stride_h;
+    p.N = (int32_t)N; p.H = (int32_t)H; p.d = (int32_t)d;
+    p.kv_group = (int32_t)(H / H_kv);
+    p.scale = scale;
+    p.causal = causal ? 1 : 0;
+    // fp16 / bf16 with d in {64, 128}, 16-byte aligned rows and no dense mask: the matrix-core kernels
+    const bool strides_ok = !(stride_b % 8) && !(stride_n % 8) && !(stride_h % 8) && !(kv_stride_b % 8) && !(kv_stride_n % 8) &&
+                            !(kv_stride_h % 8) && stride_n < (int64_t(1) << 24) && kv_stride_n < (int64_t(1) << 24);
+    if (!mask && (dtype == AHPC_F16 || dtype == AHPC_BF16) && (d == 64 || d == 128) && strides_ok && aligned16(q) &&
+        aligned16(k) && aligned16(v) && aligned16(d_out) && aligned16(d_q) && aligned16(d_k) && aligned16(d_v)) {
+        FlashBwdParams m{};
+        m.q = q; m.k = k; m.v = v; m.d_out = d_out;
+        m.d_q = d_q; m.d_k = d_k; m.d_v = d_v;
+        m.lse2 = p.lse; m.delta = p.delta; m.rows_padded = p.rows_padded;
+        m.stride_b = stride_b; m.stride_n = stride_n; m.stride_h = stride_h;
+        m.kv_stride_b = kv_stride_b; m.kv_stride_n = kv_stride_n; m.kv_stride_h = kv_stride_h;
+        m.N = (int32_t)N; m.H = (int32_t)H; m.kv_group = p.kv_group;
+        m.scale = scale;
+        m.scale_log2 = scale * kLog2e;
+        return dtype == AHPC_F16 ? launch_mfma<f16_t>(m, B, H_kv, (int)d, causal != 0, p.lse, p.delta, st)
+                                 : launch_mfma<bf16_t>(m, B, H_kv, (int)d, causal != 0, p.lse, p.delta, st);
+    }
+    switch (dtype) {
+        case AHPC_F32: return launch_simple<float>(p, B, H_kv, st);
+        case AHPC_F16: return launch_simple<f16_t>(p, B, H_kv, st);
+        default: return launch_simple<bf16_t>(p, B, H_kv, st);
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,405 @@
+// FlashAttention backward on the gfx950 matrix cores (fp16 / bf16 storage, fp32 accumulate), dense batches.
+//
+// Input: Q, K, V, dO and the per-row statistics of the forward (lse2 = log2 sum_j exp2(c q.k_j) with
+// c = scale*log2(e), delta = dO.O; written by flash_bwd_stats_mfma_kernel).  With P = exp2(c q.k - lse2):
+//
+//   flash_bwd_dq_mfma_kernel    a workgroup owns 128 query rows (32 per wavefront) and walks the keys in
+//       tiles of 64, exactly like the forward:  S^T = K Q^T and dP^T = V dO^T  (A = rows of the K / V tile
+//       in LDS, B = Q / dO held in registers; the products start from accumulators holding -lse2 and
+//       -delta, so they deliver c q.k - lse2 and dO.v - delta directly),  dS^T = exp2(S^T) o dP^T,
+//       dQ^T += K^T dS^T  (A = K^T by transposing LDS reads, B = dS^T straight from the registers it was
+//       computed in, as P^T in the forward).  dQ = scale * dQ^T^T.
+//
+//   flash_bwd_dkv_mfma_kernel   the mirror image: a workgroup owns 128 key rows (32 per wavefront, held in
+//       registers as B operands) and walks the queries in tiles of 64:  S = Q K^T, dP = dO V^T  (A = rows
+//       of the Q / dO tile in LDS, accumulators start from the tile's -lse2 / -delta per row),
+//       P = exp2(S), dS = P o dP,  dV^T += dO^T P,  dK^T += Q^T dS  (A = dO^T / Q^T by transposing LDS reads,
+//       B = P / dS from registers).  With grouped heads the query heads of the group are walked one after
+//       the other into the same accumulators.  dK = scale * dK^T^T, dV = dV^T^T.
+//
+// In both kernels a lane owns one row of the output (a query, a key) and the masks are per-lane
+// comparisons.  Tiles are streamed with direct-to-LDS loads and double buffered as in the forward; every
+// tile is read by rows (first two products) and by transposing reads (last products), with the row-read
+// swizzle.  No atomics: every output element is written once.
+#pragma once
+
+#include "flash_fwd_mfma.hpp"
+
+namespace ahpc {
+
+struct FlashBwdParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* d_out;
+    void* d_q;
+    void* d_k;
+    void* d_v;
+    const float* lse2;          // [B*H][rows_padded]
+    const float* delta;
+    int64_t rows_padded;
+    int64_t stride_b, stride_n, stride_h;           // Q, dO, dQ
+    int64_t kv_stride_b, kv_stride_n, kv_stride_h;  // K, V, dK, dV
+    int32_t N;
+    int32_t H;                  // query heads
+    int32_t kv_group;           // query heads per key/value head
+    float scale;
+    float scale_log2;           // scale * log2(e)
+};
+
+// Byte offset inside a row-swizzled tile of the 8 bytes a lane hands to a transposing read that fetches
+// the 4 tile rows 16*g + 8*a + 4*(lane/32) + 0..3 for column quad (32*mb + 16*((lane/16)%2) + 4*(lane%4)):
+// the part that does not depend on g.  Adding 16*g rows keeps the swizzle (it has period 16 rows).
+template <int D>
+__device__ inline int tr_offset_rowswizzled(int lane, int mb, int a) {
+    typedef FlashTile<D> TL;
+    const int vi = lane & 15;
+    const int row = 8 * a + 4 * (lane >> 5) + (vi >> 2);
+    const int cch = 4 * mb + 2 * ((lane >> 4) & 1) + ((vi & 3) >> 1);
+    return row * TL::kRowBytes + ((cch ^ TL::fk(row)) << 4) + 8 * (vi & 1);
+}
+
+// Packs 8 fp32 of a 32x32 accumulator block (rows r0..r0+7 of the lane's column) as one B operand.
+template <typename T>
+__device__ inline u32x4 pack_operand(const f32x16& x, int r0) {
+    return u32x4{pack2<T>(x[r0 + 0], x[r0 + 1]), pack2<T>(x[r0 + 2], x[r0 + 3]), pack2<T>(x[r0 + 4], x[r0 + 5]),
+                 pack2<T>(x[r0 + 6], x[r0 + 7])};
+}
+
+// Loads the row `row` of a [rows][D] tensor as B operands (8 consecutive elements per k-step), scaled by c.
+template <typename T, int KS>
+__device__ inline void load_row_operands(u32x4 (&reg)[KS], const T* row_ptr, int half, float c) {
+    const T* src = row_ptr + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(src + 16 * ks);
+        u32x4 sc;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) sc[w] = pack2<T>(lo_f32<T>(raw[w]) * c, hi_f32<T>(raw[w]) * c);
+        reg[ks] = sc;
+    }
+}
+
+// Stores the transposed accumulators of one output row (a lane holds 4 runs of 4 consecutive elements per
+// 32-element block), scaled by f.
+template <typename T, int MB>
+__device__ inline void store_row(T* dst_row, const f32x16 (&acc)[MB], int half, float f) {
+    T* dst = dst_row + 4 * half;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            const f32x16& a = acc[mb];
+            const u32x2 w = u32x2{pack2<T>(a[4 * g4 + 0] * f, a[4 * g4 + 1] * f), pack2<T>(a[4 * g4 + 2] * f, a[4 * g4 + 3] * f)};
+            *reinterpret_cast<u32x2*>(dst + 32 * mb + 8 * g4) = w;
+        }
+}
+
+// grid: (query tiles of 128, query heads, sequences)
+template <typename T, int D, bool CAUSAL>
+__global__ __launch_bounds__(kFlashThreads) void flash_bwd_dq_mfma_kernel(const FlashBwdParams p) {
+    typedef FlashTile<D> TL;
+    constexpr int KS = D / 16;
+    constexpr int MB = D / 32;
+    constexpr int RB = TL::kRowBytes;
+
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[TL::kBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[TL::kBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_k1[TL::kBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[TL::kBytes];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int col = lane & 31;
+    const int half = lane >> 5;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int hk = h / p.kv_group;
+    const int L = p.N;
+    // long tiles first: under a causal mask the late query tiles walk the most keys
+    const int q_tile0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * kFlashRows;
+    if (q_tile0 >= L) return;
+
+    const int64_t base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+    const int64_t kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
+    const T* const gq = static_cast<const T*>(p.q) + base;
+    const T* const gdo = static_cast<const T*>(p.d_out) + base;
+    const T* const gk = static_cast<const T*>(p.k) + kv_base;
+    const T* const gv = static_cast<const T*>(p.v) + kv_base;
+    const int64_t sn = p.stride_n;
+    const int64_t skv = p.kv_stride_n;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+
+    int dma_off[TL::kInstrPerWave];
+#pragma unroll
+    for (int i = 0; i < TL::kInstrPerWave; ++i) {
+        const int r = (wave * TL::kInstrPerWave + i) * TL::kRowsPerInstr + lane / TL::kChunks;
+        const int pc = lane % TL::kChunks;
+        dma_off[i] = (int)(r * skv * 2) + ((pc ^ TL::fk(r)) << 4);
+    }
+    auto dma_both = [&](int k0, unsigned char* dst_k, unsigned char* dst_v) {
+        const int64_t rem = (int64_t)(L - k0 - 1) * skv * 2 + 2 * D;
+        const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
+        dma_tile<D>(gk + (int64_t)k0 * skv, nrec, dma_off, dst_k, wave_u);
+        dma_tile<D>(gv + (int64_t)k0 * skv, nrec, dma_off, dst_v, wave_u);
+    };
+
+    int row_off[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * RB + (((2 * ks + half) ^ TL::fk(col)) << 4);
+    int tr_off[MB][2];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int a = 0; a < 2; ++a) tr_off[mb][a] = tr_offset_rowswizzled<D>(lane, mb, a);
+
+    int k_end = L;
+    if (CAUSAL) k_end = (q_tile0 + kFlashRows) < L ? (q_tile0 + kFlashRows) : L;
+    const int n_tiles = (k_end + kFlashKeys - 1) / kFlashKeys;
+    dma_both(0, lds_k0, lds_v0);
+
+    const int qw = q_tile0 + wave * 32;
+    const int qrow = qw + col;
+    const int row = qrow < L ? qrow : L - 1;
+    u32x4 qreg[KS], doreg[KS];
+    load_row_operands<T, KS>(qreg, gq + (int64_t)row * sn, half, p.scale_log2);
+    load_row_operands<T, KS>(doreg, gdo + (int64_t)row * sn, half, 1.0f);
+    const int64_t stat = ((int64_t)b * p.H + h) * p.rows_padded + qrow;  // qrow < rows_padded always
+    f32x16 neg_lse, neg_delta;
+    {
+        const float a = -p.lse2[stat], d0 = -p.delta[stat];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            neg_lse[r] = a;
+            neg_delta[r] = d0;
+        }
+    }
+    f32x16 acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[mb][r] = 0.0f;
+
+    auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int k0) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            const int kblock0 = k0 + 32 * kb;
+            if (kblock0 >= L) continue;                        // nothing but padding
+            if (CAUSAL && kblock0 > qw + 31) continue;        // every key of the block is in the future
+            f32x16 s = neg_lse, dp = neg_delta;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const u32x4 ak = *reinterpret_cast<const u32x4*>(tile_k + 32 * kb * RB + row_off[ks]);
+                const u32x4 av = *reinterpret_cast<const u32x4*>(tile_v + 32 * kb * RB + row_off[ks]);
+                s = mfma_32x32x16<T>(ak, qreg[ks], s);
+                dp = mfma_32x32x16<T>(av, doreg[ks], dp);
+            }
+            // key = kblock0 + 4*half + 8*(r/4) + r%4 is visible iff key <= min(qrow, L-1)
+            int lim = L - 1;
+            if (CAUSAL) lim = qrow < lim ? qrow : lim;
+            lim -= kblock0 + 4 * half;
+            f32x16 ds;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int off = 8 * (r >> 2) + (r & 3);
+                ds[r] = off <= lim ? fast_exp2(s[r]) * dp[r] : 0.0f;
+            }
+#pragma unroll
+            for (int g2 = 0; g2 < 2; ++g2) {
+                const u32x4 bop = pack_operand<T>(ds, 8 * g2);
+                const int rows = (32 * kb + 16 * g2) * RB;
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    const u32x2 lo = TrRead<T>::load(tile_k + rows + tr_off[mb][0]);
+                    const u32x2 hi = TrRead<T>::load(tile_k + rows + tr_off[mb][1]);
+                    acc[mb] = mfma_32x32x16<T>(u32x4{lo[0], lo[1], hi[0], hi[1]}, bop, acc[mb]);
+                }
+            }
+        }
+    };
+
+    auto step = [&](unsigned char* cur_k, unsigned char* cur_v, unsigned char* nxt_k, unsigned char* nxt_v, int t) {
+        const int k0 = t * kFlashKeys;
+        const bool more = t + 1 < n_tiles;
+        if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
+        compute_tile(cur_k, cur_v, k0);
+        if (more) {
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+        }
+    };
+
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    for (int t = 0; t < n_tiles; t += 2) {
+        step(lds_k0, lds_v0, lds_k1, lds_v1, t);
+        if (t + 1 < n_tiles) step(lds_k1, lds_v1, lds_k0, lds_v0, t + 1);
+    }
+    if (qrow < L) store_row<T, MB>(static_cast<T*>(p.d_q) + base + (int64_t)qrow * sn, acc, half, p.scale);
+}
+
+// grid: (key tiles of 128, key/value heads, sequences)
+template <typename T, int D, bool CAUSAL>
+__global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const FlashBwdParams p) {
+    typedef FlashTile<D> TL;
+    constexpr int KS = D / 16;
+    constexpr int MB = D / 32;
+    constexpr int RB = TL::kRowBytes;
+
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_q0[TL::kBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_o0[TL::kBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_q1[TL::kBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_o1[TL::kBytes];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int col = lane & 31;
+    const int half = lane >> 5;
+    const int hk = blockIdx.y, b = blockIdx.z;
+    const int L = p.N;
+    // under a causal mask the early key tiles see the most queries: they go first
+    const int k_tile0 = (int)blockIdx.x * kFlashRows;
+    if (k_tile0 >= L) return;
+
+    const int64_t kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
+    const T* const gk = static_cast<const T*>(p.k) + kv_base;
+    const T* const gv = static_cast<const T*>(p.v) + kv_base;
+    const int64_t sn = p.stride_n;
+    const int64_t skv = p.kv_stride_n;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+
+    int dma_off[TL::kInstrPerWave];
+#pragma unroll
+    for (int i = 0; i < TL::kInstrPerWave; ++i) {
+        const int r = (wave * TL::kInstrPerWave + i) * TL::kRowsPerInstr + lane / TL::kChunks;
+        const int pc = lane % TL::kChunks;
+        dma_off[i] = (int)(r * sn * 2) + ((pc ^ TL::fk(r)) << 4);
+    }
+    int row_off[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * RB + (((2 * ks + half) ^ TL::fk(col)) << 4);
+    int tr_off[MB][2];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int a = 0; a < 2; ++a) tr_off[mb][a] = tr_offset_rowswizzled<D>(lane, mb, a);
+
+    const int kw = k_tile0 + wave * 32;  // first key of this wavefront
+    const int key = kw + col;
+    const int krow = key < L ? key : L - 1;
+    u32x4 kreg[KS], vreg[KS];
+    load_row_operands<T, KS>(kreg, gk + (int64_t)krow * skv, half, p.scale_log2);
+    load_row_operands<T, KS>(vreg, gv + (int64_t)krow * skv, half, 1.0f);
+
+    f32x16 acc_k[MB], acc_v[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            acc_k[mb][r] = 0.0f;
+            acc_v[mb][r] = 0.0f;
+        }
+
+    // queries before the first key of the workgroup see none of its keys under a causal mask
+    const int t_begin = CAUSAL ? k_tile0 / kFlashKeys : 0;
+    const int n_tiles = (L + kFlashKeys - 1) / kFlashKeys;
+
+    for (int g = 0; g < p.kv_group; ++g) {
+        const int h = hk * p.kv_group + g;
+        const int64_t base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+        const T* const gq = static_cast<const T*>(p.q) + base;
+        const T* const gdo = static_cast<const T*>(p.d_out) + base;
+        const float* const lse2 = p.lse2 + ((int64_t)b * p.H + h) * p.rows_padded;
+        const float* const delta = p.delta + ((int64_t)b * p.H + h) * p.rows_padded;
+
+        auto dma_both = [&](int i0, unsigned char* dst_q, unsigned char* dst_o) {
+            const int64_t rem = (int64_t)(L - i0 - 1) * sn * 2 + 2 * D;
+            const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
+            dma_tile<D>(gq + (int64_t)i0 * sn, nrec, dma_off, dst_q, wave_u);
+            dma_tile<D>(gdo + (int64_t)i0 * sn, nrec, dma_off, dst_o, wave_u);
+        };
+
+        auto compute_tile = [&](const unsigned char* tile_q, const unsigned char* tile_o, int i0) {
+#pragma unroll
+            for (int ib = 0; ib < 2; ++ib) {
+                const int iblock0 = i0 + 32 * ib;
+                if (iblock0 >= L) continue;                      // nothing but padding
+                if (CAUSAL && iblock0 + 31 < kw) continue;      // every query of the block precedes the keys
+                // the block's rows of statistics: this lane's 16 rows are 4 runs of 4 consecutive rows
+                f32x16 s, dp;
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const f32x4 a = *reinterpret_cast<const f32x4*>(lse2 + iblock0 + 8 * g4 + 4 * half);
+                    const f32x4 d0 = *reinterpret_cast<const f32x4*>(delta + iblock0 + 8 * g4 + 4 * half);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        s[4 * g4 + x] = -a[x];
+                        dp[4 * g4 + x] = -d0[x];
+                    }
+                }
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const u32x4 aq = *reinterpret_cast<const u32x4*>(tile_q + 32 * ib * RB + row_off[ks]);
+                    const u32x4 ao = *reinterpret_cast<const u32x4*>(tile_o + 32 * ib * RB + row_off[ks]);
+                    s = mfma_32x32x16<T>(aq, kreg[ks], s);
+                    dp = mfma_32x32x16<T>(ao, vreg[ks], dp);
+                }
+                // query = iblock0 + 4*half + 8*(r/4) + r%4 contributes iff it exists, the key exists, and
+                // (causal) query >= key
+                int first = 0;
+                if (CAUSAL) first = key - (iblock0 + 4 * half);
+                const int last = (key < L ? L : 0) - (iblock0 + 4 * half);  // off < last
+                f32x16 pw, ds;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int off = 8 * (r >> 2) + (r & 3);
+                    const bool on = off >= first && off < last;
+                    pw[r] = on ? fast_exp2(s[r]) : 0.0f;
+                    ds[r] = on ? pw[r] * dp[r] : 0.0f;
+                }
+#pragma unroll
+                for (int g2 = 0; g2 < 2; ++g2) {
+                    const u32x4 bp = pack_operand<T>(pw, 8 * g2);
+                    const u32x4 bs = pack_operand<T>(ds, 8 * g2);
+                    const int rows = (32 * ib + 16 * g2) * RB;
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) {
+                        const u32x2 olo = TrRead<T>::load(tile_o + rows + tr_off[mb][0]);
+                        const u32x2 ohi = TrRead<T>::load(tile_o + rows + tr_off[mb][1]);
+                        acc_v[mb] = mfma_32x32x16<T>(u32x4{olo[0], olo[1], ohi[0], ohi[1]}, bp, acc_v[mb]);
+                        const u32x2 qlo = TrRead<T>::load(tile_q + rows + tr_off[mb][0]);
+                        const u32x2 qhi = TrRead<T>::load(tile_q + rows + tr_off[mb][1]);
+                        acc_k[mb] = mfma_32x32x16<T>(u32x4{qlo[0], qlo[1], qhi[0], qhi[1]}, bs, acc_k[mb]);
+                    }
+                }
+            }
+        };
+
+        auto step = [&](unsigned char* cur_q, unsigned char* cur_o, unsigned char* nxt_q, unsigned char* nxt_o, int t) {
+            const int i0 = t * kFlashKeys;
+            const bool more = t + 1 < n_tiles;
+            if (more) dma_both(i0 + kFlashKeys, nxt_q, nxt_o);
+            compute_tile(cur_q, cur_o, i0);
+            if (more) {
+                __builtin_amdgcn_s_waitcnt(0);
+                __syncthreads();
+            }
+        };
+
+        dma_both(t_begin * kFlashKeys, lds_q0, lds_o0);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        for (int t = t_begin; t < n_tiles; t += 2) {
+            step(lds_q0, lds_o0, lds_q1, lds_o1, t);
+            if (t + 1 < n_tiles) step(lds_q1, lds_o1, lds_q0, lds_o0, t + 1);
+        }
+        __syncthreads();  // the next head's first load reuses the buffers
+    }
+    if (key < L) {
+        store_row<T, MB>(static_cast<T*>(p.d_k) + kv_base + (int64_t)key * skv, acc_k, half, p.scale);
+        store_row<T, MB>(static_cast<T*>(p.d_v) + kv_base + (int64_t)key * skv, acc_v, half, 1.0f);
+    }
+}
+
+}  // namespace ahpc

@@ -150,35 +150,9 @@ static int dispatch_simple(int dtype, const SimpleParams& p, int64_t B, hipStrea
 }
 
 // ---------------------------------------------------------------------------------------------
-// Fills the launch geometry of the MFMA kernel (query tiles, pairing, workgroup count, interleaving of
-// heads) from N, H and the batch size already in `p`.  Shared by the launcher and by the host-side dump
-// of the workgroup map.
-static int plan_mfma(FlashParams& p, int64_t B, bool causal) {
-    p.n_qtiles = (p.N + kFlashRows - 1) / kFlashRows;
-    int64_t total = B * p.H * (int64_t)p.n_qtiles;
-    if (total > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
-    // Causal launches with enough workgroups to fill the chip twice over pair a late query tile with an
-    // early one, so that every workgroup walks the same number of key tiles.
-    p.paired = (causal && p.n_qtiles >= 2 && total >= 1024) ? 1 : 0;
-    if (p.paired) total = B * p.H * (int64_t)((p.n_qtiles + 1) / 2);
-    p.total_blocks = (int32_t)total;
-    p.blocks_per_xcd = (int32_t)((total + 7) / 8);
-    // AHPC_FLASH_HEADS_TOGETHER = n lets n heads advance side by side on an XCD (default: one after the
-    // other); AHPC_FLASH_ROUND_SLOTS sets how many workgroups a head contributes per round (default 64 / n:
-    // an XCD holds 64 workgroups of this kernel).  Tuning knobs; every setting computes the same result.
-    int ht = 1, rs = 0;
-    if (const char* e = std::getenv("AHPC_FLASH_HEADS_TOGETHER")) ht = std::atoi(e);
-    if (const char* e = std::getenv("AHPC_FLASH_ROUND_SLOTS")) rs = std::atoi(e);
-    if (ht < 1 || ht > 64) ht = 1;
-    if (rs < 1) rs = 64 / ht;
-    p.heads_together = ht;
-    p.round_slots = rs;
-    return AHPC_OK;
-}
-
 template <typename T, int D, bool VARLEN>
 static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
-    if (int rc = plan_mfma(p, B, causal)) return rc;
+    if (int rc = flash_plan_launch(p, B, causal)) return rc;
     dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
     if (causal) hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, true, VARLEN>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, false, VARLEN>), grid, block, 0, stream, p);
@@ -255,7 +229,7 @@ int ahpc_hip_flash_block_map(int64_t B, int64_t N, int64_t H, int causal, int64_
     if (B <= 0 || N <= 0 || H <= 0 || B > 65535 || H > 65535 || N > 0x7FFFFF00ll) return AHPC_ERR_BAD_SHAPE;
     FlashParams p{};
     p.N = (int32_t)N; p.H = (int32_t)H; p.kv_group = 1;
-    if (int rc = plan_mfma(p, B, causal != 0)) return rc;
+    if (int rc = flash_plan_launch(p, B, causal != 0)) return rc;
     const int64_t grid = (int64_t)p.blocks_per_xcd * 8;
     *n_blocks = grid;
     if (!seq_head && !first_tile && !second_tile) return AHPC_OK;

@@ -39,6 +39,8 @@
 // mask all workgroups then walk the same number of key tiles, which evens out the end of the launch.
 #pragma once
 
+#include <cstdlib>
+
 #include "ahpc_device.hpp"
 
 namespace ahpc {
@@ -170,8 +172,20 @@ __host__ __device__ inline int flash_qtile_of_part(const FlashParams& p, int slo
     return part == 0 ? p.n_qtiles - 1 - slot : -1;
 }
 
-template <typename T, int D, bool CAUSAL, bool VARLEN>
-__global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const FlashParams p) {
+// What the statistics variant of the kernel writes instead of O (first step of the backward):
+// per (sequence, head, query row)  lse2 = log2 sum_j exp2(c q.k_j)  (c = scale*log2(e), the units the kernel
+// works in) and delta = dO . O.  Rows are laid out [B*H][rows_padded], rows_padded a multiple of the
+// 128-row query tile; rows beyond the sequence receive lse2 = +inf (every weight exp2(s - inf) is 0 later
+// on) and delta = 0, so that whole tiles of statistics can be read without a bounds check.
+struct FlashStatsOut {
+    const void* d_out;     // dO, laid out like Q and O
+    float* lse2;
+    float* delta;
+    int64_t rows_padded;
+};
+
+template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS>
+__device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const FlashStatsOut& st) {
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;  // k-steps of the first product
     constexpr int MB = D / 32;  // 32-row blocks of O^T
@@ -429,7 +443,29 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
         // ---- normalise and store: lane holds, per 32-row block, 4 runs of 4 consecutive lanes of d ---
         const float l = halves_sum(l_run);
         const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-        if (qrow < L) {
+        if constexpr (STATS) {
+            // delta = dO . O over the elements this lane holds, then over the two lanes of the query
+            float part = 0.0f;
+            if (qrow < L) {
+                const T* src = static_cast<const T*>(st.d_out) + base + (int64_t)qrow * sn + 4 * half;
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        const u32x2 w = *reinterpret_cast<const u32x2*>(src + 32 * mb + 8 * g4);
+                        const f32x16& a = oacc[mb];
+                        part += a[4 * g4 + 0] * lo_f32<T>(w[0]) + a[4 * g4 + 1] * hi_f32<T>(w[0]) +
+                                a[4 * g4 + 2] * lo_f32<T>(w[1]) + a[4 * g4 + 3] * hi_f32<T>(w[1]);
+                    }
+            }
+            const float delta = halves_sum(part) * inv;
+            if (half == 0 && qrow < q_tile0 + kFlashRows) {
+                const int64_t row = (int64_t)bh * st.rows_padded + qrow;
+                const bool live = qrow < L && l > 0.0f;
+                st.lse2[row] = live ? __builtin_log2f(l) - neg_m[0] : INFINITY;
+                st.delta[row] = live ? delta : 0.0f;
+            }
+        } else if (qrow < L) {
             T* dst = go + (int64_t)qrow * sn + 4 * half;
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
@@ -443,6 +479,43 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
         }
         __syncthreads();  // the next query tile's first DMA reuses the buffers
     }
+}
+
+// Fills the launch geometry of the MFMA kernel (query tiles, pairing, workgroup count, interleaving of
+// heads) from N, H and the batch size already in `p`.  Shared by the launcher and by the host-side dump
+// of the workgroup map.
+inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal) {
+    p.n_qtiles = (p.N + kFlashRows - 1) / kFlashRows;
+    int64_t total = B * p.H * (int64_t)p.n_qtiles;
+    if (total > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
+    // Causal launches with enough workgroups to fill the chip twice over pair a late query tile with an
+    // early one, so that every workgroup walks the same number of key tiles.
+    p.paired = (causal && p.n_qtiles >= 2 && total >= 1024) ? 1 : 0;
+    if (p.paired) total = B * p.H * (int64_t)((p.n_qtiles + 1) / 2);
+    p.total_blocks = (int32_t)total;
+    p.blocks_per_xcd = (int32_t)((total + 7) / 8);
+    // AHPC_FLASH_HEADS_TOGETHER = n lets n heads advance side by side on an XCD (default: one after the
+    // other); AHPC_FLASH_ROUND_SLOTS sets how many workgroups a head contributes per round (default 64 / n:
+    // an XCD holds 64 workgroups of this kernel).  Tuning knobs; every setting computes the same result.
+    int ht = 1, rs = 0;
+    if (const char* e = std::getenv("AHPC_FLASH_HEADS_TOGETHER")) ht = std::atoi(e);
+    if (const char* e = std::getenv("AHPC_FLASH_ROUND_SLOTS")) rs = std::atoi(e);
+    if (ht < 1 || ht > 64) ht = 1;
+    if (rs < 1) rs = 64 / ht;
+    p.heads_together = ht;
+    p.round_slots = rs;
+    return AHPC_OK;
+}
+
+template <typename T, int D, bool CAUSAL, bool VARLEN>
+__global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const FlashParams p) {
+    flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, false>(p, FlashStatsOut{});
+}
+
+// The forward pass with its output kept in registers: writes the softmax statistics the backward needs.
+template <typename T, int D, bool CAUSAL>
+__global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_stats_mfma_kernel(const FlashParams p, const FlashStatsOut st) {
+    flash_fwd_mfma_body<T, D, CAUSAL, false, true>(p, st);
 }
 
 }  // namespace ahpc

@@ -157,6 +157,31 @@ int ahpc_hip_flash_fwd_varlen_gqa(const void* q, const void* k, const void* v, v
 int ahpc_hip_flash_block_map(int64_t B, int64_t N, int64_t H, int causal, int64_t capacity, int64_t* n_blocks,
                              int32_t* seq_head, int32_t* first_tile, int32_t* second_tile);
 
+/* ---- FlashAttention backward ------------------------------------------------------------------
+ * Gradients of ahpc_hip_flash_fwd_gqa: given d_out = dLoss/dO it writes d_q = dLoss/dQ (layout and strides
+ * of Q) and d_k, d_v (layout and strides of K, V; with grouped heads each K/V head receives the sum over
+ * its query heads).  Replaces FlashAttention::backward -> compute_query_gradients /
+ * compute_key_value_gradients, src/algorithms/flash_attention.cpp:114-174, :496-580, and the
+ * launch_flash_attention_backward_kernel slot of src/backends/cuda/cuda_flash_attention.hpp:50-56
+ * (flash_attention_backward_kernel, src/backends/cuda/cuda_kernels.cu:280-365).  Those are placeholders
+ * (sums that ignore the attention weights; a kernel that expects stored N x N weights): what is computed
+ * here is the derivative of the forward,  P = softmax(scale Q K^T + mask),  dV = P^T dO,
+ * dS = P o (dO V^T - rowsum(dO o O)),  dQ = scale dS K,  dK = scale dS^T Q,  with the softmax statistics
+ * recomputed (the interface passes neither O nor them).  All seven tensors share one dtype; fp32
+ * accumulation throughout; the gradient tensors are fully overwritten, rows that see no key get zeros.
+ * workspace: device memory of at least ahpc_hip_flash_bwd_workspace_bytes(B, N, H) bytes, 16-byte aligned,
+ * for two floats per (sequence, head, row of a whole 128-row tile); its contents afterwards are unspecified.
+ * fp16/bf16 with d in {64, 128} and no mask run on the MFMA kernels, everything else on fp32-FMA kernels.
+ * mask: NULL or fp32 [B,N,N] as in the forward. */
+size_t ahpc_hip_flash_bwd_workspace_bytes(int64_t B, int64_t N, int64_t H);
+int ahpc_hip_flash_bwd(const void* d_out, const void* q, const void* k, const void* v,
+                       void* d_q, void* d_k, void* d_v, int dtype,
+                       int64_t B, int64_t N, int64_t H, int64_t H_kv, int64_t d,
+                       int64_t stride_b, int64_t stride_n, int64_t stride_h,
+                       int64_t kv_stride_b, int64_t kv_stride_n, int64_t kv_stride_h,
+                       float scale, int causal, const float* mask,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- paged KV pool ---------------------------------------------------------------------------
  * Pool layout: K and V are separate slabs  [page][slot 0..P-1][head][d]  (the layout
  * update_kv_cache_kernel writes, src/backends/cuda/cuda_kernels.cu:547-556).

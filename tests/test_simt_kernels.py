@@ -282,3 +282,78 @@ def test_paired_query_tiles(emu):
     q, k, v = qkv((B, N, H, d), 18, O.F16)
     got = flash(emu, q, k, v, O.F16, B, N, H, d, 0.125, True)
     assert np.abs(got - O.attention(q, k, v, B, N, H, d, 0.125, True)).max() <= 2e-2
+
+
+# ---- FlashAttention backward -----------------------------------------------------------------------------
+def backward(emu, q, k, v, do, dtype, B, N, H, H_kv, d, scale, causal, mask=None, front=False):
+    dq_, dk_, dv_, ddo = dev(q, dtype, front), dev(k, dtype, front), dev(v, dtype, front), dev(do, dtype, front)
+    gq = S.guarded(S.empty_storage((B, N, H, d), dtype), front)
+    gk = S.guarded(S.empty_storage((B, N, H_kv, d), dtype), front)
+    gv = S.guarded(S.empty_storage((B, N, H_kv, d), dtype), front)
+    dm = None if mask is None else S.guarded(mask, front)
+    ws_bytes = emu.flash_bwd_workspace_bytes(B, N, H)
+    ws = S.guarded(np.full(ws_bytes // 4, np.nan, np.float32), front)
+    emu.flash_bwd(S.ptr(ddo), S.ptr(dq_), S.ptr(dk_), S.ptr(dv_), S.ptr(gq), S.ptr(gk), S.ptr(gv), dtype, B, N, H, H_kv, d,
+                  (N * H * d, H * d, d), (N * H_kv * d, H_kv * d, d), scale, causal, S.ptr(ws), ws_bytes, None,
+                  None if dm is None else S.ptr(dm))
+    return tuple(S.from_storage(x, dtype) for x in (gq, gk, gv))
+
+
+def bwd_inputs(B, N, H, H_kv, d, seed, dtype):
+    q = O.round_to(O.fill_normal((B, N, H, d), seed, 1), dtype)
+    k = O.round_to(O.fill_normal((B, N, H_kv, d), seed, 2), dtype)
+    v = O.round_to(O.fill_normal((B, N, H_kv, d), seed, 3), dtype)
+    do = O.round_to(O.fill_normal((B, N, H, d), seed, 7), dtype)
+    return q, k, v, do
+
+
+def check_gradients(got, want, dtype):
+    """fp32: 1e-4 max-abs as in the forward.  16-bit: 2e-2 relative to the largest entry of the gradient
+    (entries are sums over up to N terms, so their size, unlike the forward's, grows with the problem)."""
+    for name, g, w in zip(("dQ", "dK", "dV"), got, want):
+        assert np.isfinite(g).all(), name
+        bar = 1e-4 * max(1.0, np.abs(w).max()) if dtype == O.F32 else 2e-2 * max(1.0, np.abs(w).max())
+        assert np.abs(g - w).max() <= bar, (name, np.abs(g - w).max(), bar)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,N,H,H_kv,d", [(2, 16, 4, 4, 64), (1, 150, 2, 1, 32), (1, 40, 3, 3, 80), (1, 1, 2, 2, 128), (1, 20, 2, 2, 256)])
+def test_backward_fp32_kernels(emu, B, N, H, H_kv, d, causal):
+    q, k, v, do = bwd_inputs(B, N, H, H_kv, d, 31, O.F32)
+    scale = 1.0 / np.sqrt(d)
+    got = backward(emu, q, k, v, do, O.F32, B, N, H, H_kv, d, scale, causal)
+    check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), O.F32)
+
+
+def test_backward_fp32_kernels_dense_mask(emu):
+    B, N, H, d = 2, 37, 2, 64
+    q, k, v, do = bwd_inputs(B, N, H, H, d, 32, O.F32)
+    mask = (O.fill_uniform((B, N, N), 12, 6) > 0.3).astype(np.float32)
+    mask[0, 5, :] = 0.0  # a row that sees nothing: no gradient flows through it
+    got = backward(emu, q, k, v, do, O.F32, B, N, H, H, d, 0.125, False, mask=mask)
+    assert not got[0][0, 5].any()
+    check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, 0.125, False, H, mask), O.F32)
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16])
+def test_backward_fp32_kernels_16bit_storage(emu, dtype):
+    B, N, H, H_kv, d = 1, 70, 4, 2, 32   # d = 32 is not taken by the matrix-core kernels
+    q, k, v, do = bwd_inputs(B, N, H, H_kv, d, 33, dtype)
+    got = backward(emu, q, k, v, do, dtype, B, N, H, H_kv, d, 0.2, True, front=True)
+    check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, 0.2, True, H_kv), dtype)
+
+
+@pytest.mark.parametrize("dma_late", [False, True])
+@pytest.mark.parametrize("dtype", [O.BF16, O.F16])
+@pytest.mark.parametrize("B,N,H,H_kv,d,causal", [
+    (1, 64, 1, 1, 128, False), (2, 129, 2, 2, 128, True), (1, 300, 2, 2, 64, True), (1, 200, 2, 1, 64, False),
+    (1, 1, 2, 2, 128, True), (1, 260, 4, 2, 128, True)])
+def test_backward_matrix_core_kernels(emu, dtype, B, N, H, H_kv, d, causal, dma_late):
+    q, k, v, do = bwd_inputs(B, N, H, H_kv, d, 34, dtype)
+    scale = 1.0 / np.sqrt(d)
+    S.configure(dma_late, seed=N + d)
+    try:
+        got = backward(emu, q, k, v, do, dtype, B, N, H, H_kv, d, scale, causal, front=dma_late)
+    finally:
+        S.configure(False, 1)
+    check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), dtype)
