@@ -1,4 +1,4 @@
-// FlashAttention (HIP backend): validation, host/device pointer staging, one launch per forward.
+// FlashAttention (HIP backend): validation, host/device pointer staging, one launch per forward, three per backward.
 #include "algorithms/flash_attention.hpp"
 
 #include <algorithm>
@@ -16,6 +16,7 @@ struct FlashAttention::Impl {
     bool configured = false;
     hipsup::Stream stream;
     hipsup::DeviceBuffer dq, dk, dv, dout, dmask, dcu;
+    hipsup::DeviceBuffer ddo, gq, gk, gv, ws;  // backward: staged dO, gradients, statistics workspace
     std::vector<std::pair<std::string, double>> profile;
 };
 
@@ -186,10 +187,76 @@ void FlashAttention::forward_varlen(const TensorShape& shape, const void* q, con
     impl_->stream.sync();
 }
 
-void FlashAttention::backward(const TensorShape&, const void*, const TensorShape&, const void*, const TensorShape&,
-                              const void*, const TensorShape&, const void*, const TensorShape&, void*, const TensorShape&,
-                              void*, const TensorShape&, void*, const void*) {
-    throw AttentionException(AttentionError::UNSUPPORTED_OPERATION, "HIP FlashAttention implements the forward pass only");
+// Reference: FlashAttention::backward, src/algorithms/flash_attention.cpp:114-174.  The reference converts,
+// calls two placeholder gradient loops (:496-580) and converts back; here the gradients are the derivative of
+// forward(): three launches behind ahpc_hip_flash_bwd.  Validation as in forward(); the gradient tensors
+// must have the shapes of the tensors they belong to.
+void FlashAttention::backward(const TensorShape& gos, const void* go, const TensorShape& qs, const void* q,
+                              const TensorShape& ks, const void* k, const TensorShape& vs, const void* v,
+                              const TensorShape& gqs, void* gq, const TensorShape& gks, void* gk, const TensorShape& gvs,
+                              void* gv, const void* mask) {
+    if (!impl_->configured)
+        throw AttentionException(AttentionError::INVALID_PARAMETERS, "FlashAttention not configured. Call configure() first.");
+    if (!go || !q || !k || !v || !gq || !gk || !gv) throw AttentionException(AttentionError::INVALID_INPUT, "null tensor pointer");
+    if (validate_inputs(qs, ks, vs, gos, current_params_) != AttentionError::SUCCESS ||
+        validate_inputs(gqs, gks, gvs, gos, current_params_) != AttentionError::SUCCESS)
+        throw AttentionException(AttentionError::INVALID_INPUT, "tensor shapes do not match the configured parameters");
+    const size_t N = qs.dimensions[1];
+    for (const TensorShape* s : {&gos, &qs, &ks, &vs, &gqs, &gks, &gvs}) {
+        if (s->dimensions[1] != N)
+            throw AttentionException(AttentionError::INVALID_INPUT, "all tensors must share one sequence length");
+        if (s->data_type != qs.data_type)
+            throw AttentionException(AttentionError::INVALID_INPUT, "all tensors must share one data type");
+        if (s->layout != MemoryLayout::ROW_MAJOR)
+            throw AttentionException(AttentionError::UNSUPPORTED_OPERATION, "only ROW_MAJOR tensors are supported");
+    }
+    const size_t B = current_params_.batch_size, H = current_params_.num_heads, d = current_params_.head_dimension;
+    const size_t Hkv = kv_heads(current_params_);
+    const size_t bytes = qs.total_bytes(), kv_bytes = ks.total_bytes();
+    void* st = impl_->stream.get();
+    hipsup::EventTimer timer;
+    const auto wall0 = std::chrono::steady_clock::now();
+
+    const void* d_go = stage_in(go, bytes, impl_->ddo, st);
+    const void* d_q = stage_in(q, bytes, impl_->dq, st);
+    const void* d_k = stage_in(k, kv_bytes, impl_->dk, st);
+    const void* d_v = stage_in(v, kv_bytes, impl_->dv, st);
+    const bool gq_dev = hipsup::is_device_pointer(gq), gk_dev = hipsup::is_device_pointer(gk), gv_dev = hipsup::is_device_pointer(gv);
+    void* d_gq = gq_dev ? gq : impl_->gq.reserve(bytes);
+    void* d_gk = gk_dev ? gk : impl_->gk.reserve(kv_bytes);
+    void* d_gv = gv_dev ? gv : impl_->gv.reserve(kv_bytes);
+    const float* dmask = nullptr;
+    if (mask) dmask = static_cast<const float*>(stage_in(mask, B * N * N * sizeof(float), impl_->dmask, st));
+    const size_t ws_bytes = ahpc_hip_flash_bwd_workspace_bytes((int64_t)B, (int64_t)N, (int64_t)H);
+    void* ws = impl_->ws.reserve(ws_bytes);
+
+    float scale = impl_->cfg.softmax_scale > 0.0f ? impl_->cfg.softmax_scale : current_params_.scale_factor;
+    if (!(scale > 0.0f)) scale = 1.0f / std::sqrt(static_cast<float>(d));
+    const int causal = (current_params_.causal_mask || impl_->cfg.use_causal_mask) ? 1 : 0;
+    int64_t sb, sn, sh, kb, kn, kh;
+    if (impl_->cfg.tensor_layout_bhnd) {
+        sb = (int64_t)(H * N * d); sh = (int64_t)(N * d); sn = (int64_t)d;
+        kb = (int64_t)(Hkv * N * d); kh = sh; kn = sn;
+    } else {
+        sb = (int64_t)(N * H * d); sn = (int64_t)(H * d); sh = (int64_t)d;
+        kb = (int64_t)(N * Hkv * d); kn = (int64_t)(Hkv * d); kh = sh;
+    }
+    if (profiling_enabled_) timer.start(st);
+    check(ahpc_hip_flash_bwd(d_go, d_q, d_k, d_v, d_gq, d_gk, d_gv, hipsup::dtype_code(qs.data_type), (int64_t)B, (int64_t)N,
+                             (int64_t)H, (int64_t)Hkv, (int64_t)d, sb, sn, sh, kb, kn, kh, scale, causal, dmask, ws, ws_bytes, st),
+          "flash backward");
+    if (profiling_enabled_) timer.stop(st);
+    if (!gq_dev) check(ahpc_hip_memcpy_d2h(gq, d_gq, bytes, st), "copy from device");
+    if (!gk_dev) check(ahpc_hip_memcpy_d2h(gk, d_gk, kv_bytes, st), "copy from device");
+    if (!gv_dev) check(ahpc_hip_memcpy_d2h(gv, d_gv, kv_bytes, st), "copy from device");
+    impl_->stream.sync();
+
+    if (profiling_enabled_) {
+        // "backward_pass": wall-clock ms of the whole call, as in the reference (src/algorithms/flash_attention.cpp:169-173)
+        const double wall_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - wall0).count();
+        impl_->profile.emplace_back("backward_pass", wall_ms);
+        impl_->profile.emplace_back("backward_kernel_ms", timer.elapsed_ms());
+    }
 }
 
 // Device bytes this object stages when every tensor arrives in host memory (nothing when they are

@@ -267,6 +267,18 @@ def bench_extras(hip, stream, steps, warmup):
                                   (N * Hkv * d, Hkv * d, d), sc, True, stream),
         flops=2.0 * B * H * N * N * d)
 
+    # backward at the headline shape.  FLOP by the usual convention: 2.5 x the forward's (five products
+    # against two); the three launches here execute nine, because the interface passes neither the forward
+    # output nor its softmax statistics and they are recomputed.
+    go = randn((B, N, H, d), torch.bfloat16)
+    gq, gk, gv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    wsb = hip.flash_bwd_workspace_bytes(B, N, H)
+    wsf = torch.empty(wsb // 4, dtype=torch.float32, device="cuda")
+    run("flash_bwd bf16 causal B=4 N=4096 H=32 d=128",
+        lambda: hip.flash_bwd(go.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), gq.data_ptr(), gk.data_ptr(),
+                              gv.data_ptr(), hip.BF16, B, N, H, H, d, st, st, sc, True, wsf.data_ptr(), wsb, stream),
+        flops=2.5 * 2.0 * B * H * N * N * d)
+
     # ragged fp16 causal batch: 16 sequences, lengths U[128,8192], H=32, d=64 (sigma 0.5)
     rng = np.random.default_rng(0xA77E0005)
     lens = rng.integers(128, 8193, size=16).astype(np.int32)

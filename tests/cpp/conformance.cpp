@@ -190,14 +190,66 @@ CASE(Flash_DifferentBlockSizes, true) {  // :360-402: result must not depend on 
     EXPECT(run_flash_and_compare(fa, p, 6) <= 1e-4f);
 }
 
-CASE(Flash_BackwardIsUnsupported, true) {  // :405-480 only checks "non-zero"; this backend has no backward
+CASE(Flash_BackwardPass, true) {  // :405-480 (forward, then backward; the reference only asks for non-zero gradients)
     FlashAttention fa;
     AttentionParams p = fixture_params();
     fa.configure(p);
-    const TensorShape s = shape4(2, 16, 4, 64);
-    std::vector<float> x(2 * 16 * 4 * 64, 0.1f);
-    EXPECT_THROWS(fa.backward(s, x.data(), s, x.data(), s, x.data(), s, x.data(), s, x.data(), s, x.data(), s, x.data()),
-                  AttentionError::UNSUPPORTED_OPERATION);
+    const size_t B = p.batch_size, N = p.sequence_length, H = p.num_heads, d = p.head_dimension, n = B * N * H * d;
+    auto q = uniform(n, 11, 1), k = uniform(n, 11, 2), v = uniform(n, 11, 3);
+    auto go = uniform(n, 11, 7, 0.01f, 0.1f);  // as in the reference's test
+    std::vector<float> out(n), gq(n, 0.0f), gk(n, 0.0f), gv(n, 0.0f);
+    const TensorShape s = shape4(B, N, H, d);
+    fa.forward(s, q.data(), s, k.data(), s, v.data(), s, out.data());
+    fa.backward(s, go.data(), s, q.data(), s, k.data(), s, v.data(), s, gq.data(), s, gk.data(), s, gv.data());
+    auto nonzero = [](const std::vector<float>& x) {
+        for (float e : x)
+            if (std::fabs(e) > 1e-6f) return true;
+        return false;
+    };
+    EXPECT(nonzero(gq) && nonzero(gk) && nonzero(gv));  // :449-478
+    std::vector<float> wq(n), wk(n), wv(n);
+    ahpc_oracle_attention_backward(q.data(), k.data(), v.data(), go.data(), wq.data(), wk.data(), wv.data(), B, N, H, H, d,
+                                   p.scale_factor, 0, nullptr, 4);
+    EXPECT(max_abs_diff(gq, wq) <= 1e-4f && max_abs_diff(gk, wk) <= 1e-4f && max_abs_diff(gv, wv) <= 1e-4f);
+}
+
+CASE(Flash_BackwardCausalGroupedHalf, true) {  // bf16 tensors, causal, 4 query heads over 2 K/V heads: the matrix-core kernels
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    p.sequence_length = 200;
+    p.head_dimension = 128;
+    p.key_value_heads = 2;
+    p.causal_mask = true;
+    p.scale_factor = 1.0f / std::sqrt(128.0f);
+    fa.configure(p);
+    const size_t B = p.batch_size, N = p.sequence_length, H = p.num_heads, Hkv = 2, d = p.head_dimension;
+    const size_t n = B * N * H * d, nkv = B * N * Hkv * d;
+    auto q = uniform(n, 12, 1), k = uniform(nkv, 12, 2), v = uniform(nkv, 12, 3), go = uniform(n, 12, 7);
+    auto to_bf16 = [](std::vector<float>& x) {
+        std::vector<bfloat16> y(x.size());
+        for (size_t i = 0; i < x.size(); ++i) {
+            y[i] = bfloat16(x[i]);
+            x[i] = static_cast<float>(y[i]);  // the oracle sees the rounded values
+        }
+        return y;
+    };
+    auto hq = to_bf16(q), hk = to_bf16(k), hv = to_bf16(v), hgo = to_bf16(go);
+    std::vector<bfloat16> gq(n), gk(nkv), gv(nkv);
+    const TensorShape s = shape4(B, N, H, d, DataType::BFLOAT16), skv = shape4(B, N, Hkv, d, DataType::BFLOAT16);
+    fa.backward(s, hgo.data(), s, hq.data(), skv, hk.data(), skv, hv.data(), s, gq.data(), skv, gk.data(), skv, gv.data());
+    std::vector<float> wq(n), wk(nkv), wv(nkv);
+    ahpc_oracle_attention_backward(q.data(), k.data(), v.data(), go.data(), wq.data(), wk.data(), wv.data(), B, N, H, Hkv, d,
+                                   p.scale_factor, 1, nullptr, 4);
+    auto close = [](const std::vector<bfloat16>& got, const std::vector<float>& want) {
+        float top = 1.0f, worst = 0.0f;
+        for (float w : want) top = std::max(top, std::fabs(w));
+        for (size_t i = 0; i < want.size(); ++i) worst = std::max(worst, std::fabs(static_cast<float>(got[i]) - want[i]));
+        return worst <= 2e-2f * top;
+    };
+    EXPECT(close(gq, wq) && close(gk, wk) && close(gv, wv));
+    // wrong gradient shape is refused
+    EXPECT_THROWS(fa.backward(s, hgo.data(), s, hq.data(), skv, hk.data(), skv, hv.data(), s, gq.data(), s, gk.data(), skv, gv.data()),
+                  AttentionError::INVALID_INPUT);
 }
 
 CASE(Flash_AttentionMask, true) {  // :483-582: mask [B,N,N] float, 0 = masked

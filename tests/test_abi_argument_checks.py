@@ -43,6 +43,23 @@ def test_grouped_heads_argument_checks(lib):
     assert lib.ahpc_hip_flash_fwd_varlen(P, P, P, P, F16, None, 2, 16, 8, 64, 8 * 64, 64, 0.0, 1, None) == NULL_POINTER
 
 
+def test_flash_backward_argument_checks(lib):
+    def bwd(go=P, q=P, gq=P, dtype=F16, B=1, N=16, H=4, Hkv=2, d=64, ws=P, ws_bytes=1 << 20, sn=None):
+        sn = H * d if sn is None else sn
+        return lib.ahpc_hip_flash_bwd(go, q, P, P, gq, P, P, dtype, B, N, H, Hkv, d, N * H * d, sn, d, N * Hkv * d, Hkv * d, d,
+                                      0.0, 1, None, ws, ws_bytes, None)
+    assert bwd(go=None) == NULL_POINTER and bwd(q=None) == NULL_POINTER and bwd(gq=None) == NULL_POINTER
+    assert bwd(ws=None) == NULL_POINTER
+    assert bwd(dtype=7) == BAD_DTYPE
+    assert bwd(N=0) == BAD_SHAPE and bwd(H=6, Hkv=4) == BAD_SHAPE and bwd(sn=8) == BAD_SHAPE
+    assert bwd(d=512, sn=4 * 512) == HEAD_DIM
+    need = lib.ahpc_hip_flash_bwd_workspace_bytes(1, 16, 4)
+    assert need == 1 * 4 * 128 * 2 * 4          # rows padded to a whole 128-row tile, two floats each
+    assert bwd(ws_bytes=need - 1) == WORKSPACE
+    assert bwd(ws=P + 4) == BAD_ALIGNMENT
+    assert lib.ahpc_hip_flash_bwd_workspace_bytes(0, 16, 4) == 0
+
+
 def decode(lib, q=P, o=P, kp=P, vp=P, table=P, lens=P, qo=F16, pool=F16, B=2, H=8, Hkv=8, d=128, Pg=16, max_pages=4, max_len=64,
            ws=None, ws_bytes=0, chunk=0):
     return lib.ahpc_hip_paged_decode_gqa(q, o, qo, kp, vp, pool, table, lens, None, B, H, Hkv, d, Pg, max_pages, max_len, 0.0, chunk,

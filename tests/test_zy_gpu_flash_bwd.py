@@ -1,0 +1,156 @@
+"""FlashAttention backward on the GPU (through the C ABI) against the CPU oracle's double-precision gradients.
+
+Bars: fp32 tensors 1e-4 max-abs (relative to the largest entry when that exceeds 1); fp16/bf16 tensors 2e-2 of
+the largest entry of the gradient (gradient entries are sums over up to N terms, so their size grows with
+the problem, unlike the forward's convex combinations).  The reference has no working backward to compare with
+(src/algorithms/flash_attention.cpp:496-580 is a placeholder): parity is to the oracle, which is pinned by
+tests/test_oracle_backward.py.  This file is collected after the other GPU parity tests on purpose."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    from attention_amd import hip
+    hip.load()
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return hip
+
+
+def inputs(B, N, H, H_kv, d, seed, dtype):
+    q = O.round_to(O.fill_normal((B, N, H, d), seed, 1), dtype)
+    k = O.round_to(O.fill_normal((B, N, H_kv, d), seed, 2), dtype)
+    v = O.round_to(O.fill_normal((B, N, H_kv, d), seed, 3), dtype)
+    do = O.round_to(O.fill_normal((B, N, H, d), seed, 7), dtype)
+    return q, k, v, do
+
+
+def run_backward(hip, q, k, v, do, dtype, B, N, H, H_kv, d, scale, causal, mask=None):
+    import torch
+    from gpu_util import to_dev, to_host, stream_ptr
+    tq, tk, tv, tdo = (to_dev(x, dtype) for x in (q, k, v, do))
+    gq, gk, gv = torch.full_like(tq, float("nan")), torch.full_like(tk, float("nan")), torch.full_like(tv, float("nan"))
+    tm = None if mask is None else torch.from_numpy(mask).cuda()
+    ws_bytes = hip.flash_bwd_workspace_bytes(B, N, H)
+    ws = torch.full((ws_bytes // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    hip.flash_bwd(tdo.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), gq.data_ptr(), gk.data_ptr(), gv.data_ptr(),
+                  dtype, B, N, H, H_kv, d, (N * H * d, H * d, d), (N * H_kv * d, H_kv * d, d), scale, causal, ws.data_ptr(),
+                  ws_bytes, stream_ptr(), None if tm is None else tm.data_ptr())
+    torch.cuda.synchronize()
+    return to_host(gq), to_host(gk), to_host(gv)
+
+
+def check(got, want, dtype):
+    for name, g, w in zip(("dQ", "dK", "dV"), got, want):
+        assert np.isfinite(g).all(), name
+        bar = (1e-4 if dtype == O.F32 else 2e-2) * max(1.0, np.abs(w).max())
+        assert np.abs(g - w).max() <= bar, (name, float(np.abs(g - w).max()), bar)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,N,H,H_kv,d", [(2, 16, 4, 4, 64), (1, 150, 2, 1, 32), (1, 40, 3, 3, 80), (1, 1, 2, 2, 128), (1, 300, 2, 2, 128)])
+def test_fp32_tensors(gpu, B, N, H, H_kv, d, causal):
+    # the first shape is the fixture of tests/test_flash_attention.cpp:103-108, whose backward test (:405-480)
+    # only asks for non-zero gradients
+    q, k, v, do = inputs(B, N, H, H_kv, d, 31, O.F32)
+    scale = 1.0 / np.sqrt(d)
+    got = run_backward(gpu, q, k, v, do, O.F32, B, N, H, H_kv, d, scale, causal)
+    assert all(np.abs(g).max() > 1e-6 for g in got) or N == 1
+    check(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), O.F32)
+
+
+def test_dense_mask(gpu):
+    B, N, H, d = 2, 37, 2, 64
+    q, k, v, do = inputs(B, N, H, H, d, 32, O.F32)
+    mask = (O.fill_uniform((B, N, N), 12, 6) > 0.3).astype(np.float32)
+    mask[0, 5, :] = 0.0
+    got = run_backward(gpu, q, k, v, do, O.F32, B, N, H, H, d, 0.125, False, mask=mask)
+    assert not got[0][0, 5].any()
+    check(got, O.attention_backward(q, k, v, do, B, N, H, d, 0.125, False, H, mask), O.F32)
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16])
+@pytest.mark.parametrize("B,N,H,H_kv,d,causal", [
+    (1, 64, 1, 1, 128, False), (2, 129, 2, 2, 128, True), (1, 300, 2, 2, 64, True), (1, 200, 2, 1, 64, False),
+    (1, 1, 2, 2, 128, True), (1, 260, 4, 2, 128, True), (2, 1024, 4, 4, 128, True), (1, 517, 3, 3, 64, False),
+    (1, 70, 4, 2, 32, True)])
+def test_16bit_tensors(gpu, dtype, B, N, H, H_kv, d, causal):
+    # d = 64, 128: matrix-core kernels; d = 32: fp32-FMA kernels with 16-bit storage
+    q, k, v, do = inputs(B, N, H, H_kv, d, 34, dtype)
+    scale = 1.0 / np.sqrt(d)
+    got = run_backward(gpu, q, k, v, do, dtype, B, N, H, H_kv, d, scale, causal)
+    check(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), dtype)
+
+
+def test_closed_forms_16bit(gpu):
+    B, N, H, d = 1, 256, 2, 128
+    q, k, v, do = inputs(B, N, H, H, d, 35, O.BF16)
+    # V with equal rows => dP is constant along a row => dS = 0 => dQ = dK = 0
+    vc = np.repeat(v[:, :1], N, axis=1)
+    gq, gk, gv = run_backward(gpu, q, k, vc, do, O.BF16, B, N, H, H, d, 0.1, True)
+    assert np.abs(gq).max() <= 2e-2 and np.abs(gk).max() <= 2e-2
+    # K with equal rows => uniform weights: dQ = 0 and (no mask) dV_j = mean_i dO_i
+    kc = np.repeat(k[:, :1], N, axis=1)
+    gq, gk, gv = run_backward(gpu, q, kc, v, do, O.BF16, B, N, H, H, d, 0.1, False)
+    assert np.abs(gq).max() <= 2e-2
+    assert np.abs(gv - do.mean(axis=1, keepdims=True)).max() <= 2e-2
+
+
+def test_headline_shape_bf16_causal(gpu):
+    """B=4, N=4096, H=32, d=128, causal, bf16: properties that hold at any size over the whole result, and one
+    (sequence, head) against the oracle."""
+    import torch
+    from gpu_util import stream_ptr
+    B, N, H, d = 4, 4096, 32, 128
+    g = torch.Generator(device="cuda").manual_seed(0xA77E0006)
+    tq, tk, tv, tdo = (torch.randn((B, N, H, d), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+                       for _ in range(4))
+    gq, gk, gv = (torch.full_like(tq, float("nan")) for _ in range(3))
+    ws_bytes = gpu.flash_bwd_workspace_bytes(B, N, H)
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device="cuda")
+    scale = 1.0 / np.sqrt(d)
+    gpu.flash_bwd(tdo.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), gq.data_ptr(), gk.data_ptr(), gv.data_ptr(),
+                  O.BF16, B, N, H, H, d, (N * H * d, H * d, d), (N * H * d, H * d, d), scale, True, ws.data_ptr(), ws_bytes,
+                  stream_ptr())
+    torch.cuda.synchronize()
+    for t in (gq, gk, gv):
+        assert torch.isfinite(t.float()).all()
+    # the weights of a query row sum to one: sum_j dV_j = sum_i dO_i per (sequence, head)
+    lhs, rhs = gv.double().sum(dim=1), tdo.double().sum(dim=1)
+    assert (lhs - rhs).abs().max().item() <= 2e-2 * max(1.0, rhs.abs().max().item())
+    # sum_i q_i.dQ_i = sum_j k_j.dK_j (both are scale * sum_ij dS_ij q_i.k_j)
+    a = (tq.double() * gq.double()).sum(dim=(1, 3))
+    b = (tk.double() * gk.double()).sum(dim=(1, 3))
+    assert (a - b).abs().max().item() <= 2e-2 * max(1.0, a.abs().max().item(), b.abs().max().item())
+    # the last key is seen by the last query only: dV_last = P_last,last * dO_last, a multiple of dO_last
+    # one (sequence, head) against the oracle
+    bi, hi = 2, 17
+    sl = lambda t: t[bi:bi + 1, :, hi:hi + 1].float().cpu().numpy()
+    want = O.attention_backward(sl(tq), sl(tk), sl(tv), sl(tdo), 1, N, 1, d, scale, True)
+    for name, got, w in zip(("dQ", "dK", "dV"), (sl(gq), sl(gk), sl(gv)), want):
+        assert np.abs(got - w).max() <= 2e-2 * max(1.0, np.abs(w).max()), name
+
+
+def test_bad_arguments_are_rejected_without_launch(gpu):
+    import torch
+    x = torch.zeros(1 << 16, device="cuda")
+    p = x.data_ptr()
+    ok = dict(dtype=O.F32, B=1, N=16, H=2, H_kv=2, d=64, strides=(2048, 128, 64), kv_strides=(2048, 128, 64), scale=0.1,
+              causal=False, workspace=p, workspace_bytes=1 << 16)
+    call = lambda **kw: gpu.flash_bwd(p, p, p, p, p, p, p, **{**ok, **kw})
+    with pytest.raises(gpu.HipError):
+        call(H_kv=3)
+    with pytest.raises(gpu.HipError):
+        call(d=300)
+    with pytest.raises(gpu.HipError):
+        call(workspace_bytes=16)
+    with pytest.raises(gpu.HipError):
+        call(workspace=None)
+    with pytest.raises(gpu.HipError):
+        gpu.flash_bwd(p, p, p, p, 0, p, p, **ok)
+    torch.cuda.synchronize()
