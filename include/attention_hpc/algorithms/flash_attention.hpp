@@ -70,10 +70,16 @@ public:
     void forward_varlen(const TensorShape& packed_shape, const void* query_data, const void* key_data,
                         const void* value_data, void* output_data, const int32_t* cu_seqlens, size_t n_seqs);
 
-    // Always throws UNSUPPORTED_OPERATION: this backend is inference-forward only.
-    void backward(const TensorShape&, const void*, const TensorShape&, const void*, const TensorShape&, const void*,
-                  const TensorShape&, const void*, const TensorShape&, void*, const TensorShape&, void*,
-                  const TensorShape&, void*, const void* = nullptr) override;
+    // Gradients of forward() for a given grad_output: grad_query has the shape of the query tensor,
+    // grad_key / grad_value those of key / value (with grouped heads each K/V head receives the sum over its
+    // query heads).  All tensors share one data type; pointers may be host or device memory.  The forward
+    // output is not needed (it is recomputed).  Reference: src/algorithms/flash_attention.cpp:114-174, whose
+    // gradient loops (:496-580) are placeholders.
+    void backward(const TensorShape& grad_output_shape, const void* grad_output_data, const TensorShape& query_shape,
+                  const void* query_data, const TensorShape& key_shape, const void* key_data, const TensorShape& value_shape,
+                  const void* value_data, const TensorShape& grad_query_shape, void* grad_query_data,
+                  const TensorShape& grad_key_shape, void* grad_key_data, const TensorShape& grad_value_shape,
+                  void* grad_value_data, const void* attention_mask = nullptr) override;
 
     size_t get_workspace_size(const AttentionParams& params) const override;
     void set_workspace(void* workspace_ptr, size_t workspace_size) override;
