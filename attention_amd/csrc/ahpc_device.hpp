@@ -83,6 +83,17 @@ template <> __device__ inline float dot2<bf16_t>(uint32_t a, uint32_t b, float a
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), acc, false);
 }
 
+// ---- LDS ----------------------------------------------------------------------------------------
+// 16-byte LDS read (ds_read_b128).  The CPU executor the tests use defines AHPC_TRACED_LDS_READ_B128 to
+// a read that also records the lanes' addresses, so that bank conflicts can be counted there.
+__device__ inline u32x4 lds_read_b128(const unsigned char* p) {
+#if defined(AHPC_TRACED_LDS_READ_B128)
+    return AHPC_TRACED_LDS_READ_B128(p);
+#else
+    return *reinterpret_cast<const u32x4*>(p);
+#endif
+}
+
 // ---- MFMA ----------------------------------------------------------------------------------
 // D(32x32) += A(32x16) * B(16x32).  Lane l supplies A[row l%32][k 8*(l/32)..+7] and
 // B[k 8*(l/32)..+7][col l%32]; it receives D[row 8*(r/4) + 4*(l/32) + r%4][col l%32] in acc[r].

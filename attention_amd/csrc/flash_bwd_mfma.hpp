@@ -19,8 +19,8 @@
 //
 // In both kernels a lane owns one row of the output (a query, a key) and the masks are per-lane
 // comparisons.  Tiles are streamed with direct-to-LDS loads and double buffered as in the forward; every
-// tile is read by rows (first two products) and by transposing reads (last products), with the row-read
-// swizzle.  No atomics: every output element is written once.
+// tile is read by rows (first two products) and by transposing reads (last products); its swizzle
+// (FlashTile::fb) keeps both kinds of read free of LDS bank conflicts.  No atomics: every output element is written once.
 #pragma once
 
 #include "flash_fwd_mfma.hpp"
@@ -47,7 +47,7 @@ struct FlashBwdParams {
     float scale_log2;           // scale * log2(e)
 };
 
-// Byte offset inside a row-swizzled tile of the 8 bytes a lane hands to a transposing read that fetches
+// Byte offset inside a tile swizzled with FlashTile::fb of the 8 bytes a lane hands to a transposing read that fetches
 // the 4 tile rows 16*g + 8*a + 4*(lane/32) + 0..3 for column quad (32*mb + 16*((lane/16)%2) + 4*(lane%4)):
 // the part that does not depend on g.  Adding 16*g rows keeps the swizzle (it has period 16 rows).
 template <int D>
@@ -56,7 +56,7 @@ __device__ inline int tr_offset_rowswizzled(int lane, int mb, int a) {
     const int vi = lane & 15;
     const int row = 8 * a + 4 * (lane >> 5) + (vi >> 2);
     const int cch = 4 * mb + 2 * ((lane >> 4) & 1) + ((vi & 3) >> 1);
-    return row * TL::kRowBytes + ((cch ^ TL::fk(row)) << 4) + 8 * (vi & 1);
+    return row * TL::kRowBytes + ((cch ^ TL::fb(row)) << 4) + 8 * (vi & 1);
 }
 
 // Packs 8 fp32 of a 32x32 accumulator block (rows r0..r0+7 of the lane's column) as one B operand.
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dq_mfma_kernel(const 
     for (int i = 0; i < TL::kInstrPerWave; ++i) {
         const int r = (wave * TL::kInstrPerWave + i) * TL::kRowsPerInstr + lane / TL::kChunks;
         const int pc = lane % TL::kChunks;
-        dma_off[i] = (int)(r * skv * 2) + ((pc ^ TL::fk(r)) << 4);
+        dma_off[i] = (int)(r * skv * 2) + ((pc ^ TL::fb(r)) << 4);
     }
     auto dma_both = [&](int k0, unsigned char* dst_k, unsigned char* dst_v) {
         const int64_t rem = (int64_t)(L - k0 - 1) * skv * 2 + 2 * D;
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dq_mfma_kernel(const 
 
     int row_off[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * RB + (((2 * ks + half) ^ TL::fk(col)) << 4);
+    for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * RB + (((2 * ks + half) ^ TL::fb(col)) << 4);
     int tr_off[MB][2];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -189,8 +189,8 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dq_mfma_kernel(const 
             f32x16 s = neg_lse, dp = neg_delta;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const u32x4 ak = *reinterpret_cast<const u32x4*>(tile_k + 32 * kb * RB + row_off[ks]);
-                const u32x4 av = *reinterpret_cast<const u32x4*>(tile_v + 32 * kb * RB + row_off[ks]);
+                const u32x4 ak = lds_read_b128(tile_k + 32 * kb * RB + row_off[ks]);
+                const u32x4 av = lds_read_b128(tile_v + 32 * kb * RB + row_off[ks]);
                 s = mfma_32x32x16<T>(ak, qreg[ks], s);
                 dp = mfma_32x32x16<T>(av, doreg[ks], dp);
             }
@@ -274,11 +274,11 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
     for (int i = 0; i < TL::kInstrPerWave; ++i) {
         const int r = (wave * TL::kInstrPerWave + i) * TL::kRowsPerInstr + lane / TL::kChunks;
         const int pc = lane % TL::kChunks;
-        dma_off[i] = (int)(r * sn * 2) + ((pc ^ TL::fk(r)) << 4);
+        dma_off[i] = (int)(r * sn * 2) + ((pc ^ TL::fb(r)) << 4);
     }
     int row_off[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * RB + (((2 * ks + half) ^ TL::fk(col)) << 4);
+    for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * RB + (((2 * ks + half) ^ TL::fb(col)) << 4);
     int tr_off[MB][2];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -340,8 +340,8 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
                 }
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    const u32x4 aq = *reinterpret_cast<const u32x4*>(tile_q + 32 * ib * RB + row_off[ks]);
-                    const u32x4 ao = *reinterpret_cast<const u32x4*>(tile_o + 32 * ib * RB + row_off[ks]);
+                    const u32x4 aq = lds_read_b128(tile_q + 32 * ib * RB + row_off[ks]);
+                    const u32x4 ao = lds_read_b128(tile_o + 32 * ib * RB + row_off[ks]);
                     s = mfma_32x32x16<T>(aq, kreg[ks], s);
                     dp = mfma_32x32x16<T>(ao, vreg[ks], dp);
                 }

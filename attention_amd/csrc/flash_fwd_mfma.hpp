@@ -108,6 +108,12 @@ template <int D> struct FlashTile {
     // swizzles (XOR on the 16-byte chunk index)
     __device__ static int fk(int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); }
     __device__ static int fv(int row) { return D == 128 ? 4 * (row & 3) : 4 * ((row >> 1) & 1); }
+    // for tiles that are read both ways (backward): 16 consecutive rows get 16 different chunks (row reads),
+    // and the 4 rows of a transposing read get chunk quads that do not overlap
+    __device__ static int fb(int row) {
+        const int b0 = row & 1, b1 = (row >> 1) & 1, b2 = (row >> 2) & 1, b3 = (row >> 3) & 1;
+        return D == 128 ? (((b1 ^ b3) << 3) | (b0 << 2) | (b2 << 1) | b1) : (((b1 ^ b0) << 2) | (b2 << 1) | (b3 ^ b0));
+    }
 };
 
 // Streams one 64-key tile (K or V) from global memory into LDS through a buffer descriptor.
@@ -320,8 +326,8 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                 u32x4 a0[KS], a1[KS];
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    a0[ks] = *reinterpret_cast<const u32x4*>(tile_k + k_off[ks]);
-                    a1[ks] = *reinterpret_cast<const u32x4*>(tile_k + 32 * RB + k_off[ks]);
+                    a0[ks] = lds_read_b128(tile_k + k_off[ks]);
+                    a1[ks] = lds_read_b128(tile_k + 32 * RB + k_off[ks]);
                 }
                 s[0] = mfma_32x32x16<T>(a0[0], qreg[0], neg_m);
                 s[1] = mfma_32x32x16<T>(a1[0], qreg[0], neg_m);

@@ -12,6 +12,8 @@
 //   * global -> LDS direct loads are asynchronous: their data lands either at issue or only at the next
 //     s_waitcnt of the issuing lane (chosen per run), which exposes a missing wait or a buffer reused
 //     too early; buffer descriptors clamp out-of-range reads to zero like the hardware;
+//   * 16-byte LDS reads made through lds_read_b128 and transposing reads are checked for bank conflicts under
+//     a model of 64 banks of 4 bytes (16 lanes per pass for 16-byte reads, 32 for 8-byte reads);
 //   * __shared__ arrays live in one linker section, filled with a NaN pattern before every workgroup,
 //     and LDS accesses made through intrinsics are range-checked against it.
 // Plain loads and stores through pointers are ordinary host accesses; run the build under
@@ -54,6 +56,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 void launch(dim3 grid, dim3 block, const std::function<void()>& body);
 hipError_t last_error();
@@ -64,6 +67,7 @@ int lane_id();
 f32x16 mfma_32x32x16_f16(f16x8 a, f16x8 b, f32x16 c);
 f32x16 mfma_32x32x16_bf16(bf16x8 a, bf16x8 b, f32x16 c);
 uint64_t ds_read_tr16_b64(const void* lds_ptr);
+u32x4 lds_read_b128(const void* lds_ptr);  // a plain 16-byte LDS read whose addresses are recorded
 u32x2 permlane32_swap(unsigned a, unsigned b);
 uint64_t ballot(bool pred);
 int readfirstlane(int x);
@@ -169,6 +173,7 @@ inline hipError_t hipGetLastError() { return ::simt::last_error(); }
     ::simt::bits_to<__attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16>(::simt::ds_read_tr16_b64((const void*)(p)))
 #define __builtin_amdgcn_ds_read_tr16_b64_v4f16(p) \
     ::simt::bits_to<__attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16>(::simt::ds_read_tr16_b64((const void*)(p)))
+#define AHPC_TRACED_LDS_READ_B128(p) ::simt::lds_read_b128((p))
 #define __builtin_amdgcn_permlane32_swap(a, b, fi, bc) ::simt::permlane32_swap((a), (b))
 #define __builtin_amdgcn_ballot_w64(p) ::simt::ballot((p))
 #define __builtin_amdgcn_readfirstlane(x) ::simt::readfirstlane((x))

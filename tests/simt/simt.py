@@ -130,3 +130,14 @@ def guarded(a, front=False):
     out = np.frombuffer(m, dtype=a.dtype, count=a.size, offset=off).reshape(a.shape)
     out[...] = a
     return out
+
+
+def lds_stats(reset=False):
+    """(16-byte LDS reads, their bank-conflict cycles, transposing reads, their bank-conflict cycles) per
+    wavefront instruction, under the executor's model of 64 banks of 4 bytes."""
+    lib = load()
+    out = (C.c_long * 4)()
+    lib.simt_lds_stats(out)
+    if reset:
+        lib.simt_lds_stats_reset()
+    return tuple(out)

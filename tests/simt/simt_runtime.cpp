@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 #include <ucontext.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <mutex>
 #include <string>
@@ -31,7 +32,7 @@ constexpr int kWaveSize = 64;
 constexpr int kPayload = 64;          // bytes a lane can publish per cross-lane operation
 constexpr size_t kStackBytes = 512 * 1024;
 
-enum Kind : int { K_NONE = 0, K_MFMA, K_TR, K_SWAP, K_BALLOT, K_RFL, K_RL, K_DPP, K_SHFL };
+enum Kind : int { K_NONE = 0, K_MFMA, K_TR, K_SWAP, K_BALLOT, K_RFL, K_RL, K_DPP, K_SHFL, K_LDS128 };
 
 struct PendingDma {
     unsigned char* dst;
@@ -82,6 +83,7 @@ bool g_dma_late = false;
 uint64_t g_rng = 0x9E3779B97F4A7C15ull;
 std::vector<unsigned char*> g_stacks;  // reused between launches
 long g_switches = 0;
+long g_lds_stats[4] = {0, 0, 0, 0};  // 16-byte reads, their conflict cycles, transposing reads, theirs
 
 uint64_t next_rand() {
     g_rng ^= g_rng << 13;
@@ -221,6 +223,40 @@ bool in_lds(const void* p, size_t n) {
     return q >= __start_simt_lds && q + n <= __stop_simt_lds;
 }
 
+// Extra cycles a wave-wide LDS read costs under a model of 64 banks of 4 bytes: the lanes are served
+// `lanes_per_pass` at a time (256 bytes per pass); a pass takes as many cycles as the largest number of
+// different dwords that fall into one bank.
+long conflict_cycles(const View& v, int bytes_per_lane, int lanes_per_pass) {
+    long extra = 0;
+    for (int first = 0; first < kWaveSize; first += lanes_per_pass) {
+        uint64_t dwords[64][16];
+        int count[64] = {0};
+        for (int l = first; l < first + lanes_per_pass; ++l) {
+            if (!v.has(l)) continue;
+            uint64_t addr;
+            std::memcpy(&addr, v.of(l) + 16, 8);
+            addr -= reinterpret_cast<uint64_t>(__start_simt_lds);
+            for (int o = 0; o < bytes_per_lane; o += 4) {
+                const uint64_t dw = (addr + o) / 4;
+                const int bank = (int)(dw % 64);
+                bool seen = false;
+                for (int i = 0; i < count[bank]; ++i) seen = seen || dwords[bank][i] == dw;
+                if (!seen && count[bank] < 16) dwords[bank][count[bank]++] = dw;
+            }
+        }
+        int worst = 1;
+        for (int b = 0; b < 64; ++b) worst = std::max(worst, count[b]);
+        extra += worst - 1;
+    }
+    return extra;
+}
+
+bool first_live_lane(const View& v, int lane) {
+    for (int l = 0; l < lane; ++l)
+        if (v.has(l)) return false;
+    return true;
+}
+
 template <typename T> float to_f32(T x) { return (float)x; }
 
 template <typename V> f32x16 mfma_impl(V a, V b, f32x16 c) {
@@ -279,8 +315,16 @@ uint64_t ds_read_tr16_b64(const void* lds_ptr) {
     if (!in_lds(lds_ptr, 8)) fail("transposing LDS read outside the workgroup's LDS");
     if ((reinterpret_cast<uintptr_t>(lds_ptr) & 7) != 0) fail("transposing LDS read not 8-byte aligned");
     std::memcpy(&mine, lds_ptr, 8);
-    const View v = exchange(K_TR, &mine, 8);
+    unsigned char payload[24] = {0};
+    std::memcpy(payload, &mine, 8);
+    const uint64_t addr = reinterpret_cast<uint64_t>(lds_ptr);
+    std::memcpy(payload + 16, &addr, 8);
+    const View v = exchange(K_TR, payload, sizeof payload);
     const int lane = g_cur->lane, row0 = lane & ~15, j = lane & 15;
+    if (first_live_lane(v, lane)) {
+        g_lds_stats[2] += 1;
+        g_lds_stats[3] += conflict_cycles(v, 8, 32);
+    }
     uint16_t out[4];
     for (int r = 0; r < 4; ++r) {
         uint16_t src[4];
@@ -290,6 +334,22 @@ uint64_t ds_read_tr16_b64(const void* lds_ptr) {
     uint64_t res;
     std::memcpy(&res, out, 8);
     return res;
+}
+
+u32x4 lds_read_b128(const void* lds_ptr) {
+    if (!in_lds(lds_ptr, 16)) fail("16-byte LDS read outside the workgroup's LDS");
+    if ((reinterpret_cast<uintptr_t>(lds_ptr) & 15) != 0) fail("16-byte LDS read not 16-byte aligned");
+    unsigned char payload[24] = {0};
+    const uint64_t addr = reinterpret_cast<uint64_t>(lds_ptr);
+    std::memcpy(payload + 16, &addr, 8);
+    const View v = exchange(K_LDS128, payload, sizeof payload);
+    if (first_live_lane(v, g_cur->lane)) {
+        g_lds_stats[0] += 1;
+        g_lds_stats[1] += conflict_cycles(v, 16, 16);
+    }
+    u32x4 r;
+    std::memcpy(&r, lds_ptr, 16);
+    return r;
 }
 
 // v_permlane32_swap a, b: the upper 32 lanes of a and the lower 32 lanes of b change places.
@@ -488,4 +548,12 @@ void simt_clear_error() {
     simt::g_status = hipSuccess;
 }
 long simt_switch_count() { return simt::g_switches; }
+// out[0..3] = 16-byte LDS reads executed (per wavefront), their extra cycles from bank conflicts, transposing
+// reads, their extra cycles; counted since the last reset.
+void simt_lds_stats(long* out) {
+    for (int i = 0; i < 4; ++i) out[i] = simt::g_lds_stats[i];
+}
+void simt_lds_stats_reset() {
+    for (long& x : simt::g_lds_stats) x = 0;
+}
 }

@@ -357,3 +357,19 @@ def test_backward_matrix_core_kernels(emu, dtype, B, N, H, H_kv, d, causal, dma_
     finally:
         S.configure(False, 1)
     check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), dtype)
+
+
+# ---- LDS bank conflicts (model: 64 banks of 4 bytes) --------------------------------------------------------
+@pytest.mark.parametrize("dtype,d", [(O.BF16, 128), (O.F16, 64)])
+def test_operand_reads_are_free_of_bank_conflicts(emu, dtype, d):
+    """Every 16-byte operand read and every transposing read of the matrix-core kernels, forward and backward.
+    (The GPU's own conflict counter reads zero for the forward kernel, which is what anchors the model.)"""
+    B, N, H = 1, 200, 2
+    q, k, v, do = bwd_inputs(B, N, H, H, d, 36, dtype)
+    S.lds_stats(reset=True)
+    flash(emu, q, k, v, dtype, B, N, H, d, 0.1, True)
+    reads, read_conflicts, tr, tr_conflicts = S.lds_stats(reset=True)
+    assert reads > 0 and tr > 0 and read_conflicts == 0 and tr_conflicts == 0
+    backward(emu, q, k, v, do, dtype, B, N, H, H, d, 0.1, True)
+    reads, read_conflicts, tr, tr_conflicts = S.lds_stats(reset=True)
+    assert reads > 0 and tr > 0 and read_conflicts == 0 and tr_conflicts == 0
