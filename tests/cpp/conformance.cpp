@@ -925,15 +925,17 @@ CASE(Paged_SequenceLifecycle, true) {  // extend / truncate / reset, src/algorit
 // ---- main ------------------------------------------------------------------------------------------------------
 int main(int argc, char** argv) {
     bool no_gpu = false;
-    std::string filter;
+    std::string filter, skip;   // run cases whose name contains `filter`, leave out those containing `skip`
     for (int i = 1; i < argc; ++i) {
         if (std::string(argv[i]) == "--no-gpu") no_gpu = true;
+        else if (std::string(argv[i]) == "--skip" && i + 1 < argc) skip = argv[++i];
         else filter = argv[i];
     }
     int ran = 0, failed = 0;
     for (const Case& c : cases()) {
         if (no_gpu && c.needs_gpu) continue;
         if (!filter.empty() && std::string(c.name).find(filter) == std::string::npos) continue;
+        if (!skip.empty() && std::string(c.name).find(skip) != std::string::npos) continue;
         std::printf("[ RUN  ] %s\n", c.name);
         std::fflush(stdout);
         const int before = g_failures;

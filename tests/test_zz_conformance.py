@@ -34,5 +34,10 @@ def test_all_cases_on_the_cpu_executor():
 
 
 @pytest.mark.gpu
-def test_all_cases_on_gpu():
-    run([])
+def test_forward_decode_and_pool_cases_on_gpu():
+    run(["--skip", "Backward"])
+
+
+@pytest.mark.gpu
+def test_backward_cases_on_gpu():
+    run(["Backward"])

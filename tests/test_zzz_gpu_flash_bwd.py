@@ -4,7 +4,7 @@ Bars: fp32 tensors 1e-4 max-abs (relative to the largest entry when that exceeds
 the largest entry of the gradient (gradient entries are sums over up to N terms, so their size grows with
 the problem, unlike the forward's convex combinations).  The reference has no working backward to compare with
 (src/algorithms/flash_attention.cpp:496-580 is a placeholder): parity is to the oracle, which is pinned by
-tests/test_oracle_backward.py.  This file is collected after the other GPU parity tests on purpose."""
+tests/test_oracle_backward.py.  This file is collected after every other GPU test on purpose: these kernels are the newest."""
 import numpy as np
 import pytest
 
