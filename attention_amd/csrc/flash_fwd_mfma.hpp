@@ -131,6 +131,15 @@ __device__ inline void dma_tile(const void* base, unsigned nrec, const int* off,
 #endif
 }
 
+// One direct-to-LDS load instruction on its own: lane i's 16 bytes at base + off (bytes; anything not inside
+// [0, nrec) reads as zero) land at lds + 16*i.
+__device__ inline void dma_instr(const void* base, unsigned nrec, int off, unsigned char* lds) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the descriptor type exists only in the device pass
+    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, nrec, 0x00020000);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (AHPC_LDS void*)lds, 16, off, 0, 0, 0);
+#endif
+}
+
 // Workgroup id -> work.  Hardware deals consecutive workgroup ids to the 8 XCDs in turn; `logical` undoes
 // that, so that consecutive logical ids run on the same XCD and share its L2.  A head owns `per_head`
 // consecutive logical ids (its query tiles, or pairs of them), late (long) tiles first.  With

@@ -454,6 +454,12 @@ __global__ __launch_bounds__(256) void paged_merge_kernel(const DecodeParams p) 
     store_qo(p.o, p.qo_dtype, idx, l > 0.0f ? acc / l : 0.0f);
 }
 
+}  // namespace ahpc
+
+#include "paged_decode_mfma.hpp"  // uses DecodeParams and the q/o vector helpers above
+
+namespace ahpc {
+
 static int env_int(const char* name, int dflt) {
     const char* e = std::getenv(name);
     return e ? std::atoi(e) : dflt;
@@ -498,6 +504,16 @@ static int launch_decode_dp(const DecodeParams& p, dim3 grid, dim3 block, hipStr
         case 8: return launch_decode_dpg<T, PT, 8>(p, grid, block, st);
         default: return AHPC_ERR_UNSUPPORTED_GROUP;
     }
+}
+
+// Matrix-core kernel for grouped heads: one wavefront per (pool head, chunk, batch entry).
+template <typename T>
+static int launch_decode_mfma(const DecodeParams& p, hipStream_t st) {
+    const dim3 grid((unsigned)p.H_kv, (unsigned)p.n_chunks, (unsigned)p.B), block(64);
+    if (p.d == 128) hipLaunchKernelGGL((paged_decode_mfma_kernel<T, 128>), grid, block, 0, st, p);
+    else if (p.d == 64) hipLaunchKernelGGL((paged_decode_mfma_kernel<T, 64>), grid, block, 0, st, p);
+    else return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+    return static_cast<int>(hipGetLastError());
 }
 
 template <typename T>
@@ -643,7 +659,13 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
                               float scale, int64_t chunk_tokens, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !o || !k_pool || !v_pool || !block_table || !seq_lens) return AHPC_ERR_NULL_POINTER;
     if (H_kv <= 0 || H <= 0 || H % H_kv) return AHPC_ERR_BAD_SHAPE;
-    { const int64_t g = H / H_kv; if (g != 1 && g != 2 && g != 4 && g != 8) return AHPC_ERR_UNSUPPORTED_GROUP; }
+    // Groups of 1, 2, 4, 8 query heads: lane-per-element kernel, any pool type.  Groups of 16 and 32 exist on
+    // the matrix-core kernel only (16-bit pool, d 64 or 128, pages of 16 tokens); AHPC_DECODE_MFMA=1 sends
+    // groups of 4 and 8 there as well.
+    const int64_t group = H / H_kv;
+    const bool mfma_shape = (pool_dtype == AHPC_F16 || pool_dtype == AHPC_BF16) && (d == 64 || d == 128) && P == 16 && H_kv <= 65535;
+    if (group != 1 && group != 2 && group != 4 && group != 8 && !((group == 16 || group == 32) && mfma_shape))
+        return AHPC_ERR_UNSUPPORTED_GROUP;
     if (qo_dtype < AHPC_F32 || qo_dtype > AHPC_BF16 || pool_dtype < AHPC_F32 || pool_dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
     if (B <= 0 || B > 65535 || max_len <= 0 || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;
     if ((max_len + P - 1) / P > max_pages) return AHPC_ERR_BAD_SHAPE;
@@ -688,6 +710,10 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
 
     dim3 grid((unsigned)head_groups, (unsigned)n_chunks, (unsigned)B), block(64 * waves);
     int rc;
+    const bool use_mfma = mfma_shape && (group >= 16 || (group >= 4 && env_int("AHPC_DECODE_MFMA", 0) == 1));
+    if (use_mfma) {
+        rc = pool_dtype == AHPC_F16 ? launch_decode_mfma<f16_t>(p, st) : launch_decode_mfma<bf16_t>(p, st);
+    } else
     switch (pool_dtype) {
         case AHPC_F32: rc = launch_decode_d<float>(p, grid, block, st); break;
         case AHPC_F16: rc = launch_decode_d<f16_t>(p, grid, block, st); break;

@@ -21,7 +21,7 @@ inline size_t dtype_size(DataType t) { return t == DataType::FLOAT32 ? 4 : 2; }
 inline void check(int status, const char* what, bool is_alloc = false) {
     if (status == 0) return;
     AttentionError code = AttentionError::COMPUTATION_FAILED;
-    if (status == AHPC_ERR_UNSUPPORTED_HEAD_DIM) code = AttentionError::UNSUPPORTED_OPERATION;
+    if (status == AHPC_ERR_UNSUPPORTED_HEAD_DIM || status == AHPC_ERR_UNSUPPORTED_GROUP) code = AttentionError::UNSUPPORTED_OPERATION;
     else if (status == AHPC_ERR_NO_DEVICE) code = AttentionError::BACKEND_NOT_AVAILABLE;
     else if (status < 0) code = AttentionError::INVALID_INPUT;
     else if (is_alloc) code = AttentionError::MEMORY_ALLOCATION_FAILED;

@@ -43,7 +43,7 @@ typedef enum ahpc_status {
     AHPC_ERR_WORKSPACE_TOO_SMALL = -5,
     AHPC_ERR_NO_DEVICE = -6,
     AHPC_ERR_BAD_ALIGNMENT = -7,   /* pointers/strides must allow 16-byte vector access */
-    AHPC_ERR_UNSUPPORTED_GROUP = -8 /* query heads per K/V head: decode takes 1, 2, 4 or 8 */
+    AHPC_ERR_UNSUPPORTED_GROUP = -8 /* query heads per K/V head: decode takes 1, 2, 4, 8 (16, 32: see paged_decode_gqa) */
 } ahpc_status;
 
 const char* ahpc_hip_error_string(int code);
@@ -258,6 +258,8 @@ int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype,
 /* Decode with grouped K/V heads: the pool holds H_kv heads per token (its kv_scatter / kv_gather /
  * gather_indices calls take H = H_kv), q and o hold H = g * H_kv heads, g in {1, 2, 4, 8}; query
  * head h reads pool head h / g.  Every K/V byte is still read once and serves g query heads.
+ * g = 16 and 32 (up to multi-query attention with 32 heads) are served by a matrix-core kernel that needs
+ * an fp16/bf16 pool, d in {64, 128} and P = 16; other combinations return AHPC_ERR_UNSUPPORTED_GROUP.
  * Workspace size: ahpc_hip_paged_decode_workspace_bytes with the QUERY head count. */
 int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype,
                               const void* k_pool, const void* v_pool, int pool_dtype,

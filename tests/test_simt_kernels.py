@@ -373,3 +373,35 @@ def test_operand_reads_are_free_of_bank_conflicts(emu, dtype, d):
     backward(emu, q, k, v, do, dtype, B, N, H, H, d, 0.1, True)
     reads, read_conflicts, tr, tr_conflicts = S.lds_stats(reset=True)
     assert reads > 0 and tr > 0 and read_conflicts == 0 and tr_conflicts == 0
+
+
+# ---- grouped decode on the matrix cores --------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,d", [(O.F16, 128), (O.BF16, 64)])
+@pytest.mark.parametrize("G", [4, 8, 16, 32])
+def test_decode_grouped_heads_matrix_core_kernel(emu, G, dtype, d, monkeypatch):
+    monkeypatch.setenv("AHPC_DECODE_MFMA", "1")   # groups of 4 and 8 take this kernel only when asked to
+    B, H_kv, P = 4, 2, 16
+    H = G * H_kv
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [70, 5, 129, 32], 23, dtype)
+    lens = lens.copy()
+    lens[3] = 0                                     # an empty sequence: zeros
+    q = O.round_to(O.fill_normal((B, H, d), 23, 1), dtype)
+    scale = 1.0 / np.sqrt(d)
+    rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
+    want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    S.lds_stats(reset=True)
+    for chunk, qo in ((0, dtype), (48, O.F32), (16, dtype)):
+        got = decode(emu, q, kp, vp, table, lens, None, B, H, H_kv, d, P, dtype, qo, scale, chunk)
+        assert np.all(got[3] == 0.0)
+        assert np.abs(got - want).max() <= 2e-2, (chunk, qo)
+    reads, read_conflicts, tr, tr_conflicts = S.lds_stats(reset=True)
+    assert reads > 0 and tr > 0 and read_conflicts == 0 and tr_conflicts == 0
+
+
+def test_wide_groups_need_the_matrix_core_shape(emu):
+    # 16 query heads per pool head on an fp32 pool: refused
+    B, H_kv, d, P, G = 1, 1, 64, 16, 16
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [20], 24, O.F32)
+    q = O.fill_normal((B, G * H_kv, d), 24, 1)
+    with pytest.raises(emu.HipError):
+        decode(emu, q, kp, vp, table, lens, None, B, G * H_kv, H_kv, d, P, O.F32, O.F32, 0.125)

@@ -35,9 +35,14 @@ def test_all_cases_on_the_cpu_executor():
 
 @pytest.mark.gpu
 def test_forward_decode_and_pool_cases_on_gpu():
-    run(["--skip", "Backward"])
+    run(["--skip", "Backward,WideGroups"])
 
 
 @pytest.mark.gpu
 def test_backward_cases_on_gpu():
     run(["Backward"])
+
+
+@pytest.mark.gpu
+def test_wide_group_decode_cases_on_gpu():
+    run(["WideGroups"])

@@ -1,0 +1,81 @@
+"""Grouped-head decode on the matrix-core kernel, on the GPU through the C ABI, against the CPU oracle fed a pool
+whose heads are repeated (the definition of grouped heads).  16 and 32 query heads per pool head exist on this
+kernel only; 4 and 8 take it when AHPC_DECODE_MFMA=1.  Collected after the established GPU tests on purpose:
+this kernel is newer than they are."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from test_gpu_paged import build_problem, gpu_decode  # noqa: F401  (problem builder; gpu_decode documents the call)
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    from attention_amd import hip
+    hip.load()
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return hip
+
+
+def run(hip, q, kp, vp, table, lens, B, H, H_kv, d, P, dtype, qo_dtype, scale, chunk):
+    import torch
+    from gpu_util import to_dev, to_host, stream_ptr, dev_i32
+    dq = to_dev(q, qo_dtype)
+    do = torch.full_like(dq, float("nan"))
+    kd, vd = to_dev(kp, dtype), to_dev(vp, dtype)
+    dt, dl = dev_i32(table), dev_i32(lens)
+    max_len = int(max(1, lens.max()))
+    ws_bytes = hip.paged_decode_workspace_bytes(B, H, d, max_len, P, chunk)
+    ws = torch.full((max(ws_bytes, 4) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    hip.paged_decode_gqa(dq.data_ptr(), do.data_ptr(), qo_dtype, kd.data_ptr(), vd.data_ptr(), dtype, dt.data_ptr(),
+                         dl.data_ptr(), None, B, H, H_kv, d, P, table.shape[1], max_len, scale, chunk, ws.data_ptr(), ws_bytes,
+                         stream_ptr())
+    torch.cuda.synchronize()
+    return to_host(do)
+
+
+@pytest.mark.parametrize("dtype,d", [(O.F16, 128), (O.BF16, 64), (O.BF16, 128)])
+@pytest.mark.parametrize("G", [4, 8, 16, 32])
+def test_matrix_core_decode_equals_repeated_heads(gpu, G, dtype, d, monkeypatch):
+    monkeypatch.setenv("AHPC_DECODE_MFMA", "1")
+    B, H_kv, P = 5, 2, 16
+    H = G * H_kv
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [700, 5, 129, 32, 1000], 23, dtype)
+    lens = lens.copy()
+    lens[3] = 0
+    q = O.round_to(O.fill_normal((B, H, d), 23, 1), dtype)
+    scale = 1.0 / np.sqrt(d)
+    rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
+    want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    for chunk, qo in ((0, dtype), (48, O.F32), (16, dtype), (1024, dtype)):
+        got = run(gpu, q, kp, vp, table, lens, B, H, H_kv, d, P, dtype, qo, scale, chunk)
+        assert np.isfinite(got).all()
+        assert np.all(got[3] == 0.0)
+        assert np.abs(got - want).max() <= 2e-2, (chunk, qo)
+
+
+def test_both_kernels_agree_for_groups_of_four(gpu, monkeypatch):
+    B, H_kv, d, P, G = 3, 8, 128, 16, 4
+    H = G * H_kv
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [2000, 77, 513], 25, O.F16)
+    q = O.round_to(O.fill_normal((B, H, d), 25, 1), O.F16)
+    scale = 1.0 / np.sqrt(d)
+    monkeypatch.delenv("AHPC_DECODE_MFMA", raising=False)
+    a = run(gpu, q, kp, vp, table, lens, B, H, H_kv, d, P, O.F16, O.F32, scale, 0)
+    monkeypatch.setenv("AHPC_DECODE_MFMA", "1")
+    b = run(gpu, q, kp, vp, table, lens, B, H, H_kv, d, P, O.F16, O.F32, scale, 0)
+    assert np.abs(a - b).max() <= 5e-3   # same inputs, fp32 outputs: only P's rounding to 16 bits differs
+
+
+def test_wide_groups_on_other_pools_are_refused(gpu):
+    import torch
+    x = torch.zeros(1 << 16, device="cuda")
+    p = x.data_ptr()
+    with pytest.raises(gpu.HipError):   # fp32 pool
+        gpu.paged_decode_gqa(p, p, O.F32, p, p, O.F32, p, p, None, 1, 16, 1, 64, 16, 4, 64, 0.1, 0, None, 0, None)
+    with pytest.raises(gpu.HipError):   # pages of 8 tokens
+        gpu.paged_decode_gqa(p, p, O.F16, p, p, O.F16, p, p, None, 1, 32, 1, 64, 8, 8, 64, 0.1, 0, None, 0, None)
+    torch.cuda.synchronize()
