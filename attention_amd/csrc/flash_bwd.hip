@@ -313,16 +313,21 @@ static int launch_mfma_d(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool 
     const FlashStatsOut st{p.d_out, lse2, delta, p.rows_padded};
     const dim3 block(kFlashThreads);
     const dim3 grid_stats((unsigned)(f.blocks_per_xcd * 8));
-    const unsigned tiles = (unsigned)((p.N + kFlashRows - 1) / kFlashRows);
-    const dim3 grid_q(tiles, (unsigned)p.H, (unsigned)B), grid_kv(tiles, (unsigned)H_kv, (unsigned)B);
+    FlashBwdParams m = p;
+    m.n_tiles = (p.N + kFlashRows - 1) / kFlashRows;
+    const int64_t total_q = B * p.H * (int64_t)m.n_tiles, total_kv = B * H_kv * (int64_t)m.n_tiles;
+    if (total_q > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
+    m.total_q = (int32_t)total_q; m.per_xcd_q = (int32_t)((total_q + 7) / 8);
+    m.total_kv = (int32_t)total_kv; m.per_xcd_kv = (int32_t)((total_kv + 7) / 8);
+    const dim3 grid_q((unsigned)(m.per_xcd_q * 8)), grid_kv((unsigned)(m.per_xcd_kv * 8));
     if (causal) {
         hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, true>), grid_stats, block, 0, stream, f, st);
-        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, true>), grid_q, block, 0, stream, p);
-        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, true>), grid_kv, block, 0, stream, p);
+        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, true>), grid_q, block, 0, stream, m);
+        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, true>), grid_kv, block, 0, stream, m);
     } else {
         hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, false>), grid_stats, block, 0, stream, f, st);
-        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, false>), grid_q, block, 0, stream, p);
-        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, false>), grid_kv, block, 0, stream, p);
+        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, false>), grid_q, block, 0, stream, m);
+        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, false>), grid_kv, block, 0, stream, m);
     }
     return static_cast<int>(hipGetLastError());
 }

@@ -43,9 +43,26 @@ struct FlashBwdParams {
     int32_t N;
     int32_t H;                  // query heads
     int32_t kv_group;           // query heads per key/value head
+    int32_t n_tiles;            // 128-row tiles per sequence
+    int32_t total_q, per_xcd_q;     // dQ kernel: workgroups (B * H * n_tiles) and ceil(that / 8)
+    int32_t total_kv, per_xcd_kv;   // dK/dV kernel: workgroups (B * H_kv * n_tiles) and ceil(that / 8)
     float scale;
     float scale_log2;           // scale * log2(e)
 };
+
+// Workgroup id -> (sequence * heads + head, tile).  Both kernels are launched on a 1-D grid of 8 * per_xcd
+// workgroups.  Hardware deals consecutive ids to the 8 XCDs in turn; `logical` undoes that, so that the tiles
+// of one head (consecutive logical ids) run on one XCD and find the head's K/V (Q/dO) in its L2.
+struct BwdWork {
+    int bh, tile;
+    bool valid;
+};
+__host__ __device__ inline BwdWork bwd_work_of_block(unsigned block_id, int total, int per_xcd, int n_tiles) {
+    const int logical = (int)(block_id & 7u) * per_xcd + (int)(block_id >> 3);
+    if (logical >= total) return BwdWork{0, 0, false};
+    const int bh = logical / n_tiles;
+    return BwdWork{bh, logical - bh * n_tiles, true};
+}
 
 // Byte offset inside a tile swizzled with FlashTile::fb of the 8 bytes a lane hands to a transposing read that fetches
 // the 4 tile rows 16*g + 8*a + 4*(lane/32) + 0..3 for column quad (32*mb + 16*((lane/16)%2) + 4*(lane%4)):
@@ -95,7 +112,7 @@ __device__ inline void store_row(T* dst_row, const f32x16 (&acc)[MB], int half, 
         }
 }
 
-// grid: (query tiles of 128, query heads, sequences)
+// grid: 8 * per_xcd_q workgroups, see bwd_work_of_block
 template <typename T, int D, bool CAUSAL>
 __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dq_mfma_kernel(const FlashBwdParams p) {
     typedef FlashTile<D> TL;
@@ -113,12 +130,13 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dq_mfma_kernel(const 
     const int lane = tid & 63;
     const int col = lane & 31;
     const int half = lane >> 5;
-    const int h = blockIdx.y, b = blockIdx.z;
+    const BwdWork work = bwd_work_of_block(blockIdx.x, p.total_q, p.per_xcd_q, p.n_tiles);
+    if (!work.valid) return;
+    const int b = work.bh / p.H, h = work.bh - b * p.H;
     const int hk = h / p.kv_group;
     const int L = p.N;
     // long tiles first: under a causal mask the late query tiles walk the most keys
-    const int q_tile0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * kFlashRows;
-    if (q_tile0 >= L) return;
+    const int q_tile0 = (p.n_tiles - 1 - work.tile) * kFlashRows;
 
     const int64_t base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
     const int64_t kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
@@ -238,7 +256,7 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dq_mfma_kernel(const 
     if (qrow < L) store_row<T, MB>(static_cast<T*>(p.d_q) + base + (int64_t)qrow * sn, acc, half, p.scale);
 }
 
-// grid: (key tiles of 128, key/value heads, sequences)
+// grid: 8 * per_xcd_kv workgroups, see bwd_work_of_block
 template <typename T, int D, bool CAUSAL>
 __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const FlashBwdParams p) {
     typedef FlashTile<D> TL;
@@ -256,11 +274,13 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
     const int lane = tid & 63;
     const int col = lane & 31;
     const int half = lane >> 5;
-    const int hk = blockIdx.y, b = blockIdx.z;
+    const BwdWork work = bwd_work_of_block(blockIdx.x, p.total_kv, p.per_xcd_kv, p.n_tiles);
+    if (!work.valid) return;
+    const int heads_kv = p.H / p.kv_group;
+    const int b = work.bh / heads_kv, hk = work.bh - b * heads_kv;
     const int L = p.N;
     // under a causal mask the early key tiles see the most queries: they go first
-    const int k_tile0 = (int)blockIdx.x * kFlashRows;
-    if (k_tile0 >= L) return;
+    const int k_tile0 = work.tile * kFlashRows;
 
     const int64_t kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
     const T* const gk = static_cast<const T*>(p.k) + kv_base;
