@@ -405,3 +405,4 @@ def test_wide_groups_need_the_matrix_core_shape(emu):
     q = O.fill_normal((B, G * H_kv, d), 24, 1)
     with pytest.raises(emu.HipError):
         decode(emu, q, kp, vp, table, lens, None, B, G * H_kv, H_kv, d, P, O.F32, O.F32, 0.125)
+
