@@ -358,6 +358,32 @@ def run_calibration(steps):
     dt = (time.perf_counter() - t0) / steps
     print(json.dumps({"workload": "calibration copy", "bytes_read": n, "bytes_written": n, "launches": steps,
                       "ms_per_launch": round(dt * 1e3, 4), "GBps_read_plus_write": round(2 * n / dt / 1e9, 1)}))
+    # Two yardsticks from the vendor libraries, for context next to the roofline fractions: what a plain
+    # streaming read and a plain bf16 matrix product reach on this box (both well below the published peaks).
+    del dst
+    x = src.view(torch.float32)
+    x.zero_()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        x.sum()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    print(json.dumps({"workload": "streaming read (torch sum over 1 GiB)", "ms_per_launch": round(dt * 1e3, 4),
+                      "GBps_read": round(n / dt / 1e9, 1)}))
+    m = 8192
+    a = torch.randn((m, m), device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    b = torch.randn((m, m), device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    for _ in range(3):
+        torch.matmul(a, b)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        torch.matmul(a, b)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    print(json.dumps({"workload": "bf16 matrix product 8192^3 (torch.matmul)", "ms_per_launch": round(dt * 1e3, 4),
+                      "TFLOPs": round(2.0 * m ** 3 / dt / 1e12, 1)}))
 
 
 def main():
