@@ -29,6 +29,7 @@ struct BwdParams {
     void* d_k;
     void* d_v;
     const float* mask;          // [B,N,N] or null
+    const int32_t* cu_seqlens;  // ragged batches: sequence b owns token rows cu_seqlens[b] .. cu_seqlens[b+1]-1
     float* lse;                 // [B*H][rows_padded]
     float* delta;               // [B*H][rows_padded]
     int64_t rows_padded;
@@ -59,6 +60,20 @@ __device__ inline void stage_rows(float (*dst)[DP], const T* src, int64_t stride
     }
 }
 
+// Length of sequence b and the element offsets of its first row for head h (Q, dO, dQ) and K/V head hk.
+__device__ inline void bwd_sequence(const BwdParams& p, int b, int h, int hk, int& L, int64_t& base, int64_t& kv_base) {
+    if (p.cu_seqlens) {
+        const int s0 = p.cu_seqlens[b];
+        L = p.cu_seqlens[b + 1] - s0;
+        base = (int64_t)s0 * p.stride_n + (int64_t)h * p.stride_h;
+        kv_base = (int64_t)s0 * p.kv_stride_n + (int64_t)hk * p.kv_stride_h;
+    } else {
+        L = p.N;
+        base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+        kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
+    }
+}
+
 template <typename T, int DP>
 __global__ __launch_bounds__(kBwdRows) void flash_bwd_stats_simple_kernel(const BwdParams p) {
     __shared__ float sk[kBwdTile][DP];
@@ -66,13 +81,14 @@ __global__ __launch_bounds__(kBwdRows) void flash_bwd_stats_simple_kernel(const 
     const int tid = threadIdx.x;
     const int h = blockIdx.y, b = blockIdx.z;
     const int hk = h / p.kv_group;
-    const int L = p.N, d = p.d;
+    const int d = p.d;
+    int L;
+    int64_t base, kv_base;
+    bwd_sequence(p, b, h, hk, L, base, kv_base);
     const int row0 = blockIdx.x * kBwdRows;
     if (row0 >= L) return;
     const int n = row0 + tid;
     const bool active = n < L;
-    const int64_t base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
-    const int64_t kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
     const T* gq = static_cast<const T*>(p.q) + base;
     const T* gdo = static_cast<const T*>(p.d_out) + base;
     const T* gk = static_cast<const T*>(p.k) + kv_base;
@@ -141,13 +157,14 @@ __global__ __launch_bounds__(kBwdRows) void flash_bwd_dq_simple_kernel(const Bwd
     const int tid = threadIdx.x;
     const int h = blockIdx.y, b = blockIdx.z;
     const int hk = h / p.kv_group;
-    const int L = p.N, d = p.d;
+    const int d = p.d;
+    int L;
+    int64_t base, kv_base;
+    bwd_sequence(p, b, h, hk, L, base, kv_base);
     const int row0 = blockIdx.x * kBwdRows;
     if (row0 >= L) return;
     const int n = row0 + tid;
     const bool active = n < L;
-    const int64_t base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
-    const int64_t kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
     const T* gq = static_cast<const T*>(p.q) + base;
     const T* gdo = static_cast<const T*>(p.d_out) + base;
     const T* gk = static_cast<const T*>(p.k) + kv_base;
@@ -205,12 +222,14 @@ __global__ __launch_bounds__(kBwdRows) void flash_bwd_dkv_simple_kernel(const Bw
     __shared__ float s_delta[kBwdTile];
     const int tid = threadIdx.x;
     const int hk = blockIdx.y, b = blockIdx.z;
-    const int L = p.N, d = p.d;
+    const int d = p.d;
+    int L;
+    int64_t base0, kv_base;
+    bwd_sequence(p, b, hk * p.kv_group, hk, L, base0, kv_base);
     const int row0 = blockIdx.x * kBwdRows;
     if (row0 >= L) return;
     const int j = row0 + tid;
     const bool active = j < L;
-    const int64_t kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
     const T* gk = static_cast<const T*>(p.k) + kv_base;
     const T* gv = static_cast<const T*>(p.v) + kv_base;
 
@@ -228,7 +247,7 @@ __global__ __launch_bounds__(kBwdRows) void flash_bwd_dkv_simple_kernel(const Bw
 
     for (int g = 0; g < p.kv_group; ++g) {
         const int h = hk * p.kv_group + g;
-        const int64_t base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+        const int64_t base = base0 + (int64_t)g * p.stride_h;
         const T* gq = static_cast<const T*>(p.q) + base;
         const T* gdo = static_cast<const T*>(p.d_out) + base;
         const int64_t stat0 = ((int64_t)b * p.H + h) * p.rows_padded;
@@ -299,15 +318,16 @@ static bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr
 
 static int64_t padded_rows(int64_t N) { return (N + kFlashRows - 1) / kFlashRows * kFlashRows; }
 
-template <typename T, int D>
-static int launch_mfma_d(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool causal, float* lse2, float* delta,
-                         hipStream_t stream) {
+template <typename T, int D, bool VARLEN>
+static int launch_mfma_dv(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool causal, float* lse2, float* delta,
+                          hipStream_t stream) {
     // 1. statistics: the forward kernel with its output kept in registers
     FlashParams f{};
     f.q = p.q; f.k = p.k; f.v = p.v; f.o = nullptr;
     f.stride_b = p.stride_b; f.stride_n = p.stride_n; f.stride_h = p.stride_h;
     f.kv_stride_b = p.kv_stride_b; f.kv_stride_n = p.kv_stride_n; f.kv_stride_h = p.kv_stride_h;
     f.N = p.N; f.H = p.H; f.kv_group = p.kv_group;
+    f.cu_seqlens = p.cu_seqlens;
     f.scale_log2 = p.scale_log2;
     if (int rc = flash_plan_launch(f, B, causal)) return rc;
     const FlashStatsOut st{p.d_out, lse2, delta, p.rows_padded};
@@ -321,13 +341,13 @@ static int launch_mfma_d(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool 
     m.total_kv = (int32_t)total_kv; m.per_xcd_kv = (int32_t)((total_kv + 7) / 8);
     const dim3 grid_q((unsigned)(m.per_xcd_q * 8)), grid_kv((unsigned)(m.per_xcd_kv * 8));
     if (causal) {
-        hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, true>), grid_stats, block, 0, stream, f, st);
-        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, true>), grid_q, block, 0, stream, m);
-        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, true>), grid_kv, block, 0, stream, m);
+        hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, true, VARLEN>), grid_stats, block, 0, stream, f, st);
+        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, true, VARLEN>), grid_q, block, 0, stream, m);
+        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, true, VARLEN>), grid_kv, block, 0, stream, m);
     } else {
-        hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, false>), grid_stats, block, 0, stream, f, st);
-        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, false>), grid_q, block, 0, stream, m);
-        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, false>), grid_kv, block, 0, stream, m);
+        hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, false, VARLEN>), grid_stats, block, 0, stream, f, st);
+        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, false, VARLEN>), grid_q, block, 0, stream, m);
+        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, false, VARLEN>), grid_kv, block, 0, stream, m);
     }
     return static_cast<int>(hipGetLastError());
 }
@@ -335,8 +355,13 @@ static int launch_mfma_d(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool 
 template <typename T>
 static int launch_mfma(const FlashBwdParams& p, int64_t B, int64_t H_kv, int d, bool causal, float* lse2, float* delta,
                        hipStream_t stream) {
-    if (d == 128) return launch_mfma_d<T, 128>(p, B, H_kv, causal, lse2, delta, stream);
-    if (d == 64) return launch_mfma_d<T, 64>(p, B, H_kv, causal, lse2, delta, stream);
+    if (p.cu_seqlens) {
+        if (d == 128) return launch_mfma_dv<T, 128, true>(p, B, H_kv, causal, lse2, delta, stream);
+        if (d == 64) return launch_mfma_dv<T, 64, true>(p, B, H_kv, causal, lse2, delta, stream);
+    } else {
+        if (d == 128) return launch_mfma_dv<T, 128, false>(p, B, H_kv, causal, lse2, delta, stream);
+        if (d == 64) return launch_mfma_dv<T, 64, false>(p, B, H_kv, causal, lse2, delta, stream);
+    }
     return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
 }
 
@@ -352,10 +377,12 @@ size_t ahpc_hip_flash_bwd_workspace_bytes(int64_t B, int64_t N, int64_t H) {
     return (size_t)B * (size_t)H * (size_t)padded_rows(N) * 2 * sizeof(float);
 }
 
-int ahpc_hip_flash_bwd(const void* d_out, const void* q, const void* k, const void* v, void* d_q, void* d_k, void* d_v,
-                       int dtype, int64_t B, int64_t N, int64_t H, int64_t H_kv, int64_t d, int64_t stride_b, int64_t stride_n,
-                       int64_t stride_h, int64_t kv_stride_b, int64_t kv_stride_n, int64_t kv_stride_h, float scale, int causal,
-                       const float* mask, void* workspace, size_t workspace_bytes, void* stream) {
+// B sequences of N tokens (dense), or - cu_seqlens given - B sequences packed one after the other, the longest N tokens.
+static int flash_bwd_any(const void* d_out, const void* q, const void* k, const void* v, void* d_q, void* d_k, void* d_v,
+                         int dtype, const int32_t* cu_seqlens, int64_t B, int64_t N, int64_t H, int64_t H_kv, int64_t d,
+                         int64_t stride_b, int64_t stride_n, int64_t stride_h, int64_t kv_stride_b, int64_t kv_stride_n,
+                         int64_t kv_stride_h, float scale, int causal, const float* mask, void* workspace,
+                         size_t workspace_bytes, void* stream) {
     if (!d_out || !q || !k || !v || !d_q || !d_k || !d_v) return AHPC_ERR_NULL_POINTER;
     if (dtype < AHPC_F32 || dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
     if (B <= 0 || N <= 0 || H <= 0 || d <= 0 || H_kv <= 0) return AHPC_ERR_BAD_SHAPE;
@@ -374,6 +401,7 @@ int ahpc_hip_flash_bwd(const void* d_out, const void* q, const void* k, const vo
     p.q = q; p.k = k; p.v = v; p.d_out = d_out;
     p.d_q = d_q; p.d_k = d_k; p.d_v = d_v;
     p.mask = mask;
+    p.cu_seqlens = cu_seqlens;
     p.lse = static_cast<float*>(workspace);
     p.rows_padded = padded_rows(N);
     p.delta = p.lse + (size_t)B * (size_t)H * (size_t)p.rows_padded;
@@ -392,6 +420,7 @@ int ahpc_hip_flash_bwd(const void* d_out, const void* q, const void* k, const vo
         m.q = q; m.k = k; m.v = v; m.d_out = d_out;
         m.d_q = d_q; m.d_k = d_k; m.d_v = d_v;
         m.lse2 = p.lse; m.delta = p.delta; m.rows_padded = p.rows_padded;
+        m.cu_seqlens = cu_seqlens;
         m.stride_b = stride_b; m.stride_n = stride_n; m.stride_h = stride_h;
         m.kv_stride_b = kv_stride_b; m.kv_stride_n = kv_stride_n; m.kv_stride_h = kv_stride_h;
         m.N = (int32_t)N; m.H = (int32_t)H; m.kv_group = p.kv_group;
@@ -405,6 +434,23 @@ int ahpc_hip_flash_bwd(const void* d_out, const void* q, const void* k, const vo
         case AHPC_F16: return launch_simple<f16_t>(p, B, H_kv, st);
         default: return launch_simple<bf16_t>(p, B, H_kv, st);
     }
+}
+
+int ahpc_hip_flash_bwd(const void* d_out, const void* q, const void* k, const void* v, void* d_q, void* d_k, void* d_v,
+                       int dtype, int64_t B, int64_t N, int64_t H, int64_t H_kv, int64_t d, int64_t stride_b, int64_t stride_n,
+                       int64_t stride_h, int64_t kv_stride_b, int64_t kv_stride_n, int64_t kv_stride_h, float scale, int causal,
+                       const float* mask, void* workspace, size_t workspace_bytes, void* stream) {
+    return flash_bwd_any(d_out, q, k, v, d_q, d_k, d_v, dtype, nullptr, B, N, H, H_kv, d, stride_b, stride_n, stride_h,
+                         kv_stride_b, kv_stride_n, kv_stride_h, scale, causal, mask, workspace, workspace_bytes, stream);
+}
+
+int ahpc_hip_flash_bwd_varlen(const void* d_out, const void* q, const void* k, const void* v, void* d_q, void* d_k, void* d_v,
+                              int dtype, const int32_t* cu_seqlens, int64_t n_seqs, int64_t max_len, int64_t H, int64_t H_kv,
+                              int64_t d, int64_t stride_t, int64_t stride_h, int64_t kv_stride_t, int64_t kv_stride_h,
+                              float scale, int causal, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!cu_seqlens) return AHPC_ERR_NULL_POINTER;
+    return flash_bwd_any(d_out, q, k, v, d_q, d_k, d_v, dtype, cu_seqlens, n_seqs, max_len, H, H_kv, d, 0, stride_t, stride_h, 0,
+                         kv_stride_t, kv_stride_h, scale, causal, nullptr, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -37,10 +37,11 @@ struct FlashBwdParams {
     void* d_v;
     const float* lse2;          // [B*H][rows_padded]
     const float* delta;
+    const int32_t* cu_seqlens;  // ragged batches only
     int64_t rows_padded;
     int64_t stride_b, stride_n, stride_h;           // Q, dO, dQ
     int64_t kv_stride_b, kv_stride_n, kv_stride_h;  // K, V, dK, dV
-    int32_t N;
+    int32_t N;                  // sequence length (dense) / longest sequence (ragged)
     int32_t H;                  // query heads
     int32_t kv_group;           // query heads per key/value head
     int32_t n_tiles;            // 128-row tiles per sequence
@@ -113,7 +114,7 @@ __device__ inline void store_row(T* dst_row, const f32x16 (&acc)[MB], int half, 
 }
 
 // grid: 8 * per_xcd_q workgroups, see bwd_work_of_block
-template <typename T, int D, bool CAUSAL>
+template <typename T, int D, bool CAUSAL, bool VARLEN>
 __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dq_mfma_kernel(const FlashBwdParams p) {
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;
@@ -134,12 +135,22 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dq_mfma_kernel(const 
     if (!work.valid) return;
     const int b = work.bh / p.H, h = work.bh - b * p.H;
     const int hk = h / p.kv_group;
-    const int L = p.N;
+    int L;
+    int64_t base, kv_base;
+    if (VARLEN) {
+        const int s0 = p.cu_seqlens[b];
+        L = p.cu_seqlens[b + 1] - s0;
+        base = (int64_t)s0 * p.stride_n + (int64_t)h * p.stride_h;
+        kv_base = (int64_t)s0 * p.kv_stride_n + (int64_t)hk * p.kv_stride_h;
+    } else {
+        L = p.N;
+        base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+        kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
+    }
     // long tiles first: under a causal mask the late query tiles walk the most keys
     const int q_tile0 = (p.n_tiles - 1 - work.tile) * kFlashRows;
+    if (q_tile0 >= L) return;  // ragged batches: a sequence shorter than the longest one
 
-    const int64_t base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
-    const int64_t kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
     const T* const gq = static_cast<const T*>(p.q) + base;
     const T* const gdo = static_cast<const T*>(p.d_out) + base;
     const T* const gk = static_cast<const T*>(p.k) + kv_base;
@@ -257,7 +268,7 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dq_mfma_kernel(const 
 }
 
 // grid: 8 * per_xcd_kv workgroups, see bwd_work_of_block
-template <typename T, int D, bool CAUSAL>
+template <typename T, int D, bool CAUSAL, bool VARLEN>
 __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const FlashBwdParams p) {
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;
@@ -278,11 +289,18 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
     if (!work.valid) return;
     const int heads_kv = p.H / p.kv_group;
     const int b = work.bh / heads_kv, hk = work.bh - b * heads_kv;
-    const int L = p.N;
+    int seq0 = 0;
+    int L = p.N;
+    if (VARLEN) {
+        seq0 = p.cu_seqlens[b];
+        L = p.cu_seqlens[b + 1] - seq0;
+    }
     // under a causal mask the early key tiles see the most queries: they go first
     const int k_tile0 = work.tile * kFlashRows;
+    if (k_tile0 >= L) return;  // ragged batches: a sequence shorter than the longest one
 
-    const int64_t kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
+    const int64_t kv_base = VARLEN ? (int64_t)seq0 * p.kv_stride_n + (int64_t)hk * p.kv_stride_h
+                                   : (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
     const T* const gk = static_cast<const T*>(p.k) + kv_base;
     const T* const gv = static_cast<const T*>(p.v) + kv_base;
     const int64_t sn = p.stride_n;
@@ -327,7 +345,8 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
 
     for (int g = 0; g < p.kv_group; ++g) {
         const int h = hk * p.kv_group + g;
-        const int64_t base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+        const int64_t base = VARLEN ? (int64_t)seq0 * p.stride_n + (int64_t)h * p.stride_h
+                                    : (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
         const T* const gq = static_cast<const T*>(p.q) + base;
         const T* const gdo = static_cast<const T*>(p.d_out) + base;
         const float* const lse2 = p.lse2 + ((int64_t)b * p.H + h) * p.rows_padded;

@@ -528,9 +528,9 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
 }
 
 // The forward pass with its output kept in registers: writes the softmax statistics the backward needs.
-template <typename T, int D, bool CAUSAL>
+template <typename T, int D, bool CAUSAL, bool VARLEN>
 __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_stats_mfma_kernel(const FlashParams p, const FlashStatsOut st) {
-    flash_fwd_mfma_body<T, D, CAUSAL, false, true>(p, st);
+    flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, true>(p, st);
 }
 
 }  // namespace ahpc

@@ -63,6 +63,7 @@ SIGNATURES = {
     "ahpc_hip_flash_block_map": (_ci, [_i64, _i64, _i64, _ci, _i64, C.POINTER(_i64), _vp, _vp, _vp]),
     "ahpc_hip_flash_bwd_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "ahpc_hip_flash_bwd": (_ci, [_vp] * 7 + [_ci] + [_i64] * 11 + [_f32, _ci, _vp, _vp, _sz, _vp]),
+    "ahpc_hip_flash_bwd_varlen": (_ci, [_vp] * 7 + [_ci, _vp] + [_i64] * 9 + [_f32, _ci, _vp, _sz, _vp]),
     "ahpc_hip_flash_fwd_masked": (_ci, [_vp, _vp, _vp, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp, _vp]),
     "ahpc_hip_flash_fwd_varlen": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp]),
     "ahpc_hip_flash_fwd_varlen_gqa": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp]),
@@ -152,6 +153,13 @@ def flash_bwd(d_out, q, k, v, d_q, d_k, d_v, dtype, B, N, H, H_kv, d, strides, k
     kb, kn, kh = kv_strides
     _check(load().ahpc_hip_flash_bwd(d_out, q, k, v, d_q, d_k, d_v, dtype, B, N, H, H_kv, d, sb, sn, sh, kb, kn, kh, scale,
                                     int(causal), mask, workspace, workspace_bytes, stream), "flash_bwd")
+
+
+def flash_bwd_varlen(d_out, q, k, v, d_q, d_k, d_v, dtype, cu_seqlens, n_seqs, max_len, H, H_kv, d, stride_t, stride_h,
+                     kv_stride_t, kv_stride_h, scale, causal, workspace, workspace_bytes, stream=None):
+    _check(load().ahpc_hip_flash_bwd_varlen(d_out, q, k, v, d_q, d_k, d_v, dtype, cu_seqlens, n_seqs, max_len, H, H_kv, d,
+                                           stride_t, stride_h, kv_stride_t, kv_stride_h, scale, int(causal), workspace,
+                                           workspace_bytes, stream), "flash_bwd_varlen")
 
 
 def flash_fwd_varlen_gqa(q, k, v, o, dtype, cu_seqlens, n_seqs, max_len, H, H_kv, d, stride_t, stride_h, kv_stride_t,

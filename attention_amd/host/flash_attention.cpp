@@ -259,6 +259,52 @@ void FlashAttention::backward(const TensorShape& gos, const void* go, const Tens
     }
 }
 
+void FlashAttention::backward_varlen(const TensorShape& shape, const void* go, const void* q, const void* k, const void* v,
+                                     void* gq, void* gk, void* gv, const int32_t* cu_seqlens, size_t n_seqs) {
+    if (!impl_->configured)
+        throw AttentionException(AttentionError::INVALID_PARAMETERS, "FlashAttention not configured. Call configure() first.");
+    if (!go || !q || !k || !v || !gq || !gk || !gv || !cu_seqlens) throw AttentionException(AttentionError::INVALID_INPUT, "null pointer");
+    const size_t H = current_params_.num_heads, d = current_params_.head_dimension;
+    if (shape.dimensions.size() != 3 || shape.dimensions[1] != H || shape.dimensions[2] != d || n_seqs == 0)
+        throw AttentionException(AttentionError::INVALID_INPUT, "packed tensors must be [total_tokens, heads, head_dim]");
+    int64_t max_len = 0;
+    if (cu_seqlens[0] != 0) throw AttentionException(AttentionError::INVALID_INPUT, "cu_seqlens must start at 0");
+    for (size_t i = 0; i < n_seqs; ++i) {
+        const int64_t len = (int64_t)cu_seqlens[i + 1] - cu_seqlens[i];
+        if (len < 0) throw AttentionException(AttentionError::INVALID_INPUT, "cu_seqlens must not decrease");
+        max_len = std::max(max_len, len);
+    }
+    if ((size_t)cu_seqlens[n_seqs] != shape.dimensions[0])
+        throw AttentionException(AttentionError::INVALID_INPUT, "cu_seqlens must end at total_tokens");
+    if (max_len == 0) return;
+    void* st = impl_->stream.get();
+    const size_t Hkv = kv_heads(current_params_);
+    const size_t bytes = shape.total_bytes(), kv_bytes = bytes / H * Hkv;
+    const void* d_go = stage_in(go, bytes, impl_->ddo, st);
+    const void* d_q = stage_in(q, bytes, impl_->dq, st);
+    const void* d_k = stage_in(k, kv_bytes, impl_->dk, st);
+    const void* d_v = stage_in(v, kv_bytes, impl_->dv, st);
+    const bool gq_dev = hipsup::is_device_pointer(gq), gk_dev = hipsup::is_device_pointer(gk), gv_dev = hipsup::is_device_pointer(gv);
+    void* d_gq = gq_dev ? gq : impl_->gq.reserve(bytes);
+    void* d_gk = gk_dev ? gk : impl_->gk.reserve(kv_bytes);
+    void* d_gv = gv_dev ? gv : impl_->gv.reserve(kv_bytes);
+    void* dcu = impl_->dcu.reserve((n_seqs + 1) * sizeof(int32_t));
+    check(ahpc_hip_memcpy_h2d(dcu, cu_seqlens, (n_seqs + 1) * sizeof(int32_t), st), "copy cu_seqlens");
+    const size_t ws_bytes = ahpc_hip_flash_bwd_workspace_bytes((int64_t)n_seqs, max_len, (int64_t)H);
+    void* ws = impl_->ws.reserve(ws_bytes);
+    float scale = impl_->cfg.softmax_scale > 0.0f ? impl_->cfg.softmax_scale : current_params_.scale_factor;
+    if (!(scale > 0.0f)) scale = 1.0f / std::sqrt(static_cast<float>(d));
+    const int causal = (current_params_.causal_mask || impl_->cfg.use_causal_mask) ? 1 : 0;
+    check(ahpc_hip_flash_bwd_varlen(d_go, d_q, d_k, d_v, d_gq, d_gk, d_gv, hipsup::dtype_code(shape.data_type),
+                                    static_cast<const int32_t*>(dcu), (int64_t)n_seqs, max_len, (int64_t)H, (int64_t)Hkv,
+                                    (int64_t)d, (int64_t)(H * d), (int64_t)d, (int64_t)(Hkv * d), (int64_t)d, scale, causal, ws,
+                                    ws_bytes, st), "flash backward (ragged)");
+    if (!gq_dev) check(ahpc_hip_memcpy_d2h(gq, d_gq, bytes, st), "copy from device");
+    if (!gk_dev) check(ahpc_hip_memcpy_d2h(gk, d_gk, kv_bytes, st), "copy from device");
+    if (!gv_dev) check(ahpc_hip_memcpy_d2h(gv, d_gv, kv_bytes, st), "copy from device");
+    impl_->stream.sync();
+}
+
 // Device bytes this object stages when every tensor arrives in host memory (nothing when they are
 // already on the device).  Reference: FlashAttention::get_workspace_size,
 // src/algorithms/flash_attention.cpp:176-199, whose fp32 conversion buffers have no counterpart here.

@@ -182,6 +182,18 @@ int ahpc_hip_flash_bwd(const void* d_out, const void* q, const void* k, const vo
                        float scale, int causal, const float* mask,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same for a ragged batch packed as in ahpc_hip_flash_fwd_varlen_gqa: token t, head h, element e of Q, dO and
+ * dQ is at t*stride_t + h*stride_h + e (K, V, dK, dV: kv_stride_t, kv_stride_h); sequence i owns tokens
+ * cu_seqlens[i] .. cu_seqlens[i+1]-1 (n_seqs+1 device integers) and max_len is the longest sequence.
+ * Workspace: ahpc_hip_flash_bwd_workspace_bytes(n_seqs, max_len, H).  No counterpart in the reference. */
+int ahpc_hip_flash_bwd_varlen(const void* d_out, const void* q, const void* k, const void* v,
+                              void* d_q, void* d_k, void* d_v, int dtype,
+                              const int32_t* cu_seqlens, int64_t n_seqs, int64_t max_len,
+                              int64_t H, int64_t H_kv, int64_t d,
+                              int64_t stride_t, int64_t stride_h, int64_t kv_stride_t, int64_t kv_stride_h,
+                              float scale, int causal,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- paged KV pool ---------------------------------------------------------------------------
  * Pool layout: K and V are separate slabs  [page][slot 0..P-1][head][d]  (the layout
  * update_kv_cache_kernel writes, src/backends/cuda/cuda_kernels.cu:547-556).

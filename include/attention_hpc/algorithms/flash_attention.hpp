@@ -81,6 +81,12 @@ public:
                   const TensorShape& grad_key_shape, void* grad_key_data, const TensorShape& grad_value_shape,
                   void* grad_value_data, const void* attention_mask = nullptr) override;
 
+    // Gradients for a ragged batch packed as in forward_varlen: grad_output, query, grad_query are
+    // [total_tokens, num_heads, head_dim]; key, value, grad_key, grad_value [total_tokens, key_value_heads, head_dim].
+    void backward_varlen(const TensorShape& packed_shape, const void* grad_output_data, const void* query_data,
+                         const void* key_data, const void* value_data, void* grad_query_data, void* grad_key_data,
+                         void* grad_value_data, const int32_t* cu_seqlens, size_t n_seqs);
+
     size_t get_workspace_size(const AttentionParams& params) const override;
     void set_workspace(void* workspace_ptr, size_t workspace_size) override;
 

@@ -252,6 +252,30 @@ CASE(Flash_BackwardCausalGroupedHalf, true) {  // bf16 tensors, causal, 4 query 
                   AttentionError::INVALID_INPUT);
 }
 
+CASE(Flash_BackwardRaggedBatch, true) {  // packed sequences: each one's gradients equal the dense oracle's on it
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    p.causal_mask = true;
+    fa.configure(p);
+    const size_t H = p.num_heads, d = p.head_dimension;
+    const std::vector<int32_t> cu = {0, 5, 5, 140, 141};  // lengths 5, 0, 135, 1
+    const size_t T = 141, n = T * H * d;
+    auto q = uniform(n, 13, 1), k = uniform(n, 13, 2), v = uniform(n, 13, 3), go = uniform(n, 13, 7);
+    std::vector<float> gq(n, 9.0f), gk(n, 9.0f), gv(n, 9.0f);
+    const TensorShape s({T, H, d}, DataType::FLOAT32);
+    fa.backward_varlen(s, go.data(), q.data(), k.data(), v.data(), gq.data(), gk.data(), gv.data(), cu.data(), cu.size() - 1);
+    for (size_t i = 0; i + 1 < cu.size(); ++i) {
+        const size_t a = (size_t)cu[i] * H * d, len = (size_t)(cu[i + 1] - cu[i]), m = len * H * d;
+        if (!len) continue;
+        std::vector<float> wq(m), wk(m), wv(m);
+        ahpc_oracle_attention_backward(q.data() + a, k.data() + a, v.data() + a, go.data() + a, wq.data(), wk.data(), wv.data(), 1,
+                                       len, H, H, d, p.scale_factor, 1, nullptr, 4);
+        EXPECT(max_abs_diff(std::vector<float>(gq.begin() + a, gq.begin() + a + m), wq) <= 1e-4f);
+        EXPECT(max_abs_diff(std::vector<float>(gk.begin() + a, gk.begin() + a + m), wk) <= 1e-4f);
+        EXPECT(max_abs_diff(std::vector<float>(gv.begin() + a, gv.begin() + a + m), wv) <= 1e-4f);
+    }
+}
+
 CASE(Flash_AttentionMask, true) {  // :483-582: mask [B,N,N] float, 0 = masked
     FlashAttention fa;
     AttentionParams p = fixture_params();

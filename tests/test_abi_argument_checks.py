@@ -58,6 +58,10 @@ def test_flash_backward_argument_checks(lib):
     assert bwd(ws_bytes=need - 1) == WORKSPACE
     assert bwd(ws=P + 4) == BAD_ALIGNMENT
     assert lib.ahpc_hip_flash_bwd_workspace_bytes(0, 16, 4) == 0
+    # ragged: cu_seqlens is required, the rest is checked like the dense call
+    rag = lambda cu, H=4, Hkv=2: lib.ahpc_hip_flash_bwd_varlen(P, P, P, P, P, P, P, F16, cu, 2, 16, H, Hkv, 64, H * 64, 64, Hkv * 64, 64,
+                                                                0.0, 1, P, 1 << 20, None)
+    assert rag(None) == NULL_POINTER and rag(P, H=6, Hkv=4) == BAD_SHAPE
 
 
 def decode(lib, q=P, o=P, kp=P, vp=P, table=P, lens=P, qo=F16, pool=F16, B=2, H=8, Hkv=8, d=128, Pg=16, max_pages=4, max_len=64,

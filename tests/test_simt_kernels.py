@@ -406,3 +406,30 @@ def test_wide_groups_need_the_matrix_core_shape(emu):
     with pytest.raises(emu.HipError):
         decode(emu, q, kp, vp, table, lens, None, B, G * H_kv, H_kv, d, P, O.F32, O.F32, 0.125)
 
+
+@pytest.mark.parametrize("dtype,d,H,H_kv", [(O.F16, 64, 2, 2), (O.BF16, 128, 4, 2), (O.F32, 32, 2, 1)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_backward_ragged_batch(emu, dtype, d, H, H_kv, causal):
+    """Packed sequences of different lengths: every sequence's gradients equal the dense oracle's on that sequence."""
+    lens = np.array([1, 130, 64, 257], np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    q = O.round_to(O.fill_normal((T, H, d), 37, 1), dtype)
+    k = O.round_to(O.fill_normal((T, H_kv, d), 37, 2), dtype)
+    v = O.round_to(O.fill_normal((T, H_kv, d), 37, 3), dtype)
+    do = O.round_to(O.fill_normal((T, H, d), 37, 7), dtype)
+    tq, tk, tv, tdo = dev(q, dtype), dev(k, dtype), dev(v, dtype), dev(do, dtype)
+    gq = S.guarded(S.empty_storage((T, H, d), dtype))
+    gk = S.guarded(S.empty_storage((T, H_kv, d), dtype))
+    gv = S.guarded(S.empty_storage((T, H_kv, d), dtype))
+    dcu = S.guarded(cu)
+    ws_bytes = emu.flash_bwd_workspace_bytes(len(lens), int(lens.max()), H)
+    ws = S.guarded(np.full(ws_bytes // 4, np.nan, np.float32))
+    scale = 1.0 / np.sqrt(d)
+    emu.flash_bwd_varlen(S.ptr(tdo), S.ptr(tq), S.ptr(tk), S.ptr(tv), S.ptr(gq), S.ptr(gk), S.ptr(gv), dtype, S.ptr(dcu),
+                         len(lens), int(lens.max()), H, H_kv, d, H * d, d, H_kv * d, d, scale, causal, S.ptr(ws), ws_bytes)
+    got = tuple(S.from_storage(x, dtype) for x in (gq, gk, gv))
+    for i, n in enumerate(lens):
+        a, b = cu[i], cu[i + 1]
+        want = O.attention_backward(q[a:b][None], k[a:b][None], v[a:b][None], do[a:b][None], 1, int(n), H, d, scale, causal, H_kv)
+        check_gradients(tuple(g[a:b][None] for g in got), want, dtype)

@@ -154,3 +154,33 @@ def test_bad_arguments_are_rejected_without_launch(gpu):
     with pytest.raises(gpu.HipError):
         gpu.flash_bwd(p, p, p, p, 0, p, p, **ok)
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dtype,d,H,H_kv", [(O.F16, 64, 4, 4), (O.BF16, 128, 4, 2), (O.F32, 32, 2, 1)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_ragged_batch(gpu, dtype, d, H, H_kv, causal):
+    """Packed sequences of different lengths: every sequence's gradients equal the dense oracle's on that sequence."""
+    import torch
+    from gpu_util import to_dev, to_host, stream_ptr, dev_i32
+    lens = np.array([5, 130, 1, 64, 257, 128], np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    q = O.round_to(O.fill_normal((T, H, d), 37, 1), dtype)
+    k = O.round_to(O.fill_normal((T, H_kv, d), 37, 2), dtype)
+    v = O.round_to(O.fill_normal((T, H_kv, d), 37, 3), dtype)
+    do = O.round_to(O.fill_normal((T, H, d), 37, 7), dtype)
+    tq, tk, tv, tdo = (to_dev(x, dtype) for x in (q, k, v, do))
+    gq, gk, gv = torch.full_like(tq, float("nan")), torch.full_like(tk, float("nan")), torch.full_like(tv, float("nan"))
+    dcu = dev_i32(cu)
+    ws_bytes = gpu.flash_bwd_workspace_bytes(len(lens), int(lens.max()), H)
+    ws = torch.full((ws_bytes // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    scale = 1.0 / np.sqrt(d)
+    gpu.flash_bwd_varlen(tdo.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), gq.data_ptr(), gk.data_ptr(),
+                         gv.data_ptr(), dtype, dcu.data_ptr(), len(lens), int(lens.max()), H, H_kv, d, H * d, d, H_kv * d, d,
+                         scale, causal, ws.data_ptr(), ws_bytes, stream_ptr())
+    torch.cuda.synchronize()
+    got = (to_host(gq), to_host(gk), to_host(gv))
+    for i, n in enumerate(lens):
+        a, b = cu[i], cu[i + 1]
+        want = O.attention_backward(q[a:b][None], k[a:b][None], v[a:b][None], do[a:b][None], 1, int(n), H, d, scale, causal, H_kv)
+        check(tuple(g[a:b][None] for g in got), want, dtype)
