@@ -390,8 +390,12 @@ def test_decode_grouped_heads_matrix_core_kernel(emu, G, dtype, d, monkeypatch):
     rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
     want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
     S.lds_stats(reset=True)
-    for chunk, qo in ((0, dtype), (48, O.F32), (16, dtype)):
-        got = decode(emu, q, kp, vp, table, lens, None, B, H, H_kv, d, P, dtype, qo, scale, chunk)
+    for chunk, qo, dma_late in ((0, dtype, False), (48, O.F32, True), (16, dtype, False), (0, dtype, True)):
+        S.configure(dma_late, seed=G + chunk)
+        try:
+            got = decode(emu, q, kp, vp, table, lens, None, B, H, H_kv, d, P, dtype, qo, scale, chunk)
+        finally:
+            S.configure(False, 1)
         assert np.all(got[3] == 0.0)
         assert np.abs(got - want).max() <= 2e-2, (chunk, qo)
     reads, read_conflicts, tr, tr_conflicts = S.lds_stats(reset=True)
