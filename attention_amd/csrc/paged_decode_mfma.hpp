@@ -144,15 +144,20 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_kernel(const DecodeParam
             s[r] = off < lim ? s[r] : -INFINITY;
             mx = fmaxf(mx, s[r]);
         }
-        mx = halves_max(mx);  // a tile holds at least one token, so this is finite
-        const float m_new = fmaxf(m_run, mx);
-        const float alpha = fast_exp2(m_run - m_new);  // first tile: exp2(-inf) = 0
-        m_run = m_new;
-        l_run *= alpha;
+        // The reference maximum is raised only when a score tops it by more than 2^8 (and on the first tile):
+        // p stays in (0, 256], O/l is unchanged, and the accumulators are rescaled rarely.
+        if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.0f) != 0) {  // always on the first tile: m_run is -inf there
+            mx = halves_max(mx);  // a tile holds at least one token, so this is finite
+            const float m_new = fmaxf(m_run, mx);
+            const float alpha = fast_exp2(m_run - m_new);  // first tile: exp2(-inf) = 0
+            m_run = m_new;
+            l_run *= alpha;
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
+            for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[mb][r] *= alpha;
+                for (int r = 0; r < 16; ++r) oacc[mb][r] *= alpha;
+        }
+        const float m_new = m_run;
         float sum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
