@@ -140,6 +140,14 @@ __device__ inline void dma_instr(const void* base, unsigned nrec, int off, unsig
 #endif
 }
 
+// The 4-byte form of the same instruction: lane i's dword lands at lds + 4*i.
+__device__ inline void dma_dword(const void* base, unsigned nrec, int off, unsigned char* lds) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, nrec, 0x00020000);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (AHPC_LDS void*)lds, 4, off, 0, 0, 0);
+#endif
+}
+
 // Workgroup id -> work.  Hardware deals consecutive workgroup ids to the 8 XCDs in turn; `logical` undoes
 // that, so that consecutive logical ids run on the same XCD and share its L2.  A head owns `per_head`
 // consecutive logical ids (its query tiles, or pairs of them), late (long) tiles first.  With
@@ -199,7 +207,10 @@ struct FlashStatsOut {
     int64_t rows_padded;
 };
 
-template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS>
+// TOUCH: while tile t is computed and tile t+1 streams into LDS, one dword of every 128-byte line of tile
+// t+2 is requested as well (into an LDS area nobody reads), so that what misses the L2 is on its way a tile
+// earlier than the stream needs it.  The wait at the end of a step then leaves that one request outstanding.
+template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS, bool TOUCH = false>
 __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const FlashStatsOut& st) {
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;  // k-steps of the first product
@@ -263,6 +274,21 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
         const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
         dma_tile<D>(gk + (int64_t)k0 * skv, nrec, dma_off_k, dst_k, wave_u);
         dma_tile<D>(gv + (int64_t)k0 * skv, nrec, dma_off_v, dst_v, wave_u);
+    };
+
+    // Requests one dword of each 128-byte line of the K and V tiles that start at key k0 (TOUCH only).
+    auto touch_tile = [&](int k0) {
+        if constexpr (TOUCH) {
+            __shared__ __attribute__((aligned(1024))) unsigned char lds_touch[1024];
+            constexpr int kLinesPerRow = RB / 128;                    // 2 (d = 128) or 1 (d = 64)
+            constexpr int kLines = kFlashKeys * kLinesPerRow;         // lines per tile
+            const int i = tid % kLines;                               // the line this thread asks for
+            const bool is_v = (tid / kLines) & 1;                     // first group of threads: K, second: V
+            const int64_t rem = (int64_t)(L - k0 - 1) * skv * 2 + 2 * D;
+            const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
+            const int off = (int)((i / kLinesPerRow) * skv * 2) + (i % kLinesPerRow) * 128;
+            dma_dword((is_v ? gv : gk) + (int64_t)k0 * skv, nrec, off, lds_touch + wave_u * 256);
+        }
     };
 
     // ---- LDS operand addresses (byte offsets inside a tile) -------------------------------------
@@ -440,10 +466,15 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
             const int k0 = t * kFlashKeys;
             const bool more = t + 1 < n_tiles;
             if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
+            const bool touched = TOUCH && t + 2 < n_tiles;
+            if (touched) touch_tile(k0 + 2 * kFlashKeys);
             // a wavefront whose queries all precede this tile has nothing to add
             if (!(CAUSAL && k0 > qw + 31)) compute_tile(cur_k, cur_v, k0);
             if (more) {
-                __builtin_amdgcn_s_waitcnt(0);  // this wave's part of the next tile has landed
+                // this wave's part of the next tile has landed (requests complete in order: the one request for
+                // the tile after it, issued last, may still be under way)
+                if (touched) __builtin_amdgcn_s_waitcnt(1);
+                else __builtin_amdgcn_s_waitcnt(0);
                 __syncthreads();                // everyone's has, and everyone is done with the current one
             }
         };
@@ -525,6 +556,12 @@ inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal) {
 template <typename T, int D, bool CAUSAL, bool VARLEN>
 __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const FlashParams p) {
     flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, false>(p, FlashStatsOut{});
+}
+
+// The same kernel with the L2 warm-up described at flash_fwd_mfma_body (AHPC_FLASH_L2_PREFETCH=1).
+template <typename T, int D, bool CAUSAL, bool VARLEN>
+__global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_touch_kernel(const FlashParams p) {
+    flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, false, true>(p, FlashStatsOut{});
 }
 
 // The forward pass with its output kept in registers: writes the softmax statistics the backward needs.

@@ -37,6 +37,7 @@ enum Kind : int { K_NONE = 0, K_MFMA, K_TR, K_SWAP, K_BALLOT, K_RFL, K_RL, K_DPP
 struct PendingDma {
     unsigned char* dst;
     const unsigned char* src;  // null: zeros
+    int bytes;
 };
 
 struct Wave {
@@ -146,12 +147,16 @@ void fail(const std::string& what) {
     }
 }
 
-void flush_dma(Fiber* f) {
-    for (const PendingDma& d : f->dma) {
-        if (d.src) std::memcpy(d.dst, d.src, 16);
-        else std::memset(d.dst, 0, 16);
+// Lands this lane's outstanding direct-to-LDS loads, oldest first, until at most `leave` are outstanding
+// (loads complete in the order they were issued).
+void flush_dma(Fiber* f, size_t leave = 0) {
+    size_t n = f->dma.size() > leave ? f->dma.size() - leave : 0;
+    for (size_t i = 0; i < n; ++i) {
+        const PendingDma& d = f->dma[i];
+        if (d.src) std::memcpy(d.dst, d.src, (size_t)d.bytes);
+        else std::memset(d.dst, 0, (size_t)d.bytes);
     }
-    f->dma.clear();
+    f->dma.erase(f->dma.begin(), f->dma.begin() + (long)n);
 }
 
 void wait_until(const int* counter, const int* target) {
@@ -431,14 +436,14 @@ int shfl_xor_bits(int x, int mask, int width) {
 // not completely inside the descriptor reads as zeros.
 void buffer_load_lds(BufferRsrc r, void* lds_base, int size, int voffset, int soffset, int imm, int aux) {
     (void)aux;
-    if (size != 16) fail("buffer_load_lds: only 16-byte loads are modelled");
+    if (size != 16 && size != 4) fail("buffer_load_lds: only 4- and 16-byte loads are modelled");
     Fiber* f = g_cur;
-    unsigned char* dst = static_cast<unsigned char*>(lds_base) + imm + 16 * f->lane;
-    if (!in_lds(dst, 16)) fail("buffer_load_lds writes outside the workgroup's LDS");
+    unsigned char* dst = static_cast<unsigned char*>(lds_base) + imm + size * f->lane;
+    if (!in_lds(dst, (size_t)size)) fail("buffer_load_lds writes outside the workgroup's LDS");
     const uint64_t off = (uint64_t)(uint32_t)voffset + (uint64_t)(uint32_t)soffset + (uint64_t)(uint32_t)imm;
     if (voffset < 0) fail("buffer_load_lds: negative lane offset");
-    const bool inside = off + 16 <= (uint64_t)r.num_records;
-    PendingDma d{dst, inside ? r.base + off : nullptr};
+    const bool inside = off + (uint64_t)size <= (uint64_t)r.num_records;
+    PendingDma d{dst, inside ? r.base + off : nullptr, size};
     if (g_dma_late) f->dma.push_back(d);
     else {
         f->dma.push_back(d);
@@ -446,9 +451,11 @@ void buffer_load_lds(BufferRsrc r, void* lds_base, int size, int voffset, int so
     }
 }
 
+// s_waitcnt with the gfx9 encoding: vmcnt in bits 3:0 and 15:14; the other counters are not modelled
+// (LDS and scalar accesses are synchronous here).
 void waitcnt(int imm) {
-    if (imm != 0) fail("s_waitcnt: only the wait-for-everything form is modelled");
-    if (g_cur) flush_dma(g_cur);
+    const int vmcnt = (imm & 0xF) | (((imm >> 14) & 3) << 4);
+    if (g_cur) flush_dma(g_cur, (size_t)vmcnt);
 }
 
 void launch(dim3 grid, dim3 block, const std::function<void()>& body) {
