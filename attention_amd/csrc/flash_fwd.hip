@@ -154,12 +154,21 @@ template <typename T, int D, bool VARLEN>
 static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
     if (int rc = flash_plan_launch(p, B, causal)) return rc;
     dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
-    // AHPC_FLASH_L2_PREFETCH=1: the variant that asks for the tile after next a step early (tuning knob, same results)
-    const char* touch = std::getenv("AHPC_FLASH_L2_PREFETCH");
-    if (touch && std::atoi(touch) == 1) {
-        if (causal) hipLaunchKernelGGL((flash_fwd_mfma_touch_kernel<T, D, true, VARLEN>), grid, block, 0, stream, p);
-        else hipLaunchKernelGGL((flash_fwd_mfma_touch_kernel<T, D, false, VARLEN>), grid, block, 0, stream, p);
-        return static_cast<int>(hipGetLastError());
+    // AHPC_FLASH_VARIANT = 1 (L2 warm-up), 2 (issue priority) or 3 (both): tuning variants of the dense kernel
+    // that compute the same results (see flash_fwd_mfma_body)
+    if constexpr (!VARLEN) {
+        const char* e = std::getenv("AHPC_FLASH_VARIANT");
+        const int variant = e ? std::atoi(e) : 0;
+#define AHPC_LAUNCH_VARIANT(V)                                                                                        \
+    if (variant == V) {                                                                                               \
+        if (causal) hipLaunchKernelGGL((flash_fwd_mfma_variant_kernel<T, D, true, V>), grid, block, 0, stream, p);   \
+        else hipLaunchKernelGGL((flash_fwd_mfma_variant_kernel<T, D, false, V>), grid, block, 0, stream, p);         \
+        return static_cast<int>(hipGetLastError());                                                                   \
+    }
+        AHPC_LAUNCH_VARIANT(1)
+        AHPC_LAUNCH_VARIANT(2)
+        AHPC_LAUNCH_VARIANT(3)
+#undef AHPC_LAUNCH_VARIANT
     }
     if (causal) hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, true, VARLEN>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, false, VARLEN>), grid, block, 0, stream, p);

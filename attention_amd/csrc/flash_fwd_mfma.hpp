@@ -207,11 +207,21 @@ struct FlashStatsOut {
     int64_t rows_padded;
 };
 
-// TOUCH: while tile t is computed and tile t+1 streams into LDS, one dword of every 128-byte line of tile
-// t+2 is requested as well (into an LDS area nobody reads), so that what misses the L2 is on its way a tile
-// earlier than the stream needs it.  The wait at the end of a step then leaves that one request outstanding.
-template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS, bool TOUCH = false>
+// VARIANT: tuning variants of the same computation, compiled as separate kernels and chosen by the launcher.
+//   kVariantTouch     while tile t is computed and tile t+1 streams into LDS, one dword of every 128-byte line
+//                     of tile t+2 is requested as well (into an LDS area nobody reads), so that what misses the
+//                     L2 is on its way a tile earlier than the stream needs it.  The wait at the end of a step
+//                     then leaves that one request outstanding.
+//   kVariantPriority  a wavefront raises its issue priority (s_setprio) while it feeds the matrix cores and
+//                     lowers it for the stretch of pure softmax arithmetic, so that of the two wavefronts that
+//                     share a SIMD the one with matrix instructions ready goes first.
+constexpr int kVariantTouch = 1;
+constexpr int kVariantPriority = 2;
+
+template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS, int VARIANT = 0>
 __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const FlashStatsOut& st) {
+    constexpr bool TOUCH = (VARIANT & kVariantTouch) != 0;
+    constexpr bool PRIORITY = (VARIANT & kVariantPriority) != 0;
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;  // k-steps of the first product
     constexpr int MB = D / 32;  // 32-row blocks of O^T
@@ -357,6 +367,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
             // ---- S^T = c*K Q^T - m  (log2 units).  The two 32-key blocks alternate, kAhead operand
             //      pairs are requested before the first product and one more after every two products.
             f32x16 s[2];
+            if constexpr (PRIORITY) __builtin_amdgcn_s_setprio(1);
             {
                 u32x4 a0[KS], a1[KS];
 #pragma unroll
@@ -389,6 +400,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                 vf[0][mb][1] = TrRead<T>::load(tile_v + v_off[mb] + 8 * RB);
             }
 
+            if constexpr (PRIORITY) __builtin_amdgcn_s_setprio(0);
             const bool need_mask = (k0 + kFlashKeys > L) || (CAUSAL && (k0 + kFlashKeys - 1 > qw));
             if (need_mask) {
                 // key = k0 + 4*half + off(kb, r); visible iff key <= min(qrow, L-1)  <=>  off <= lim
@@ -442,6 +454,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                 }
             };
             make_pb(0);
+            if constexpr (PRIORITY) __builtin_amdgcn_s_setprio(1);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
@@ -459,6 +472,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if constexpr (PRIORITY) __builtin_amdgcn_s_setprio(0);
             l_run += sum;
         };
 
@@ -558,10 +572,10 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
     flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, false>(p, FlashStatsOut{});
 }
 
-// The same kernel with the L2 warm-up described at flash_fwd_mfma_body (AHPC_FLASH_L2_PREFETCH=1).
-template <typename T, int D, bool CAUSAL, bool VARLEN>
-__global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_touch_kernel(const FlashParams p) {
-    flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, false, true>(p, FlashStatsOut{});
+// The tuning variants described at flash_fwd_mfma_body (dense batches; AHPC_FLASH_VARIANT = 1, 2 or 3).
+template <typename T, int D, bool CAUSAL, int VARIANT>
+__global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_variant_kernel(const FlashParams p) {
+    flash_fwd_mfma_body<T, D, CAUSAL, false, false, VARIANT>(p, FlashStatsOut{});
 }
 
 // The forward pass with its output kept in registers: writes the softmax statistics the backward needs.
