@@ -550,7 +550,10 @@ inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal) {
     if (total > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
     // Causal launches with enough workgroups to fill the chip twice over pair a late query tile with an
     // early one, so that every workgroup walks the same number of key tiles.
-    p.paired = (causal && p.n_qtiles >= 2 && total >= 1024) ? 1 : 0;
+    // (AHPC_FLASH_PAIR_MIN moves the threshold; 1024 tiles = two rounds of two workgroups on each of 256 CUs.)
+    int64_t pair_min = 1024;
+    if (const char* e = std::getenv("AHPC_FLASH_PAIR_MIN")) pair_min = std::atoi(e) > 0 ? std::atoi(e) : pair_min;
+    p.paired = (causal && p.n_qtiles >= 2 && total >= pair_min) ? 1 : 0;
     if (p.paired) total = B * p.H * (int64_t)((p.n_qtiles + 1) / 2);
     p.total_blocks = (int32_t)total;
     p.blocks_per_xcd = (int32_t)((total + 7) / 8);
