@@ -6,6 +6,7 @@
 
 #include "ahpc_device.hpp"
 #include "flash_fwd_mfma.hpp"
+#include "flash_fwd_wide.hpp"
 
 namespace ahpc {
 
@@ -152,6 +153,18 @@ static int dispatch_simple(int dtype, const SimpleParams& p, int64_t B, hipStrea
 // ---------------------------------------------------------------------------------------------
 template <typename T, int D, bool VARLEN>
 static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
+    // AHPC_FLASH_WIDE=1: the experimental variant in which a wavefront owns 64 query rows (flash_fwd_wide.hpp; dense
+    // batches only).  Same results; not the default until it has been timed.
+    if constexpr (!VARLEN) {
+        const char* wide = std::getenv("AHPC_FLASH_WIDE");
+        if (wide && std::atoi(wide) == 1) {
+            if (int rc = flash_plan_launch(p, B, causal, kWideRows)) return rc;
+            dim3 wgrid((unsigned)(p.blocks_per_xcd * 8)), wblock(kFlashThreads);
+            if (causal) hipLaunchKernelGGL((flash_fwd_wide_kernel<T, D, true, false>), wgrid, wblock, 0, stream, p);
+            else hipLaunchKernelGGL((flash_fwd_wide_kernel<T, D, false, false>), wgrid, wblock, 0, stream, p);
+            return static_cast<int>(hipGetLastError());
+        }
+    }
     if (int rc = flash_plan_launch(p, B, causal)) return rc;
     dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
     // AHPC_FLASH_VARIANT = 1 (L2 warm-up), 2 (issue priority) or 3 (both): tuning variants of the dense kernel

@@ -544,8 +544,8 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
 // Fills the launch geometry of the MFMA kernel (query tiles, pairing, workgroup count, interleaving of
 // heads) from N, H and the batch size already in `p`.  Shared by the launcher and by the host-side dump
 // of the workgroup map.
-inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal) {
-    p.n_qtiles = (p.N + kFlashRows - 1) / kFlashRows;
+inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal, int rows_per_workgroup = kFlashRows) {
+    p.n_qtiles = (p.N + rows_per_workgroup - 1) / rows_per_workgroup;
     int64_t total = B * p.H * (int64_t)p.n_qtiles;
     if (total > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
     // Causal launches with enough workgroups to fill the chip twice over pair a late query tile with an
@@ -553,7 +553,7 @@ inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal) {
     // (AHPC_FLASH_PAIR_MIN moves the threshold; 1024 tiles = two rounds of two workgroups on each of 256 CUs.)
     int64_t pair_min = 1024;
     if (const char* e = std::getenv("AHPC_FLASH_PAIR_MIN")) pair_min = std::atoi(e) > 0 ? std::atoi(e) : pair_min;
-    p.paired = (causal && p.n_qtiles >= 2 && total >= pair_min) ? 1 : 0;
+    p.paired = (causal && p.n_qtiles >= 2 && total * rows_per_workgroup >= pair_min * kFlashRows) ? 1 : 0;
     if (p.paired) total = B * p.H * (int64_t)((p.n_qtiles + 1) / 2);
     p.total_blocks = (int32_t)total;
     p.blocks_per_xcd = (int32_t)((total + 7) / 8);

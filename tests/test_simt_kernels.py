@@ -460,3 +460,61 @@ def test_forward_tuning_variants_compute_the_same(emu, dtype, N, d, causal, dma_
         S.configure(False, 1)
     assert np.array_equal(plain, warmed)
     assert np.abs(plain - O.attention(q, k, v, B, N, H, d, 0.1, causal)).max() <= TOL[dtype]
+
+# ---- forward, wide variant (a wavefront owns 64 query rows; AHPC_FLASH_WIDE=1) ------------------------------
+@pytest.mark.parametrize("dma_late", [False, True])
+@pytest.mark.parametrize("dtype", [O.BF16, O.F16])
+@pytest.mark.parametrize("N,d,causal", [(64, 128, False), (129, 128, True), (300, 64, True), (520, 64, False), (1, 128, True),
+                                        (700, 128, True)])
+def test_wide_forward_kernel(emu, dtype, N, d, causal, dma_late, monkeypatch):
+    monkeypatch.setenv("AHPC_FLASH_WIDE", "1")
+    B, H = 2, 2
+    q, k, v = qkv((B, N, H, d), 19, dtype)
+    scale = 1.0 / np.sqrt(d)
+    S.configure(dma_late, seed=N + d)
+    S.lds_stats(reset=True)
+    try:
+        got = flash(emu, q, k, v, dtype, B, N, H, d, scale, causal, front=dma_late)
+    finally:
+        S.configure(False, 1)
+    assert np.isfinite(got).all()
+    assert np.abs(got - O.attention(q, k, v, B, N, H, d, scale, causal)).max() <= TOL[dtype]
+    reads, read_conflicts, tr, tr_conflicts = S.lds_stats(reset=True)
+    assert read_conflicts == 0 and tr_conflicts == 0
+
+
+@pytest.mark.parametrize("dtype", [O.BF16, O.F16])
+@pytest.mark.parametrize("causal", [False, True])
+def test_wide_forward_kernel_scores_that_outgrow_the_first_block(emu, dtype, causal, monkeypatch):
+    """Keys whose scores top those of the first key block by far more than 2^15: the fast pass gives up and the
+    workgroup repeats the query tile with the rescaling pass.  Only some wavefronts are affected."""
+    monkeypatch.setenv("AHPC_FLASH_WIDE", "1")
+    B, N, H, d = 1, 400, 2, 128
+    q, k, v = qkv((B, N, H, d), 26, dtype, sigma=0.25)
+    q[:, 100:130, 0, 0] = 1.0          # these queries (second wavefront of the first tile) ...
+    k[:, 77, 0, 0] = 80.0              # ... see one key with a logit of 80 (scale 1): the output is that V row
+    k[:, 333, 1, :] *= 30.0            # head 1: a late key with large scores of both signs
+    q, k = O.round_to(q, dtype), O.round_to(k, dtype)
+    got = flash(emu, q, k, v, dtype, B, N, H, d, 1.0, causal)
+    want = O.attention(q, k, v, B, N, H, d, 1.0, causal)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= TOL[dtype]
+    assert np.abs(got[0, 100:130, 0] - v[0, 77, 0]).max() <= 1e-2
+
+
+def test_wide_forward_kernel_grouped_and_paired(emu, monkeypatch):
+    monkeypatch.setenv("AHPC_FLASH_WIDE", "1")
+    # grouped heads
+    B, N, H, H_kv, d = 1, 300, 4, 2, 128
+    q = O.round_to(O.fill_normal((B, N, H, d), 21, 1), O.BF16)
+    k = O.round_to(O.fill_normal((B, N, H_kv, d), 21, 2), O.BF16)
+    v = O.round_to(O.fill_normal((B, N, H_kv, d), 21, 3), O.BF16)
+    got = flash(emu, q, k, v, O.BF16, B, N, H, d, 0.1, True, H_kv=H_kv)
+    want = O.attention(q, np.repeat(k, 2, axis=2), np.repeat(v, 2, axis=2), B, N, H, d, 0.1, True)
+    assert np.abs(got - want).max() <= 2e-2
+    # paired query tiles (threshold lowered): a workgroup takes a late 256-row tile and then an early one
+    monkeypatch.setenv("AHPC_FLASH_PAIR_MIN", "1")
+    B, N, H, d = 1, 1100, 2, 64
+    q, k, v = qkv((B, N, H, d), 22, O.F16)
+    got = flash(emu, q, k, v, O.F16, B, N, H, d, 0.125, True)
+    assert np.abs(got - O.attention(q, k, v, B, N, H, d, 0.125, True)).max() <= 2e-2
