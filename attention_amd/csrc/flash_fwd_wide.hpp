@@ -369,8 +369,7 @@ __global__ __launch_bounds__(kFlashThreads, 1) void flash_fwd_wide_kernel(const 
                 if (blk < 3) {
 #pragma unroll
                     for (int i = 0; i < KS; ++i) {
-                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);       // one K operand read
-                        __builtin_amdgcn_sched_group_barrier(0x008, QB, 0);      // the matrix instructions it feeds
+                        __builtin_amdgcn_sched_group_barrier(0x008, QB, 0);      // the matrix instructions of one k-step
                         __builtin_amdgcn_sched_group_barrier(0x400, 16 / KS, 0); // exponentials
                         __builtin_amdgcn_sched_group_barrier(0x002, 24 / KS, 0); // conversions, row sums
                     }
