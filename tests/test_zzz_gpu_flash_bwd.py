@@ -184,3 +184,17 @@ def test_ragged_batch(gpu, dtype, d, H, H_kv, causal):
         a, b = cu[i], cu[i + 1]
         want = O.attention_backward(q[a:b][None], k[a:b][None], v[a:b][None], do[a:b][None], 1, int(n), H, d, scale, causal, H_kv)
         check(tuple(g[a:b][None] for g in got), want, dtype)
+
+
+def test_golden_backward_vectors(gpu):
+    """tests/golden/*.npz: gradients from a float64 computation that shares no code with the oracle."""
+    import os
+    from test_golden_vectors import FILES, load, dense_inputs
+    for path in FILES:
+        c = load(path)
+        if "dq" not in c:
+            continue
+        (B, N, H, Hkv, d), q, k, v, do, mask = dense_inputs(c)
+        got = run_backward(gpu, q, k, v, do, O.F32, B, N, H, Hkv, d, float(c["scale"]), bool(c["causal"]), mask)
+        for g, name in zip(got, ("dq", "dk", "dv")):
+            assert np.abs(g - c[name]).max() <= 1e-4, (os.path.basename(path), name)
