@@ -363,16 +363,43 @@ __global__ __launch_bounds__(kFlashThreads, 1) void flash_fwd_wide_kernel(const 
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int blk = 0; blk < 4; ++blk) {
-                // stage A: scores of the next block | P of this block, first 16 keys
-                if (blk < 3) scores(blk + 1, s_nxt);
-                make_pb(s_cur, 0, pb0, sum);
+                // stage A: scores of the next block | P of this block, first 16 keys.  One k-step of the scores
+                // (an operand read, two matrix instructions) alternates with one slice of the P arithmetic; the
+                // empty asm statements make, as far as the instruction scheduler can tell, each slice depend on
+                // the k-step's operand and the next k-step's operand depend on the slice, which pins that order.
                 if (blk < 3) {
+                    const unsigned char* tk = tile_k + 32 * (blk + 1) * RB;
+                    constexpr int kItems = QB * 4;             // (query block, register pair) items of make_pb
+                    constexpr int kPerStep = kItems / KS > 0 ? kItems / KS : 1;
+                    float pinned = 0.0f;
 #pragma unroll
-                    for (int i = 0; i < KS; ++i) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, QB, 0);      // the matrix instructions of one k-step
-                        __builtin_amdgcn_sched_group_barrier(0x400, 16 / KS, 0); // exponentials
-                        __builtin_amdgcn_sched_group_barrier(0x002, 24 / KS, 0); // conversions, row sums
+                    for (int ks = 0; ks < KS; ++ks) {
+                        u32x4 a = lds_read_b128(tk + k_off[ks]);
+                        if (ks > 0) asm("" : "+v"(a) : "v"(pinned));
+#pragma unroll
+                        for (int qb = 0; qb < QB; ++qb)
+                            s_nxt[qb] = mfma_32x32x16<T>(a, qreg[qb][ks], ks == 0 ? neg_m[qb] : s_nxt[qb]);
+#pragma unroll
+                        for (int it = ks * kPerStep; it < (ks + 1) * kPerStep && it < kItems; ++it) {
+                            const int qb = it / 4, w = it % 4;
+                            float x0 = s_cur[qb][2 * w], x1 = s_cur[qb][2 * w + 1];
+                            asm("" : "+v"(x0), "+v"(x1) : "v"(a));
+                            const float p0 = fast_exp2(x0), p1 = fast_exp2(x1);
+                            pb0[qb][w] = pack2<T>(p0, p1);
+                            sum[qb] += p0 + p1;
+                            pinned = p1;
+                        }
                     }
+                    // items the k-steps did not cover (more items than k-steps times kPerStep)
+#pragma unroll
+                    for (int it = KS * kPerStep; it < kItems; ++it) {
+                        const int qb = it / 4, w = it % 4;
+                        const float p0 = fast_exp2(s_cur[qb][2 * w]), p1 = fast_exp2(s_cur[qb][2 * w + 1]);
+                        pb0[qb][w] = pack2<T>(p0, p1);
+                        sum[qb] += p0 + p1;
+                    }
+                } else {
+                    make_pb(s_cur, 0, pb0, sum);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 // stage B: second product, first 16 keys | P of this block, last 16 keys
@@ -391,8 +418,17 @@ __global__ __launch_bounds__(kFlashThreads, 1) void flash_fwd_wide_kernel(const 
                 if (blk < 3) v_operands(blk + 1, 0, vf0);
                 second_product(vf1, pb1);
                 if (blk < 3) {
+                    // (the empty asm ties each copy out of the accumulation registers to a value of stage B, so that
+                    // the copies are made here, between this stage's matrix instructions, and not right behind the
+                    // matrix instructions that produce the scores, where they would wait for them)
 #pragma unroll
-                    for (int qb = 0; qb < QB; ++qb) s_cur[qb] = s_nxt[qb];
+                    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            float t = s_nxt[qb][r];
+                            asm("" : "+v"(t) : "v"(pb1[qb][r & 3]));
+                            s_cur[qb][r] = t;
+                        }
                     beyond = beyond | beyond_frame(s_cur);
 #pragma unroll
                     for (int i = 0; i < MB; ++i) {
