@@ -69,7 +69,7 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_kernel(const DecodeParam
         }
         return;
     }
-    my_page = my_page < 0 ? 0 : my_page;  // a missing page reads page 0 (the host never hands out such a table)
+    my_page = my_page < 0 ? 0 : my_page;  // entries behind a sequence's last page are never dereferenced
     const int t1 = (t0 + p.chunk_tokens) < L ? (t0 + p.chunk_tokens) : L;
     const int n_tok = t1 - t0;
     const int n_tiles = (n_tok + kDecodeTile - 1) / kDecodeTile;
@@ -95,17 +95,22 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_kernel(const DecodeParam
         off_k[i] = (lane / TL::kChunks) * tok_bytes + ((pc ^ TL::fk(r)) << 4);
         off_v[i] = (lane / TL::kChunks) * tok_bytes + ((pc ^ TL::fv(r)) << 4);
     }
-    const unsigned span = (unsigned)((RPI - 1) * tok_bytes + 2 * D);  // bytes one instruction may touch
     const unsigned char* const kpool = static_cast<const unsigned char*>(p.k_pool);
     const unsigned char* const vpool = static_cast<const unsigned char*>(p.v_pool);
-    auto gather_tile = [&](int tile, unsigned char* dst_k, unsigned char* dst_v) {
+    auto gather_tile = [&](int tile, unsigned char* dst_k, unsigned char* dst_v) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             const int ti = tile * kDecodeTile + i * RPI;  // chunk-relative token of the instruction's first row
             const int page_id = __builtin_amdgcn_readlane(my_page, ti >> 4);
             const int64_t byte0 = (((int64_t)page_id * P + (ti & 15)) * p.H_kv + hk) * (int64_t)(D * (int)sizeof(T));
-            dma_instr(kpool + byte0, span, off_k[i], dst_k + i * 1024);
-            dma_instr(vpool + byte0, span, off_v[i], dst_v + i * 1024);
+            // Token rows at or beyond the end of the chunk are outside the descriptor and land as zeros: what the
+            // pool holds there may be any bit pattern, and 0 * NaN in the second product would poison the row.
+            // (An instruction with no token row left touches no memory, whatever its page id is.)
+            const int rows = n_tok - ti;
+            const int rc = rows < RPI ? rows : RPI;  // token rows of this instruction that exist (may be <= 0)
+            const unsigned nrec = rc > 0 ? (unsigned)((rc - 1) * tok_bytes + 2 * D) : 0u;  // bytes it may touch
+            dma_instr(kpool + byte0, nrec, off_k[i], dst_k + i * 1024);
+            dma_instr(vpool + byte0, nrec, off_v[i], dst_v + i * 1024);
         }
     };
 
@@ -129,7 +134,7 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_kernel(const DecodeParam
         for (int r = 0; r < 16; ++r) oacc[mb][r] = 0.0f;
     float m_run = -INFINITY, l_run = 0.0f;
 
-    auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int tile) {
+    auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int tile) __attribute__((always_inline)) {
         f32x16 s;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = 0.0f;
@@ -178,7 +183,7 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_kernel(const DecodeParam
         }
     };
 
-    auto step = [&](unsigned char* cur_k, unsigned char* cur_v, unsigned char* nxt_k, unsigned char* nxt_v, int t) {
+    auto step = [&](unsigned char* cur_k, unsigned char* cur_v, unsigned char* nxt_k, unsigned char* nxt_v, int t) __attribute__((always_inline)) {
         const bool more = t + 1 < n_tiles;
         if (more) gather_tile(t + 1, nxt_k, nxt_v);
         compute_tile(cur_k, cur_v, t);

@@ -41,6 +41,23 @@ def build_problem(B, H, d, P, lens, seed, dtype, extra_pages=5):
     return q, kp, vp, table, lens, news, n_pages
 
 
+def poison_unused(kp, vp, table, lens, P, H, d, wild_page=None):
+    """Copies of the pools with NaN in every token slot that no sequence owns (the tail of a last page, free pages,
+    the pages of a sequence whose length was set to zero), and of the table with `wild_page` (if given) in the
+    entries behind each sequence's last page.  A decode must neither read the former into its result nor
+    dereference the latter."""
+    kp, vp, table = kp.copy(), vp.copy(), table.copy()
+    used = np.zeros(kp.size // (H * d), bool)
+    for b, n in enumerate(np.asarray(lens)):
+        t = np.arange(int(n))
+        used[table[b, t // P].astype(np.int64) * P + t % P] = True
+        if wild_page is not None:
+            table[b, (int(n) + P - 1) // P:] = wild_page
+    kp.reshape(-1, H * d)[~used] = np.nan
+    vp.reshape(-1, H * d)[~used] = np.nan
+    return kp, vp, table
+
+
 def gpu_decode(hip, q, kp_dev, vp_dev, table, lens, rows, B, H, d, P, dtype, qo_dtype, scale, chunk=0, max_len=None):
     import torch
     from gpu_util import to_dev, to_host, stream_ptr, dev_i32

@@ -135,7 +135,7 @@ def test_interleaved_workgroup_map_computes_the_same(emu, together, slots, monke
 
 
 # ---- paged KV pool and decode -----------------------------------------------------------------------------
-from test_gpu_paged import build_problem, _tables_for  # problem builders only (pure numpy + oracle)
+from test_gpu_paged import build_problem, poison_unused, _tables_for  # problem builders only (pure numpy + oracle)
 
 
 def decode(emu, q, kp, vp, table, lens, rows, B, H, H_kv, d, P, dtype, qo_dtype, scale, chunk=0):
@@ -160,6 +160,7 @@ def test_decode(emu, dtype, H, d, P):
     q, kp, vp, table, lens, _, _ = build_problem(B, H, d, P, [33, 1, 16, 150], 21, dtype)
     scale = 1.0 / np.sqrt(d)
     want = O.paged_decode(q, kp, vp, table, lens, None, B, H, d, P, scale)
+    kp, vp, table = poison_unused(kp, vp, table, lens, P, H, d, wild_page=1 << 24)
     for chunk in (0, P, 4 * P):
         got = decode(emu, q, kp, vp, table, lens, None, B, H, H, d, P, dtype, dtype, scale, chunk)
         assert np.isfinite(got).all()
@@ -176,6 +177,7 @@ def test_decode_grouped_heads(emu, G):
     # the ordinary oracle on a pool whose heads are repeated G times
     rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
     want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    kp, vp, table = poison_unused(kp, vp, table, lens, P, H_kv, d, wild_page=1 << 24)
     for chunk in (0, 32):
         got = decode(emu, q, kp, vp, table, lens, None, B, H, H_kv, d, P, O.F16, O.F16, scale, chunk)
         assert np.abs(got - want).max() <= 2e-2
@@ -392,6 +394,8 @@ def test_decode_grouped_heads_matrix_core_kernel(emu, G, dtype, d, monkeypatch):
     scale = 1.0 / np.sqrt(d)
     rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
     want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    # slots that hold no token of a sequence are NaN, table entries behind a last page point far outside the pool
+    kp, vp, table = poison_unused(kp, vp, table, lens, P, H_kv, d, wild_page=1 << 24)
     S.lds_stats(reset=True)
     for chunk, qo, dma_late in ((0, dtype, False), (48, O.F32, True), (16, dtype, False), (0, dtype, True)):
         S.configure(dma_late, seed=G + chunk)

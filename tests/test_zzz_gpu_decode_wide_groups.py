@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 from oracle import oracle as O
-from test_gpu_paged import build_problem, gpu_decode  # noqa: F401  (problem builder; gpu_decode documents the call)
+from test_gpu_paged import build_problem, poison_unused, gpu_decode  # noqa: F401  (builders; gpu_decode documents the call)
 
 pytestmark = pytest.mark.gpu
 
@@ -50,6 +50,7 @@ def test_matrix_core_decode_equals_repeated_heads(gpu, G, dtype, d, monkeypatch)
     scale = 1.0 / np.sqrt(d)
     rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
     want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    kp, vp, table = poison_unused(kp, vp, table, lens, P, H_kv, d)   # NaN wherever the pool holds no token of a sequence
     for chunk, qo in ((0, dtype), (48, O.F32), (16, dtype), (1024, dtype)):
         got = run(gpu, q, kp, vp, table, lens, B, H, H_kv, d, P, dtype, qo, scale, chunk)
         assert np.isfinite(got).all()
