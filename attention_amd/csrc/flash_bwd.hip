@@ -42,26 +42,42 @@ struct BwdParams {
 };
 
 // ---------------------------------------------------------------------------------------------
-// fp32-FMA kernels: any dtype, head dimension up to 256, optional dense mask.  One thread owns one row
-// (query row in the first two kernels, key row in the third) and keeps it in registers; the rows it walks
-// over are staged in LDS as fp32, 16 at a time, by the 128 threads of the workgroup.  This is the accuracy
-// path (fp32 tensors, 1e-4 tolerance) and the fallback for what the matrix-core kernels do not take.
-constexpr int kBwdRows = 128;
+// fp32-FMA kernels: any dtype, head dimension up to 256, optional dense mask.  A row (query row in the first
+// two kernels, key row in the third) is owned by S neighbouring lanes that keep it in registers, 16-byte
+// granules dealt round-robin (S = 1, 2, 4 for padded head dimensions up to 64, 128, 256: at most 64 elements
+// of each per-row vector per lane, which is what fits the register file); the rows they walk over are staged in
+// LDS as fp32, 16 at a time, by the 128 threads of the workgroup, and dot products are summed across the S
+// lanes with shuffles.  Everything between two barriers is straight-line per key with the row's conditions as
+// predicates, so that the shuffles run with all lanes.  This is the accuracy path (fp32 tensors, 1e-4
+// tolerance) and the fallback for what the matrix-core kernels do not take.
+constexpr int kBwdThreads = 128;
 constexpr int kBwdTile = 16;
 
 // Stages rows [r0, r0+16) of a [rows][d] tensor (row stride `stride`) into dst[16][DP] as fp32; rows at or
 // beyond `n_rows` and columns at or beyond d become zero.
 template <typename T, int DP>
 __device__ inline void stage_rows(float (*dst)[DP], const T* src, int64_t stride, int r0, int n_rows, int d, int tid) {
-    for (int i = tid; i < kBwdTile * DP; i += kBwdRows) {
+    for (int i = tid; i < kBwdTile * DP; i += kBwdThreads) {
         const int r = i / DP, e = i - r * DP;
         const int row = r0 + r;
         dst[r][e] = (row < n_rows && e < d) ? Storage<T>::load(src + (int64_t)row * stride + e) : 0.0f;
     }
 }
 
+// Element of the row that register i of lane part `part` holds (S lanes per row, 16-byte granules round-robin).
+template <int S>
+__device__ inline int row_elem(int i, int part) { return (((i >> 2) * S + part) << 2) + (i & 3); }
+
+// Sum over the S neighbouring lanes of a row; every lane of the wavefront takes part.
+template <int S>
+__device__ inline float row_sum(float x) {
+    if (S >= 2) x += __shfl_xor(x, 1, kWave);
+    if (S >= 4) x += __shfl_xor(x, 2, kWave);
+    return x;
+}
+
 // Length of sequence b and the element offsets of its first row for head h (Q, dO, dQ) and K/V head hk.
-__device__ inline void bwd_sequence(const BwdParams& p, int b, int h, int hk, int& L, int64_t& base, int64_t& kv_base) {
+__device__ __forceinline__ void bwd_sequence(const BwdParams& p, int b, int h, int hk, int& L, int64_t& base, int64_t& kv_base) {
     if (p.cu_seqlens) {
         const int s0 = p.cu_seqlens[b];
         L = p.cu_seqlens[b + 1] - s0;
@@ -74,35 +90,39 @@ __device__ inline void bwd_sequence(const BwdParams& p, int b, int h, int hk, in
     }
 }
 
-template <typename T, int DP>
-__global__ __launch_bounds__(kBwdRows) void flash_bwd_stats_simple_kernel(const BwdParams p) {
+template <typename T, int DP, int S>
+__global__ __launch_bounds__(kBwdThreads) void flash_bwd_stats_simple_kernel(const BwdParams p) {
+    constexpr int EP = DP / S;            // elements of a row per lane
+    constexpr int R = kBwdThreads / S;    // rows per workgroup
     __shared__ float sk[kBwdTile][DP];
     __shared__ float sv[kBwdTile][DP];
     const int tid = threadIdx.x;
+    const int part = tid % S;
     const int h = blockIdx.y, b = blockIdx.z;
     const int hk = h / p.kv_group;
     const int d = p.d;
     int L;
     int64_t base, kv_base;
     bwd_sequence(p, b, h, hk, L, base, kv_base);
-    const int row0 = blockIdx.x * kBwdRows;
+    const int row0 = blockIdx.x * R;
     if (row0 >= L) return;
-    const int n = row0 + tid;
+    const int n = row0 + tid / S;
     const bool active = n < L;
     const T* gq = static_cast<const T*>(p.q) + base;
     const T* gdo = static_cast<const T*>(p.d_out) + base;
     const T* gk = static_cast<const T*>(p.k) + kv_base;
     const T* gv = static_cast<const T*>(p.v) + kv_base;
 
-    float qv[DP], acc[DP];
+    float qv[EP], acc[EP];
 #pragma unroll
-    for (int e = 0; e < DP; ++e) {
-        qv[e] = (active && e < d) ? Storage<T>::load(gq + (int64_t)n * p.stride_n + e) : 0.0f;
-        acc[e] = 0.0f;
+    for (int i = 0; i < EP; ++i) {
+        const int e = row_elem<S>(i, part);
+        qv[i] = (active && e < d) ? Storage<T>::load(gq + (int64_t)n * p.stride_n + e) : 0.0f;
+        acc[i] = 0.0f;
     }
     float m = -INFINITY, l = 0.0f;
     int k_end = L;
-    if (p.causal) k_end = (row0 + kBwdRows) < L ? (row0 + kBwdRows) : L;
+    if (p.causal) k_end = (row0 + R) < L ? (row0 + R) : L;
     const float* mrow = (p.mask && active) ? p.mask + ((int64_t)b * p.N + n) * p.N : nullptr;
 
     for (int k0 = 0; k0 < k_end; k0 += kBwdTile) {
@@ -110,78 +130,80 @@ __global__ __launch_bounds__(kBwdRows) void flash_bwd_stats_simple_kernel(const 
         stage_rows<T, DP>(sk, gk, p.kv_stride_n, k0, L, d, tid);
         stage_rows<T, DP>(sv, gv, p.kv_stride_n, k0, L, d, tid);
         __syncthreads();
-        if (!active) continue;
-        for (int kr = 0; kr < kBwdTile; ++kr) {
+        const int kr_end = (k_end - k0) < kBwdTile ? (k_end - k0) : kBwdTile;
+        for (int kr = 0; kr < kr_end; ++kr) {
             const int key = k0 + kr;
-            if (key >= L) break;
-            if (p.causal && key > n) break;
-            if (mrow && mrow[key] == 0.0f) continue;
             float dot = 0.0f;
 #pragma unroll
-            for (int e = 0; e < DP; ++e) dot = __builtin_fmaf(qv[e], sk[kr][e], dot);
-            const float s = dot * p.scale;
+            for (int i = 0; i < EP; ++i) dot = __builtin_fmaf(qv[i], sk[kr][row_elem<S>(i, part)], dot);
+            const float s = row_sum<S>(dot) * p.scale;
+            const bool seen = active && !(p.causal && key > n) && !(mrow && mrow[key] == 0.0f);
+            if (!seen) continue;
             if (s > m) {
                 const float a = __expf(m - s);  // first key: exp(-inf) = 0
                 l = l * a + 1.0f;
 #pragma unroll
-                for (int e = 0; e < DP; ++e) acc[e] = __builtin_fmaf(acc[e], a, sv[kr][e]);
+                for (int i = 0; i < EP; ++i) acc[i] = __builtin_fmaf(acc[i], a, sv[kr][row_elem<S>(i, part)]);
                 m = s;
             } else {
                 const float w = __expf(s - m);
                 l += w;
 #pragma unroll
-                for (int e = 0; e < DP; ++e) acc[e] = __builtin_fmaf(w, sv[kr][e], acc[e]);
+                for (int i = 0; i < EP; ++i) acc[i] = __builtin_fmaf(w, sv[kr][row_elem<S>(i, part)], acc[i]);
             }
         }
     }
-    if (!active) return;
-    // a row that sees no key: every weight is exp(s - inf) = 0 later on, and nothing flows through it
-    float lse = INFINITY, delta = 0.0f;
-    if (l > 0.0f) {
-        lse = m + logf(l);
-        float dot = 0.0f;
+    // delta = dO . O, summed over the lanes of the row (rows beyond the sequence take part with zeros)
+    float dot = 0.0f;
 #pragma unroll
-        for (int e = 0; e < DP; ++e)
-            if (e < d) dot = __builtin_fmaf(acc[e], Storage<T>::load(gdo + (int64_t)n * p.stride_n + e), dot);
-        delta = dot / l;
+    for (int i = 0; i < EP; ++i) {
+        const int e = row_elem<S>(i, part);
+        if (active && e < d) dot = __builtin_fmaf(acc[i], Storage<T>::load(gdo + (int64_t)n * p.stride_n + e), dot);
     }
+    dot = row_sum<S>(dot);
+    if (!active || part != 0) return;
+    // a row that sees no key: every weight is exp(s - inf) = 0 later on, and nothing flows through it
     const int64_t row = ((int64_t)b * p.H + h) * p.rows_padded + n;
-    p.lse[row] = lse;
-    p.delta[row] = delta;
+    p.lse[row] = l > 0.0f ? m + logf(l) : INFINITY;
+    p.delta[row] = l > 0.0f ? dot / l : 0.0f;
 }
 
-template <typename T, int DP>
-__global__ __launch_bounds__(kBwdRows) void flash_bwd_dq_simple_kernel(const BwdParams p) {
+template <typename T, int DP, int S>
+__global__ __launch_bounds__(kBwdThreads) void flash_bwd_dq_simple_kernel(const BwdParams p) {
+    constexpr int EP = DP / S;
+    constexpr int R = kBwdThreads / S;
     __shared__ float sk[kBwdTile][DP];
     __shared__ float sv[kBwdTile][DP];
     const int tid = threadIdx.x;
+    const int part = tid % S;
     const int h = blockIdx.y, b = blockIdx.z;
     const int hk = h / p.kv_group;
     const int d = p.d;
     int L;
     int64_t base, kv_base;
     bwd_sequence(p, b, h, hk, L, base, kv_base);
-    const int row0 = blockIdx.x * kBwdRows;
+    const int row0 = blockIdx.x * R;
     if (row0 >= L) return;
-    const int n = row0 + tid;
+    const int n = row0 + tid / S;
     const bool active = n < L;
     const T* gq = static_cast<const T*>(p.q) + base;
     const T* gdo = static_cast<const T*>(p.d_out) + base;
     const T* gk = static_cast<const T*>(p.k) + kv_base;
     const T* gv = static_cast<const T*>(p.v) + kv_base;
 
-    float qv[DP], dov[DP], dq[DP];
+    float qv[EP], dov[EP], dq[EP];
 #pragma unroll
-    for (int e = 0; e < DP; ++e) {
+    for (int i = 0; i < EP; ++i) {
+        const int e = row_elem<S>(i, part);
         const bool in = active && e < d;
-        qv[e] = in ? Storage<T>::load(gq + (int64_t)n * p.stride_n + e) : 0.0f;
-        dov[e] = in ? Storage<T>::load(gdo + (int64_t)n * p.stride_n + e) : 0.0f;
-        dq[e] = 0.0f;
+        qv[i] = in ? Storage<T>::load(gq + (int64_t)n * p.stride_n + e) : 0.0f;
+        dov[i] = in ? Storage<T>::load(gdo + (int64_t)n * p.stride_n + e) : 0.0f;
+        dq[i] = 0.0f;
     }
     const int64_t row = ((int64_t)b * p.H + h) * p.rows_padded + (active ? n : 0);
     const float lse = p.lse[row], delta = p.delta[row];
     int k_end = L;
-    if (p.causal) k_end = (row0 + kBwdRows) < L ? (row0 + kBwdRows) : L;
+    if (p.causal) k_end = (row0 + R) < L ? (row0 + R) : L;
     const float* mrow = (p.mask && active) ? p.mask + ((int64_t)b * p.N + n) * p.N : nullptr;
 
     for (int k0 = 0; k0 < k_end; k0 += kBwdTile) {
@@ -189,58 +211,66 @@ __global__ __launch_bounds__(kBwdRows) void flash_bwd_dq_simple_kernel(const Bwd
         stage_rows<T, DP>(sk, gk, p.kv_stride_n, k0, L, d, tid);
         stage_rows<T, DP>(sv, gv, p.kv_stride_n, k0, L, d, tid);
         __syncthreads();
-        if (!active) continue;
-        for (int kr = 0; kr < kBwdTile; ++kr) {
+        const int kr_end = (k_end - k0) < kBwdTile ? (k_end - k0) : kBwdTile;
+        for (int kr = 0; kr < kr_end; ++kr) {
             const int key = k0 + kr;
-            if (key >= L) break;
-            if (p.causal && key > n) break;
-            if (mrow && mrow[key] == 0.0f) continue;
             float dot = 0.0f, dp = 0.0f;
 #pragma unroll
-            for (int e = 0; e < DP; ++e) {
-                dot = __builtin_fmaf(qv[e], sk[kr][e], dot);
-                dp = __builtin_fmaf(dov[e], sv[kr][e], dp);
+            for (int i = 0; i < EP; ++i) {
+                const int e = row_elem<S>(i, part);
+                dot = __builtin_fmaf(qv[i], sk[kr][e], dot);
+                dp = __builtin_fmaf(dov[i], sv[kr][e], dp);
             }
+            dot = row_sum<S>(dot);
+            dp = row_sum<S>(dp);
+            const bool seen = active && !(p.causal && key > n) && !(mrow && mrow[key] == 0.0f);
+            if (!seen) continue;
             const float ds = __expf(dot * p.scale - lse) * (dp - delta);
 #pragma unroll
-            for (int e = 0; e < DP; ++e) dq[e] = __builtin_fmaf(ds, sk[kr][e], dq[e]);
+            for (int i = 0; i < EP; ++i) dq[i] = __builtin_fmaf(ds, sk[kr][row_elem<S>(i, part)], dq[i]);
         }
     }
     if (!active) return;
     T* out = static_cast<T*>(p.d_q) + base + (int64_t)n * p.stride_n;
 #pragma unroll
-    for (int e = 0; e < DP; ++e)
-        if (e < d) Storage<T>::store(out + e, dq[e] * p.scale);
+    for (int i = 0; i < EP; ++i) {
+        const int e = row_elem<S>(i, part);
+        if (e < d) Storage<T>::store(out + e, dq[i] * p.scale);
+    }
 }
 
 // grid.y = key/value heads: the query heads of a group are walked one after the other
-template <typename T, int DP>
-__global__ __launch_bounds__(kBwdRows) void flash_bwd_dkv_simple_kernel(const BwdParams p) {
+template <typename T, int DP, int S>
+__global__ __launch_bounds__(kBwdThreads) void flash_bwd_dkv_simple_kernel(const BwdParams p) {
+    constexpr int EP = DP / S;
+    constexpr int R = kBwdThreads / S;
     __shared__ float sq[kBwdTile][DP];
     __shared__ float sdo[kBwdTile][DP];
     __shared__ float s_lse[kBwdTile];
     __shared__ float s_delta[kBwdTile];
     const int tid = threadIdx.x;
+    const int part = tid % S;
     const int hk = blockIdx.y, b = blockIdx.z;
     const int d = p.d;
     int L;
     int64_t base0, kv_base;
     bwd_sequence(p, b, hk * p.kv_group, hk, L, base0, kv_base);
-    const int row0 = blockIdx.x * kBwdRows;
+    const int row0 = blockIdx.x * R;
     if (row0 >= L) return;
-    const int j = row0 + tid;
+    const int j = row0 + tid / S;
     const bool active = j < L;
     const T* gk = static_cast<const T*>(p.k) + kv_base;
     const T* gv = static_cast<const T*>(p.v) + kv_base;
 
-    float kv[DP], vv[DP], dk[DP], dv[DP];
+    float kv[EP], vv[EP], dk[EP], dv[EP];
 #pragma unroll
-    for (int e = 0; e < DP; ++e) {
+    for (int i = 0; i < EP; ++i) {
+        const int e = row_elem<S>(i, part);
         const bool in = active && e < d;
-        kv[e] = in ? Storage<T>::load(gk + (int64_t)j * p.kv_stride_n + e) : 0.0f;
-        vv[e] = in ? Storage<T>::load(gv + (int64_t)j * p.kv_stride_n + e) : 0.0f;
-        dk[e] = 0.0f;
-        dv[e] = 0.0f;
+        kv[i] = in ? Storage<T>::load(gk + (int64_t)j * p.kv_stride_n + e) : 0.0f;
+        vv[i] = in ? Storage<T>::load(gv + (int64_t)j * p.kv_stride_n + e) : 0.0f;
+        dk[i] = 0.0f;
+        dv[i] = 0.0f;
     }
     // under a causal mask only queries at or after the first key of this workgroup contribute
     const int i_begin = p.causal ? (row0 / kBwdTile) * kBwdTile : 0;
@@ -261,24 +291,27 @@ __global__ __launch_bounds__(kBwdRows) void flash_bwd_dkv_simple_kernel(const Bw
                 s_delta[tid] = i < L ? p.delta[stat0 + i] : 0.0f;
             }
             __syncthreads();
-            if (!active) continue;
-            for (int r = 0; r < kBwdTile; ++r) {
+            const int r_end = (L - i0) < kBwdTile ? (L - i0) : kBwdTile;
+            for (int r = 0; r < r_end; ++r) {
                 const int i = i0 + r;
-                if (i >= L) break;
-                if (p.causal && i < j) continue;
-                if (p.mask && p.mask[((int64_t)b * p.N + i) * p.N + j] == 0.0f) continue;
                 float dot = 0.0f, dp = 0.0f;
 #pragma unroll
-                for (int e = 0; e < DP; ++e) {
-                    dot = __builtin_fmaf(sq[r][e], kv[e], dot);
-                    dp = __builtin_fmaf(sdo[r][e], vv[e], dp);
+                for (int x = 0; x < EP; ++x) {
+                    const int e = row_elem<S>(x, part);
+                    dot = __builtin_fmaf(sq[r][e], kv[x], dot);
+                    dp = __builtin_fmaf(sdo[r][e], vv[x], dp);
                 }
+                dot = row_sum<S>(dot);
+                dp = row_sum<S>(dp);
+                const bool seen = active && !(p.causal && i < j) && !(p.mask && p.mask[((int64_t)b * p.N + i) * p.N + j] == 0.0f);
+                if (!seen) continue;
                 const float pw = __expf(dot * p.scale - s_lse[r]);
                 const float ds = pw * (dp - s_delta[r]);
 #pragma unroll
-                for (int e = 0; e < DP; ++e) {
-                    dv[e] = __builtin_fmaf(pw, sdo[r][e], dv[e]);
-                    dk[e] = __builtin_fmaf(ds, sq[r][e], dk[e]);
+                for (int x = 0; x < EP; ++x) {
+                    const int e = row_elem<S>(x, part);
+                    dv[x] = __builtin_fmaf(pw, sdo[r][e], dv[x]);
+                    dk[x] = __builtin_fmaf(ds, sq[r][e], dk[x]);
                 }
             }
         }
@@ -287,20 +320,24 @@ __global__ __launch_bounds__(kBwdRows) void flash_bwd_dkv_simple_kernel(const Bw
     T* out_k = static_cast<T*>(p.d_k) + kv_base + (int64_t)j * p.kv_stride_n;
     T* out_v = static_cast<T*>(p.d_v) + kv_base + (int64_t)j * p.kv_stride_n;
 #pragma unroll
-    for (int e = 0; e < DP; ++e)
+    for (int x = 0; x < EP; ++x) {
+        const int e = row_elem<S>(x, part);
         if (e < d) {
-            Storage<T>::store(out_k + e, dk[e] * p.scale);
-            Storage<T>::store(out_v + e, dv[e]);
+            Storage<T>::store(out_k + e, dk[x] * p.scale);
+            Storage<T>::store(out_v + e, dv[x]);
         }
+    }
 }
 
 template <typename T, int DP>
 static int launch_simple_dp(const BwdParams& p, int64_t B, int64_t H_kv, hipStream_t stream) {
-    const unsigned tiles = (unsigned)((p.N + kBwdRows - 1) / kBwdRows);
-    dim3 block(kBwdRows);
-    hipLaunchKernelGGL((flash_bwd_stats_simple_kernel<T, DP>), dim3(tiles, (unsigned)p.H, (unsigned)B), block, 0, stream, p);
-    hipLaunchKernelGGL((flash_bwd_dq_simple_kernel<T, DP>), dim3(tiles, (unsigned)p.H, (unsigned)B), block, 0, stream, p);
-    hipLaunchKernelGGL((flash_bwd_dkv_simple_kernel<T, DP>), dim3(tiles, (unsigned)H_kv, (unsigned)B), block, 0, stream, p);
+    constexpr int S = DP <= 64 ? 1 : DP / 64;  // lanes per row
+    constexpr int R = kBwdThreads / S;
+    const unsigned tiles = (unsigned)((p.N + R - 1) / R);
+    dim3 block(kBwdThreads);
+    hipLaunchKernelGGL((flash_bwd_stats_simple_kernel<T, DP, S>), dim3(tiles, (unsigned)p.H, (unsigned)B), block, 0, stream, p);
+    hipLaunchKernelGGL((flash_bwd_dq_simple_kernel<T, DP, S>), dim3(tiles, (unsigned)p.H, (unsigned)B), block, 0, stream, p);
+    hipLaunchKernelGGL((flash_bwd_dkv_simple_kernel<T, DP, S>), dim3(tiles, (unsigned)H_kv, (unsigned)B), block, 0, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 
