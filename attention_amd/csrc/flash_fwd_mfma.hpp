@@ -262,7 +262,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
     const T* const gq = static_cast<const T*>(p.q) + base;
     const T* const gk = static_cast<const T*>(p.k) + kv_base;
     const T* const gv = static_cast<const T*>(p.v) + kv_base;
-    T* const go = static_cast<T*>(p.o) + base;
+    T* const go = STATS ? nullptr : static_cast<T*>(p.o) + base;  // the statistics pass has no output tensor
     const int64_t sn = p.stride_n;
     const int64_t skv = p.kv_stride_n;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
