@@ -11,13 +11,16 @@ import numpy as np
 from attention_amd import hip
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libahpc_simt.so")
+# AHPC_SIMT_LIB names another build of the same library (the sanitizer build of the Makefile's `ubsan` target)
+LIB_PATH = os.environ.get("AHPC_SIMT_LIB") or os.path.join(_HERE, "libahpc_simt.so")
 
 F32, F16, BF16 = 0, 1, 2
 _lib = None
 
 
 def build():
+    if os.environ.get("AHPC_SIMT_LIB"):
+        return  # a build the caller made
     subprocess.run(["make", "-C", _HERE], check=True, capture_output=True)
 
 
