@@ -39,6 +39,27 @@ __global__ void dma_round_trip(const unsigned char* src, unsigned char* dst, int
     for (int i = 0; i < 16; ++i) dst[threadIdx.x * 16 + i] = tile[threadIdx.x * 16 + i];
 }
 
+// Two wavefronts and one 1 KiB tile.  mode 0 (correct): wavefront 0 loads the tile, waits, barrier, wavefront 1
+// reads it.  mode 1: the barrier is missing.  mode 2: after a correct round both wavefronts read the tile and
+// wavefront 0 loads into it again without a barrier in between.
+__global__ void lds_ordering(const unsigned char* src, unsigned char* dst, int mode) {
+    __shared__ __attribute__((aligned(1024))) unsigned char tile[1024];
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(src), 0, 2048, 0x00020000);
+    if (wave == 0) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, tile, 16, lane * 16, 0, 0, 0);
+        __builtin_amdgcn_s_waitcnt(0);
+    }
+    if (mode != 1) __syncthreads();
+    simt::u32x4 x = simt::lds_read_b128(tile + lane * 16);
+    if (mode == 2 && wave == 0) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, tile, 16, 1024 + lane * 16, 0, 0, 0);
+        __builtin_amdgcn_s_waitcnt(0);
+    }
+    if (wave == 1)
+        for (int i = 0; i < 4; ++i) reinterpret_cast<unsigned*>(dst)[lane * 4 + i] = x[i];
+}
+
 // D = A * B + C with A[i][k] = a[i*16+k], B[k][j] = b[k*32+j], operands and result laid out as documented
 // for v_mfma_f32_32x32x16_bf16
 __global__ void matrix_instruction(const float* a, const float* b, const float* c, float* d) {
@@ -87,6 +108,10 @@ int simt_selftest_reads_a_finished_lane(int* out) {
 }
 int simt_selftest_dma_round_trip(const unsigned char* src, unsigned char* dst, int wait) {
     hipLaunchKernelGGL(dma_round_trip, dim3(1), dim3(64), 0, nullptr, src, dst, wait);
+    return hipGetLastError();
+}
+int simt_selftest_lds_ordering(const unsigned char* src, unsigned char* dst, int mode) {
+    hipLaunchKernelGGL(lds_ordering, dim3(1), dim3(128), 0, nullptr, src, dst, mode);
     return hipGetLastError();
 }
 int simt_selftest_matrix_instruction(const float* a, const float* b, const float* c, float* d) {

@@ -14,6 +14,10 @@
 //     too early; buffer descriptors clamp out-of-range reads to zero like the hardware;
 //   * 16-byte LDS reads made through lds_read_b128 and transposing reads are checked for bank conflicts under
 //     a model of 64 banks of 4 bytes (16 lanes per pass for 16-byte reads, 32 for 8-byte reads);
+//   * the same reads and the direct loads are checked for ordering between wavefronts: a direct load's write and
+//     another wavefront's read (or direct load) of the same LDS word need a workgroup barrier between them,
+//     where a load occupies the span from its issue to its lane's wait; violations are reported as errors
+//     whatever order the run happened to execute the wavefronts in (plain C++ accesses to LDS are not seen);
 //   * __shared__ arrays live in one linker section, filled with a NaN pattern before every workgroup,
 //     and LDS accesses made through intrinsics are range-checked against it.
 // Plain loads and stores through pointers are ordinary host accesses; run the build under

@@ -86,6 +86,40 @@ std::vector<unsigned char*> g_stacks;  // reused between launches
 long g_switches = 0;
 long g_lds_stats[4] = {0, 0, 0, 0};  // 16-byte reads, their conflict cycles, transposing reads, theirs
 
+// ---- ordering of LDS traffic between wavefronts ----------------------------------------------------
+// A work-item's epoch is the number of workgroup barriers it has passed.  Per 4-byte word of LDS: which
+// wavefront last wrote it with a direct-to-LDS load, in which epoch the load was issued and in which epoch
+// the issuing lane waited for it (-1: not yet), and per wavefront the last epoch in which it read the word
+// with one of the traced reads (16-byte operand reads, transposing reads).  Two accesses of different
+// wavefronts to one word, one of them a load's write, are ordered only by a barrier between them; a load
+// is "between" its issue and its wait.  Plain C++ accesses to LDS are not seen.
+constexpr int kMaxWaves = 16;
+struct WordState {
+    uint64_t workgroup = 0;  // serial number of the workgroup this state belongs to; older states count as fresh
+    int16_t writer = -1;
+    int32_t issued = 0, waited = -1;
+    int32_t read_epoch[kMaxWaves];
+};
+std::vector<WordState> g_words;
+uint64_t g_workgroup_serial = 0;
+
+void reset_word_states() {
+    ++g_workgroup_serial;
+    const size_t n = (size_t)(__stop_simt_lds - __start_simt_lds) / 4;
+    if (g_words.size() != n) g_words.assign(n, WordState());
+}
+WordState* word_state(const void* p) {
+    WordState* w = &g_words[(size_t)(static_cast<const unsigned char*>(p) - __start_simt_lds) / 4];
+    return w;
+}
+void freshen(WordState* w) {
+    if (w->workgroup == g_workgroup_serial) return;
+    w->workgroup = g_workgroup_serial;
+    w->writer = -1;
+    w->waited = -1;
+    for (int& e : w->read_epoch) e = -1;
+}
+
 uint64_t next_rand() {
     g_rng ^= g_rng << 13;
     g_rng ^= g_rng >> 7;
@@ -147,6 +181,8 @@ void fail(const std::string& what) {
     }
 }
 
+void note_dma_landed(const struct Fiber* f, const void* p, int bytes);
+
 // Lands this lane's outstanding direct-to-LDS loads, oldest first, until at most `leave` are outstanding
 // (loads complete in the order they were issued).
 void flush_dma(Fiber* f, size_t leave = 0) {
@@ -155,8 +191,51 @@ void flush_dma(Fiber* f, size_t leave = 0) {
         const PendingDma& d = f->dma[i];
         if (d.src) std::memcpy(d.dst, d.src, (size_t)d.bytes);
         else std::memset(d.dst, 0, (size_t)d.bytes);
+        note_dma_landed(f, d.dst, d.bytes);
     }
     f->dma.erase(f->dma.begin(), f->dma.begin() + (long)n);
+}
+
+// A traced read of `bytes` bytes at p by the running work-item.
+void note_lds_read(const void* p, int bytes) {
+    Fiber* f = g_cur;
+    const int e = (int)f->bar_gen;
+    WordState* w = word_state(p);
+    for (int i = 0; i < bytes / 4; ++i, ++w) {
+        freshen(w);
+        if (w->writer >= 0) {
+            if (w->waited < 0)
+                fail(w->writer == f->wave ? "LDS read of a direct-to-LDS load that its wavefront has not waited for"
+                                          : "LDS read of a direct-to-LDS load of another wavefront that is still in flight");
+            else if (w->writer != f->wave && w->waited >= e)
+                fail("LDS read races with a direct-to-LDS load of another wavefront: no barrier between the wait for the load and the read");
+        }
+        if (f->wave < kMaxWaves) w->read_epoch[f->wave] = e;
+    }
+}
+
+// A direct-to-LDS load of `bytes` bytes to p issued by the running work-item.
+void note_dma_issue(const void* p, int bytes) {
+    Fiber* f = g_cur;
+    const int e = (int)f->bar_gen;
+    WordState* w = word_state(p);
+    for (int i = 0; i < bytes / 4; ++i, ++w) {
+        freshen(w);
+        for (int v = 0; v < kMaxWaves; ++v)
+            if (v != f->wave && w->read_epoch[v] == e)
+                fail("direct-to-LDS load overwrites LDS that another wavefront has read since the last barrier");
+        if (w->writer >= 0 && w->writer != f->wave && (w->waited < 0 || w->waited >= e))
+            fail("direct-to-LDS loads of two wavefronts write the same LDS without a barrier between them");
+        w->writer = (int16_t)f->wave;
+        w->issued = e;
+        w->waited = -1;
+    }
+}
+
+void note_dma_landed(const Fiber* f, const void* p, int bytes) {
+    WordState* w = word_state(p);
+    for (int i = 0; i < bytes / 4; ++i, ++w)
+        if (w->workgroup == g_workgroup_serial && w->writer == f->wave && w->waited < 0) w->waited = (int32_t)f->bar_gen;
 }
 
 void wait_until(const int* counter, const int* target) {
@@ -325,6 +404,7 @@ uint64_t ds_read_tr16_b64(const void* lds_ptr) {
     const uint64_t addr = reinterpret_cast<uint64_t>(lds_ptr);
     std::memcpy(payload + 16, &addr, 8);
     const View v = exchange(K_TR, payload, sizeof payload);
+    note_lds_read(lds_ptr, 8);
     const int lane = g_cur->lane, row0 = lane & ~15, j = lane & 15;
     if (first_live_lane(v, lane)) {
         g_lds_stats[2] += 1;
@@ -352,6 +432,7 @@ u32x4 lds_read_b128(const void* lds_ptr) {
         g_lds_stats[0] += 1;
         g_lds_stats[1] += conflict_cycles(v, 16, 16);
     }
+    note_lds_read(lds_ptr, 16);
     u32x4 r;
     std::memcpy(&r, lds_ptr, 16);
     return r;
@@ -443,6 +524,7 @@ void buffer_load_lds(BufferRsrc r, void* lds_base, int size, int voffset, int so
     const uint64_t off = (uint64_t)(uint32_t)voffset + (uint64_t)(uint32_t)soffset + (uint64_t)(uint32_t)imm;
     if (voffset < 0) fail("buffer_load_lds: negative lane offset");
     const bool inside = off + (uint64_t)size <= (uint64_t)r.num_records;
+    note_dma_issue(dst, size);
     PendingDma d{dst, inside ? r.base + off : nullptr, size};
     if (g_dma_late) f->dma.push_back(d);
     else {
@@ -483,6 +565,7 @@ void launch(dim3 grid, dim3 block, const std::function<void()>& body) {
             for (unsigned bx = 0; bx < grid.x && g_status == hipSuccess; ++bx) {
                 blockIdx = dim3(bx, by, bz);
                 std::memset(__start_simt_lds, 0xFF, (size_t)(__stop_simt_lds - __start_simt_lds));
+                reset_word_states();
                 Block& b = g_block;
                 b.fibers.assign(n, Fiber());
                 b.waves.assign(n_waves, Wave());

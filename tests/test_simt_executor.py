@@ -59,6 +59,23 @@ def test_direct_to_lds_load_without_wait_is_exposed(lib):
     S.configure(False, 1)
 
 
+def test_lds_traffic_of_two_wavefronts_needs_a_barrier_between(lib):
+    src = S.guarded(np.arange(2048, dtype=np.uint16).view(np.uint8)[:2048].copy())
+    for seed in (1, 2, 3, 4):
+        for late in (False, True):
+            S.configure(late, seed)
+            dst = np.zeros(1024, np.uint8)
+            assert lib.simt_selftest_lds_ordering(C.c_void_p(src.ctypes.data), C.c_void_p(dst.ctypes.data), 0) == 0
+            assert np.array_equal(dst, src[:1024])
+            # no barrier between the wait for a load and another wavefront's read of its data
+            text = failing(lib, lib.simt_selftest_lds_ordering, C.c_void_p(src.ctypes.data), C.c_void_p(dst.ctypes.data), 1)
+            assert "direct-to-LDS load" in text and "another wavefront" in text
+            # a load into LDS that the other wavefront reads in the same barrier interval
+            text = failing(lib, lib.simt_selftest_lds_ordering, C.c_void_p(src.ctypes.data), C.c_void_p(dst.ctypes.data), 2)
+            assert "direct-to-LDS load" in text and "another wavefront" in text
+    S.configure(False, 1)
+
+
 def test_matrix_instruction_equals_matmul(lib):
     rng = np.random.default_rng(5)
     a = rng.integers(-8, 9, (32, 16)).astype(np.float32)
