@@ -87,37 +87,42 @@ long g_switches = 0;
 long g_lds_stats[4] = {0, 0, 0, 0};  // 16-byte reads, their conflict cycles, transposing reads, theirs
 
 // ---- ordering of LDS traffic between wavefronts ----------------------------------------------------
-// A work-item's epoch is the number of workgroup barriers it has passed.  Per 4-byte word of LDS: which
-// wavefront last wrote it with a direct-to-LDS load, in which epoch the load was issued and in which epoch
-// the issuing lane waited for it (-1: not yet), and per wavefront the last epoch in which it read the word
-// with one of the traced reads (16-byte operand reads, transposing reads).  Two accesses of different
-// wavefronts to one word, one of them a load's write, are ordered only by a barrier between them; a load
-// is "between" its issue and its wait.  Plain C++ accesses to LDS are not seen.
+// A work-item's epoch is the number of workgroup barriers it has passed (at any moment all running
+// work-items of a workgroup are in the same epoch).  Per 8-byte granule of LDS: which wavefront last wrote
+// it with a direct-to-LDS load and in which epoch the issuing lane waited for it (-1: not yet), and which
+// wavefronts have read it with one of the traced reads (16-byte operand reads, transposing reads) in the
+// latest epoch it was read in.  Two accesses of different wavefronts to one granule, one of them a load's
+// write, are ordered only by a barrier between them; a load is "between" its issue and its wait.  Plain
+// C++ accesses to LDS are not seen.
 constexpr int kMaxWaves = 16;
-struct WordState {
+constexpr int kGranule = 8;
+struct GranuleState {
     uint64_t workgroup = 0;  // serial number of the workgroup this state belongs to; older states count as fresh
+    int32_t waited = -1;
+    int32_t read_epoch = -1;
     int16_t writer = -1;
-    int32_t issued = 0, waited = -1;
-    int32_t read_epoch[kMaxWaves];
+    uint16_t readers = 0;    // wavefronts that read it in read_epoch
 };
-std::vector<WordState> g_words;
+std::vector<GranuleState> g_granules;
 uint64_t g_workgroup_serial = 0;
 
-void reset_word_states() {
+void reset_granule_states() {
     ++g_workgroup_serial;
-    const size_t n = (size_t)(__stop_simt_lds - __start_simt_lds) / 4;
-    if (g_words.size() != n) g_words.assign(n, WordState());
+    const size_t n = (size_t)(__stop_simt_lds - __start_simt_lds + kGranule - 1) / kGranule;
+    if (g_granules.size() != n) g_granules.assign(n, GranuleState());
 }
-WordState* word_state(const void* p) {
-    WordState* w = &g_words[(size_t)(static_cast<const unsigned char*>(p) - __start_simt_lds) / 4];
-    return w;
-}
-void freshen(WordState* w) {
-    if (w->workgroup == g_workgroup_serial) return;
-    w->workgroup = g_workgroup_serial;
-    w->writer = -1;
-    w->waited = -1;
-    for (int& e : w->read_epoch) e = -1;
+// The states of the granules that [p, p + bytes) touches, made fresh if they belong to an earlier workgroup.
+GranuleState* granules_of(const void* p, int bytes, int* count) {
+    const size_t off = (size_t)(static_cast<const unsigned char*>(p) - __start_simt_lds);
+    const size_t first = off / kGranule, last = (off + (size_t)bytes - 1) / kGranule;
+    *count = (int)(last - first + 1);
+    GranuleState* g = &g_granules[first];
+    for (int i = 0; i < *count; ++i)
+        if (g[i].workgroup != g_workgroup_serial) {
+            g[i] = GranuleState();
+            g[i].workgroup = g_workgroup_serial;
+        }
+    return g;
 }
 
 uint64_t next_rand() {
@@ -200,17 +205,21 @@ void flush_dma(Fiber* f, size_t leave = 0) {
 void note_lds_read(const void* p, int bytes) {
     Fiber* f = g_cur;
     const int e = (int)f->bar_gen;
-    WordState* w = word_state(p);
-    for (int i = 0; i < bytes / 4; ++i, ++w) {
-        freshen(w);
-        if (w->writer >= 0) {
-            if (w->waited < 0)
-                fail(w->writer == f->wave ? "LDS read of a direct-to-LDS load that its wavefront has not waited for"
+    int n;
+    GranuleState* g = granules_of(p, bytes, &n);
+    for (int i = 0; i < n; ++i, ++g) {
+        if (g->writer >= 0) {
+            if (g->waited < 0)
+                fail(g->writer == f->wave ? "LDS read of a direct-to-LDS load that its wavefront has not waited for"
                                           : "LDS read of a direct-to-LDS load of another wavefront that is still in flight");
-            else if (w->writer != f->wave && w->waited >= e)
+            else if (g->writer != f->wave && g->waited >= e)
                 fail("LDS read races with a direct-to-LDS load of another wavefront: no barrier between the wait for the load and the read");
         }
-        if (f->wave < kMaxWaves) w->read_epoch[f->wave] = e;
+        if (g->read_epoch != e) {
+            g->read_epoch = e;
+            g->readers = 0;
+        }
+        if (f->wave < kMaxWaves) g->readers |= (uint16_t)(1u << f->wave);
     }
 }
 
@@ -218,24 +227,24 @@ void note_lds_read(const void* p, int bytes) {
 void note_dma_issue(const void* p, int bytes) {
     Fiber* f = g_cur;
     const int e = (int)f->bar_gen;
-    WordState* w = word_state(p);
-    for (int i = 0; i < bytes / 4; ++i, ++w) {
-        freshen(w);
-        for (int v = 0; v < kMaxWaves; ++v)
-            if (v != f->wave && w->read_epoch[v] == e)
-                fail("direct-to-LDS load overwrites LDS that another wavefront has read since the last barrier");
-        if (w->writer >= 0 && w->writer != f->wave && (w->waited < 0 || w->waited >= e))
+    const uint16_t me = f->wave < kMaxWaves ? (uint16_t)(1u << f->wave) : 0;
+    int n;
+    GranuleState* g = granules_of(p, bytes, &n);
+    for (int i = 0; i < n; ++i, ++g) {
+        if (g->read_epoch == e && (g->readers & ~me) != 0)
+            fail("direct-to-LDS load overwrites LDS that another wavefront has read since the last barrier");
+        if (g->writer >= 0 && g->writer != f->wave && (g->waited < 0 || g->waited >= e))
             fail("direct-to-LDS loads of two wavefronts write the same LDS without a barrier between them");
-        w->writer = (int16_t)f->wave;
-        w->issued = e;
-        w->waited = -1;
+        g->writer = (int16_t)f->wave;
+        g->waited = -1;
     }
 }
 
 void note_dma_landed(const Fiber* f, const void* p, int bytes) {
-    WordState* w = word_state(p);
-    for (int i = 0; i < bytes / 4; ++i, ++w)
-        if (w->workgroup == g_workgroup_serial && w->writer == f->wave && w->waited < 0) w->waited = (int32_t)f->bar_gen;
+    int n;
+    GranuleState* g = granules_of(p, bytes, &n);
+    for (int i = 0; i < n; ++i, ++g)
+        if (g->writer == f->wave && g->waited < 0) g->waited = (int32_t)f->bar_gen;
 }
 
 void wait_until(const int* counter, const int* target) {
@@ -565,7 +574,7 @@ void launch(dim3 grid, dim3 block, const std::function<void()>& body) {
             for (unsigned bx = 0; bx < grid.x && g_status == hipSuccess; ++bx) {
                 blockIdx = dim3(bx, by, bz);
                 std::memset(__start_simt_lds, 0xFF, (size_t)(__stop_simt_lds - __start_simt_lds));
-                reset_word_states();
+                reset_granule_states();
                 Block& b = g_block;
                 b.fibers.assign(n, Fiber());
                 b.waves.assign(n_waves, Wave());
