@@ -1,11 +1,13 @@
 """Grouped-head decode on the matrix-core kernel, on the GPU through the C ABI, against the CPU oracle fed a pool
 whose heads are repeated (the definition of grouped heads).  16 and 32 query heads per pool head exist on this
 kernel only; 4 and 8 take it when AHPC_DECODE_MFMA=1.  Collected after the established GPU tests on purpose:
-this kernel is newer than they are."""
+this kernel is newer than they are, and the tests that launch it wait for a first run by hand
+(gpu_util.first_hardware_run)."""
 import numpy as np
 import pytest
 
 from oracle import oracle as O
+from gpu_util import first_hardware_run
 from test_gpu_paged import build_problem, poison_unused, gpu_decode  # noqa: F401  (builders; gpu_decode documents the call)
 
 pytestmark = pytest.mark.gpu
@@ -37,6 +39,7 @@ def run(hip, q, kp, vp, table, lens, B, H, H_kv, d, P, dtype, qo_dtype, scale, c
     return to_host(do)
 
 
+@first_hardware_run
 @pytest.mark.parametrize("dtype,d", [(O.F16, 128), (O.BF16, 64), (O.BF16, 128)])
 @pytest.mark.parametrize("G", [4, 8, 16, 32])
 def test_matrix_core_decode_equals_repeated_heads(gpu, G, dtype, d, monkeypatch):
@@ -58,6 +61,7 @@ def test_matrix_core_decode_equals_repeated_heads(gpu, G, dtype, d, monkeypatch)
         assert np.abs(got - want).max() <= 2e-2, (chunk, qo)
 
 
+@first_hardware_run
 def test_both_kernels_agree_for_groups_of_four(gpu, monkeypatch):
     B, H_kv, d, P, G = 3, 8, 128, 16, 4
     H = G * H_kv
