@@ -73,12 +73,11 @@ def test_dense_vectors(path):
             assert np.abs(got - c[name]).max() <= 1e-4, name
 
 
-@pytest.mark.parametrize("path", [f for f in FILES if "decode" in os.path.basename(f)], ids=os.path.basename)
-def test_decode_vectors(path):
-    c = load(path)
+def decode_inputs(c):
+    """Rebuilds the decode problem of a fixture: queries, the two pools (fp32, `Hkv` heads per token), block table, lengths."""
     H, Hkv, d, P = (int(x) for x in c["shape"])
-    lens, seed, scale = c["lens"].astype(np.int32), int(c["seed"]), float(c["scale"])
-    B, g = len(lens), H // Hkv
+    lens, seed = c["lens"].astype(np.int32), int(c["seed"])
+    B = len(lens)
     q = O.fill_normal((B, H, d), seed, 1)
     pages_per = (lens + P - 1) // P
     n_pages = int(pages_per.sum()) + 3
@@ -93,6 +92,14 @@ def test_decode_vectors(path):
         kb = O.fill_normal((int(n), Hkv, d), seed + 10 + b, 2)
         vb = O.fill_normal((int(n), Hkv, d), seed + 10 + b, 3)
         O.kv_scatter(kb, vb, kp, vp, table, b, 0, P, Hkv, d)
+    return (B, H, Hkv, d, P), q, kp, vp, table, lens
+
+
+@pytest.mark.parametrize("path", [f for f in FILES if "decode" in os.path.basename(f)], ids=os.path.basename)
+def test_decode_vectors(path):
+    c = load(path)
+    (B, H, Hkv, d, P), q, kp, vp, table, lens = decode_inputs(c)
+    scale, g = float(c["scale"]), H // Hkv
     rep = lambda pool: np.repeat(pool.reshape(-1, Hkv, d), g, axis=1).reshape(-1)
     o = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
     assert np.abs(o - c["o"]).max() <= 2e-6
