@@ -167,7 +167,8 @@ static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream
     }
     if (int rc = flash_plan_launch(p, B, causal)) return rc;
     dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
-    // AHPC_FLASH_VARIANT = 1 (L2 warm-up), 2 (issue priority) or 3 (both): tuning variants of the dense kernel
+    // AHPC_FLASH_VARIANT = 1 (L2 warm-up), 2 (issue priority by phase), 3 (both), 4 (issue priority by workgroup role)
+    // or 6 (by phase, then by role): tuning variants of the dense kernel
     // that compute the same results (see flash_fwd_mfma_body)
     if constexpr (!VARLEN) {
         const char* e = std::getenv("AHPC_FLASH_VARIANT");
@@ -181,6 +182,8 @@ static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream
         AHPC_LAUNCH_VARIANT(1)
         AHPC_LAUNCH_VARIANT(2)
         AHPC_LAUNCH_VARIANT(3)
+        AHPC_LAUNCH_VARIANT(4)
+        AHPC_LAUNCH_VARIANT(6)
 #undef AHPC_LAUNCH_VARIANT
     }
     if (causal) hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, true, VARLEN>), grid, block, 0, stream, p);

@@ -215,13 +215,32 @@ struct FlashStatsOut {
 //   kVariantPriority  a wavefront raises its issue priority (s_setprio) while it feeds the matrix cores and
 //                     lowers it for the stretch of pure softmax arithmetic, so that of the two wavefronts that
 //                     share a SIMD the one with matrix instructions ready goes first.
+//   kVariantRole      the two workgroups that share a CU get different issue priorities for their whole life:
+//                     the one whose LDS allocation starts at offset 0 goes first whenever both have an
+//                     instruction of a kind ready, the other one fills the gaps.  Two equal wavefronts on a
+//                     SIMD that are served in turn stay in step (both in their matrix phase, then both in
+//                     their softmax phase) and their times add up; unequal ones drift into opposite phases.
+//                     Together with kVariantPriority the phase decides first (matrix work of either
+//                     wavefront before softmax work of either), the role second.
 constexpr int kVariantTouch = 1;
 constexpr int kVariantPriority = 2;
+constexpr int kVariantRole = 4;
+
+// First 12 bits of the LDS allocation register of the wavefront: the offset of the workgroup's LDS inside
+// the CU's, in allocation granules.  0 for the workgroup that came first (or took the first one's place).
+__device__ inline unsigned lds_allocation_base() {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_s_getreg(6 /* HW_REG_LDS_ALLOC */ | (0 << 6) | ((12 - 1) << 11));
+#else
+    return 0;
+#endif
+}
 
 template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS, int VARIANT = 0>
 __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const FlashStatsOut& st) {
     constexpr bool TOUCH = (VARIANT & kVariantTouch) != 0;
     constexpr bool PRIORITY = (VARIANT & kVariantPriority) != 0;
+    constexpr bool ROLE = (VARIANT & kVariantRole) != 0;
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;  // k-steps of the first product
     constexpr int MB = D / 32;  // 32-row blocks of O^T
@@ -241,6 +260,18 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
 
     const FlashWork work = flash_work_of_block(blockIdx.x, p);
     if (!work.valid) return;
+    // issue priority of this wavefront while it feeds the matrix cores (`busy`) and otherwise
+    bool leads = false;
+    if constexpr (ROLE) leads = lds_allocation_base() == 0;
+    auto set_priority = [&](bool busy) {
+        if constexpr (ROLE && PRIORITY) {
+            if (busy) { if (leads) __builtin_amdgcn_s_setprio(3); else __builtin_amdgcn_s_setprio(2); }
+            else { if (leads) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0); }
+        } else if constexpr (PRIORITY) {
+            if (busy) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0);
+        }
+    };
+    if constexpr (ROLE && !PRIORITY) { if (leads) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(0); }
     const int bh = work.bh;
     const int slot = work.slot;
     const int b = bh / p.H;
@@ -367,7 +398,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
             // ---- S^T = c*K Q^T - m  (log2 units).  The two 32-key blocks alternate, kAhead operand
             //      pairs are requested before the first product and one more after every two products.
             f32x16 s[2];
-            if constexpr (PRIORITY) __builtin_amdgcn_s_setprio(1);
+            set_priority(true);
             {
                 u32x4 a0[KS], a1[KS];
 #pragma unroll
@@ -400,7 +431,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                 vf[0][mb][1] = TrRead<T>::load(tile_v + v_off[mb] + 8 * RB);
             }
 
-            if constexpr (PRIORITY) __builtin_amdgcn_s_setprio(0);
+            set_priority(false);
             const bool need_mask = (k0 + kFlashKeys > L) || (CAUSAL && (k0 + kFlashKeys - 1 > qw));
             if (need_mask) {
                 // key = k0 + 4*half + off(kb, r); visible iff key <= min(qrow, L-1)  <=>  off <= lim
@@ -454,7 +485,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                 }
             };
             make_pb(0);
-            if constexpr (PRIORITY) __builtin_amdgcn_s_setprio(1);
+            set_priority(true);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
@@ -472,7 +503,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if constexpr (PRIORITY) __builtin_amdgcn_s_setprio(0);
+            set_priority(false);
             l_run += sum;
         };
 
@@ -575,7 +606,7 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
     flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, false>(p, FlashStatsOut{});
 }
 
-// The tuning variants described at flash_fwd_mfma_body (dense batches; AHPC_FLASH_VARIANT = 1, 2 or 3).
+// The tuning variants described at flash_fwd_mfma_body (dense batches; AHPC_FLASH_VARIANT = 1 ... 7, a sum of the bits).
 template <typename T, int D, bool CAUSAL, int VARIANT>
 __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_variant_kernel(const FlashParams p) {
     flash_fwd_mfma_body<T, D, CAUSAL, false, false, VARIANT>(p, FlashStatsOut{});

@@ -191,6 +191,9 @@ inline hipError_t hipGetLastError() { return ::simt::last_error(); }
 #define __builtin_amdgcn_sched_group_barrier(a, b, c) ((void)0)
 #define __builtin_amdgcn_sched_barrier(a) ((void)0)
 #define __builtin_amdgcn_s_setprio(a) ((void)0)
+// hardware register reads: the only one the kernels use is the LDS allocation base, which the executor answers with
+// 0 for even workgroups and a non-zero offset for odd ones (both roles of a pair of workgroups get exercised)
+#define __builtin_amdgcn_s_getreg(which) ((unsigned)((blockIdx.x & 1u) * 64u))
 #define __builtin_amdgcn_exp2f(x) exp2f(x)
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))
 #define __builtin_amdgcn_fdot2(a, b, c, clamp) ::simt::fdot2_f16((a), (b), (c))

@@ -446,13 +446,15 @@ def test_backward_ragged_batch(emu, dtype, d, H, H_kv, causal):
         check_gradients(tuple(g[a:b][None] for g in got), want, dtype)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 6])
 @pytest.mark.parametrize("dma_late", [False, True])
 @pytest.mark.parametrize("dtype,N,d,causal", [(O.BF16, 700, 128, True), (O.F16, 520, 64, False), (O.BF16, 129, 128, True),
                                              (O.F16, 64, 128, False)])
 def test_forward_tuning_variants_compute_the_same(emu, dtype, N, d, causal, dma_late, variant, monkeypatch):
     """AHPC_FLASH_VARIANT: 1 requests the tile after next a step early (and leaves that request outstanding at the
-    end-of-step wait), 2 changes issue priorities, 3 does both.  Results must be bit-identical."""
+    end-of-step wait), 2 changes issue priorities by phase, 3 does both, 4 gives the two workgroups of a CU different
+    priorities (the executor tells even workgroups that they came first and odd ones that they did not), 6 = 2 + 4.
+    Results must be bit-identical."""
     B, H = 1, 2
     q, k, v = qkv((B, N, H, d), 27, dtype)
     plain = flash(emu, q, k, v, dtype, B, N, H, d, 0.1, causal)
