@@ -62,6 +62,7 @@ struct FlashParams {
     int32_t blocks_per_xcd;     // ceil(total_blocks / 8)
     int32_t heads_together;     // <= 1: a head's workgroups are consecutive; n: n heads advance side by side
     int32_t round_slots;        // with heads_together > 1: workgroups one head contributes per round
+    int32_t pingpong_low_bit;   // alternating variant only: 1 = wavefronts w and w^1 form a pair (default: w and w+4)
     float scale_log2;           // scale * log2(e)
 };
 

@@ -168,6 +168,7 @@ inline hipError_t hipEventElapsedTime(float* ms, hipEvent_t, hipEvent_t) { *ms =
 inline hipError_t hipGetLastError() { return ::simt::last_error(); }
 
 #define __syncthreads() ::simt::syncthreads()
+#define __builtin_amdgcn_s_barrier() ::simt::syncthreads()
 #define __shfl_xor(x, mask, width) ::simt::shfl_xor((x), (mask), (width))
 #define __expf(x) expf(x)
 

@@ -524,3 +524,50 @@ def test_wide_forward_kernel_grouped_and_paired(emu, monkeypatch):
     q, k, v = qkv((B, N, H, d), 22, O.F16)
     got = flash(emu, q, k, v, O.F16, B, N, H, d, 0.125, True)
     assert np.abs(got - O.attention(q, k, v, B, N, H, d, 0.125, True)).max() <= 2e-2
+
+
+# ---- forward, alternating variant (8 wavefronts, two groups in opposite phases; AHPC_FLASH_PINGPONG=1 or 2) ---
+@pytest.mark.parametrize("mode", ["1", "2"])
+@pytest.mark.parametrize("dma_late", [False, True])
+@pytest.mark.parametrize("dtype,N,d,causal", [(O.BF16, 64, 128, False), (O.F16, 129, 128, True), (O.BF16, 300, 64, True),
+                                             (O.F16, 520, 64, False), (O.BF16, 1, 128, True), (O.BF16, 700, 128, True),
+                                             (O.F16, 257, 128, False)])
+def test_alternating_forward_kernel(emu, dtype, N, d, causal, dma_late, mode, monkeypatch):
+    """Parity with the oracle and bit-identity with the standard kernel (same arithmetic in the same order per
+    wavefront; only the schedule differs), with tile requests that land as late as their wait allows, under the
+    executor's LDS ordering check (every tile request against every operand read, by barrier epochs)."""
+    B, H = 2, 2
+    q, k, v = qkv((B, N, H, d), 29, dtype)
+    scale = 1.0 / np.sqrt(d)
+    plain = flash(emu, q, k, v, dtype, B, N, H, d, scale, causal)
+    monkeypatch.setenv("AHPC_FLASH_PINGPONG", mode)
+    S.configure(dma_late, seed=N + d)
+    S.lds_stats(reset=True)
+    try:
+        got = flash(emu, q, k, v, dtype, B, N, H, d, scale, causal, front=dma_late)
+    finally:
+        S.configure(False, 1)
+    assert np.isfinite(got).all()
+    assert np.abs(got - O.attention(q, k, v, B, N, H, d, scale, causal)).max() <= TOL[dtype]
+    assert np.array_equal(got, plain)
+    reads, read_conflicts, tr, tr_conflicts = S.lds_stats(reset=True)
+    assert read_conflicts == 0 and tr_conflicts == 0
+
+
+def test_alternating_forward_kernel_grouped_and_paired(emu, monkeypatch):
+    monkeypatch.setenv("AHPC_FLASH_PINGPONG", "1")
+    # grouped heads
+    B, N, H, H_kv, d = 1, 300, 4, 2, 128
+    q = O.round_to(O.fill_normal((B, N, H, d), 21, 1), O.BF16)
+    k = O.round_to(O.fill_normal((B, N, H_kv, d), 21, 2), O.BF16)
+    v = O.round_to(O.fill_normal((B, N, H_kv, d), 21, 3), O.BF16)
+    got = flash(emu, q, k, v, O.BF16, B, N, H, d, 0.1, True, H_kv=H_kv)
+    want = O.attention(q, np.repeat(k, 2, axis=2), np.repeat(v, 2, axis=2), B, N, H, d, 0.1, True)
+    assert np.abs(got - want).max() <= 2e-2
+    # a workgroup that takes a late query tile and then an early one of the same head (odd tile count: the middle
+    # one has no partner); the pairing threshold is lowered so that a small problem pairs
+    monkeypatch.setenv("AHPC_FLASH_PAIR_MIN", "1")
+    B, N, H, d = 1, 1100, 1, 64
+    q, k, v = qkv((B, N, H, d), 22, O.F16)
+    got = flash(emu, q, k, v, O.F16, B, N, H, d, 0.125, True)
+    assert np.abs(got - O.attention(q, k, v, B, N, H, d, 0.125, True)).max() <= 2e-2
