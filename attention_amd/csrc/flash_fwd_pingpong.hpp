@@ -145,7 +145,7 @@ __global__ __launch_bounds__(kPingPongThreads, 1) void flash_fwd_pingpong_kernel
         request(gk, dma_off_k, 0, lds_k0);  // K(0), before anything else
 
         // ---- Q^T operands, pre-multiplied by c = scale*log2(e) ------------------------------------
-        const int qw = q_tile0 + wave * 32;
+        const int qw = q_tile0 + wave_u * 32;  // first query row of this wavefront (a scalar: conditions on it are branches)
         const int qrow = qw + col;
         u32x4 qreg[KS];
         {
@@ -296,6 +296,9 @@ __global__ __launch_bounds__(kPingPongThreads, 1) void flash_fwd_pingpong_kernel
         };
         // Matrix phase of tile t: the second product of tile t-1 (its V is in the other buffer), the first of tile t.
         auto matrix_phase = [&](int t, const unsigned char* k_cur, const unsigned char* v_prev) __attribute__((always_inline)) {
+            // the wavefront that feeds the matrix cores goes first when its SIMD has to choose: the other one's
+            // softmax arithmetic fits into the shadow of the matrix instructions
+            __builtin_amdgcn_s_setprio(1);
             if (active(t - 1)) weighted_values(v_prev);
             __builtin_amdgcn_sched_barrier(0);
             if (active(t)) {
@@ -307,6 +310,7 @@ __global__ __launch_bounds__(kPingPongThreads, 1) void flash_fwd_pingpong_kernel
                 for (int r = 0; r < 16; ++r) s[0][r] = s[1][r] = 0.0f;
             }
             __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(0);
         };
 
         // One tile of either group.  (k_cur, v_cur): buffers of parity t; (k_nxt, v_nxt): of parity t+1, which
