@@ -74,6 +74,7 @@ SIGNATURES = {
     "ahpc_hip_paged_decode": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp, _sz, _vp]),
     "ahpc_hip_paged_decode_gqa": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp, _sz, _vp]),
     "ahpc_hip_paged_gather_indices": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp]),
+    "ahpc_hip_probe_matrix_rate": (_ci, [_ci, _ci, _i64, _i64, _vp, _sz, C.POINTER(C.c_double), _vp]),
 }
 
 _lib = None
@@ -213,3 +214,11 @@ def paged_decode_gqa(q, o, qo_dtype, k_pool, v_pool, pool_dtype, table, seq_lens
 def paged_gather_indices(table, seq_lens, batch_rows, B, H, d, P, max_pages, max_len, offsets, stream=None):
     _check(load().ahpc_hip_paged_gather_indices(table, seq_lens, batch_rows, B, H, d, P, max_pages, max_len, offsets,
                                                stream), "paged_gather_indices")
+
+
+def probe_matrix_rate(dtype, mix, workgroups, iterations, sink, sink_bytes, stream=None):
+    """Launches the matrix-rate calibration kernel; returns the floating-point operations of the launch."""
+    flop = C.c_double(0.0)
+    _check(load().ahpc_hip_probe_matrix_rate(dtype, mix, workgroups, iterations, sink, sink_bytes, C.byref(flop), stream),
+           "probe_matrix_rate")
+    return flop.value

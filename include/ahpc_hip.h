@@ -288,6 +288,18 @@ int ahpc_hip_paged_gather_indices(const int32_t* block_table, const int32_t* seq
                                   int64_t B, int64_t H, int64_t d, int64_t P, int64_t max_pages, int64_t max_len,
                                   int64_t* offsets, void* stream);
 
+/* ---- calibration ------------------------------------------------------------------------------------
+ * One launch that does nothing but matrix instructions on register operands: `workgroups` workgroups of 4
+ * wavefronts, each wavefront `iterations` x 4 independent v_mfma_f32_32x32x16 of `dtype` (AHPC_F16 / AHPC_BF16);
+ * mix = 1 adds the VALU work of a softmax between them (an exponential, two additions, a maximum, a packing
+ * conversion and a bit operation per matrix instruction: somewhat more than the flash forward's).  *flop (optional) receives the floating-point operations of the launch;
+ * the caller times it (events on `stream`).  sink: workgroups * 256 floats of device memory that receive the
+ * accumulators' sums, so that the work cannot be optimised away.  Measures what "matrix-bound" means on the box
+ * in hand, next to the published peak.  No counterpart in the reference (its benchmark,
+ * benchmarks/benchmark_attention.cpp:129-255, times whole attention calls only). */
+int ahpc_hip_probe_matrix_rate(int dtype, int mix, int64_t workgroups, int64_t iterations, float* sink,
+                               size_t sink_bytes, double* flop, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

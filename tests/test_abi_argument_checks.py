@@ -115,3 +115,13 @@ def test_error_strings_cover_every_code(lib):
         seen.add(text)
     assert len(seen) == 9
     assert hip.error_string(-99) == "unknown error code"
+
+
+def test_calibration_probe_argument_checks(lib):
+    probe = lambda dtype=F16, mix=0, wgs=4, it=10, sink=P, nbytes=4 * 256 * 4: lib.ahpc_hip_probe_matrix_rate(
+        dtype, mix, wgs, it, sink, nbytes, None, None)
+    assert probe(sink=None) == NULL_POINTER
+    assert probe(dtype=0) == BAD_DTYPE and probe(dtype=7) == BAD_DTYPE
+    for bad in (dict(wgs=0), dict(it=0), dict(mix=2), dict(it=1 << 25), dict(wgs=1 << 21)):
+        assert probe(**bad) == BAD_SHAPE, bad
+    assert probe(nbytes=4 * 256 * 4 - 1) == WORKSPACE

@@ -571,3 +571,18 @@ def test_alternating_forward_kernel_grouped_and_paired(emu, monkeypatch):
     q, k, v = qkv((B, N, H, d), 22, O.F16)
     got = flash(emu, q, k, v, O.F16, B, N, H, d, 0.125, True)
     assert np.abs(got - O.attention(q, k, v, B, N, H, d, 0.125, True)).max() <= 2e-2
+
+
+# ---- calibration probe -------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16])
+@pytest.mark.parametrize("mix", [0, 1])
+def test_matrix_rate_probe_runs_and_counts_its_work(emu, dtype, mix):
+    """The probe has no result worth checking beyond being finite and written by every lane; its operation count is
+    what the benchmark divides by the measured time."""
+    import ctypes as C
+    wgs, it = 2, 3
+    sink = S.guarded(np.full(wgs * 256, np.nan, np.float32))
+    flop = C.c_double(0.0)
+    assert S.load().ahpc_hip_probe_matrix_rate(dtype, mix, wgs, it, S.ptr(sink), sink.nbytes, C.byref(flop), None) == 0
+    assert np.isfinite(sink).all()
+    assert flop.value == 2.0 * 32 * 32 * 16 * 4 * it * 4 * wgs
