@@ -167,17 +167,17 @@ static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream
         }
     }
     // AHPC_FLASH_PINGPONG=1 (or 2: the other pairing of wavefronts): the experimental variant with one workgroup of 8
-    // wavefronts per CU whose two halves alternate between matrix and softmax phases (flash_fwd_pingpong.hpp; dense
-    // batches only).  Same results; not the default until it has been timed.
-    if constexpr (!VARLEN) {
+    // wavefronts per CU whose two halves alternate between matrix and softmax phases (flash_fwd_pingpong.hpp).
+    // Same results; not the default until it has been timed.
+    {
         const char* pp = std::getenv("AHPC_FLASH_PINGPONG");
         const int mode = pp ? std::atoi(pp) : 0;
         if (mode == 1 || mode == 2) {
             if (int rc = flash_plan_launch(p, B, causal, kPingPongRows)) return rc;
             p.pingpong_low_bit = mode == 2 ? 1 : 0;
             dim3 pgrid((unsigned)(p.blocks_per_xcd * 8)), pblock(kPingPongThreads);
-            if (causal) hipLaunchKernelGGL((flash_fwd_pingpong_kernel<T, D, true>), pgrid, pblock, 0, stream, p);
-            else hipLaunchKernelGGL((flash_fwd_pingpong_kernel<T, D, false>), pgrid, pblock, 0, stream, p);
+            if (causal) hipLaunchKernelGGL((flash_fwd_pingpong_kernel<T, D, true, VARLEN>), pgrid, pblock, 0, stream, p);
+            else hipLaunchKernelGGL((flash_fwd_pingpong_kernel<T, D, false, VARLEN>), pgrid, pblock, 0, stream, p);
             return static_cast<int>(hipGetLastError());
         }
     }

@@ -30,8 +30,8 @@
 // Which wavefronts form a group: waves w and w+4 of a workgroup are taken to share a SIMD (group = w / 4);
 // FlashParams::pingpong_low_bit = 1 pairs w and w^1 instead (group = w % 2).
 //
-// Selected with AHPC_FLASH_PINGPONG=1 (or 2 for the other pairing); dense batches; the standard kernel stays the
-// default until both have been timed.
+// Selected with AHPC_FLASH_PINGPONG=1 (or 2 for the other pairing); dense and ragged batches; the standard kernel
+// stays the default until both have been timed.
 #pragma once
 
 #include <type_traits>
@@ -50,7 +50,7 @@ __device__ inline void bare_barrier() {
     asm volatile("" ::: "memory");
 }
 
-template <typename T, int D, bool CAUSAL>
+template <typename T, int D, bool CAUSAL, bool VARLEN>
 __global__ __launch_bounds__(kPingPongThreads, 1) void flash_fwd_pingpong_kernel(const FlashParams p) {
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;
@@ -77,9 +77,18 @@ __global__ __launch_bounds__(kPingPongThreads, 1) void flash_fwd_pingpong_kernel
     const int h = bh - b * p.H;
     const int hk = h / p.kv_group;
 
-    const int L = p.N;
-    const int64_t base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
-    const int64_t kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
+    int L;
+    int64_t base, kv_base;
+    if (VARLEN) {  // packed sequences: this one's tokens start at cu_seqlens[b]
+        const int s0 = p.cu_seqlens[b];
+        L = p.cu_seqlens[b + 1] - s0;
+        base = (int64_t)s0 * p.stride_n + (int64_t)h * p.stride_h;
+        kv_base = (int64_t)s0 * p.kv_stride_n + (int64_t)hk * p.kv_stride_h;
+    } else {
+        L = p.N;
+        base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+        kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
+    }
     const T* const gq = static_cast<const T*>(p.q) + base;
     const T* const gk = static_cast<const T*>(p.k) + kv_base;
     const T* const gv = static_cast<const T*>(p.v) + kv_base;
