@@ -188,12 +188,22 @@ __global__ __launch_bounds__(kPingPongThreads, 1) void flash_fwd_pingpong_kernel
         auto active = [&](int t) __attribute__((always_inline)) { return t >= 0 && t < n_tiles && !(CAUSAL && t * kFlashKeys > qw + 31); };
 
         // ---- S^T = c*K Q^T - m (log2 units) ---------------------------------------------------------
-        auto scores = [&](const unsigned char* tile_k) __attribute__((always_inline)) {
+        // The first product's operands are requested in two goes: the first kAhead pairs early (before the second
+        // product of the previous tile, whose tail then hides their latency), the rest between the matrix instructions.
+        constexpr int kAhead = KS < 4 ? KS : 4;
+        auto scores_head = [&](const unsigned char* tile_k, u32x4* h0, u32x4* h1) __attribute__((always_inline)) {
+#pragma unroll
+            for (int ks = 0; ks < kAhead; ++ks) {
+                h0[ks] = lds_read_b128(tile_k + k_off[ks]);
+                h1[ks] = lds_read_b128(tile_k + 32 * RB + k_off[ks]);
+            }
+        };
+        auto scores = [&](const unsigned char* tile_k, const u32x4* h0, const u32x4* h1) __attribute__((always_inline)) {
             u32x4 a0[KS], a1[KS];
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                a0[ks] = lds_read_b128(tile_k + k_off[ks]);
-                a1[ks] = lds_read_b128(tile_k + 32 * RB + k_off[ks]);
+                a0[ks] = ks < kAhead ? h0[ks] : lds_read_b128(tile_k + k_off[ks]);
+                a1[ks] = ks < kAhead ? h1[ks] : lds_read_b128(tile_k + 32 * RB + k_off[ks]);
             }
             // the products start from accumulators holding -m, so that the matrix core delivers c*s - m (the
             // standard kernel keeps a 16-register copy of -m for this; here the registers are worth more)
@@ -204,12 +214,11 @@ __global__ __launch_bounds__(kPingPongThreads, 1) void flash_fwd_pingpong_kernel
                 s[0] = mfma_32x32x16<T>(a0[ks], qreg[ks], s[0]);
                 s[1] = mfma_32x32x16<T>(a1[ks], qreg[ks], s[1]);
             }
-            constexpr int kAhead = KS < 4 ? KS : 4;
-            __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);  // LDS reads
+            // two matrix instructions, then the next operand pair's reads, until the reads run out
 #pragma unroll
             for (int i = 0; i < KS - kAhead; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // matrix instructions
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // LDS reads
             }
 #pragma unroll
             for (int i = 0; i < kAhead; ++i) __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
@@ -308,10 +317,14 @@ __global__ __launch_bounds__(kPingPongThreads, 1) void flash_fwd_pingpong_kernel
             // the wavefront that feeds the matrix cores goes first when its SIMD has to choose: the other one's
             // softmax arithmetic fits into the shadow of the matrix instructions
             __builtin_amdgcn_s_setprio(1);
+            // the first operands of this tile's first product are requested before the previous tile's second product,
+            // whose matrix instructions then hide their latency
+            u32x4 h0[kAhead], h1[kAhead];
+            const bool act = active(t);
+            if (act) scores_head(k_cur, h0, h1);
             if (active(t - 1)) weighted_values(v_prev);
-            __builtin_amdgcn_sched_barrier(0);
-            if (active(t)) {
-                scores(k_cur);
+            if (act) {
+                scores(k_cur, h0, h1);
             } else {
                 // nobody reads these scores; defining them on this path too tells the register allocator that the
                 // previous tile's scores are dead by now
