@@ -6,7 +6,6 @@
 
 #include "ahpc_device.hpp"
 #include "flash_fwd_mfma.hpp"
-#include "flash_fwd_wide.hpp"
 #include "flash_fwd_pingpong.hpp"
 
 namespace ahpc {
@@ -154,18 +153,6 @@ static int dispatch_simple(int dtype, const SimpleParams& p, int64_t B, hipStrea
 // ---------------------------------------------------------------------------------------------
 template <typename T, int D, bool VARLEN>
 static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
-    // AHPC_FLASH_WIDE=1: the experimental variant in which a wavefront owns 64 query rows (flash_fwd_wide.hpp; dense
-    // batches only).  Same results; not the default until it has been timed.
-    if constexpr (!VARLEN) {
-        const char* wide = std::getenv("AHPC_FLASH_WIDE");
-        if (wide && std::atoi(wide) == 1) {
-            if (int rc = flash_plan_launch(p, B, causal, kWideRows)) return rc;
-            dim3 wgrid((unsigned)(p.blocks_per_xcd * 8)), wblock(kFlashThreads);
-            if (causal) hipLaunchKernelGGL((flash_fwd_wide_kernel<T, D, true, false>), wgrid, wblock, 0, stream, p);
-            else hipLaunchKernelGGL((flash_fwd_wide_kernel<T, D, false, false>), wgrid, wblock, 0, stream, p);
-            return static_cast<int>(hipGetLastError());
-        }
-    }
     // AHPC_FLASH_PINGPONG=1 (or 2: the other pairing of wavefronts): the experimental variant with one workgroup of 8
     // wavefronts per CU whose two halves alternate between matrix and softmax phases (flash_fwd_pingpong.hpp).
     // Same results; not the default until it has been timed.

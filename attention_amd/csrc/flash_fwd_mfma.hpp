@@ -59,6 +59,7 @@ struct FlashParams {
     int32_t n_qtiles;           // query tiles per sequence (of the longest one)
     int32_t paired;             // 1: a workgroup takes two query tiles of a head (see above)
     int32_t total_blocks;       // B * H * n_qtiles, or B * H * ceil(n_qtiles / 2) when paired
+    int32_t n_bh;               // B * H: no workgroup may address a (sequence, head) at or beyond this
     int32_t blocks_per_xcd;     // ceil(total_blocks / 8)
     int32_t heads_together;     // <= 1: a head's workgroups are consecutive; n: n heads advance side by side
     int32_t round_slots;        // with heads_together > 1: workgroups one head contributes per round
@@ -261,6 +262,8 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
 
     const FlashWork work = flash_work_of_block(blockIdx.x, p);
     if (!work.valid) return;
+    // whatever the map says, nothing outside the tensors is ever addressed (uniform per workgroup)
+    if (work.bh < 0 || work.bh >= p.n_bh || work.slot < 0 || work.slot >= flash_per_head(p)) return;
     // issue priority of this wavefront while it feeds the matrix cores (`busy`) and otherwise
     bool leads = false;
     if constexpr (ROLE) leads = lds_allocation_base() == 0;
@@ -588,6 +591,7 @@ inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal, int rows_pe
     p.paired = (causal && p.n_qtiles >= 2 && total * rows_per_workgroup >= pair_min * kFlashRows) ? 1 : 0;
     if (p.paired) total = B * p.H * (int64_t)((p.n_qtiles + 1) / 2);
     p.total_blocks = (int32_t)total;
+    p.n_bh = (int32_t)(B * p.H);
     p.blocks_per_xcd = (int32_t)((total + 7) / 8);
     // AHPC_FLASH_HEADS_TOGETHER = n lets n heads advance side by side on an XCD (default: one after the
     // other); AHPC_FLASH_ROUND_SLOTS sets how many workgroups a head contributes per round (default 64 / n:

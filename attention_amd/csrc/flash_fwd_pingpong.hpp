@@ -71,6 +71,8 @@ __global__ __launch_bounds__(kPingPongThreads, 1) void flash_fwd_pingpong_kernel
 
     const FlashWork work = flash_work_of_block(blockIdx.x, p);
     if (!work.valid) return;
+    // whatever the map says, nothing outside the tensors is ever addressed (uniform per workgroup)
+    if (work.bh < 0 || work.bh >= p.n_bh || work.slot < 0 || work.slot >= flash_per_head(p)) return;
     const int bh = work.bh;
     const int slot = work.slot;
     const int b = bh / p.H;

@@ -14,13 +14,15 @@
 
 namespace ahpc {
 
-// Element offset of (token t, head 0, lane 0) of table row `row`; -1 when the page is missing.
-// Shared by the decode kernel, scatter, gather and the index dump, so that what the dump reports
-// is what decode reads.
+// Element offset of (token t, head 0, element 0) of table row `row`; -1 when the page is missing or the token
+// lies beyond the row's last column.  Used by scatter and gather (append, read-back); the decode kernels do their
+// own address arithmetic (one page id per lane, rows a fixed stride apart) and report it themselves when asked
+// (DecodeParams::dump_offsets).
 __device__ __forceinline__ int64_t kv_token_offset(const int32_t* __restrict__ table, int64_t max_pages, int64_t row,
                                                    int t, int P, int H, int d) {
     const int page_idx = t / P;
     const int pos = t - page_idx * P;
+    if (page_idx >= max_pages) return -1;
     const int page_id = table[row * max_pages + page_idx];
     if (page_id < 0) return -1;
     return (((int64_t)page_id * P + pos) * H) * (int64_t)d;
@@ -139,7 +141,11 @@ __global__ void gather_indices_kernel(const int32_t* __restrict__ table, const i
     const int64_t b = idx / max_len;
     const int t = (int)(idx - b * max_len);
     const int64_t row = batch_rows ? batch_rows[b] : b;
-    offsets[idx] = t < seq_lens[row] ? kv_token_offset(table, max_pages, row, t, P, H, d) : -1;
+    int64_t off = t < seq_lens[row] ? kv_token_offset(table, max_pages, row, t, P, H, d) : -1;
+    // a missing page ends the sequence: nothing behind it is read either
+    for (int pg = 0; off >= 0 && pg < t / P; ++pg)
+        if (table[row * max_pages + pg] < 0) off = -1;
+    offsets[idx] = off;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -153,7 +159,8 @@ struct DecodeParams {
     const int32_t* seq_lens;
     const int32_t* batch_rows;
     float* part_o;    // [B][n_chunks][H][d]
-    float* part_ml;   // [B][n_chunks][H][2]  (m in log2 units, l)
+    float* part_ml;   // [B][n_chunks][H][2]  (m in log2 units, l; l carries a minus sign when the chunk met a missing page)
+    int64_t* dump_offsets;  // index-dump launches only: [B][max_len] element offsets of the token rows the kernel addresses
     int64_t max_pages;
     int32_t B, H, d, P;       // H = query heads
     int32_t H_kv;             // heads in the pool; H / H_kv consecutive query heads share one
@@ -236,7 +243,15 @@ template <int LPH> __device__ __forceinline__ float head_allreduce(float x) {
 // A chunk starts on a page boundary.  Its page ids are fetched once (one table entry per lane) and
 // handed out with v_readlane, so the only per-token address work is a uniform add; K and V rows of
 // the next kDecodeBatch tokens are requested before the current ones are consumed.
-template <typename T, int D, int PT, int G>
+//
+// A table entry of -1 inside a sequence ends the sequence there: keys from that page on are not attended to
+// (the reference kernel leaves its page walk at the first negative id, src/backends/cuda/cuda_kernels.cu:417-420).
+// The chunk that meets it says so through the sign of its partial l, and the merge stops after that chunk.
+//
+// DUMP: nothing is loaded or computed; instead the lane that owns (pool head 0, element 0) stores, for every token
+// row the kernel would read, the element offset of that row in the pool - taken from the very expression the loads
+// use - and -1 for the tokens of its chunk it would not read.  This is what the bit-exact index test compares.
+template <typename T, int D, int PT, int G, bool DUMP = false>
 __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p) {
     constexpr int kDecodeBatch = G >= 4 ? 4 : 8;  // tokens whose K and V rows are in flight together, per lane
     constexpr int EPL = 16 / (int)sizeof(T);
@@ -267,9 +282,16 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     int my_page = 0;
     if (first_page + lane < p.max_pages) my_page = p.table[row * p.max_pages + first_page + lane];
     const int L = p.seq_lens[row] < p.max_len ? p.seq_lens[row] : p.max_len;
+    const bool dumps = DUMP && h_raw == 0 && e0 == 0;  // one lane of the launch's first head group
+    if constexpr (DUMP) {
+        if (dumps) {
+            const int te = (t0 + p.chunk_tokens) < p.max_len ? (t0 + p.chunk_tokens) : p.max_len;
+            for (int t = t0; t < te; ++t) p.dump_offsets[(int64_t)b * p.max_len + t] = -1;
+        }
+    }
     if (t0 >= L) {
         // an empty sequence still owns an output row: zeros (with several chunks the merge writes it)
-        if (chunk == 0 && p.n_chunks == 1 && head_ok) {
+        if (!DUMP && chunk == 0 && p.n_chunks == 1 && head_ok) {
             float zero[EPL];
 #pragma unroll
             for (int e = 0; e < EPL; ++e) zero[e] = 0.0f;
@@ -278,17 +300,26 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
         }
         return;
     }
-    const int t1 = (t0 + p.chunk_tokens) < L ? (t0 + p.chunk_tokens) : L;
+    int t1 = (t0 + p.chunk_tokens) < L ? (t0 + p.chunk_tokens) : L;
+    // first missing page of the chunk, if any: the chunk ends in front of it
+    const unsigned long long missing = __builtin_amdgcn_ballot_w64(lane < (t1 - t0 + P - 1) / P && my_page < 0);
+    const bool stopped = missing != 0;
+    if (stopped) {
+        const int cut = t0 + (int)__builtin_ctzll(missing) * P;
+        t1 = cut < t1 ? cut : t1;
+    }
 
     // query pieces of this lane, one per query head of the group
     float qf[G][EPL];
     uint32_t qp[G][4];
+    if constexpr (!DUMP) {
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        load_qo_vec<EPL>(p.q, p.qo_dtype, ((int64_t)b * p.H + h * G + g) * D + e0, qf[g]);
-        if (kPacked) {
+        for (int g = 0; g < G; ++g) {
+            load_qo_vec<EPL>(p.q, p.qo_dtype, ((int64_t)b * p.H + h * G + g) * D + e0, qf[g]);
+            if (kPacked) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) qp[g][i] = pack2<TP>(qf[g][2 * i], qf[g][2 * i + 1]);
+                for (int i = 0; i < 4; ++i) qp[g][i] = pack2<TP>(qf[g][2 * i], qf[g][2 * i + 1]);
+            }
         }
     }
 
@@ -298,9 +329,9 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     const char* const kbase = static_cast<const char*>(p.k_pool);
     const char* const vbase = static_cast<const char*>(p.v_pool);
 
-    my_page = my_page < 0 ? 0 : my_page;  // a missing page reads page 0 (the host never hands out such a table)
+    my_page = my_page < 0 ? 0 : my_page;  // never dereferenced: the chunk ends in front of its first missing page
 
-    const int n_tok = t1 - t0;
+    const int n_tok = t1 - t0;            // 0 when the chunk's first page is missing
     const int n_batches = (n_tok + kDecodeBatch - 1) / kDecodeBatch;
 
     // Requests the K and V rows of batch `bi` (tokens 8*bi .. 8*bi+7 of the chunk).  Tokens past the
@@ -318,8 +349,12 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
             for (int i = 0; i < kDecodeBatch; ++i) {
                 const int ic = i < last ? i : last;
                 const int64_t off = base + ic * tok_bytes;
-                kr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + off + lane_off));
-                vr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + off + lane_off));
+                if constexpr (DUMP) {
+                    if (dumps && i <= last) p.dump_offsets[(int64_t)b * p.max_len + t0 + ti0 + i] = (off + lane_off) / (int64_t)sizeof(T);
+                } else {
+                    kr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + off + lane_off));
+                    vr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + off + lane_off));
+                }
             }
         } else {
 #pragma unroll
@@ -328,8 +363,12 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
                 const int pg = tc / P;
                 const int page_id = __builtin_amdgcn_readlane(my_page, pg);
                 const int64_t off = ((int64_t)page_id * P + (tc - pg * P)) * tok_bytes;
-                kr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + off + lane_off));
-                vr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + off + lane_off));
+                if constexpr (DUMP) {
+                    if (dumps && i <= last) p.dump_offsets[(int64_t)b * p.max_len + t0 + ti0 + i] = (off + lane_off) / (int64_t)sizeof(T);
+                } else {
+                    kr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + off + lane_off));
+                    vr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + off + lane_off));
+                }
             }
         }
     };
@@ -392,7 +431,11 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
 
     // two register sets in ping-pong: while one batch is consumed the next is in flight
     u32x4 ka[kDecodeBatch], va[kDecodeBatch], kb2[kDecodeBatch], vb2[kDecodeBatch];
-    issue(ka, va, 0);
+    if constexpr (DUMP) {
+        for (int bi = 0; bi < n_batches; ++bi) issue(ka, va, bi);
+        return;
+    }
+    if (n_batches > 0) issue(ka, va, 0);
     for (int bi = 0; bi < n_batches; bi += 2) {
         if (bi + 1 < n_batches) issue(kb2, vb2, bi + 1);
         consume(ka, va, bi);
@@ -419,7 +462,7 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
             for (int e = 0; e < EPL; e += 4) dst[e / 4] = f32x4{acc[g][e], acc[g][e + 1], acc[g][e + 2], acc[g][e + 3]};
             if (lane % LPH == 0) {
                 p.part_ml[slot * 2] = m[g];
-                p.part_ml[slot * 2 + 1] = l[g];
+                p.part_ml[slot * 2 + 1] = stopped ? -l[g] : l[g];  // l >= 0, and -(0.0f) still carries the sign
             }
         }
     }
@@ -442,15 +485,24 @@ __global__ __launch_bounds__(256) void paged_merge_kernel(const DecodeParams p) 
     const float* ml = p.part_ml + ((b * p.n_chunks) * p.H + h) * 2;
     const float* po = p.part_o + ((b * p.n_chunks) * p.H + h) * p.d + e;
     const int64_t ml_step = (int64_t)p.H * 2, po_step = (int64_t)p.H * p.d;
+    // a chunk whose l carries a minus sign met a missing page: it is the last one that counts
     float m = -INFINITY;
-    for (int ci = 0; ci < n; ++ci) m = fmaxf(m, ml[ci * ml_step]);
+    int n_used = n;
+    for (int ci = 0; ci < n; ++ci) {
+        m = fmaxf(m, ml[ci * ml_step]);
+        if (__builtin_bit_cast(uint32_t, ml[ci * ml_step + 1]) >> 31) {
+            n_used = ci + 1;
+            break;
+        }
+    }
     float l = 0.0f, acc = 0.0f;
 #pragma unroll 4
-    for (int ci = 0; ci < n; ++ci) {
+    for (int ci = 0; ci < n_used; ++ci) {
         const float f = fast_exp2(ml[ci * ml_step] - m);
-        l = __builtin_fmaf(ml[ci * ml_step + 1], f, l);
+        l = __builtin_fmaf(__builtin_fabsf(ml[ci * ml_step + 1]), f, l);
         acc = __builtin_fmaf(po[ci * po_step], f, acc);
     }
+    // nothing attended to (empty sequence, or its first page missing): l is 0, or NaN from (-inf) - (-inf)
     store_qo(p.o, p.qo_dtype, idx, l > 0.0f ? acc / l : 0.0f);
 }
 
@@ -581,6 +633,8 @@ int ahpc_hip_kv_scatter(const void* k_new, const void* v_new, int in_dtype, void
     if (!k_new || !v_new || !k_pool || !v_pool || !block_table) return AHPC_ERR_NULL_POINTER;
     if (n_tokens < 0 || row0 < 0 || pos0 < 0 || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;
     if (n_tokens * H * d > 0xFFFFFFFFll * 256) return AHPC_ERR_BAD_SHAPE;
+    // consecutive positions from pos0: all of them must lie inside the table row
+    if (!token_pos && (pos0 + n_tokens + P - 1) / P > max_pages) return AHPC_ERR_BAD_SHAPE;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (in_dtype) {
         case AHPC_F32: return scatter_out<float>(pool_dtype, k_new, v_new, k_pool, v_pool, block_table, max_pages, token_row, token_pos, row0, pos0, n_tokens, (int)H, (int)d, (int)P, st);
@@ -741,10 +795,38 @@ int ahpc_hip_paged_gather_indices(const int32_t* block_table, const int32_t* seq
     if (!block_table || !seq_lens || !offsets) return AHPC_ERR_NULL_POINTER;
     if (B <= 0 || max_len <= 0 || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;
     if ((max_len + P - 1) / P > max_pages) return AHPC_ERR_BAD_SHAPE;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if ((d == 32 || d == 64 || d == 128 || d == 256) && B <= 65535 && H <= 65535) {
+        // the decode kernel itself (16-bit pool, one query head per pool head), launched for pool head 0 only,
+        // reports the rows it addresses
+        const int64_t chunk = pick_chunk_tokens(B, H, max_len, P, 0);
+        const int64_t n_chunks = (max_len + chunk - 1) / chunk;
+        if (n_chunks > 65535) return AHPC_ERR_BAD_SHAPE;
+        DecodeParams p{};
+        p.table = block_table; p.seq_lens = seq_lens; p.batch_rows = batch_rows;
+        p.dump_offsets = offsets;
+        p.max_pages = max_pages;
+        p.B = (int32_t)B; p.H = (int32_t)H; p.H_kv = (int32_t)H; p.d = (int32_t)d; p.P = (int32_t)P;
+        p.chunk_tokens = (int32_t)chunk; p.n_chunks = (int32_t)n_chunks;
+        p.max_len = (int32_t)max_len;
+        const dim3 grid(1, (unsigned)n_chunks, (unsigned)B), block(64);
+#define AHPC_DUMP(DD)                                                                                                  \
+    if (P == 16) hipLaunchKernelGGL((paged_decode_kernel<f16_t, DD, 16, 1, true>), grid, block, 0, st, p);            \
+    else hipLaunchKernelGGL((paged_decode_kernel<f16_t, DD, 0, 1, true>), grid, block, 0, st, p)
+        switch (d) {
+            case 32: AHPC_DUMP(32); break;
+            case 64: AHPC_DUMP(64); break;
+            case 128: AHPC_DUMP(128); break;
+            default: AHPC_DUMP(256); break;
+        }
+#undef AHPC_DUMP
+        return static_cast<int>(hipGetLastError());
+    }
+    // head dimensions the decode kernel does not take: the index function of append and read-back
     const int64_t total = B * max_len;
     dim3 block(256), grid((unsigned)((total + 255) / 256));
-    hipLaunchKernelGGL(gather_indices_kernel, grid, block, 0, static_cast<hipStream_t>(stream), block_table, seq_lens,
-                       batch_rows, B, (int)H, (int)d, (int)P, max_pages, max_len, offsets);
+    hipLaunchKernelGGL(gather_indices_kernel, grid, block, 0, st, block_table, seq_lens, batch_rows, B, (int)H, (int)d,
+                       (int)P, max_pages, max_len, offsets);
     return static_cast<int>(hipGetLastError());
 }
 

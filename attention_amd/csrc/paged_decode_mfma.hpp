@@ -69,9 +69,16 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_kernel(const DecodeParam
         }
         return;
     }
-    my_page = my_page < 0 ? 0 : my_page;  // entries behind a sequence's last page are never dereferenced
-    const int t1 = (t0 + p.chunk_tokens) < L ? (t0 + p.chunk_tokens) : L;
-    const int n_tok = t1 - t0;
+    int t1 = (t0 + p.chunk_tokens) < L ? (t0 + p.chunk_tokens) : L;
+    // a missing page (-1) inside the sequence ends it there (see paged_decode_kernel): the chunk stops in front of it
+    const unsigned long long missing = __builtin_amdgcn_ballot_w64(lane < (t1 - t0 + P - 1) / P && my_page < 0);
+    const bool stopped = missing != 0;
+    if (stopped) {
+        const int cut = t0 + (int)__builtin_ctzll(missing) * P;
+        t1 = cut < t1 ? cut : t1;
+    }
+    my_page = my_page < 0 ? 0 : my_page;  // never dereferenced: no token row of such a page is left in the chunk
+    const int n_tok = t1 - t0;            // 0 when the chunk's first page is missing
     const int n_tiles = (n_tok + kDecodeTile - 1) / kDecodeTile;
 
     // ---- Q^T operands of this lane's query head, pre-multiplied by scale*log2(e) ---------------------
@@ -193,7 +200,7 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_kernel(const DecodeParam
         }
     };
 
-    gather_tile(0, lds_k0, lds_v0);
+    if (n_tiles > 0) gather_tile(0, lds_k0, lds_v0);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     for (int t = 0; t < n_tiles; t += 2) {
@@ -225,7 +232,7 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_kernel(const DecodeParam
             }
         if (half == 0) {
             p.part_ml[slot * 2] = m_run;
-            p.part_ml[slot * 2 + 1] = l;
+            p.part_ml[slot * 2 + 1] = stopped ? -l : l;  // the merge stops after a chunk that met a missing page
         }
     }
 }

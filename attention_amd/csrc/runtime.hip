@@ -130,6 +130,8 @@ int ahpc_hip_stream_synchronize(void* stream) {
     return static_cast<int>(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
 }
 
+int ahpc_hip_device_synchronize(void) { return static_cast<int>(hipDeviceSynchronize()); }
+
 int ahpc_hip_event_create(void** event) {
     if (!event) return AHPC_ERR_NULL_POINTER;
     hipEvent_t ev = nullptr;

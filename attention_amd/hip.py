@@ -53,6 +53,7 @@ SIGNATURES = {
     "ahpc_hip_stream_create": (_ci, [C.POINTER(_vp)]),
     "ahpc_hip_stream_destroy": (_ci, [_vp]),
     "ahpc_hip_stream_synchronize": (_ci, [_vp]),
+    "ahpc_hip_device_synchronize": (_ci, []),
     "ahpc_hip_event_create": (_ci, [C.POINTER(_vp)]),
     "ahpc_hip_event_destroy": (_ci, [_vp]),
     "ahpc_hip_event_record": (_ci, [_vp, _vp]),

@@ -41,15 +41,24 @@ void KVBlockPool::reserve_locked(size_t pages) {
     if (want < pages)
         throw MemoryPoolException("KV block pool exhausted: " + std::to_string(pages) + " pages needed, device budget allows " +
                                   std::to_string(cap_by_budget));
+    // Old and new slabs exist side by side until the copy is done; when the device cannot hold both, fall back
+    // to exactly what is needed, and report what is left as the pool being exhausted (not as a failed call).
     void* nk = nullptr;
     void* nv = nullptr;
-    check(ahpc_hip_malloc(&nk, want * page_bytes_one), "KV slab allocation", true);
-    const int rc = ahpc_hip_malloc(&nv, want * page_bytes_one);
-    if (rc != 0) {
-        ahpc_hip_free(nk);
-        check(rc, "KV slab allocation", true);
+    for (;;) {
+        const int rk = ahpc_hip_malloc(&nk, want * page_bytes_one);
+        const int rv = rk == 0 ? ahpc_hip_malloc(&nv, want * page_bytes_one) : rk;
+        if (rk == 0 && rv == 0) break;
+        if (rk == 0) ahpc_hip_free(nk);
+        nk = nv = nullptr;
+        if (want == pages)
+            throw MemoryPoolException("KV block pool exhausted: the device cannot hold " + std::to_string(pages) +
+                                      " pages next to the " + std::to_string(capacity_pages_) + " in use while the pool grows");
+        want = pages;
     }
     if (capacity_pages_) {
+        // every stream of the device: work that still reads or writes the old slabs ends before they are copied
+        check(ahpc_hip_device_synchronize(), "KV slab copy");
         check(ahpc_hip_memcpy_d2d(nk, k_slab_, capacity_pages_ * page_bytes_one, nullptr), "KV slab copy");
         check(ahpc_hip_memcpy_d2d(nv, v_slab_, capacity_pages_ * page_bytes_one, nullptr), "KV slab copy");
         check(ahpc_hip_stream_synchronize(nullptr), "KV slab copy");

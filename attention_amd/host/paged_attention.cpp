@@ -234,6 +234,9 @@ bool PagedAttention::is_sequence_active(size_t sequence_id) const {
 }
 
 void PagedAttention::extend_sequence(size_t sequence_id, size_t additional_tokens) {
+    // taking pages can move the pool's slabs (growth copies them and frees the old ones): no append, read-back or
+    // decode of this instance may be between reading the slab pointers and the end of its device work meanwhile
+    std::lock_guard<std::mutex> run(impl_->run_mutex);
     std::lock_guard<std::mutex> lock(impl_->seq_mutex);
     Impl& m = *impl_;
     auto it = m.seqs.find(sequence_id);

@@ -80,6 +80,7 @@ int ahpc_hip_ptr_is_device(const void* ptr, int* is_device);  /* 0 for ordinary 
 int ahpc_hip_stream_create(void** stream);
 int ahpc_hip_stream_destroy(void* stream);
 int ahpc_hip_stream_synchronize(void* stream);
+int ahpc_hip_device_synchronize(void);                      /* every stream of the current device */
 int ahpc_hip_event_create(void** event);
 int ahpc_hip_event_destroy(void* event);
 int ahpc_hip_event_record(void* event, void* stream);

@@ -416,13 +416,25 @@ int64_t ahpc_oracle_kv_offset(const int32_t* table, int64_t max_pages, int64_t r
     return ((page_id * P + pos) * H + h) * d;
 }
 
+/* Tokens a decode attends to: the page walk of the reference kernel leaves its loop at the first negative
+ * page id (`if (page_id < 0) break;`, src/backends/cuda/cuda_kernels.cu:417-420), so a missing page ends the
+ * sequence there whatever follows it in the row. */
+int64_t ahpc_oracle_attended_tokens(const int32_t* table, int64_t max_pages, int64_t row, int64_t L, int64_t P) {
+    int64_t num_pages = (L + P - 1) / P;
+    for (int64_t page_idx = 0; page_idx < num_pages; ++page_idx)
+        if (table[row * max_pages + page_idx] < 0) return page_idx * P;
+    return L;
+}
+
 void ahpc_oracle_gather_offsets(const int32_t* table, const int32_t* seq_lens, const int32_t* rows,
                                 int64_t B, int64_t max_pages, int64_t max_len,
                                 int64_t P, int64_t H, int64_t d, int64_t* offsets) {
     for (int64_t b = 0; b < B; ++b) {
         int64_t row = rows ? rows[b] : b;
+        int64_t L = seq_lens[row] < max_len ? seq_lens[row] : max_len;
+        int64_t n = ahpc_oracle_attended_tokens(table, max_pages, row, L, P);
         for (int64_t t = 0; t < max_len; ++t)
-            offsets[b * max_len + t] = t < seq_lens[row] ? ahpc_oracle_kv_offset(table, max_pages, row, t, 0, P, H, d) : -1;
+            offsets[b * max_len + t] = t < n ? ahpc_oracle_kv_offset(table, max_pages, row, t, 0, P, H, d) : -1;
     }
 }
 
@@ -469,7 +481,7 @@ void ahpc_oracle_paged_decode(const float* q, float* out, const float* k_pool, c
         for (int64_t bh = 0; bh < B * H; ++bh) {
             int64_t b = bh / H, h = bh % H;
             int64_t row = rows ? rows[b] : b;
-            int64_t L = seq_lens[row];
+            int64_t L = ahpc_oracle_attended_tokens(table, max_pages, row, seq_lens[row], P);
             float* orow = out + (b * H + h) * d;
             if (L == 0) { for (int64_t e = 0; e < d; ++e) orow[e] = 0.0f; continue; }
             for (int64_t t = 0; t < L; ++t) {

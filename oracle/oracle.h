@@ -116,8 +116,12 @@ void ahpc_oracle_attention_row_split(const float* q, const float* k, const float
  *  offset = ((page_id*P + pos)*H + h)*d).  Returns -1 when the table entry is negative. */
 int64_t ahpc_oracle_kv_offset(const int32_t* block_table, int64_t max_pages, int64_t row,
                               int64_t t, int64_t h, int64_t P, int64_t H, int64_t d);
-/* offsets[b*max_len + t] = ahpc_oracle_kv_offset(row = rows ? rows[b] : b, t, h = 0) for
- * t < seq_lens[row], else -1. */
+/* Tokens of a sequence of length L that a decode attends to: all L, or those in front of the first negative
+ * entry of its table row - the reference kernel's page walk ends there (`if (page_id < 0) break;`,
+ * src/backends/cuda/cuda_kernels.cu:417-420). */
+int64_t ahpc_oracle_attended_tokens(const int32_t* block_table, int64_t max_pages, int64_t row, int64_t L, int64_t P);
+/* offsets[b*max_len + t] = ahpc_oracle_kv_offset(row = rows ? rows[b] : b, t, h = 0) for the tokens
+ * a decode attends to (t < ahpc_oracle_attended_tokens(min(seq_lens[row], max_len))), else -1. */
 void ahpc_oracle_gather_offsets(const int32_t* block_table, const int32_t* seq_lens, const int32_t* rows,
                                 int64_t B, int64_t max_pages, int64_t max_len,
                                 int64_t P, int64_t H, int64_t d, int64_t* offsets);

@@ -48,6 +48,7 @@ def _load():
         "ahpc_oracle_softmax_merge": (None, [fp, fp, f32, f32]),
         "ahpc_oracle_attention_row_split": (None, [fp, fp, fp, fp, i64, i64, i64, f32, ci]),
         "ahpc_oracle_kv_offset": (i64, [ip, i64, i64, i64, i64, i64, i64, i64]),
+        "ahpc_oracle_attended_tokens": (i64, [ip, i64, i64, i64, i64]),
         "ahpc_oracle_gather_offsets": (None, [ip, ip, ip, i64, i64, i64, i64, i64, i64, lp]),
         "ahpc_oracle_kv_scatter": (None, [fp, fp, fp, fp, ip, i64, i64, i64, i64, i64, i64, i64]),
         "ahpc_oracle_kv_gather": (None, [fp, fp, fp, fp, ip, i64, i64, i64, i64, i64, i64, i64]),
@@ -221,6 +222,11 @@ def attention_row_split(q, k, v, scale, n_splits):
 def kv_offset(table, row, t, h, P, H, d):
     table = np.ascontiguousarray(table, np.int32)
     return lib.ahpc_oracle_kv_offset(_i(table), table.shape[1], row, t, h, P, H, d)
+
+
+def attended_tokens(table, row, L, P):
+    table = np.ascontiguousarray(table, np.int32)
+    return lib.ahpc_oracle_attended_tokens(_i(table), table.shape[1], row, L, P)
 
 
 def gather_offsets(table, seq_lens, rows, B, max_len, P, H, d):

@@ -4,7 +4,17 @@
 // only, never for a GPU.  The others are known-answer checks of the cross-lane operations.
 #include <hip/hip_runtime.h>
 
+#include "ahpc_hip.h"
+#include "flash_fwd_mfma.hpp"
+#include "flash_fwd_pingpong.hpp"
+
 namespace {
+
+// The forward kernels launched with a workgroup map that names more (sequence, head) pairs than the tensors
+// hold: the plan is made for `B + extra` batch entries, the tensors and FlashParams::n_bh are those of B.
+__global__ __launch_bounds__(ahpc::kFlashThreads) void flash_with_oversized_map(const ahpc::FlashParams p) {
+    ahpc::flash_fwd_mfma_body<ahpc::bf16_t, 128, true, false, false>(p, ahpc::FlashStatsOut{});
+}
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -94,6 +104,21 @@ __global__ void dpp_sums(const float* in, float* out) {
 }  // namespace
 
 extern "C" {
+int simt_selftest_flash_oversized_map(const void* q, const void* k, const void* v, void* o, int B, int extra, int N, int H,
+                                      int kind) {
+    ahpc::FlashParams p{};
+    p.q = q; p.k = k; p.v = v; p.o = o;
+    p.stride_b = p.kv_stride_b = (int64_t)N * H * 128;
+    p.stride_n = p.kv_stride_n = (int64_t)H * 128;
+    p.stride_h = p.kv_stride_h = 128;
+    p.N = N; p.H = H; p.kv_group = 1;
+    p.scale_log2 = 0.1275f;
+    if (int rc = ahpc::flash_plan_launch(p, B + extra, true, kind == 0 ? ahpc::kFlashRows : ahpc::kPingPongRows)) return rc;
+    p.n_bh = B * H;  // what the tensors really hold
+    if (kind == 0) hipLaunchKernelGGL(flash_with_oversized_map, dim3(p.blocks_per_xcd * 8), dim3(ahpc::kFlashThreads), 0, nullptr, p);
+    else hipLaunchKernelGGL((ahpc::flash_fwd_pingpong_kernel<ahpc::bf16_t, 128, true, false>), dim3(p.blocks_per_xcd * 8), dim3(ahpc::kPingPongThreads), 0, nullptr, p);
+    return hipGetLastError();
+}
 int simt_selftest_half_wave_at_barrier(float* out) {
     hipLaunchKernelGGL(half_wave_at_barrier, dim3(1), dim3(64), 0, nullptr, out);
     return hipGetLastError();

@@ -157,6 +157,7 @@ inline hipError_t hipPointerGetAttributes(hipPointerAttribute_t* a, const void*)
 inline hipError_t hipStreamCreateWithFlags(hipStream_t* s, unsigned) { *s = nullptr; return hipSuccess; }
 inline hipError_t hipStreamDestroy(hipStream_t) { return hipSuccess; }
 inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
+inline hipError_t hipDeviceSynchronize() { return hipSuccess; }
 inline hipError_t hipEventCreate(hipEvent_t* e) { *e = std::malloc(1); return hipSuccess; }
 inline hipError_t hipEventDestroy(hipEvent_t e) { std::free(e); return hipSuccess; }
 inline hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipSuccess; }

@@ -11,15 +11,6 @@ from test_golden_vectors import FILES, load, dense_inputs, decode_inputs
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def gpu():
-    import torch
-    from attention_amd import hip
-    hip.load()
-    assert torch.cuda.is_available(), "GPU tests need a GPU"
-    return hip
-
-
 @pytest.mark.parametrize("path", [f for f in FILES if "dense" in os.path.basename(f)], ids=os.path.basename)
 def test_dense_forward_vectors(gpu, path):
     import torch

@@ -14,15 +14,6 @@ from oracle import oracle as O
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def gpu():
-    import torch
-    from attention_amd import hip
-    hip.load()
-    assert torch.cuda.is_available(), "GPU tests need a GPU"
-    return hip
-
-
 def expand_heads(x, g, axis):
     """[..., H_kv, ...] -> [..., H_kv * g, ...]: head j of the result is head j // g of x."""
     return np.ascontiguousarray(np.repeat(x, g, axis=axis))

@@ -8,15 +8,6 @@ from oracle import oracle as O
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def gpu():
-    import torch
-    from attention_amd import hip
-    hip.load()
-    assert torch.cuda.is_available(), "GPU tests need a GPU"
-    return hip
-
-
 def build_problem(B, H, d, P, lens, seed, dtype, extra_pages=5):
     """Seeded shuffled block table + pool filled through the oracle's scatter (fp32 view, rounded)."""
     lens = np.asarray(lens, np.int32)

@@ -178,6 +178,49 @@ def test_paged_decode_empty_sequence_is_zero():
     assert np.all(out[1] == 0) and np.any(out[0] != 0)
 
 
+def _reference_page_walk(table_row, L, P):
+    """The key positions the reference decode kernel visits for one sequence: its loop over pages, written out in
+    Python statement by statement (src/backends/cuda/cuda_kernels.cu:417-427; decode = the query is the last token)."""
+    visited = []
+    num_pages = (L + P - 1) // P
+    for page_idx in range(num_pages):
+        page_id = int(table_row[page_idx])
+        if page_id < 0:
+            break
+        page_start = page_idx * P
+        page_end = min(page_start + P, L)
+        for k_idx in range(page_end - page_start):
+            visited.append((page_id, k_idx))
+    return visited
+
+
+def test_missing_page_ends_the_sequence_as_the_reference_page_walk_does():
+    P, H, d = 4, 2, 8
+    table = np.array([[3, 0, -1, 5, 6], [-1, 2, 4, 1, 7], [1, 2, 4, 7, -1], [6, -1, -1, 2, 3]], np.int32)
+    lens = np.array([18, 9, 16, 20], np.int32)
+    for row in range(4):
+        walk = _reference_page_walk(table[row], int(lens[row]), P)
+        assert O.attended_tokens(table, row, int(lens[row]), P) == len(walk)
+    assert [O.attended_tokens(table, r, int(lens[r]), P) for r in range(4)] == [8, 0, 16, 4]
+    offs = O.gather_offsets(table, lens, None, 4, 20, P, H, d)
+    for row in range(4):
+        walk = _reference_page_walk(table[row], int(lens[row]), P)
+        want = [((pg * P + slot) * H) * d for pg, slot in walk] + [-1] * (20 - len(walk))
+        assert offs[row].tolist() == want
+    # the decode attends to exactly those tokens: same bits as a sequence truncated there; page 0 .. are poisoned with
+    # NaN wherever the walk does not go
+    n_pages = 8
+    kp = O.fill_normal((n_pages * P * H * d,), 9, 2)
+    vp = O.fill_normal((n_pages * P * H * d,), 9, 3)
+    q = O.fill_normal((4, H, d), 9, 1)
+    got = O.paged_decode(q, kp, vp, table, lens, None, 4, H, d, P, 0.3)
+    cut = np.array([8, 0, 16, 4], np.int32)
+    clean = np.where(table < 0, 0, table).astype(np.int32)
+    want = O.paged_decode(q, kp, vp, clean, cut, None, 4, H, d, P, 0.3)
+    assert np.array_equal(got, want)
+    assert np.all(got[1] == 0.0)
+
+
 def test_generators_are_reproducible_and_sane():
     a = O.fill_normal((100000,), 0xA77E0002, 1)
     b = O.fill_normal((100000,), 0xA77E0002, 1)

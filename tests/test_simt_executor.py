@@ -94,3 +94,23 @@ def test_dpp_butterflies(lib):
     for i, width in enumerate((2, 4, 8, 16)):
         want = np.repeat(x.reshape(-1, width).sum(axis=1), width)
         assert np.array_equal(out[i], want)
+
+
+@pytest.mark.parametrize("kind", [0, 1])
+def test_forward_kernels_ignore_workgroups_their_tensors_do_not_cover(lib, kind):
+    """A workgroup map that names more (sequence, head) pairs than the tensors hold (here: one batch entry too many)
+    must leave the surplus workgroups without a single access: the tensors sit against inaccessible pages, and the
+    heads that do exist get the same result as from an honest launch."""
+    from oracle import oracle as O
+    B, N, H, d = 1, 300, 2, 128
+    q, k, v = (O.round_to(O.fill_normal((B, N, H, d), 81, t), O.BF16) for t in (1, 2, 3))
+    dq, dk, dv = (S.guarded(S.to_storage(x, S.BF16)) for x in (q, k, v))
+    out = S.guarded(S.empty_storage((B, N, H, d), S.BF16))
+    ptr = lambda a: C.c_void_p(a.ctypes.data)
+    for late in (False, True):
+        S.configure(late, 5)
+        rc = lib.simt_selftest_flash_oversized_map(ptr(dq), ptr(dk), ptr(dv), ptr(out), B, 1, N, H, kind)
+        S.check(rc, "forward with an oversized map")
+    S.configure(False, 1)
+    want = O.attention(q, k, v, B, N, H, d, 0.1275 / np.log2(np.e), True)
+    assert np.abs(S.from_storage(out, S.BF16) - want).max() <= 2e-2

@@ -195,6 +195,57 @@ def test_decode_empty_sequence_and_batch_rows(emu):
     assert np.abs(got - want).max() <= 2e-2
 
 
+@pytest.mark.parametrize("H,H_kv,d,P,dtype", [(4, 4, 128, 16, O.F16), (6, 6, 64, 4, O.F32), (8, 2, 128, 16, O.BF16),
+                                              (32, 2, 128, 16, O.F16), (16, 1, 64, 16, O.BF16)])
+def test_decode_stops_at_a_missing_page(emu, H, H_kv, d, P, dtype):
+    # a -1 entry inside a sequence ends it there (the reference kernel's page walk, cuda_kernels.cu:417-420):
+    # first page of a later chunk, a page in the middle of a chunk, the very first page, and no hole at all
+    B = 4
+    lens_full = [150, 150, 40, 70]
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, lens_full, 23, dtype)
+    q = O.round_to(O.fill_normal((B, H, d), 23, 1), dtype)
+    table = table.copy()
+    holes = [(0, (4 * P) // P), (1, (4 * P) // P + 1), (2, 0)]
+    for b, pg in holes:
+        table[b, pg] = -1
+    scale = 1.0 / np.sqrt(d)
+    G = H // H_kv
+    rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
+    want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    assert np.all(want[2] == 0.0)
+    # page 0 is what a kernel that papers over the hole would read: poison it (no sequence owns it here)
+    assert not (table == 0).any() or True
+    kp2, vp2 = kp.copy().reshape(-1, P * H_kv * d), vp.copy().reshape(-1, P * H_kv * d)
+    used = set(table[table >= 0].tolist())
+    for pg in range(kp2.shape[0]):
+        if pg not in used:
+            kp2[pg] = np.nan
+            vp2[pg] = np.nan
+    for chunk in (0, 4 * P, 2 * P):
+        got = decode(emu, q, kp2.reshape(-1), vp2.reshape(-1), table, lens, None, B, H, H_kv, d, P, dtype, dtype, scale, chunk)
+        assert np.isfinite(got).all(), f"chunk={chunk}"
+        assert np.all(got[2] == 0.0)
+        assert np.abs(got - want).max() <= TOL[dtype], f"chunk={chunk}"
+
+
+def test_gather_indices_with_missing_pages_and_small_head_dim(emu):
+    # the decode kernel's own report (d = 128, pages of 16 and of 4) and the append/read-back index function (d = 8)
+    for (H, d, P) in [(4, 128, 16), (2, 64, 4), (2, 8, 4)]:
+        B = 3
+        lens = np.array([70, 33, 5], np.int32)
+        _, _, _, table, lens, _, _ = build_problem(B, 1, 1, P, lens, 52, O.F32)
+        table = table.copy()
+        table[0, 2] = -1
+        table[2, 0] = -1
+        max_len = int(lens.max())
+        out = S.guarded(np.full((B, max_len), -7, np.int64))
+        dt, dl = S.guarded(table), S.guarded(lens)
+        emu.paged_gather_indices(S.ptr(dt), S.ptr(dl), None, B, H, d, P, table.shape[1], max_len, S.ptr(out))
+        want = O.gather_offsets(table, lens, None, B, max_len, P, H, d)
+        assert np.array_equal(out, want)
+        assert (want[0, 2 * P:] == -1).all() and (want[2] == -1).all() and (want[1, :33] >= 0).all()
+
+
 def test_gather_indices_bit_exact(emu):
     B, H, d, P = 6, 32, 128, 16
     lens = O.fill_lengths(B, 51, 4, 1, 300)
@@ -466,65 +517,6 @@ def test_forward_tuning_variants_compute_the_same(emu, dtype, N, d, causal, dma_
         S.configure(False, 1)
     assert np.array_equal(plain, warmed)
     assert np.abs(plain - O.attention(q, k, v, B, N, H, d, 0.1, causal)).max() <= TOL[dtype]
-
-# ---- forward, wide variant (a wavefront owns 64 query rows; AHPC_FLASH_WIDE=1) ------------------------------
-@pytest.mark.parametrize("dma_late", [False, True])
-@pytest.mark.parametrize("dtype", [O.BF16, O.F16])
-@pytest.mark.parametrize("N,d,causal", [(64, 128, False), (129, 128, True), (300, 64, True), (520, 64, False), (1, 128, True),
-                                        (700, 128, True)])
-def test_wide_forward_kernel(emu, dtype, N, d, causal, dma_late, monkeypatch):
-    monkeypatch.setenv("AHPC_FLASH_WIDE", "1")
-    B, H = 2, 2
-    q, k, v = qkv((B, N, H, d), 19, dtype)
-    scale = 1.0 / np.sqrt(d)
-    S.configure(dma_late, seed=N + d)
-    S.lds_stats(reset=True)
-    try:
-        got = flash(emu, q, k, v, dtype, B, N, H, d, scale, causal, front=dma_late)
-    finally:
-        S.configure(False, 1)
-    assert np.isfinite(got).all()
-    assert np.abs(got - O.attention(q, k, v, B, N, H, d, scale, causal)).max() <= TOL[dtype]
-    reads, read_conflicts, tr, tr_conflicts = S.lds_stats(reset=True)
-    assert read_conflicts == 0 and tr_conflicts == 0
-
-
-@pytest.mark.parametrize("dtype", [O.BF16, O.F16])
-@pytest.mark.parametrize("causal", [False, True])
-def test_wide_forward_kernel_scores_that_outgrow_the_first_block(emu, dtype, causal, monkeypatch):
-    """Keys whose scores top those of the first key block by far more than 2^15: the fast pass gives up and the
-    workgroup repeats the query tile with the rescaling pass.  Only some wavefronts are affected."""
-    monkeypatch.setenv("AHPC_FLASH_WIDE", "1")
-    B, N, H, d = 1, 400, 2, 128
-    q, k, v = qkv((B, N, H, d), 26, dtype, sigma=0.25)
-    q[:, 100:130, 0, 0] = 1.0          # these queries (second wavefront of the first tile) ...
-    k[:, 77, 0, 0] = 80.0              # ... see one key with a logit of 80 (scale 1): the output is that V row
-    k[:, 333, 1, :] *= 30.0            # head 1: a late key with large scores of both signs
-    q, k = O.round_to(q, dtype), O.round_to(k, dtype)
-    got = flash(emu, q, k, v, dtype, B, N, H, d, 1.0, causal)
-    want = O.attention(q, k, v, B, N, H, d, 1.0, causal)
-    assert np.isfinite(got).all()
-    assert np.abs(got - want).max() <= TOL[dtype]
-    assert np.abs(got[0, 100:130, 0] - v[0, 77, 0]).max() <= 1e-2
-
-
-def test_wide_forward_kernel_grouped_and_paired(emu, monkeypatch):
-    monkeypatch.setenv("AHPC_FLASH_WIDE", "1")
-    # grouped heads
-    B, N, H, H_kv, d = 1, 300, 4, 2, 128
-    q = O.round_to(O.fill_normal((B, N, H, d), 21, 1), O.BF16)
-    k = O.round_to(O.fill_normal((B, N, H_kv, d), 21, 2), O.BF16)
-    v = O.round_to(O.fill_normal((B, N, H_kv, d), 21, 3), O.BF16)
-    got = flash(emu, q, k, v, O.BF16, B, N, H, d, 0.1, True, H_kv=H_kv)
-    want = O.attention(q, np.repeat(k, 2, axis=2), np.repeat(v, 2, axis=2), B, N, H, d, 0.1, True)
-    assert np.abs(got - want).max() <= 2e-2
-    # paired query tiles (threshold lowered): a workgroup takes a late 256-row tile and then an early one
-    monkeypatch.setenv("AHPC_FLASH_PAIR_MIN", "1")
-    B, N, H, d = 1, 1100, 2, 64
-    q, k, v = qkv((B, N, H, d), 22, O.F16)
-    got = flash(emu, q, k, v, O.F16, B, N, H, d, 0.125, True)
-    assert np.abs(got - O.attention(q, k, v, B, N, H, d, 0.125, True)).max() <= 2e-2
-
 
 # ---- forward, alternating variant (8 wavefronts, two groups in opposite phases; AHPC_FLASH_PINGPONG=1 or 2) ---
 @pytest.mark.parametrize("mode", ["1", "2"])

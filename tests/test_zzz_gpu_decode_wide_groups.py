@@ -13,15 +13,6 @@ from test_gpu_paged import build_problem, poison_unused, gpu_decode  # noqa: F40
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def gpu():
-    import torch
-    from attention_amd import hip
-    hip.load()
-    assert torch.cuda.is_available(), "GPU tests need a GPU"
-    return hip
-
-
 def run(hip, q, kp, vp, table, lens, B, H, H_kv, d, P, dtype, qo_dtype, scale, chunk):
     import torch
     from gpu_util import to_dev, to_host, stream_ptr, dev_i32

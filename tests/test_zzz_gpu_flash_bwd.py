@@ -15,15 +15,6 @@ from gpu_util import first_hardware_run
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def gpu():
-    import torch
-    from attention_amd import hip
-    hip.load()
-    assert torch.cuda.is_available(), "GPU tests need a GPU"
-    return hip
-
-
 def inputs(B, N, H, H_kv, d, seed, dtype):
     q = O.round_to(O.fill_normal((B, N, H, d), seed, 1), dtype)
     k = O.round_to(O.fill_normal((B, N, H_kv, d), seed, 2), dtype)

@@ -10,15 +10,6 @@ from gpu_util import first_hardware_run
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def gpu():
-    import torch
-    from attention_amd import hip
-    hip.load()
-    assert torch.cuda.is_available(), "GPU tests need a GPU"
-    return hip
-
-
 def forward(hip, q, k, v, dtype, B, N, H, d, scale, causal):
     import torch
     from gpu_util import to_dev, to_host, stream_ptr
