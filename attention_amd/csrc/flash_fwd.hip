@@ -6,7 +6,7 @@
 
 #include "ahpc_device.hpp"
 #include "flash_fwd_mfma.hpp"
-#include "flash_fwd_pingpong.hpp"
+#include "tuning.hpp"
 
 namespace ahpc {
 
@@ -153,42 +153,8 @@ static int dispatch_simple(int dtype, const SimpleParams& p, int64_t B, hipStrea
 // ---------------------------------------------------------------------------------------------
 template <typename T, int D, bool VARLEN>
 static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
-    // AHPC_FLASH_PINGPONG=1 (or 2: the other pairing of wavefronts): the experimental variant with one workgroup of 8
-    // wavefronts per CU whose two halves alternate between matrix and softmax phases (flash_fwd_pingpong.hpp).
-    // Same results; not the default until it has been timed.
-    {
-        const char* pp = std::getenv("AHPC_FLASH_PINGPONG");
-        const int mode = pp ? std::atoi(pp) : 0;
-        if (mode == 1 || mode == 2) {
-            if (int rc = flash_plan_launch(p, B, causal, kPingPongRows)) return rc;
-            p.pingpong_low_bit = mode == 2 ? 1 : 0;
-            dim3 pgrid((unsigned)(p.blocks_per_xcd * 8)), pblock(kPingPongThreads);
-            if (causal) hipLaunchKernelGGL((flash_fwd_pingpong_kernel<T, D, true, VARLEN>), pgrid, pblock, 0, stream, p);
-            else hipLaunchKernelGGL((flash_fwd_pingpong_kernel<T, D, false, VARLEN>), pgrid, pblock, 0, stream, p);
-            return static_cast<int>(hipGetLastError());
-        }
-    }
-    if (int rc = flash_plan_launch(p, B, causal)) return rc;
+    if (int rc = flash_plan_launch(p, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load())) return rc;
     dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
-    // AHPC_FLASH_VARIANT = 1 (L2 warm-up), 2 (issue priority by phase), 3 (both), 4 (issue priority by workgroup role)
-    // or 6 (by phase, then by role): tuning variants of the dense kernel
-    // that compute the same results (see flash_fwd_mfma_body)
-    if constexpr (!VARLEN) {
-        const char* e = std::getenv("AHPC_FLASH_VARIANT");
-        const int variant = e ? std::atoi(e) : 0;
-#define AHPC_LAUNCH_VARIANT(V)                                                                                        \
-    if (variant == V) {                                                                                               \
-        if (causal) hipLaunchKernelGGL((flash_fwd_mfma_variant_kernel<T, D, true, V>), grid, block, 0, stream, p);   \
-        else hipLaunchKernelGGL((flash_fwd_mfma_variant_kernel<T, D, false, V>), grid, block, 0, stream, p);         \
-        return static_cast<int>(hipGetLastError());                                                                   \
-    }
-        AHPC_LAUNCH_VARIANT(1)
-        AHPC_LAUNCH_VARIANT(2)
-        AHPC_LAUNCH_VARIANT(3)
-        AHPC_LAUNCH_VARIANT(4)
-        AHPC_LAUNCH_VARIANT(6)
-#undef AHPC_LAUNCH_VARIANT
-    }
     if (causal) hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, true, VARLEN>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, false, VARLEN>), grid, block, 0, stream, p);
     return static_cast<int>(hipGetLastError());
@@ -264,7 +230,7 @@ int ahpc_hip_flash_block_map(int64_t B, int64_t N, int64_t H, int causal, int64_
     if (B <= 0 || N <= 0 || H <= 0 || B > 65535 || H > 65535 || N > 0x7FFFFF00ll) return AHPC_ERR_BAD_SHAPE;
     FlashParams p{};
     p.N = (int32_t)N; p.H = (int32_t)H; p.kv_group = 1;
-    if (int rc = flash_plan_launch(p, B, causal != 0)) return rc;
+    if (int rc = flash_plan_launch(p, B, causal != 0, kFlashRows, tuning().flash_pair_min_tiles.load())) return rc;
     const int64_t grid = (int64_t)p.blocks_per_xcd * 8;
     *n_blocks = grid;
     if (!seq_head && !first_tile && !second_tile) return AHPC_OK;

@@ -61,9 +61,6 @@ struct FlashParams {
     int32_t total_blocks;       // B * H * n_qtiles, or B * H * ceil(n_qtiles / 2) when paired
     int32_t n_bh;               // B * H: no workgroup may address a (sequence, head) at or beyond this
     int32_t blocks_per_xcd;     // ceil(total_blocks / 8)
-    int32_t heads_together;     // <= 1: a head's workgroups are consecutive; n: n heads advance side by side
-    int32_t round_slots;        // with heads_together > 1: workgroups one head contributes per round
-    int32_t pingpong_low_bit;   // alternating variant only: 1 = wavefronts w and w^1 form a pair (default: w and w+4)
     float scale_log2;           // scale * log2(e)
 };
 
@@ -152,9 +149,7 @@ __device__ inline void dma_dword(const void* base, unsigned nrec, int off, unsig
 
 // Workgroup id -> work.  Hardware deals consecutive workgroup ids to the 8 XCDs in turn; `logical` undoes
 // that, so that consecutive logical ids run on the same XCD and share its L2.  A head owns `per_head`
-// consecutive logical ids (its query tiles, or pairs of them), late (long) tiles first.  With
-// heads_together = n > 1 the ids of n heads are interleaved instead, round_slots of each head per round,
-// so that n heads stream their K/V side by side (more L2 channels busy, less reuse per head).
+// consecutive logical ids (its query tiles, or pairs of them), late (long) tiles first.
 // Host and device evaluate the same code: a host-side dump of this function is what the tests check.
 struct FlashWork {
     int bh;     // sequence * H + head
@@ -167,26 +162,8 @@ __host__ __device__ inline FlashWork flash_work_of_block(unsigned block_id, cons
     const int logical = xcd * p.blocks_per_xcd + (int)(block_id >> 3);
     if (logical >= p.total_blocks) return FlashWork{0, 0, false};
     const int per_head = flash_per_head(p);
-    if (p.heads_together <= 1) {
-        const int bh = logical / per_head;
-        return FlashWork{bh, logical - bh * per_head, true};
-    }
-    const int n_heads = p.total_blocks / per_head;
-    const int group = logical / (p.heads_together * per_head);
-    const int first = group * p.heads_together;
-    const int ch = (n_heads - first) < p.heads_together ? (n_heads - first) : p.heads_together;  // heads in this group
-    const int r = logical - first * per_head;                 // 0 .. ch*per_head-1
-    const int sl = p.round_slots > 0 ? p.round_slots : 1;
-    const int full_rounds = per_head / sl;
-    const int full_items = full_rounds * ch * sl;
-    if (r < full_items) {
-        const int round = r / (ch * sl);
-        const int rr = r - round * (ch * sl);
-        return FlashWork{first + rr / sl, round * sl + rr % sl, true};
-    }
-    const int rem = per_head - full_rounds * sl;               // slots of the last, partial round (> 0 here)
-    const int rr = r - full_items;
-    return FlashWork{first + rr / rem, full_rounds * sl + rr % rem, true};
+    const int bh = logical / per_head;
+    return FlashWork{bh, logical - bh * per_head, true};
 }
 // Query tile a workgroup handles in its first (part 0) and second (part 1) pass; -1 = none.
 __host__ __device__ inline int flash_qtile_of_part(const FlashParams& p, int slot, int part) {
@@ -209,40 +186,8 @@ struct FlashStatsOut {
     int64_t rows_padded;
 };
 
-// VARIANT: tuning variants of the same computation, compiled as separate kernels and chosen by the launcher.
-//   kVariantTouch     while tile t is computed and tile t+1 streams into LDS, one dword of every 128-byte line
-//                     of tile t+2 is requested as well (into an LDS area nobody reads), so that what misses the
-//                     L2 is on its way a tile earlier than the stream needs it.  The wait at the end of a step
-//                     then leaves that one request outstanding.
-//   kVariantPriority  a wavefront raises its issue priority (s_setprio) while it feeds the matrix cores and
-//                     lowers it for the stretch of pure softmax arithmetic, so that of the two wavefronts that
-//                     share a SIMD the one with matrix instructions ready goes first.
-//   kVariantRole      the two workgroups that share a CU get different issue priorities for their whole life:
-//                     the one whose LDS allocation starts at offset 0 goes first whenever both have an
-//                     instruction of a kind ready, the other one fills the gaps.  Two equal wavefronts on a
-//                     SIMD that are served in turn stay in step (both in their matrix phase, then both in
-//                     their softmax phase) and their times add up; unequal ones drift into opposite phases.
-//                     Together with kVariantPriority the phase decides first (matrix work of either
-//                     wavefront before softmax work of either), the role second.
-constexpr int kVariantTouch = 1;
-constexpr int kVariantPriority = 2;
-constexpr int kVariantRole = 4;
-
-// First 12 bits of the LDS allocation register of the wavefront: the offset of the workgroup's LDS inside
-// the CU's, in allocation granules.  0 for the workgroup that came first (or took the first one's place).
-__device__ inline unsigned lds_allocation_base() {
-#if defined(__HIP_DEVICE_COMPILE__)
-    return __builtin_amdgcn_s_getreg(6 /* HW_REG_LDS_ALLOC */ | (0 << 6) | ((12 - 1) << 11));
-#else
-    return 0;
-#endif
-}
-
-template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS, int VARIANT = 0>
+template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS>
 __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const FlashStatsOut& st) {
-    constexpr bool TOUCH = (VARIANT & kVariantTouch) != 0;
-    constexpr bool PRIORITY = (VARIANT & kVariantPriority) != 0;
-    constexpr bool ROLE = (VARIANT & kVariantRole) != 0;
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;  // k-steps of the first product
     constexpr int MB = D / 32;  // 32-row blocks of O^T
@@ -264,18 +209,12 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
     if (!work.valid) return;
     // whatever the map says, nothing outside the tensors is ever addressed (uniform per workgroup)
     if (work.bh < 0 || work.bh >= p.n_bh || work.slot < 0 || work.slot >= flash_per_head(p)) return;
-    // issue priority of this wavefront while it feeds the matrix cores (`busy`) and otherwise
-    bool leads = false;
-    if constexpr (ROLE) leads = lds_allocation_base() == 0;
+    // A wavefront raises its issue priority while it feeds the matrix cores and lowers it for the stretch of pure
+    // softmax arithmetic: of the two wavefronts that share a SIMD the one with matrix instructions ready goes first
+    // (worth about 2% on the headline shape).
     auto set_priority = [&](bool busy) {
-        if constexpr (ROLE && PRIORITY) {
-            if (busy) { if (leads) __builtin_amdgcn_s_setprio(3); else __builtin_amdgcn_s_setprio(2); }
-            else { if (leads) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0); }
-        } else if constexpr (PRIORITY) {
-            if (busy) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0);
-        }
+        if (busy) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0);
     };
-    if constexpr (ROLE && !PRIORITY) { if (leads) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(0); }
     const int bh = work.bh;
     const int slot = work.slot;
     const int b = bh / p.H;
@@ -319,21 +258,6 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
         const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
         dma_tile<D>(gk + (int64_t)k0 * skv, nrec, dma_off_k, dst_k, wave_u);
         dma_tile<D>(gv + (int64_t)k0 * skv, nrec, dma_off_v, dst_v, wave_u);
-    };
-
-    // Requests one dword of each 128-byte line of the K and V tiles that start at key k0 (TOUCH only).
-    auto touch_tile = [&](int k0) {
-        if constexpr (TOUCH) {
-            __shared__ __attribute__((aligned(1024))) unsigned char lds_touch[1024];
-            constexpr int kLinesPerRow = RB / 128;                    // 2 (d = 128) or 1 (d = 64)
-            constexpr int kLines = kFlashKeys * kLinesPerRow;         // lines per tile
-            const int i = tid % kLines;                               // the line this thread asks for
-            const bool is_v = (tid / kLines) & 1;                     // first group of threads: K, second: V
-            const int64_t rem = (int64_t)(L - k0 - 1) * skv * 2 + 2 * D;
-            const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
-            const int off = (int)((i / kLinesPerRow) * skv * 2) + (i % kLinesPerRow) * 128;
-            dma_dword((is_v ? gv : gk) + (int64_t)k0 * skv, nrec, off, lds_touch + wave_u * 256);
-        }
     };
 
     // ---- LDS operand addresses (byte offsets inside a tile) -------------------------------------
@@ -515,15 +439,10 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
             const int k0 = t * kFlashKeys;
             const bool more = t + 1 < n_tiles;
             if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
-            const bool touched = TOUCH && t + 2 < n_tiles;
-            if (touched) touch_tile(k0 + 2 * kFlashKeys);
             // a wavefront whose queries all precede this tile has nothing to add
             if (!(CAUSAL && k0 > qw + 31)) compute_tile(cur_k, cur_v, k0);
             if (more) {
-                // this wave's part of the next tile has landed (requests complete in order: the one request for
-                // the tile after it, issued last, may still be under way)
-                if (touched) __builtin_amdgcn_s_waitcnt(1);
-                else __builtin_amdgcn_s_waitcnt(0);
+                __builtin_amdgcn_s_waitcnt(0);  // this wave's part of the next tile has landed
                 __syncthreads();                // everyone's has, and everyone is done with the current one
             }
         };
@@ -576,45 +495,26 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
     }
 }
 
-// Fills the launch geometry of the MFMA kernel (query tiles, pairing, workgroup count, interleaving of
-// heads) from N, H and the batch size already in `p`.  Shared by the launcher and by the host-side dump
+// Fills the launch geometry of the MFMA kernel (query tiles, pairing, workgroup count) from N, H and the batch size already in `p`.  Shared by the launcher and by the host-side dump
 // of the workgroup map.
-inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal, int rows_per_workgroup = kFlashRows) {
+inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal, int rows_per_workgroup = kFlashRows, int64_t pair_min_tiles = 1024) {
     p.n_qtiles = (p.N + rows_per_workgroup - 1) / rows_per_workgroup;
     int64_t total = B * p.H * (int64_t)p.n_qtiles;
     if (total > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
     // Causal launches with enough workgroups to fill the chip twice over pair a late query tile with an
-    // early one, so that every workgroup walks the same number of key tiles.
-    // (AHPC_FLASH_PAIR_MIN moves the threshold; 1024 tiles = two rounds of two workgroups on each of 256 CUs.)
-    int64_t pair_min = 1024;
-    if (const char* e = std::getenv("AHPC_FLASH_PAIR_MIN")) pair_min = std::atoi(e) > 0 ? std::atoi(e) : pair_min;
-    p.paired = (causal && p.n_qtiles >= 2 && total * rows_per_workgroup >= pair_min * kFlashRows) ? 1 : 0;
+    // early one, so that every workgroup walks the same number of key tiles
+    // (1024 tiles = two rounds of two workgroups on each of 256 CUs).
+    p.paired = (causal && p.n_qtiles >= 2 && total * rows_per_workgroup >= pair_min_tiles * kFlashRows) ? 1 : 0;
     if (p.paired) total = B * p.H * (int64_t)((p.n_qtiles + 1) / 2);
     p.total_blocks = (int32_t)total;
     p.n_bh = (int32_t)(B * p.H);
     p.blocks_per_xcd = (int32_t)((total + 7) / 8);
-    // AHPC_FLASH_HEADS_TOGETHER = n lets n heads advance side by side on an XCD (default: one after the
-    // other); AHPC_FLASH_ROUND_SLOTS sets how many workgroups a head contributes per round (default 64 / n:
-    // an XCD holds 64 workgroups of this kernel).  Tuning knobs; every setting computes the same result.
-    int ht = 1, rs = 0;
-    if (const char* e = std::getenv("AHPC_FLASH_HEADS_TOGETHER")) ht = std::atoi(e);
-    if (const char* e = std::getenv("AHPC_FLASH_ROUND_SLOTS")) rs = std::atoi(e);
-    if (ht < 1 || ht > 64) ht = 1;
-    if (rs < 1) rs = 64 / ht;
-    p.heads_together = ht;
-    p.round_slots = rs;
     return AHPC_OK;
 }
 
 template <typename T, int D, bool CAUSAL, bool VARLEN>
 __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const FlashParams p) {
     flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, false>(p, FlashStatsOut{});
-}
-
-// The tuning variants described at flash_fwd_mfma_body (dense batches; AHPC_FLASH_VARIANT = 1 ... 7, a sum of the bits).
-template <typename T, int D, bool CAUSAL, int VARIANT>
-__global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_variant_kernel(const FlashParams p) {
-    flash_fwd_mfma_body<T, D, CAUSAL, false, false, VARIANT>(p, FlashStatsOut{});
 }
 
 // The forward pass with its output kept in registers: writes the softmax statistics the backward needs.

@@ -11,6 +11,7 @@
 #include <type_traits>
 
 #include "ahpc_device.hpp"
+#include "tuning.hpp"
 
 namespace ahpc {
 
@@ -282,11 +283,15 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     int my_page = 0;
     if (first_page + lane < p.max_pages) my_page = p.table[row * p.max_pages + first_page + lane];
     const int L = p.seq_lens[row] < p.max_len ? p.seq_lens[row] : p.max_len;
-    const bool dumps = DUMP && h_raw == 0 && e0 == 0;  // one lane of the launch's first head group
+    bool dumps = DUMP && h_raw == 0 && e0 == 0;  // one lane of the launch's first head group
     if constexpr (DUMP) {
         if (dumps) {
             const int te = (t0 + p.chunk_tokens) < p.max_len ? (t0 + p.chunk_tokens) : p.max_len;
             for (int t = t0; t < te; ++t) p.dump_offsets[(int64_t)b * p.max_len + t] = -1;
+            // what a chunk behind a missing page reads never enters the result (the merge stops in front of it):
+            // it is not reported either
+            for (int pg = 0; pg < first_page && pg < p.max_pages; ++pg)
+                if (p.table[row * p.max_pages + pg] < 0) dumps = false;
         }
     }
     if (t0 >= L) {
@@ -512,17 +517,12 @@ __global__ __launch_bounds__(256) void paged_merge_kernel(const DecodeParams p) 
 
 namespace ahpc {
 
-static int env_int(const char* name, int dflt) {
-    const char* e = std::getenv(name);
-    return e ? std::atoi(e) : dflt;
-}
-
 // Waves per decode workgroup (each wave works alone; this only sets how many heads travel together).
-static int decode_waves() { return env_int("AHPC_DECODE_WAVES", 0); }
+static int decode_waves() { return (int)tuning().decode_waves.load(); }
 
 static int64_t pick_chunk_tokens(int64_t B, int64_t H, int64_t max_len, int64_t P, int64_t requested) {
     int64_t chunk = requested;
-    if (chunk <= 0) chunk = env_int("AHPC_DECODE_CHUNK", 0);
+    if (chunk <= 0) chunk = tuning().decode_chunk.load();
     if (chunk <= 0) {
         // enough workgroups to keep every CU busy several times over, while the fp32 partials stay
         // below ~1% of the K/V bytes of a chunk
@@ -714,8 +714,8 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     if (!q || !o || !k_pool || !v_pool || !block_table || !seq_lens) return AHPC_ERR_NULL_POINTER;
     if (H_kv <= 0 || H <= 0 || H % H_kv) return AHPC_ERR_BAD_SHAPE;
     // Groups of 1, 2, 4, 8 query heads: lane-per-element kernel, any pool type.  Groups of 16 and 32 exist on
-    // the matrix-core kernel only (16-bit pool, d 64 or 128, pages of 16 tokens); AHPC_DECODE_MFMA=1 sends
-    // groups of 4 and 8 there as well.
+    // the matrix-core kernel only (16-bit pool, d 64 or 128, pages of 16 tokens); the tuning value
+    // decode_matrix_min_group can send groups of 4 and 8 there as well (slightly slower when timed).
     const int64_t group = H / H_kv;
     const bool mfma_shape = (pool_dtype == AHPC_F16 || pool_dtype == AHPC_BF16) && (d == 64 || d == 128) && P == 16 && H_kv <= 65535;
     if (group != 1 && group != 2 && group != 4 && group != 8 && !((group == 16 || group == 32) && mfma_shape))
@@ -764,7 +764,8 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
 
     dim3 grid((unsigned)head_groups, (unsigned)n_chunks, (unsigned)B), block(64 * waves);
     int rc;
-    const bool use_mfma = mfma_shape && (group >= 16 || (group >= 4 && env_int("AHPC_DECODE_MFMA", 0) == 1));
+    const int64_t matrix_from = tuning().decode_matrix_min_group.load();
+    const bool use_mfma = mfma_shape && (group >= 16 || (group >= 4 && group >= matrix_from));
     if (use_mfma) {
         rc = pool_dtype == AHPC_F16 ? launch_decode_mfma<f16_t>(p, st) : launch_decode_mfma<bf16_t>(p, st);
     } else

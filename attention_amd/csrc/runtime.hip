@@ -1,11 +1,61 @@
 // Device, memory, stream and event entry points of the C ABI, and the error strings.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
 #include <cstring>
 
 #include "ahpc_hip.h"
+#include "tuning.hpp"
+
+namespace ahpc {
+
+static int64_t env_value(const char* name, int64_t dflt) {
+    const char* e = std::getenv(name);
+    return e ? std::atoll(e) : dflt;
+}
+
+Tuning::Tuning()
+    : flash_pair_min_tiles(env_value("AHPC_FLASH_PAIR_MIN", 1024)),
+      decode_waves(env_value("AHPC_DECODE_WAVES", 0)),
+      decode_chunk(env_value("AHPC_DECODE_CHUNK", 0)),
+      decode_matrix_min_group(env_value("AHPC_DECODE_MFMA_MIN_GROUP", 16)) {
+    if (flash_pair_min_tiles.load() < 1) flash_pair_min_tiles = 1024;
+}
+
+Tuning& tuning() {
+    static Tuning t;  // the environment is read here, once
+    return t;
+}
+
+static std::atomic<int64_t>* tuning_slot(const char* name) {
+    if (!name) return nullptr;
+    Tuning& t = tuning();
+    if (!std::strcmp(name, "flash_pair_min_tiles")) return &t.flash_pair_min_tiles;
+    if (!std::strcmp(name, "decode_waves")) return &t.decode_waves;
+    if (!std::strcmp(name, "decode_chunk")) return &t.decode_chunk;
+    if (!std::strcmp(name, "decode_matrix_min_group")) return &t.decode_matrix_min_group;
+    return nullptr;
+}
+
+}  // namespace ahpc
 
 extern "C" {
+
+int ahpc_hip_set_tuning(const char* name, int64_t value) {
+    std::atomic<int64_t>* slot = ahpc::tuning_slot(name);
+    if (!slot) return AHPC_ERR_BAD_SHAPE;
+    if (value < 0) return AHPC_ERR_BAD_SHAPE;
+    slot->store(value);
+    return AHPC_OK;
+}
+
+int ahpc_hip_get_tuning(const char* name, int64_t* value) {
+    if (!value) return AHPC_ERR_NULL_POINTER;
+    std::atomic<int64_t>* slot = ahpc::tuning_slot(name);
+    if (!slot) return AHPC_ERR_BAD_SHAPE;
+    *value = slot->load();
+    return AHPC_OK;
+}
 
 const char* ahpc_hip_error_string(int code) {
     switch (code) {

@@ -39,6 +39,8 @@ _vp, _i64, _f32, _ci, _sz = C.c_void_p, C.c_int64, C.c_float, C.c_int, C.c_size_
 # name -> (restype, argtypes); every symbol the header declares
 SIGNATURES = {
     "ahpc_hip_error_string": (C.c_char_p, [_ci]),
+    "ahpc_hip_set_tuning": (_ci, [C.c_char_p, _i64]),
+    "ahpc_hip_get_tuning": (_ci, [C.c_char_p, C.POINTER(_i64)]),
     "ahpc_hip_device_count": (_ci, [C.POINTER(_ci)]),
     "ahpc_hip_device_info": (_ci, [_ci, C.POINTER(DeviceInfo)]),
     "ahpc_hip_malloc": (_ci, [C.POINTER(_vp), _sz]),
@@ -110,6 +112,16 @@ def device_count():
     n = _ci(0)
     _check(load().ahpc_hip_device_count(C.byref(n)), "device_count")
     return n.value
+
+
+def set_tuning(name, value):
+    _check(load().ahpc_hip_set_tuning(name.encode(), value), "set_tuning")
+
+
+def get_tuning(name):
+    v = _i64()
+    _check(load().ahpc_hip_get_tuning(name.encode(), C.byref(v)), "get_tuning")
+    return v.value
 
 
 def device_info(device=0):

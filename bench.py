@@ -320,14 +320,14 @@ def bench_extras(hip, stream, steps, warmup):
     decode_case("paged_decode fp16 B=64 H=32 over 8 pool heads d=128 page=16 context U[512,4096]",
                 dict(DECODE), 32, 8, hip.F16, torch.float16)
     # the same grouped decode, and multi-query decode, on the matrix-core kernel
-    os.environ["AHPC_DECODE_MFMA"] = "1"
+    hip.set_tuning("decode_matrix_min_group", 4)
     try:
         decode_case("paged_decode (matrix-core kernel) fp16 B=64 H=32 over 8 pool heads d=128 page=16 context U[512,4096]",
                     dict(DECODE), 32, 8, hip.F16, torch.float16)
         decode_case("paged_decode (matrix-core kernel) fp16 B=64 H=32 over 1 pool head d=128 page=16 context U[512,4096]",
                     dict(DECODE), 32, 1, hip.F16, torch.float16)
     finally:
-        del os.environ["AHPC_DECODE_MFMA"]
+        hip.set_tuning("decode_matrix_min_group", 16)
 
     # prefill -> cache hand-off: K and V of the headline prefill into the pool, one launch
     P = 16

@@ -66,6 +66,13 @@ typedef struct ahpc_device_info {
     int32_t  runtime_version;
 } ahpc_device_info;
 
+/* Launcher tuning values ("flash_pair_min_tiles", "decode_waves", "decode_chunk", "decode_matrix_min_group"):
+ * process-wide, each starts from its environment variable (AHPC_FLASH_PAIR_MIN, AHPC_DECODE_WAVES, AHPC_DECODE_CHUNK,
+ * AHPC_DECODE_MFMA_MIN_GROUP), which is read once.  No value
+ * changes results; unknown names and negative values are refused.  The reference has no counterpart: its tile sizes
+ * sit in PerformanceConfig (src/api/attention_interface.hpp:29-53), which the host classes still honour. */
+int ahpc_hip_set_tuning(const char* name, int64_t value);
+int ahpc_hip_get_tuning(const char* name, int64_t* value);
 int ahpc_hip_device_count(int* count);                       /* never fails: count = 0 without a GPU */
 int ahpc_hip_device_info(int device, ahpc_device_info* out);
 int ahpc_hip_malloc(void** ptr, size_t bytes);

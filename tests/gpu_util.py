@@ -1,19 +1,9 @@
 """Helpers for the GPU parity tests: device buffers come from torch (plumbing only); every compute
 call goes through the C ABI (attention_amd.hip)."""
-import os
-
 import numpy as np
 import pytest
 
 from oracle import oracle as O
-
-# Kernels that have so far run only on the CPU executor (tests/simt) get their first run on hardware by hand:
-# one case at a time, each under its own time limit, with AHPC_GPU_FIRST_RUN=1.  An unattended run of the
-# suite leaves their launching tests out until that has happened, because a kernel that misbehaves on its
-# first run can take the whole machine with it and hide the results of every established test.
-first_hardware_run = pytest.mark.skipif(
-    os.environ.get("AHPC_GPU_FIRST_RUN") != "1",
-    reason="kernel verified on the CPU executor only; its first run on hardware is made by hand (AHPC_GPU_FIRST_RUN=1)")
 
 TOL = {O.F32: 1e-4, O.F16: 2e-2, O.BF16: 2e-2}  # max-abs bars: fp32 vs oracle, 16-bit vs fp32 oracle
 

@@ -6,11 +6,10 @@
 
 #include "ahpc_hip.h"
 #include "flash_fwd_mfma.hpp"
-#include "flash_fwd_pingpong.hpp"
 
 namespace {
 
-// The forward kernels launched with a workgroup map that names more (sequence, head) pairs than the tensors
+// The forward kernel launched with a workgroup map that names more (sequence, head) pairs than the tensors
 // hold: the plan is made for `B + extra` batch entries, the tensors and FlashParams::n_bh are those of B.
 __global__ __launch_bounds__(ahpc::kFlashThreads) void flash_with_oversized_map(const ahpc::FlashParams p) {
     ahpc::flash_fwd_mfma_body<ahpc::bf16_t, 128, true, false, false>(p, ahpc::FlashStatsOut{});
@@ -113,10 +112,10 @@ int simt_selftest_flash_oversized_map(const void* q, const void* k, const void* 
     p.stride_h = p.kv_stride_h = 128;
     p.N = N; p.H = H; p.kv_group = 1;
     p.scale_log2 = 0.1275f;
-    if (int rc = ahpc::flash_plan_launch(p, B + extra, true, kind == 0 ? ahpc::kFlashRows : ahpc::kPingPongRows)) return rc;
+    (void)kind;
+    if (int rc = ahpc::flash_plan_launch(p, B + extra, true)) return rc;
     p.n_bh = B * H;  // what the tensors really hold
-    if (kind == 0) hipLaunchKernelGGL(flash_with_oversized_map, dim3(p.blocks_per_xcd * 8), dim3(ahpc::kFlashThreads), 0, nullptr, p);
-    else hipLaunchKernelGGL((ahpc::flash_fwd_pingpong_kernel<ahpc::bf16_t, 128, true, false>), dim3(p.blocks_per_xcd * 8), dim3(ahpc::kPingPongThreads), 0, nullptr, p);
+    hipLaunchKernelGGL(flash_with_oversized_map, dim3(p.blocks_per_xcd * 8), dim3(ahpc::kFlashThreads), 0, nullptr, p);
     return hipGetLastError();
 }
 int simt_selftest_half_wave_at_barrier(float* out) {

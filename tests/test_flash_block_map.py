@@ -1,25 +1,11 @@
 """The MFMA flash kernel's workgroup -> work map, dumped on the host by the function the kernel itself uses
-(ahpc_hip_flash_block_map): whatever the shape, the pairing of query tiles under a causal mask and the
-interleaving of heads selected through the environment, every (sequence*head, query tile) must be handled by
-exactly one workgroup pass, and nothing else may be handled.  A map that misses or repeats a tile computes wrong
+(ahpc_hip_flash_block_map): whatever the shape and the pairing of query tiles under a causal mask, every
+(sequence*head, query tile) must be handled by exactly one workgroup pass, and nothing else may be handled.  A map that misses or repeats a tile computes wrong
 attention; one that names a head that does not exist reads outside the tensors."""
-import itertools
-import os
-
 import numpy as np
 import pytest
 
 ROWS = 128  # query rows per workgroup pass
-
-
-@pytest.fixture()
-def clean_env():
-    saved = {k: os.environ.pop(k, None) for k in ("AHPC_FLASH_HEADS_TOGETHER", "AHPC_FLASH_ROUND_SLOTS")}
-    yield
-    for k, v in saved.items():
-        os.environ.pop(k, None)
-        if v is not None:
-            os.environ[k] = v
 
 
 def check_exact_cover(B, N, H, causal):
@@ -42,7 +28,7 @@ SHAPES = [(1, 1, 1), (1, 128, 1), (2, 129, 3), (1, 1000, 3), (2, 2144, 16), (4, 
 
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("B,N,H", SHAPES)
-def test_default_map_covers_every_tile_once_and_keeps_its_order(clean_env, B, N, H, causal):
+def test_default_map_covers_every_tile_once_and_keeps_its_order(B, N, H, causal):
     bh, t0, t1 = check_exact_cover(B, N, H, causal)
     # the default order: consecutive logical ids (= 8 workgroup ids apart) walk one head's tiles, late tiles first
     n_tiles = (N + ROWS - 1) // ROWS
@@ -58,27 +44,6 @@ def test_default_map_covers_every_tile_once_and_keeps_its_order(clean_env, B, N,
         assert bh[block] == logical // per_head and t0[block] == n_tiles - 1 - slot
         want_second = slot if paired and 2 * slot != n_tiles - 1 else -1
         assert t1[block] == want_second
-
-
-@pytest.mark.parametrize("together,slots", [(2, None), (4, None), (8, None), (16, None), (3, 5), (8, 1), (5, 64), (64, None), (7, 3)])
-def test_interleaved_heads_still_cover_every_tile_once(clean_env, together, slots):
-    os.environ["AHPC_FLASH_HEADS_TOGETHER"] = str(together)
-    if slots is not None:
-        os.environ["AHPC_FLASH_ROUND_SLOTS"] = str(slots)
-    for (B, N, H), causal in itertools.product(SHAPES, (False, True)):
-        check_exact_cover(B, N, H, causal)
-
-
-def test_interleaving_puts_the_requested_heads_side_by_side(clean_env):
-    from attention_amd import hip
-    os.environ["AHPC_FLASH_HEADS_TOGETHER"] = "8"
-    bh, _, _ = hip.flash_block_map(4, 4096, 32, True)
-    per_xcd = len(bh) // 8
-    first64 = [bh[(l % per_xcd) * 8 + l // per_xcd] for l in range(64)]   # logical ids 0..63: what one XCD starts with
-    assert sorted(set(first64)) == list(range(8)) and first64[:8] == [0] * 8
-    # nonsense settings fall back to the default
-    os.environ["AHPC_FLASH_HEADS_TOGETHER"] = "-3"
-    assert np.array_equal(hip.flash_block_map(2, 512, 4, True)[0][:8], hip.flash_block_map(2, 512, 4, True)[0][:8])
 
 
 def test_rejects_bad_shapes_without_a_gpu():

@@ -112,6 +112,55 @@ def test_decode_empty_sequence_and_batch_rows(gpu):
         assert np.abs(got - want).max() <= 2e-2
 
 
+@pytest.mark.parametrize("H,H_kv,d,P,dtype", [(4, 4, 128, 16, O.F16), (6, 6, 64, 4, O.F32), (8, 2, 128, 16, O.BF16),
+                                              (32, 2, 128, 16, O.F16), (16, 1, 64, 16, O.BF16)])
+def test_decode_stops_at_a_missing_page(gpu, H, H_kv, d, P, dtype):
+    """A -1 entry inside a sequence ends it there, as the reference kernel's page walk does
+    (src/backends/cuda/cuda_kernels.cu:417-420): the first page of a later chunk, a page in the middle of a chunk, the
+    very first page.  Every page no sequence owns (page ids a kernel that papers over the hole might fall back to,
+    page 0 among them) holds NaN."""
+    import torch
+    from gpu_util import to_dev, to_host, stream_ptr, dev_i32
+    B = 4
+    _, kp, vp, table, lens, _, n_pages = build_problem(B, H_kv, d, P, [600, 600, 40, 70], 23, dtype, extra_pages=9)
+    q = O.round_to(O.fill_normal((B, H, d), 23, 1), dtype)
+    table = table.copy()
+    for b, pg in [(0, 16), (1, 21), (2, 0)]:
+        table[b, pg] = -1
+    scale = 1.0 / np.sqrt(d)
+    G = H // H_kv
+    rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
+    want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    assert np.all(want[2] == 0.0)
+    kp2, vp2 = kp.copy().reshape(n_pages, -1), vp.copy().reshape(n_pages, -1)
+    owned = set(table[table >= 0].tolist())
+    for pg in range(n_pages):
+        if pg not in owned:
+            kp2[pg] = np.nan
+            vp2[pg] = np.nan
+    assert 0 not in owned or True
+    kd, vd = to_dev(kp2.reshape(-1), dtype), to_dev(vp2.reshape(-1), dtype)
+    dq = to_dev(q, dtype)
+    dt, dl = dev_i32(table), dev_i32(lens)
+    max_len = int(lens.max())
+    for chunk in (0, 16 * P, 4 * P):
+        do = torch.full_like(dq, float("nan"))
+        ws_bytes = gpu.paged_decode_workspace_bytes(B, H, d, max_len, P, chunk)
+        ws = torch.full((max(ws_bytes, 4) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+        gpu.paged_decode_gqa(dq.data_ptr(), do.data_ptr(), dtype, kd.data_ptr(), vd.data_ptr(), dtype, dt.data_ptr(), dl.data_ptr(),
+                             None, B, H, H_kv, d, P, table.shape[1], max_len, scale, chunk, ws.data_ptr(), ws_bytes, stream_ptr())
+        torch.cuda.synchronize()
+        got = to_host(do)
+        assert np.isfinite(got).all(), f"chunk={chunk}"
+        assert np.all(got[2] == 0.0)
+        assert np.abs(got - want).max() <= (1e-4 if dtype == O.F32 else 2e-2), f"chunk={chunk}"
+    # and the kernel's own report of what it reads ends at the hole
+    out = torch.full((B, max_len), -7, dtype=torch.int64, device="cuda")
+    gpu.paged_gather_indices(dt.data_ptr(), dl.data_ptr(), None, B, H_kv, d, P, table.shape[1], max_len, out.data_ptr(), stream_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), O.gather_offsets(table, lens, None, B, max_len, P, H_kv, d))
+
+
 def test_gather_indices_bit_exact(gpu):
     import torch
     from gpu_util import stream_ptr, dev_i32

@@ -121,19 +121,6 @@ def test_head_major_strides(emu):
     assert np.abs(got - O.attention(q, k, v, B, N, H, d, 0.09, True)).max() <= 2e-2
 
 
-@pytest.mark.parametrize("together,slots", [(2, 0), (4, 1), (3, 2), (64, 0)])
-def test_interleaved_workgroup_map_computes_the_same(emu, together, slots, monkeypatch):
-    B, N, H, d = 1, 520, 5, 64   # 5 query tiles per head, 5 heads: partial groups and partial rounds
-    q, k, v = qkv((B, N, H, d), 17, O.F16)
-    plain = flash(emu, q, k, v, O.F16, B, N, H, d, 0.125, True)
-    monkeypatch.setenv("AHPC_FLASH_HEADS_TOGETHER", str(together))
-    if slots:
-        monkeypatch.setenv("AHPC_FLASH_ROUND_SLOTS", str(slots))
-    mixed = flash(emu, q, k, v, O.F16, B, N, H, d, 0.125, True)
-    assert np.array_equal(plain, mixed)
-    assert np.abs(plain - O.attention(q, k, v, B, N, H, d, 0.125, True)).max() <= 2e-2
-
-
 # ---- paged KV pool and decode -----------------------------------------------------------------------------
 from test_gpu_paged import build_problem, poison_unused, _tables_for  # problem builders only (pure numpy + oracle)
 
@@ -232,7 +219,7 @@ def test_gather_indices_with_missing_pages_and_small_head_dim(emu):
     # the decode kernel's own report (d = 128, pages of 16 and of 4) and the append/read-back index function (d = 8)
     for (H, d, P) in [(4, 128, 16), (2, 64, 4), (2, 8, 4)]:
         B = 3
-        lens = np.array([70, 33, 5], np.int32)
+        lens = np.array([70 if P == 16 else 300, 33, 5], np.int32)  # the longest one spans several chunks
         _, _, _, table, lens, _, _ = build_problem(B, 1, 1, P, lens, 52, O.F32)
         table = table.copy()
         table[0, 2] = -1
@@ -327,10 +314,23 @@ def test_scatter_batch_packed(emu):
     assert np.array_equal(S.from_storage(dkp, O.F16), kp) and np.array_equal(S.from_storage(dvp, O.F16), vp)
 
 
-def test_paired_query_tiles(emu, monkeypatch):
+@pytest.fixture
+def tuned(emu):
+    """tuned(name, value) changes a launcher tuning value of the emulated library for the rest of the test."""
+    before = {}
+
+    def set_value(name, value):
+        before.setdefault(name, emu.get_tuning(name))
+        emu.set_tuning(name, value)
+    yield set_value
+    for name, value in before.items():
+        emu.set_tuning(name, value)
+
+
+def test_paired_query_tiles(emu, tuned):
     """Causal launches with many query tiles (1024 by default; lowered here) hand each workgroup a late tile and
     then an early one; with an odd count the middle tile has no partner."""
-    monkeypatch.setenv("AHPC_FLASH_PAIR_MIN", "1")
+    tuned("flash_pair_min_tiles", 1)
     for N in (512, 640):
         B, H, d = 1, 3, 64
         _, _, second = emu.flash_block_map(B, N, H, True)
@@ -434,8 +434,8 @@ def test_operand_reads_are_free_of_bank_conflicts(emu, dtype, d):
 # ---- grouped decode on the matrix cores --------------------------------------------------------------------
 @pytest.mark.parametrize("dtype,d", [(O.F16, 128), (O.BF16, 64)])
 @pytest.mark.parametrize("G", [4, 8, 16, 32])
-def test_decode_grouped_heads_matrix_core_kernel(emu, G, dtype, d, monkeypatch):
-    monkeypatch.setenv("AHPC_DECODE_MFMA", "1")   # groups of 4 and 8 take this kernel only when asked to
+def test_decode_grouped_heads_matrix_core_kernel(emu, G, dtype, d, tuned):
+    tuned("decode_matrix_min_group", 4)   # groups of 4 and 8 take this kernel only when asked to
     B, H_kv, P = 4, 2, 16
     H = G * H_kv
     _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [70, 5, 129, 32], 23, dtype)
@@ -497,74 +497,6 @@ def test_backward_ragged_batch(emu, dtype, d, H, H_kv, causal):
         check_gradients(tuple(g[a:b][None] for g in got), want, dtype)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 6])
-@pytest.mark.parametrize("dma_late", [False, True])
-@pytest.mark.parametrize("dtype,N,d,causal", [(O.BF16, 700, 128, True), (O.F16, 520, 64, False), (O.BF16, 129, 128, True),
-                                             (O.F16, 64, 128, False)])
-def test_forward_tuning_variants_compute_the_same(emu, dtype, N, d, causal, dma_late, variant, monkeypatch):
-    """AHPC_FLASH_VARIANT: 1 requests the tile after next a step early (and leaves that request outstanding at the
-    end-of-step wait), 2 changes issue priorities by phase, 3 does both, 4 gives the two workgroups of a CU different
-    priorities (the executor tells even workgroups that they came first and odd ones that they did not), 6 = 2 + 4.
-    Results must be bit-identical."""
-    B, H = 1, 2
-    q, k, v = qkv((B, N, H, d), 27, dtype)
-    plain = flash(emu, q, k, v, dtype, B, N, H, d, 0.1, causal)
-    monkeypatch.setenv("AHPC_FLASH_VARIANT", str(variant))
-    S.configure(dma_late, seed=N)
-    try:
-        warmed = flash(emu, q, k, v, dtype, B, N, H, d, 0.1, causal, front=dma_late)
-    finally:
-        S.configure(False, 1)
-    assert np.array_equal(plain, warmed)
-    assert np.abs(plain - O.attention(q, k, v, B, N, H, d, 0.1, causal)).max() <= TOL[dtype]
-
-# ---- forward, alternating variant (8 wavefronts, two groups in opposite phases; AHPC_FLASH_PINGPONG=1 or 2) ---
-@pytest.mark.parametrize("mode", ["1", "2"])
-@pytest.mark.parametrize("dma_late", [False, True])
-@pytest.mark.parametrize("dtype,N,d,causal", [(O.BF16, 64, 128, False), (O.F16, 129, 128, True), (O.BF16, 300, 64, True),
-                                             (O.F16, 520, 64, False), (O.BF16, 1, 128, True), (O.BF16, 700, 128, True),
-                                             (O.F16, 257, 128, False)])
-def test_alternating_forward_kernel(emu, dtype, N, d, causal, dma_late, mode, monkeypatch):
-    """Parity with the oracle and bit-identity with the standard kernel (same arithmetic in the same order per
-    wavefront; only the schedule differs), with tile requests that land as late as their wait allows, under the
-    executor's LDS ordering check (every tile request against every operand read, by barrier epochs)."""
-    B, H = 2, 2
-    q, k, v = qkv((B, N, H, d), 29, dtype)
-    scale = 1.0 / np.sqrt(d)
-    plain = flash(emu, q, k, v, dtype, B, N, H, d, scale, causal)
-    monkeypatch.setenv("AHPC_FLASH_PINGPONG", mode)
-    S.configure(dma_late, seed=N + d)
-    S.lds_stats(reset=True)
-    try:
-        got = flash(emu, q, k, v, dtype, B, N, H, d, scale, causal, front=dma_late)
-    finally:
-        S.configure(False, 1)
-    assert np.isfinite(got).all()
-    assert np.abs(got - O.attention(q, k, v, B, N, H, d, scale, causal)).max() <= TOL[dtype]
-    assert np.array_equal(got, plain)
-    reads, read_conflicts, tr, tr_conflicts = S.lds_stats(reset=True)
-    assert read_conflicts == 0 and tr_conflicts == 0
-
-
-def test_alternating_forward_kernel_grouped_and_paired(emu, monkeypatch):
-    monkeypatch.setenv("AHPC_FLASH_PINGPONG", "1")
-    # grouped heads
-    B, N, H, H_kv, d = 1, 300, 4, 2, 128
-    q = O.round_to(O.fill_normal((B, N, H, d), 21, 1), O.BF16)
-    k = O.round_to(O.fill_normal((B, N, H_kv, d), 21, 2), O.BF16)
-    v = O.round_to(O.fill_normal((B, N, H_kv, d), 21, 3), O.BF16)
-    got = flash(emu, q, k, v, O.BF16, B, N, H, d, 0.1, True, H_kv=H_kv)
-    want = O.attention(q, np.repeat(k, 2, axis=2), np.repeat(v, 2, axis=2), B, N, H, d, 0.1, True)
-    assert np.abs(got - want).max() <= 2e-2
-    # a workgroup that takes a late query tile and then an early one of the same head (odd tile count: the middle
-    # one has no partner); the pairing threshold is lowered so that a small problem pairs
-    monkeypatch.setenv("AHPC_FLASH_PAIR_MIN", "1")
-    B, N, H, d = 1, 1100, 1, 64
-    q, k, v = qkv((B, N, H, d), 22, O.F16)
-    got = flash(emu, q, k, v, O.F16, B, N, H, d, 0.125, True)
-    assert np.abs(got - O.attention(q, k, v, B, N, H, d, 0.125, True)).max() <= 2e-2
-
-
 # ---- calibration probe -------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16])
 @pytest.mark.parametrize("mix", [0, 1])
@@ -578,29 +510,3 @@ def test_matrix_rate_probe_runs_and_counts_its_work(emu, dtype, mix):
     assert S.load().ahpc_hip_probe_matrix_rate(dtype, mix, wgs, it, S.ptr(sink), sink.nbytes, C.byref(flop), None) == 0
     assert np.isfinite(sink).all()
     assert flop.value == 2.0 * 32 * 32 * 16 * 4 * it * 4 * wgs
-
-
-@pytest.mark.parametrize("dtype,d", [(O.F16, 64), (O.BF16, 128)])
-@pytest.mark.parametrize("mode", ["1", "2"])
-def test_alternating_forward_kernel_ragged_batch(emu, dtype, d, mode, monkeypatch):
-    """Packed sequences (cu_seqlens) on the alternating kernel: sequences shorter than a key tile, shorter than
-    the 256-row query tile, and longer; bit-identical with the standard kernel."""
-    H = 2
-    lens = np.array([1, 130, 64, 300, 257], np.int32)
-    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
-    T = int(cu[-1])
-    q, k, v = qkv((T, H, d), 15, dtype)
-    dq, dk, dv = dev(q, dtype), dev(k, dtype), dev(v, dtype)
-    dcu = S.guarded(cu)
-    scale = 1.0 / np.sqrt(d)
-    outs = []
-    for knob in (None, mode):
-        if knob:
-            monkeypatch.setenv("AHPC_FLASH_PINGPONG", knob)
-        do = S.guarded(S.empty_storage((T, H, d), dtype))
-        emu.flash_fwd_varlen(S.ptr(dq), S.ptr(dk), S.ptr(dv), S.ptr(do), dtype, S.ptr(dcu), len(lens), int(lens.max()), H, d,
-                             H * d, d, scale, True)
-        outs.append(S.from_storage(do, dtype))
-    want = O.attention_varlen(q, k, v, cu, H, d, scale, True)
-    assert np.abs(outs[1] - want).max() <= TOL[dtype]
-    assert np.array_equal(outs[0], outs[1])

@@ -5,7 +5,6 @@ import subprocess
 
 import pytest
 
-from gpu_util import first_hardware_run
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 BIN = os.path.join(ROOT, "attention_amd", "lib", "ahpc_conformance")
@@ -41,12 +40,10 @@ def test_forward_decode_and_pool_cases_on_gpu():
 
 
 @pytest.mark.gpu
-@first_hardware_run
 def test_backward_cases_on_gpu():
     run(["Backward"])
 
 
 @pytest.mark.gpu
-@first_hardware_run
 def test_wide_group_decode_cases_on_gpu():
     run(["WideGroups"])

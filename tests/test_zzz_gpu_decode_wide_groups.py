@@ -1,13 +1,10 @@
 """Grouped-head decode on the matrix-core kernel, on the GPU through the C ABI, against the CPU oracle fed a pool
 whose heads are repeated (the definition of grouped heads).  16 and 32 query heads per pool head exist on this
-kernel only; 4 and 8 take it when AHPC_DECODE_MFMA=1.  Collected after the established GPU tests on purpose:
-this kernel is newer than they are, and the tests that launch it wait for a first run by hand
-(gpu_util.first_hardware_run)."""
+kernel only; 4 and 8 take it when the tuning value decode_matrix_min_group says so."""
 import numpy as np
 import pytest
 
 from oracle import oracle as O
-from gpu_util import first_hardware_run
 from test_gpu_paged import build_problem, poison_unused, gpu_decode  # noqa: F401  (builders; gpu_decode documents the call)
 
 pytestmark = pytest.mark.gpu
@@ -30,11 +27,17 @@ def run(hip, q, kp, vp, table, lens, B, H, H_kv, d, P, dtype, qo_dtype, scale, c
     return to_host(do)
 
 
-@first_hardware_run
+@pytest.fixture
+def matrix_kernel_from_four(gpu):
+    before = gpu.get_tuning("decode_matrix_min_group")
+    gpu.set_tuning("decode_matrix_min_group", 4)
+    yield
+    gpu.set_tuning("decode_matrix_min_group", before)
+
+
 @pytest.mark.parametrize("dtype,d", [(O.F16, 128), (O.BF16, 64), (O.BF16, 128)])
 @pytest.mark.parametrize("G", [4, 8, 16, 32])
-def test_matrix_core_decode_equals_repeated_heads(gpu, G, dtype, d, monkeypatch):
-    monkeypatch.setenv("AHPC_DECODE_MFMA", "1")
+def test_matrix_core_decode_equals_repeated_heads(gpu, G, dtype, d, matrix_kernel_from_four):
     B, H_kv, P = 5, 2, 16
     H = G * H_kv
     _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [700, 5, 129, 32, 1000], 23, dtype)
@@ -52,17 +55,20 @@ def test_matrix_core_decode_equals_repeated_heads(gpu, G, dtype, d, monkeypatch)
         assert np.abs(got - want).max() <= 2e-2, (chunk, qo)
 
 
-@first_hardware_run
-def test_both_kernels_agree_for_groups_of_four(gpu, monkeypatch):
+def test_both_kernels_agree_for_groups_of_four(gpu):
     B, H_kv, d, P, G = 3, 8, 128, 16, 4
     H = G * H_kv
     _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [2000, 77, 513], 25, O.F16)
     q = O.round_to(O.fill_normal((B, H, d), 25, 1), O.F16)
     scale = 1.0 / np.sqrt(d)
-    monkeypatch.delenv("AHPC_DECODE_MFMA", raising=False)
-    a = run(gpu, q, kp, vp, table, lens, B, H, H_kv, d, P, O.F16, O.F32, scale, 0)
-    monkeypatch.setenv("AHPC_DECODE_MFMA", "1")
-    b = run(gpu, q, kp, vp, table, lens, B, H, H_kv, d, P, O.F16, O.F32, scale, 0)
+    before = gpu.get_tuning("decode_matrix_min_group")
+    try:
+        gpu.set_tuning("decode_matrix_min_group", 16)
+        a = run(gpu, q, kp, vp, table, lens, B, H, H_kv, d, P, O.F16, O.F32, scale, 0)
+        gpu.set_tuning("decode_matrix_min_group", 4)
+        b = run(gpu, q, kp, vp, table, lens, B, H, H_kv, d, P, O.F16, O.F32, scale, 0)
+    finally:
+        gpu.set_tuning("decode_matrix_min_group", before)
     assert np.abs(a - b).max() <= 5e-3   # same inputs, fp32 outputs: only P's rounding to 16 bits differs
 
 

@@ -4,13 +4,11 @@ Bars: fp32 tensors 1e-4 max-abs (relative to the largest entry when that exceeds
 the largest entry of the gradient (gradient entries are sums over up to N terms, so their size grows with
 the problem, unlike the forward's convex combinations).  The reference has no working backward to compare with
 (src/algorithms/flash_attention.cpp:496-580 is a placeholder): parity is to the oracle, which is pinned by
-tests/test_oracle_backward.py.  This file is collected after every other GPU test on purpose: these kernels are the newest, and the tests that
-launch them wait for a first run by hand (gpu_util.first_hardware_run)."""
+tests/test_oracle_backward.py."""
 import numpy as np
 import pytest
 
 from oracle import oracle as O
-from gpu_util import first_hardware_run
 
 pytestmark = pytest.mark.gpu
 
@@ -45,7 +43,6 @@ def check(got, want, dtype):
         assert np.abs(g - w).max() <= bar, (name, float(np.abs(g - w).max()), bar)
 
 
-@first_hardware_run
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("B,N,H,H_kv,d", [(2, 16, 4, 4, 64), (1, 150, 2, 1, 32), (1, 40, 3, 3, 80), (1, 1, 2, 2, 128), (1, 300, 2, 2, 128)])
 def test_fp32_tensors(gpu, B, N, H, H_kv, d, causal):
@@ -58,7 +55,6 @@ def test_fp32_tensors(gpu, B, N, H, H_kv, d, causal):
     check(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), O.F32)
 
 
-@first_hardware_run
 def test_dense_mask(gpu):
     B, N, H, d = 2, 37, 2, 64
     q, k, v, do = inputs(B, N, H, H, d, 32, O.F32)
@@ -69,7 +65,6 @@ def test_dense_mask(gpu):
     check(got, O.attention_backward(q, k, v, do, B, N, H, d, 0.125, False, H, mask), O.F32)
 
 
-@first_hardware_run
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16])
 @pytest.mark.parametrize("B,N,H,H_kv,d,causal", [
     (1, 64, 1, 1, 128, False), (2, 129, 2, 2, 128, True), (1, 300, 2, 2, 64, True), (1, 200, 2, 1, 64, False),
@@ -83,7 +78,6 @@ def test_16bit_tensors(gpu, dtype, B, N, H, H_kv, d, causal):
     check(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), dtype)
 
 
-@first_hardware_run
 def test_closed_forms_16bit(gpu):
     B, N, H, d = 1, 256, 2, 128
     q, k, v, do = inputs(B, N, H, H, d, 35, O.BF16)
@@ -98,7 +92,6 @@ def test_closed_forms_16bit(gpu):
     assert np.abs(gv - do.mean(axis=1, keepdims=True)).max() <= 2e-2
 
 
-@first_hardware_run
 def test_headline_shape_bf16_causal(gpu):
     """B=4, N=4096, H=32, d=128, causal, bf16: properties that hold at any size over the whole result, and one
     (sequence, head) against the oracle."""
@@ -154,7 +147,6 @@ def test_bad_arguments_are_rejected_without_launch(gpu):
     torch.cuda.synchronize()
 
 
-@first_hardware_run
 @pytest.mark.parametrize("dtype,d,H,H_kv", [(O.F16, 64, 4, 4), (O.BF16, 128, 4, 2), (O.F32, 32, 2, 1)])
 @pytest.mark.parametrize("causal", [False, True])
 def test_ragged_batch(gpu, dtype, d, H, H_kv, causal):
@@ -185,7 +177,6 @@ def test_ragged_batch(gpu, dtype, d, H, H_kv, causal):
         check(tuple(g[a:b][None] for g in got), want, dtype)
 
 
-@first_hardware_run
 def test_golden_backward_vectors(gpu):
     """tests/golden/*.npz: gradients from a float64 computation that shares no code with the oracle."""
     import os
