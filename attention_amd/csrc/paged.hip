@@ -6,6 +6,8 @@
 // token with a single 16-byte load per lane.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include <cmath>
 #include <cstdlib>
 #include <type_traits>
@@ -573,6 +575,30 @@ static int launch_decode_d(const DecodeParams& p, dim3 grid, dim3 block, hipStre
     return p.P == 16 ? launch_decode_dp<T, 16>(p, grid, block, st) : launch_decode_dp<T, 0>(p, grid, block, st);
 }
 
+// ---- scratch of ahpc_hip_paged_decode_noalloc -------------------------------------------------------
+// Part of the device code, so every GPU that loads the library holds its own copy at its own address.  In
+// host code the array's name is only a handle for hipGetSymbolAddress: kernels and memory calls get the
+// looked-up device address, never the name.
+static __device__ __align__(256) unsigned char scratch[AHPC_NOALLOC_SCRATCH_BYTES];
+constexpr int kScratchDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kScratchDevices];  // per device; null until looked up
+
+static int scratch_of_current_device(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (dev < 0 || dev >= kScratchDevices) return AHPC_ERR_NO_DEVICE;
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (!ptr) return AHPC_ERR_NO_DEVICE;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // two threads racing here store the same address
+    }
+    *out = ptr;
+    return AHPC_OK;
+}
+
 }  // namespace ahpc
 
 using namespace ahpc;
@@ -780,6 +806,21 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
         return static_cast<int>(hipGetLastError());
     }
     return AHPC_OK;
+}
+
+int ahpc_hip_paged_decode_noalloc(const void* q, void* o, int qo_dtype, const void* k_pool, const void* v_pool, int pool_dtype,
+                                  const int32_t* block_table, const int32_t* seq_lens, const int32_t* batch_rows, int64_t B,
+                                  int64_t H, int64_t H_kv, int64_t d, int64_t P, int64_t max_pages, int64_t max_len,
+                                  float scale, int64_t chunk_tokens, void* stream) {
+    // (arguments that are wrong in themselves are reported by the call below, whatever this size comes out as)
+    if (ahpc_hip_paged_decode_workspace_bytes(B, H, d, max_len, P, chunk_tokens) > AHPC_NOALLOC_SCRATCH_BYTES)
+        return AHPC_ERR_SCRATCH_LIMIT;
+    void* ptr = nullptr;
+    if (int rc = scratch_of_current_device(&ptr)) return rc;
+    // The partials need no clearing between calls: the merge reads, per sequence, exactly the chunks whose
+    // decode workgroup wrote them in this call (those that start before the sequence's end).
+    return ahpc_hip_paged_decode_gqa(q, o, qo_dtype, k_pool, v_pool, pool_dtype, block_table, seq_lens, batch_rows, B, H, H_kv,
+                                     d, P, max_pages, max_len, scale, chunk_tokens, ptr, AHPC_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype, const void* k_pool, const void* v_pool, int pool_dtype,

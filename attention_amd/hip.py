@@ -76,6 +76,7 @@ SIGNATURES = {
     "ahpc_hip_paged_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64]),
     "ahpc_hip_paged_decode": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp, _sz, _vp]),
     "ahpc_hip_paged_decode_gqa": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp, _sz, _vp]),
+    "ahpc_hip_paged_decode_noalloc": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp]),
     "ahpc_hip_paged_gather_indices": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp]),
     "ahpc_hip_probe_matrix_rate": (_ci, [_ci, _ci, _i64, _i64, _vp, _sz, C.POINTER(C.c_double), _vp]),
 }
@@ -222,6 +223,14 @@ def paged_decode_gqa(q, o, qo_dtype, k_pool, v_pool, pool_dtype, table, seq_lens
     _check(load().ahpc_hip_paged_decode_gqa(q, o, qo_dtype, k_pool, v_pool, pool_dtype, table, seq_lens, batch_rows, B, H,
                                            H_kv, d, P, max_pages, max_len, scale, chunk_tokens, workspace,
                                            workspace_bytes, stream), "paged_decode_gqa")
+
+
+def paged_decode_noalloc(q, o, qo_dtype, k_pool, v_pool, pool_dtype, table, seq_lens, batch_rows, B, H, H_kv, d, P, max_pages,
+                         max_len, scale, chunk_tokens=0, stream=None):
+    """ahpc_hip_paged_decode_gqa without a workspace argument: partials in the library's built-in scratch array."""
+    _check(load().ahpc_hip_paged_decode_noalloc(q, o, qo_dtype, k_pool, v_pool, pool_dtype, table, seq_lens, batch_rows, B,
+                                               H, H_kv, d, P, max_pages, max_len, scale, chunk_tokens, stream),
+           "paged_decode_noalloc")
 
 
 def paged_gather_indices(table, seq_lens, batch_rows, B, H, d, P, max_pages, max_len, offsets, stream=None):

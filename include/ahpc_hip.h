@@ -43,7 +43,8 @@ typedef enum ahpc_status {
     AHPC_ERR_WORKSPACE_TOO_SMALL = -5,
     AHPC_ERR_NO_DEVICE = -6,
     AHPC_ERR_BAD_ALIGNMENT = -7,   /* pointers/strides must allow 16-byte vector access */
-    AHPC_ERR_UNSUPPORTED_GROUP = -8 /* query heads per K/V head: decode takes 1, 2, 4, 8 (16, 32: see paged_decode_gqa) */
+    AHPC_ERR_UNSUPPORTED_GROUP = -8, /* query heads per K/V head: decode takes 1, 2, 4, 8 (16, 32: see paged_decode_gqa) */
+    AHPC_ERR_SCRATCH_LIMIT = -9     /* ahpc_hip_paged_decode_noalloc: the call needs more than AHPC_NOALLOC_SCRATCH_BYTES */
 } ahpc_status;
 
 const char* ahpc_hip_error_string(int code);
@@ -288,10 +289,29 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype,
                               int64_t max_len, float scale, int64_t chunk_tokens,
                               void* workspace, size_t workspace_bytes, void* stream);
 
-/* Debug twin of the decode kernel's addressing: offsets[b*max_len + t] = the element offset
- * of (token t, head 0, lane 0) of batch entry b, computed by the same device function the
- * decode kernel uses, or -1 for t >= seq_lens[row] or a negative table entry.  Lets a test
- * compare the gather indices bit for bit with a host computation. */
+/* Decode for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  No counterpart in the reference.  Same arguments, kernels and results as
+ * ahpc_hip_paged_decode_gqa, without the workspace: the chunk partials live in an array that is part of the
+ * library's device code (AHPC_NOALLOC_SCRATCH_BYTES per GPU, held until the process ends).  The call performs no
+ * hipMalloc / hipFree and calls no allocating library routine; its first call on a device looks the array's
+ * address up (make that call outside a capture).  A call whose partials do not fit
+ * (ahpc_hip_paged_decode_workspace_bytes(...) > AHPC_NOALLOC_SCRATCH_BYTES) returns AHPC_ERR_SCRATCH_LIMIT and
+ * launches nothing.  Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (different
+ * streams, different threads) race; calls on one stream do not.  Nothing in the array has to start at zero. */
+#define AHPC_NOALLOC_SCRATCH_BYTES ((size_t)16 << 20)
+int ahpc_hip_paged_decode_noalloc(const void* q, void* o, int qo_dtype,
+                                  const void* k_pool, const void* v_pool, int pool_dtype,
+                                  const int32_t* block_table, const int32_t* seq_lens, const int32_t* batch_rows,
+                                  int64_t B, int64_t H, int64_t H_kv, int64_t d, int64_t P, int64_t max_pages,
+                                  int64_t max_len, float scale, int64_t chunk_tokens, void* stream);
+
+/* What the decode kernel gathers: offsets[b*max_len + t] = the element offset in the pool of (token t, head 0,
+ * element 0) of batch entry b, or -1 for a token the decode does not attend to (t >= seq_lens[row], or at and behind
+ * the first negative table entry of the row).  For the head dimensions the decode kernel takes (32, 64, 128, 256) the
+ * values are written by that kernel itself, launched in a reporting mode in which the expression that addresses a
+ * token row feeds a store instead of the loads; for other head dimensions by the index function of append and
+ * read-back.  Lets a test hold the GPU's gather indices bit for bit against the index math of the reference
+ * (src/backends/cuda/cuda_kernels.cu:417-440).  offsets: int64 [B][max_len] in device memory. */
 int ahpc_hip_paged_gather_indices(const int32_t* block_table, const int32_t* seq_lens, const int32_t* batch_rows,
                                   int64_t B, int64_t H, int64_t d, int64_t P, int64_t max_pages, int64_t max_len,
                                   int64_t* offsets, void* stream);

@@ -37,6 +37,7 @@
 #define __global__
 #define __device__
 #define __host__
+#define __align__(n) __attribute__((aligned(n)))
 #define __forceinline__ inline
 #define __launch_bounds__(...)
 #define __shared__ static __attribute__((section("simt_lds"), used))
@@ -128,6 +129,8 @@ struct hipDeviceProp_t {
 inline const char* hipGetErrorString(hipError_t e) { return e == hipSuccess ? "success" : "emulated kernel launch failed"; }
 inline hipError_t hipGetDeviceCount(int* n) { *n = 1; return hipSuccess; }
 inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
+#define HIP_SYMBOL(x) (&(x))
+template <typename S> inline hipError_t hipGetSymbolAddress(void** p, S* symbol) { *p = (void*)symbol; return hipSuccess; }
 inline hipError_t hipRuntimeGetVersion(int* v) { *v = 0; return hipSuccess; }
 inline hipError_t hipMemGetInfo(size_t* free_b, size_t* total_b) {
     *free_b = (size_t)4 << 30;  // what callers may really take from the host

@@ -510,3 +510,35 @@ def test_matrix_rate_probe_runs_and_counts_its_work(emu, dtype, mix):
     assert S.load().ahpc_hip_probe_matrix_rate(dtype, mix, wgs, it, S.ptr(sink), sink.nbytes, C.byref(flop), None) == 0
     assert np.isfinite(sink).all()
     assert flop.value == 2.0 * 32 * 32 * 16 * 4 * it * 4 * wgs
+
+
+# ---- decode without a workspace argument ----------------------------------------------------------------------
+def decode_noalloc(emu, q, kp, vp, table, lens, B, H, H_kv, d, P, dtype, scale, chunk):
+    dq = dev(q, dtype)
+    do = S.guarded(S.empty_storage((B, H, d), dtype))
+    dk, dv = dev(kp, dtype), dev(vp, dtype)
+    dt, dl = S.guarded(table), S.guarded(np.asarray(lens, np.int32))
+    emu.paged_decode_noalloc(S.ptr(dq), S.ptr(do), dtype, S.ptr(dk), S.ptr(dv), dtype, S.ptr(dt), S.ptr(dl), None, B, H, H_kv,
+                             d, P, table.shape[1], int(max(1, np.max(lens))), scale, chunk)
+    return S.from_storage(do, dtype)
+
+
+def test_decode_with_built_in_scratch_equals_decode_with_workspace(emu):
+    """Two calls in a row, the second smaller: the built-in array keeps the first call's partials."""
+    for B, H, H_kv, d, lens, seed, dtype, chunk in ((4, 4, 4, 64, [150, 5, 33, 70], 71, O.F16, 32),
+                                                    (2, 4, 4, 64, [40, 17], 72, O.F16, 32),
+                                                    (3, 8, 2, 128, [90, 0, 20], 73, O.BF16, 16)):
+        P = 16
+        _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, lens, seed, dtype)
+        q = O.round_to(O.fill_normal((B, H, d), seed, 1), dtype)
+        a = decode(emu, q, kp, vp, table, lens, None, B, H, H_kv, d, P, dtype, dtype, 0.125, chunk)
+        b = decode_noalloc(emu, q, kp, vp, table, lens, B, H, H_kv, d, P, dtype, 0.125, chunk)
+        assert np.isfinite(b).all() and np.array_equal(a, b)
+
+
+def test_decode_with_built_in_scratch_has_a_limit(emu):
+    x = S.guarded(np.zeros(64, np.float32))
+    p = S.ptr(x)
+    with pytest.raises(emu.HipError) as e:
+        emu.paged_decode_noalloc(p, p, O.F16, p, p, O.F16, p, p, None, 4096, 64, 64, 128, 16, 4096, 65536, 0.1, 16)
+    assert "scratch" in str(e.value)
