@@ -367,7 +367,7 @@ static int launch_mfma_dv(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool
     f.N = p.N; f.H = p.H; f.kv_group = p.kv_group;
     f.cu_seqlens = p.cu_seqlens;
     f.scale_log2 = p.scale_log2;
-    if (int rc = flash_plan_launch(f, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load())) return rc;
+    if (int rc = flash_plan_launch(f, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load(), VARLEN)) return rc;
     const FlashStatsOut st{p.d_out, lse2, delta, p.rows_padded};
     const dim3 block(kFlashThreads);
     const dim3 grid_stats((unsigned)(f.blocks_per_xcd * 8));

@@ -153,7 +153,7 @@ static int dispatch_simple(int dtype, const SimpleParams& p, int64_t B, hipStrea
 // ---------------------------------------------------------------------------------------------
 template <typename T, int D, bool VARLEN>
 static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
-    if (int rc = flash_plan_launch(p, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load())) return rc;
+    if (int rc = flash_plan_launch(p, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load(), VARLEN)) return rc;
     dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
     if (causal) hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, true, VARLEN>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, false, VARLEN>), grid, block, 0, stream, p);
@@ -238,8 +238,8 @@ int ahpc_hip_flash_block_map(int64_t B, int64_t N, int64_t H, int causal, int64_
     for (int64_t i = 0; i < grid; ++i) {
         const FlashWork w = flash_work_of_block((unsigned)i, p);
         seq_head[i] = w.valid ? w.bh : -1;
-        first_tile[i] = w.valid ? flash_qtile_of_part(p, w.slot, 0) : -1;
-        second_tile[i] = w.valid ? flash_qtile_of_part(p, w.slot, 1) : -1;
+        first_tile[i] = w.valid ? flash_qtile_of_part(p, p.n_qtiles, w.slot, 0) : -1;
+        second_tile[i] = w.valid ? flash_qtile_of_part(p, p.n_qtiles, w.slot, 1) : -1;
     }
     return AHPC_OK;
 }

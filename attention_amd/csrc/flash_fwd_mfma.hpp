@@ -60,6 +60,7 @@ struct FlashParams {
     int32_t paired;             // 1: a workgroup takes two query tiles of a head (see above)
     int32_t total_blocks;       // B * H * n_qtiles, or B * H * ceil(n_qtiles / 2) when paired
     int32_t n_bh;               // B * H: no workgroup may address a (sequence, head) at or beyond this
+    int32_t spread_groups;      // ragged batches: 1 = (sequence, head) pairs are dealt to the 8 XCDs in turn (see flash_work_of_block)
     int32_t blocks_per_xcd;     // ceil(total_blocks / 8)
     float scale_log2;           // scale * log2(e)
 };
@@ -150,6 +151,10 @@ __device__ inline void dma_dword(const void* base, unsigned nrec, int off, unsig
 // Workgroup id -> work.  Hardware deals consecutive workgroup ids to the 8 XCDs in turn; `logical` undoes
 // that, so that consecutive logical ids run on the same XCD and share its L2.  A head owns `per_head`
 // consecutive logical ids (its query tiles, or pairs of them), late (long) tiles first.
+// Ragged batches (spread_groups): sequences differ in length, so equal shares of the id range are not equal shares of
+// the work.  There the (sequence, head) pairs are dealt to the XCDs in turn - pair g runs on XCD g % 8, its tiles
+// still side by side on that XCD - every pair owns as many slots as the LONGEST sequence needs, and a workgroup
+// whose slot lies beyond its own sequence's tiles (counted and paired from that sequence's own length) exits at once.
 // Host and device evaluate the same code: a host-side dump of this function is what the tests check.
 struct FlashWork {
     int bh;     // sequence * H + head
@@ -159,19 +164,27 @@ struct FlashWork {
 __host__ __device__ inline int flash_per_head(const FlashParams& p) { return p.paired ? (p.n_qtiles + 1) >> 1 : p.n_qtiles; }
 __host__ __device__ inline FlashWork flash_work_of_block(unsigned block_id, const FlashParams& p) {
     const int xcd = (int)(block_id & 7u);
+    const int per_head = flash_per_head(p);
+    if (p.spread_groups) {
+        const int k = (int)(block_id >> 3);
+        const int round = k / per_head;
+        const int g = round * 8 + xcd;
+        if (g >= p.n_bh) return FlashWork{0, 0, false};
+        return FlashWork{g, k - round * per_head, true};
+    }
     const int logical = xcd * p.blocks_per_xcd + (int)(block_id >> 3);
     if (logical >= p.total_blocks) return FlashWork{0, 0, false};
-    const int per_head = flash_per_head(p);
     const int bh = logical / per_head;
     return FlashWork{bh, logical - bh * per_head, true};
 }
 // Query tile a workgroup handles in its first (part 0) and second (part 1) pass; -1 = none.
-__host__ __device__ inline int flash_qtile_of_part(const FlashParams& p, int slot, int part) {
+// n_qtiles: query tiles of the sequence in hand (p.n_qtiles for dense batches, the sequence's own count in a ragged one).
+__host__ __device__ inline int flash_qtile_of_part(const FlashParams& p, int n_qtiles, int slot, int part) {
     if (p.paired) {
-        if (part == 1 && 2 * slot == p.n_qtiles - 1) return -1;  // odd count: the middle tile has no partner
-        return part == 0 ? p.n_qtiles - 1 - slot : slot;
+        if (part == 1 && 2 * slot == n_qtiles - 1) return -1;  // odd count: the middle tile has no partner
+        return part == 0 ? n_qtiles - 1 - slot : slot;
     }
-    return part == 0 ? p.n_qtiles - 1 - slot : -1;
+    return part == 0 ? n_qtiles - 1 - slot : -1;
 }
 
 // What the statistics variant of the kernel writes instead of O (first step of the backward):
@@ -233,6 +246,10 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
         base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
         kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
     }
+    // query tiles of this sequence, and the slots they fill (a ragged batch hands every sequence as many slots as
+    // the longest one needs: the surplus exits here, before anything is requested)
+    const int n_q = VARLEN ? (L + kFlashRows - 1) / kFlashRows : p.n_qtiles;
+    if (VARLEN && slot >= (p.paired ? (n_q + 1) >> 1 : n_q)) return;
     const T* const gq = static_cast<const T*>(p.q) + base;
     const T* const gk = static_cast<const T*>(p.k) + kv_base;
     const T* const gv = static_cast<const T*>(p.v) + kv_base;
@@ -277,7 +294,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
     }
 
     for (int part = 0; part < 2; ++part) {
-        const int qt = flash_qtile_of_part(p, slot, part);
+        const int qt = flash_qtile_of_part(p, n_q, slot, part);
         if (qt < 0) break;
         const int q_tile0 = qt * kFlashRows;
         if (q_tile0 >= L) continue;
@@ -497,7 +514,8 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
 
 // Fills the launch geometry of the MFMA kernel (query tiles, pairing, workgroup count) from N, H and the batch size already in `p`.  Shared by the launcher and by the host-side dump
 // of the workgroup map.
-inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal, int rows_per_workgroup = kFlashRows, int64_t pair_min_tiles = 1024) {
+inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal, int rows_per_workgroup = kFlashRows, int64_t pair_min_tiles = 1024,
+                             bool ragged = false) {
     p.n_qtiles = (p.N + rows_per_workgroup - 1) / rows_per_workgroup;
     int64_t total = B * p.H * (int64_t)p.n_qtiles;
     if (total > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
@@ -509,6 +527,12 @@ inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal, int rows_pe
     p.total_blocks = (int32_t)total;
     p.n_bh = (int32_t)(B * p.H);
     p.blocks_per_xcd = (int32_t)((total + 7) / 8);
+    p.spread_groups = ragged ? 1 : 0;
+    if (ragged) {
+        const int64_t per_xcd = ((B * p.H + 7) / 8) * (p.paired ? (p.n_qtiles + 1) / 2 : p.n_qtiles);
+        if (per_xcd * 8 > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
+        p.blocks_per_xcd = (int32_t)per_xcd;
+    }
     return AHPC_OK;
 }
 

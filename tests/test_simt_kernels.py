@@ -109,6 +109,31 @@ def test_ragged_batch(emu, dtype, d):
     assert np.abs(S.from_storage(do, dtype) - want).max() <= TOL[dtype]
 
 
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("paired", [False, True])
+def test_ragged_batch_of_very_different_lengths(emu, causal, paired):
+    """Every sequence is tiled and paired from its own length: an empty one, some shorter than a tile, odd and even
+    tile counts, 3 heads on 8 XCDs (the surplus slots of the short sequences exit without touching anything)."""
+    if paired:
+        emu.set_tuning("flash_pair_min_tiles", 1)
+    try:
+        H, d, dtype = 3, 64, O.F16
+        lens = np.array([1, 130, 0, 64, 700, 257, 384, 129], np.int32)
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        T = int(cu[-1])
+        q, k, v = qkv((T, H, d), 16, dtype)
+        dq, dk, dv = dev(q, dtype), dev(k, dtype), dev(v, dtype)
+        do = S.guarded(S.empty_storage((T, H, d), dtype))
+        dcu = S.guarded(cu)
+        emu.flash_fwd_varlen(S.ptr(dq), S.ptr(dk), S.ptr(dv), S.ptr(do), dtype, S.ptr(dcu), len(lens), int(lens.max()), H, d,
+                             H * d, d, 0.125, causal)
+        got = S.from_storage(do, dtype)
+        assert np.isfinite(got).all()
+        assert np.abs(got - O.attention_varlen(q, k, v, cu, H, d, 0.125, causal)).max() <= TOL[dtype]
+    finally:
+        emu.set_tuning("flash_pair_min_tiles", 1024)
+
+
 def test_head_major_strides(emu):
     # the same tensors laid out [B,H,N,d]: only the strides change
     B, N, H, d = 1, 140, 3, 128
