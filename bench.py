@@ -12,7 +12,14 @@ PagedAttention decode result (fp16, B=64, H=32, d=128, page 16, context lengths 
                    events on the launch stream, against MI355X's dense bf16 MFMA peak (2.5 PFLOP/s)
                    or HBM peak (8 TB/s)
   cpu_baseline     the CPU oracle (oracle/, a restatement of the reference's algorithm) timed on this
-                   box's host cores over a bounded sample of the same workload
+                   box's host cores over a bounded sample of the same workload: on all cores (OpenMP over rows)
+                   and, under "single_thread", on one core as the reference's own CPU path runs
+  extras           the other configurations (long-context decode, ragged prefill, backward, grouped heads,
+                   batched append), one row each, timed in the same run
+
+Inputs of the two headline workloads come from the oracle's seeded generator (splitmix64 + Box-Muller, seeds
+0xA77E0002 / 0xA77E0003, tensor ids 1-5), rounded to the storage type on the host, so that the CPU legs and the
+GPU see the same values; the extras draw theirs with torch.randn on the GPU.
 """
 import argparse
 import json
@@ -28,23 +35,47 @@ sys.path.insert(0, ROOT)
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on exactly these workloads,
-# each counter scaled by its reading for a 1 GiB device copy (profiles/*.txt hold the runs).
-FLASH_TRAFFIC_BYTES = 672_100_000     # 537.9 MB fetched + 134.2 MB written (algorithmic: 536.9 MB)
-DECODE_TRAFFIC_BYTES = 2_364_900_000  # decode 2343.7 + 9.8 MB, merge 10.9 + 0.5 MB (algorithmic: 2342.9 MB)
+# HBM bytes per launch come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of exactly these workloads (each counter
+# scaled by its reading for a 1 GiB device copy).  The figure is not re-measured by this script: it is read from the
+# committed summary of those runs, together with the kernel it was taken for, and reported as null when that summary
+# is missing or names another kernel.
+PROFILE_FLASH = os.path.join(ROOT, "profiles", "flash_fwd_mfma_bf16_d128_causal_B4_N4096_H32.txt")
+PROFILE_DECODE = os.path.join(ROOT, "profiles", "paged_decode_f16_d128_B64_ctx512-4096.txt")
+
+
+def traffic_from_profile(path, kernel_word):
+    """(bytes per launch, provenance) from the lines `traffic_bytes_per_launch = N` and `measured = ...` of a profile
+    summary whose `kernel = ...` line contains kernel_word; (None, reason) otherwise."""
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, "no profile summary at " + os.path.relpath(path, ROOT)
+    fields = {}
+    for line in text.splitlines():
+        if " = " in line and not line.startswith(" "):
+            k, v = line.split(" = ", 1)
+            fields[k.strip()] = v.strip()
+    if kernel_word not in fields.get("kernel", ""):
+        return None, "profile summary is for another kernel: " + fields.get("kernel", "?")
+    try:
+        return int(fields["traffic_bytes_per_launch"]), os.path.relpath(path, ROOT) + " (" + fields.get("measured", "undated") + ")"
+    except (KeyError, ValueError):
+        return None, "profile summary holds no traffic figure"
+
 
 FLASH = dict(B=4, N=4096, H=32, d=128, causal=True, dtype="bf16", seed=0xA77E0002)
 DECODE = dict(B=64, H=32, d=128, P=16, lo=512, hi=4096, dtype="fp16", seed=0xA77E0003)
 
 
 def lengths_and_table(cfg):
-    """Seeded context lengths and a shuffled block table (numpy only)."""
-    rng = np.random.default_rng(cfg["seed"])
-    lens = rng.integers(cfg["lo"], cfg["hi"] + 1, size=cfg["B"]).astype(np.int32)
+    """Seeded context lengths (tensor id 4) and a block table that is a slice of a seeded permutation of the page
+    ids (tensor id 5), both from the oracle's generator."""
+    from oracle import oracle as O
+    lens = O.fill_lengths(cfg["B"], cfg["seed"], 4, cfg["lo"], cfg["hi"])
     P = cfg["P"]
     pages_per = (lens + P - 1) // P
     n_pages = int(pages_per.sum()) + 64
-    ids = rng.permutation(n_pages).astype(np.int32)
+    ids = O.permutation(n_pages, cfg["seed"], 5)
     table = np.full((cfg["B"], int(pages_per.max())), -1, np.int32)
     c = 0
     for b in range(cfg["B"]):
@@ -112,12 +143,32 @@ def timed_steps(hip, stream, launch, steps, warmup):
     return wall, per
 
 
+def seeded_tensor(shape, seed, tensor_id, torch_dtype, code, keep_host=False, sigma=1.0):
+    """N(0, sigma) from the oracle's generator, rounded to the storage type on the host, on the GPU.  Generated in
+    pieces of 32 Mi elements so that the host never holds more than one piece (unless keep_host)."""
+    import torch
+    from oracle import oracle as O
+    n = int(np.prod(shape))
+    dev = torch.empty(n, dtype=torch_dtype, device="cuda")
+    host = np.empty(n, np.float32) if keep_host else None
+    piece = 1 << 25
+    buf = np.empty(min(piece, n), np.float32)
+    for first in range(0, n, piece):
+        m = min(piece, n - first)
+        x = O.fill_normal_at(buf[:m], seed, tensor_id, sigma, first)
+        x = O.round_to(x, code)
+        dev[first:first + m] = torch.from_numpy(x).to(torch_dtype)
+        if keep_host:
+            host[first:first + m] = x
+    return dev.view(*shape), (host.reshape(shape) if keep_host else None)
+
+
 def bench_flash(hip, stream, steps, warmup, cpu):
     import torch
+    from oracle import oracle as O
     c = FLASH
     B, N, H, d = c["B"], c["N"], c["H"], c["d"]
-    g = torch.Generator(device="cuda").manual_seed(c["seed"])
-    q, k, v = (torch.randn((B, N, H, d), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16) for _ in range(3))
+    (q, qh), (k, kh), (v, vh) = (seeded_tensor((B, N, H, d), c["seed"], t, torch.bfloat16, O.BF16, keep_host=cpu) for t in (1, 2, 3))
     o = torch.empty_like(q)
     torch.cuda.synchronize()
     scale = 1.0 / np.sqrt(d)
@@ -131,29 +182,45 @@ def bench_flash(hip, stream, steps, warmup, cpu):
     value = flops * steps / wall / 1e12
     kern_ms = float(np.mean(per))
     achieved = flops / (kern_ms * 1e-3) / 1e12
+    flash_traffic, flash_traffic_src = traffic_from_profile(PROFILE_FLASH, "flash_fwd_mfma_kernel")
     res = {
         "metric": "FlashAttn fwd TFLOP/s (bf16, N=4096, d=128)", "value": round(value, 2), "unit": "TFLOP/s",
         "ms_per_step": round(wall / steps * 1e3, 4),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": FLASH_TRAFFIC_BYTES,
+                     "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": flash_traffic, "traffic_source": flash_traffic_src,
                      "kernel": "flash_fwd_mfma_kernel<bf16,128,causal>", "kernel_ms_mean": round(kern_ms, 4),
                      "kernel_ms_min": round(float(np.min(per)), 4), "flop_per_launch": flops},
         "config": {"workload": "flash_fwd bf16 causal B=4 N=4096 H=32 d=128 layout [B,N,H,d], fp32 accumulate, bf16 out"},
     }
     if cpu:
-        from oracle import oracle as O
-        # bounded sample: the first `nb` batch entries (all 32 heads each) on the box's host cores
+        # all cores: the whole step (the same rounded inputs the GPU got), OpenMP over rows
         nb, reps = 4, 3
-        qs, ks, vs = (t[0:nb].float().cpu().numpy() for t in (q, k, v))
         threads = O.cpu_threads()
         t0 = time.perf_counter()
         for _ in range(reps):
-            ref = O.attention(qs, ks, vs, nb, N, H, d, scale, True, threads=threads)
+            ref = O.attention(qh, kh, vh, nb, N, H, d, scale, True, threads=threads)
         dt = (time.perf_counter() - t0) / reps
         err = float(np.abs(o[0:nb].float().cpu().numpy() - ref).max())
         res["cpu_baseline"] = {"value": round(2.0 * nb * H * N * N * d / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads,
                                "kind": "port", "sample": f"the whole step ({nb}x32 heads x 4096 rows), mean of {reps} passes of "
                                f"{dt:.1f} s wall on {threads} threads", "max_abs_err_gpu_vs_cpu": err}
+        # one core, as the reference's CPU path runs (it has no threading): 1/128 of the step - one head of one batch
+        # entry, all 4096 rows - and the reference's own CPU-sized configuration in full
+        q1, k1, v1 = (np.ascontiguousarray(x[0:1, :, 0:1, :]) for x in (qh, kh, vh))
+        t0 = time.perf_counter()
+        O.attention(q1, k1, v1, 1, N, 1, d, scale, True, threads=1)
+        dt1 = time.perf_counter() - t0
+        Bc, Nc, Hc, dc = 2, 512, 8, 64
+        qc, kc, vc = (O.fill_normal((Bc, Nc, Hc, dc), 0xA77E0001, t) for t in (1, 2, 3))
+        t0 = time.perf_counter()
+        O.attention(qc, kc, vc, Bc, Nc, Hc, dc, 1.0 / np.sqrt(dc), False, threads=1)
+        dtc = time.perf_counter() - t0
+        res["cpu_baseline"]["single_thread"] = {
+            "value": round(2.0 * N * N * d / dt1 / 1e12, 6), "unit": "TFLOP/s", "cores": 1,
+            "sample": f"1/128 of the step (batch entry 0, head 0, 4096 rows), one pass of {dt1:.2f} s; the whole step "
+                      f"extrapolates to {dt1 * B * H:.0f} s",
+            "reference_cpu_config": {"workload": "flash_fwd fp32 non-causal B=2 N=512 H=8 d=64 (in full)", "seconds": round(dtc, 3),
+                                     "value": round(4.0 * Bc * Hc * Nc * Nc * dc / dtc / 1e12, 6), "unit": "TFLOP/s"}}
     return res
 
 
@@ -161,12 +228,12 @@ def bench_decode(hip, stream, steps, warmup, cpu):
     import torch
     c = DECODE
     B, H, d, P = c["B"], c["H"], c["d"], c["P"]
+    from oracle import oracle as O
     lens, table, n_pages = lengths_and_table(c)
-    g = torch.Generator(device="cuda").manual_seed(c["seed"])
     elems = n_pages * P * H * d
-    kpool = torch.randn(elems, generator=g, device="cuda", dtype=torch.float32).to(torch.float16)
-    vpool = torch.randn(elems, generator=g, device="cuda", dtype=torch.float32).to(torch.float16)
-    q = torch.randn((B, H, d), generator=g, device="cuda", dtype=torch.float32).to(torch.float16)
+    kpool, _ = seeded_tensor((elems,), c["seed"], 2, torch.float16, O.F16)
+    vpool, _ = seeded_tensor((elems,), c["seed"], 3, torch.float16, O.F16)
+    q, _ = seeded_tensor((B, H, d), c["seed"], 1, torch.float16, O.F16)
     o = torch.empty_like(q)
     dt_, dl = torch.from_numpy(table).cuda(), torch.from_numpy(lens).cuda()
     max_len, max_pages = int(lens.max()), table.shape[1]
@@ -184,18 +251,18 @@ def bench_decode(hip, stream, steps, warmup, cpu):
     value = nbytes * steps / wall / 1e9
     kern_ms = float(np.mean(per))
     achieved = nbytes / (kern_ms * 1e-3) / 1e9
+    decode_traffic, decode_traffic_src = traffic_from_profile(PROFILE_DECODE, "paged_decode_kernel")
     res = {
         "metric": "paged decode HBM GB/s", "value": round(value, 1), "unit": "GB/s",
         "ms_per_step": round(wall / steps * 1e3, 4),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": DECODE_TRAFFIC_BYTES,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": decode_traffic, "traffic_source": decode_traffic_src,
                      "kernel": "paged_decode_kernel<f16,128> + paged_merge_kernel", "kernel_ms_mean": round(kern_ms, 4),
                      "kernel_ms_min": round(float(np.min(per)), 4), "bytes_per_launch": nbytes},
         "config": {"workload": f"paged_decode fp16 B=64 H=32 d=128 page=16 context U[512,4096] (sum {int(lens.sum())} tokens), "
                                f"shuffled block table, pool {n_pages} pages"},
     }
     if cpu:
-        from oracle import oracle as O
         # bounded sample: the first 32 of the 64 sequences, their pages copied to the host; 200 passes
         nb = 32
         pages_per = (lens + P - 1) // P
@@ -223,6 +290,13 @@ def bench_decode(hip, stream, steps, warmup, cpu):
                                "kind": "port", "sample": f"first {nb} of 64 sequences ({int(lens[:nb].sum())} tokens), mean of "
                                f"{reps} passes of {dt:.2f} s on {threads} threads; bytes counted at the GPU's 2-byte storage size "
                                "(the CPU path streams fp32 copies, twice as many bytes)", "max_abs_err_gpu_vs_cpu": err}
+        reps1 = 10
+        t0 = time.perf_counter()
+        for _ in range(reps1):
+            O.paged_decode(qh, kh, vh, st, lens[:nb], None, nb, H, d, P, scale, threads=1)
+        dt1 = (time.perf_counter() - t0) / reps1
+        res["cpu_baseline"]["single_thread"] = {"value": round(decode_bytes(lens[:nb], sub) / dt1 / 1e9, 3), "unit": "GB/s", "cores": 1,
+                                                "sample": f"the same {nb} sequences, mean of {reps1} passes of {dt1:.2f} s on one thread"}
     return res
 
 
@@ -280,8 +354,8 @@ def bench_extras(hip, stream, steps, warmup):
         flops=2.5 * 2.0 * B * H * N * N * d)
 
     # ragged fp16 causal batch: 16 sequences, lengths U[128,8192], H=32, d=64 (sigma 0.5)
-    rng = np.random.default_rng(0xA77E0005)
-    lens = rng.integers(128, 8193, size=16).astype(np.int32)
+    from oracle import oracle as O
+    lens = O.fill_lengths(16, 0xA77E0005, 4, 128, 8192)
     cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     T, Hv, dv_ = int(cu[-1]), 32, 64
     qv = (randn((T, Hv, dv_), torch.float32) * 0.5).to(torch.float16)
@@ -290,7 +364,7 @@ def bench_extras(hip, stream, steps, warmup):
     ov = torch.empty_like(qv)
     dcu = torch.from_numpy(cu).cuda()
     L = lens.astype(np.float64)
-    run(f"flash_fwd_varlen fp16 causal 16 seqs U[128,8192] ({T} tokens) H=32 d=64",
+    run(f"flash_fwd_varlen fp16 causal 16 seqs U[128,8192] ({T} tokens) H=32 d=64 (BASELINE config 5)",
         lambda: hip.flash_fwd_varlen(qv.data_ptr(), kv.data_ptr(), vv.data_ptr(), ov.data_ptr(), hip.F16, dcu.data_ptr(), 16,
                                      int(lens.max()), Hv, dv_, Hv * dv_, dv_, 1.0 / np.sqrt(dv_), True, stream),
         flops=float((4.0 * Hv * dv_ * L * (L + 1) / 2).sum()))
@@ -315,19 +389,13 @@ def bench_extras(hip, stream, steps, warmup):
                                          max_len, scl, 0, ws.data_ptr(), wsb, stream),
             nbytes=nb)
 
-    decode_case("paged_decode bf16 B=8 H=32 d=128 page=16 context U[16384,32768]",
+    decode_case("paged_decode bf16 B=8 H=32 d=128 page=16 context U[16384,32768] (BASELINE config 4)",
                 dict(B=8, H=32, d=128, P=16, lo=16384, hi=32768, seed=0xA77E0004), 32, 32, hip.BF16, torch.bfloat16)
     decode_case("paged_decode fp16 B=64 H=32 over 8 pool heads d=128 page=16 context U[512,4096]",
                 dict(DECODE), 32, 8, hip.F16, torch.float16)
-    # the same grouped decode, and multi-query decode, on the matrix-core kernel
-    hip.set_tuning("decode_matrix_min_group", 4)
-    try:
-        decode_case("paged_decode (matrix-core kernel) fp16 B=64 H=32 over 8 pool heads d=128 page=16 context U[512,4096]",
-                    dict(DECODE), 32, 8, hip.F16, torch.float16)
-        decode_case("paged_decode (matrix-core kernel) fp16 B=64 H=32 over 1 pool head d=128 page=16 context U[512,4096]",
-                    dict(DECODE), 32, 1, hip.F16, torch.float16)
-    finally:
-        hip.set_tuning("decode_matrix_min_group", 16)
+    # multi-query decode (32 query heads over one pool head): the matrix-core kernel
+    decode_case("paged_decode (matrix-core kernel) fp16 B=64 H=32 over 1 pool head d=128 page=16 context U[512,4096]",
+                dict(DECODE), 32, 1, hip.F16, torch.float16)
 
     # prefill -> cache hand-off: K and V of the headline prefill into the pool, one launch
     P = 16
@@ -447,6 +515,8 @@ def main():
         out["dtype"] = "f16"
     if flash and decode:
         out["decode"] = decode
+        # the other configurations, in the same run and on the same box (inputs: torch.randn on the GPU)
+        out["extras"] = bench_extras(hip, stream, min(a.steps, 20), min(a.warmup, 5))
     info = hip.device_info(0)
     out["device"] = {"name": info.name.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units}
     hip.load().ahpc_hip_stream_destroy(stream)

@@ -44,15 +44,22 @@ static inline uint64_t draw(uint64_t seed, uint64_t tensor_id, uint64_t i) {
     return mix64(mix64(seed ^ (tensor_id * 0x9E3779B97F4A7C15ull)) + i);
 }
 
-void ahpc_oracle_fill_normal(float* out, size_t n, uint64_t seed, uint64_t tensor_id, float sigma) {
+/* Elements first .. first+n-1 of the stream (every element depends on its index only, so any split of a tensor
+ * into pieces, and any number of threads, gives the same values). */
+void ahpc_oracle_fill_normal_at(float* out, size_t n, uint64_t seed, uint64_t tensor_id, float sigma, uint64_t first) {
     const double two_pi = 6.283185307179586476925286766559;
+#pragma omp parallel for schedule(static) if (n > 65536)
     for (size_t i = 0; i < n; ++i) {
-        uint64_t z = draw(seed, tensor_id, (uint64_t)i);
+        uint64_t z = draw(seed, tensor_id, first + (uint64_t)i);
         double u1 = (double)((z >> 40) + 1) * (1.0 / 16777216.0);       /* (0, 1] */
         double u2 = (double)((z >> 16) & 0xFFFFFFu) * (1.0 / 16777216.0); /* [0, 1) */
         double r = sqrt(-2.0 * log(u1));
         out[i] = (float)(r * cos(two_pi * u2)) * sigma;
     }
+}
+
+void ahpc_oracle_fill_normal(float* out, size_t n, uint64_t seed, uint64_t tensor_id, float sigma) {
+    ahpc_oracle_fill_normal_at(out, n, seed, tensor_id, sigma, 0);
 }
 
 void ahpc_oracle_fill_uniform(float* out, size_t n, uint64_t seed, uint64_t tensor_id, float lo, float hi) {

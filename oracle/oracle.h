@@ -32,6 +32,8 @@ extern "C" {
  * tests/test_flash_attention.cpp:16-27, so there is nothing to restate: this only has to
  * be reproducible.) */
 void ahpc_oracle_fill_normal(float* out, size_t n, uint64_t seed, uint64_t tensor_id, float sigma);
+/* The same stream from element `first` on: a tensor generated in pieces holds the same values. */
+void ahpc_oracle_fill_normal_at(float* out, size_t n, uint64_t seed, uint64_t tensor_id, float sigma, uint64_t first);
 /* Same counter hash, uniform in [lo, hi) (the reference's tests draw U(-1,1),
  * tests/test_flash_attention.cpp:16-27). */
 void ahpc_oracle_fill_uniform(float* out, size_t n, uint64_t seed, uint64_t tensor_id, float lo, float hi);

@@ -32,6 +32,7 @@ def _load():
     i64, u64, f32, ci = C.c_int64, C.c_uint64, C.c_float, C.c_int
     sig = {
         "ahpc_oracle_fill_normal": (None, [fp, C.c_size_t, u64, u64, f32]),
+        "ahpc_oracle_fill_normal_at": (None, [fp, C.c_size_t, u64, u64, f32, C.c_uint64]),
         "ahpc_oracle_fill_uniform": (None, [fp, C.c_size_t, u64, u64, f32, f32]),
         "ahpc_oracle_fill_lengths": (None, [ip, C.c_size_t, u64, u64, C.c_int32, C.c_int32]),
         "ahpc_oracle_permutation": (None, [ip, C.c_size_t, u64, u64]),
@@ -101,6 +102,12 @@ def fill_normal(shape, seed, tensor_id, sigma=1.0):
 def fill_uniform(shape, seed, tensor_id, lo=-1.0, hi=1.0):
     out = np.empty(shape, np.float32)
     lib.ahpc_oracle_fill_uniform(_f(out), out.size, seed, tensor_id, lo, hi)
+    return out
+
+
+def fill_normal_at(out, seed, tensor_id, sigma, first):
+    """Fills the float32 array `out` with elements first .. first+out.size-1 of the stream fill_normal draws from."""
+    lib.ahpc_oracle_fill_normal_at(_f(out), out.size, seed, tensor_id, sigma, first)
     return out
 
 
