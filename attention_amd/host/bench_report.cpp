@@ -5,14 +5,15 @@
 // elements skipped, :490-493), same warm-up 5 / 10 timed iterations, same derived figures and the same JSON
 // field names, so that its results file can be laid beside one produced by the reference.
 //
-// Differences, all forced: the backend is BackendType::HIP; there is no backward pass
-// (backward_time_ms = 0, so total_time_ms = forward_time_ms and "gflops" - which the reference computes
-// from B*H*N^2*d*2 over the TOTAL time, :241-242 - is a forward-only figure); inputs are seeded, not
-// std::random_device.  Two extra fields per row say where the tensors lived: with --device the tensors are
-// resident in HBM (the kernel rate), without it they are host vectors exactly as in the reference and
-// forward_time_ms includes the PCIe copies of Q, K, V and O.
+// The backward pass is timed into backward_time_ms and total_time_ms exactly as the reference does (:215-235), and
+// "gflops" is the reference's figure: B*H*N^2*d*2 over the TOTAL time (:241-242).  --csv FILE also writes the table of
+// examples/performance_comparison.cpp:431-463 (same columns, same precisions).
 //
-//   ahpc_bench_report [--device] [--dtype fp32|fp16|bf16] [--causal] [--quick] [--json FILE]
+// Differences, all forced: the backend is BackendType::HIP; inputs are seeded, not std::random_device.  Two extra
+// JSON fields per row say where the tensors lived: with --device the tensors are resident in HBM (the kernel rate),
+// without it they are host vectors exactly as in the reference and the times include the PCIe copies.
+//
+//   ahpc_bench_report [--device] [--dtype fp32|fp16|bf16] [--causal] [--quick] [--json FILE] [--csv FILE]
 #include <chrono>
 #include <cmath>
 #include <cstdio>
@@ -37,6 +38,7 @@ struct Options {
     bool device = false, causal = false, quick = false;
     DataType dtype = DataType::FLOAT32;
     std::string json = "benchmark_results.json";
+    std::string csv;   // empty: no CSV file
     int warmup = 5, iters = 10;  // BenchmarkConfig::warmup_iterations / benchmark_iterations
 };
 
@@ -106,19 +108,32 @@ Metrics run_config(size_t B, size_t N, size_t H, size_t d, const Options& opt) {
         const TensorShape shape({B, N, H, d}, opt.dtype, MemoryLayout::ROW_MAJOR);
         const void *pq = q.data(), *pk = k.data(), *pv = v.data();
         void* po = o.data();
-        std::unique_ptr<DeviceTensor> dq, dk, dv, dout;
+        // backward operands: dO in, dQ, dK, dV out (:178-184)
+        auto go = random_tensor(n, opt.dtype, 4);
+        std::vector<unsigned char> gq(bytes, 0), gk(bytes, 0), gv(bytes, 0);
+        const void* pgo = go.data();
+        void *pgq = gq.data(), *pgk = gk.data(), *pgv = gv.data();
+        std::unique_ptr<DeviceTensor> dq, dk, dv, dout, dgo, dgq, dgk, dgv;
         if (opt.device) {
             dq.reset(new DeviceTensor(q)); dk.reset(new DeviceTensor(k)); dv.reset(new DeviceTensor(v)); dout.reset(new DeviceTensor(o));
+            dgo.reset(new DeviceTensor(go)); dgq.reset(new DeviceTensor(gq)); dgk.reset(new DeviceTensor(gk)); dgv.reset(new DeviceTensor(gv));
             pq = dq->p; pk = dk->p; pv = dv->p; po = dout->p;
+            pgo = dgo->p; pgq = dgq->p; pgk = dgk->p; pgv = dgv->p;
         }
-        m.memory_usage_bytes = m.peak_memory_bytes = 4 * bytes;  // Q, K, V, O (the tracker of :186-191; no workspace here)
+        m.memory_usage_bytes = m.peak_memory_bytes = 8 * bytes;  // Q, K, V, O, dO, dQ, dK, dV (the tracker of :186-191)
 
         for (int i = 0; i < opt.warmup; ++i) attention->forward(shape, pq, shape, pk, shape, pv, shape, po);
         const auto t0 = std::chrono::steady_clock::now();
         for (int i = 0; i < opt.iters; ++i) attention->forward(shape, pq, shape, pk, shape, pv, shape, po);
         const auto t1 = std::chrono::steady_clock::now();
         m.forward_time_ms = std::chrono::duration<double, std::milli>(t1 - t0).count() / opt.iters;
-        m.backward_time_ms = 0.0;  // no backward pass in this backend
+        // backward pass, timed like the forward (:215-235); one untimed call first
+        attention->backward(shape, pgo, shape, pq, shape, pk, shape, pv, shape, pgq, shape, pgk, shape, pgv);
+        const auto t2 = std::chrono::steady_clock::now();
+        for (int i = 0; i < opt.iters; ++i)
+            attention->backward(shape, pgo, shape, pq, shape, pk, shape, pv, shape, pgq, shape, pgk, shape, pgv);
+        const auto t3 = std::chrono::steady_clock::now();
+        m.backward_time_ms = std::chrono::duration<double, std::milli>(t3 - t2).count() / opt.iters;
         m.total_time_ms = m.forward_time_ms + m.backward_time_ms;
         const double flops = (double)B * H * N * N * d * 2;  // :241
         m.gflops = (flops / 1e9) / (m.total_time_ms / 1000.0);
@@ -182,6 +197,28 @@ bool save_json(const std::vector<Result>& results, const Options& opt) {  // Sav
     return true;
 }
 
+// save_results_to_csv, examples/performance_comparison.cpp:431-463: same header, same precisions
+bool save_csv(const std::vector<Result>& results, const std::string& filename) {
+    std::ofstream file(filename);
+    if (!file.is_open()) return false;
+    file << "Backend,BatchSize,SequenceLength,NumHeads,HeadDimension,";
+    file << "ForwardTimeMs,BackwardTimeMs,TotalTimeMs,MemoryUsageMB,PeakMemoryMB,";
+    file << "ThroughputTokensPerSec,GFLOPS,Success,ErrorMessage" << std::endl;
+    for (const Result& r : results) {
+        file << "HIP" << "," << r.B << "," << r.N << "," << r.H << "," << r.d << ","
+             << std::fixed << std::setprecision(6) << r.m.forward_time_ms << ","
+             << std::fixed << std::setprecision(6) << r.m.backward_time_ms << ","
+             << std::fixed << std::setprecision(6) << r.m.total_time_ms << ","
+             << std::fixed << std::setprecision(2) << r.m.memory_usage_bytes / 1024.0 / 1024.0 << ","
+             << std::fixed << std::setprecision(2) << r.m.peak_memory_bytes / 1024.0 / 1024.0 << ","
+             << std::fixed << std::setprecision(0) << r.m.throughput_tokens_per_sec << ","
+             << std::fixed << std::setprecision(4) << r.m.gflops << ","
+             << (r.m.success ? "true" : "false") << ","
+             << "\"" << r.m.error_message << "\"" << std::endl;
+    }
+    return true;
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
@@ -192,11 +229,12 @@ int main(int argc, char** argv) {
         else if (a == "--causal") opt.causal = true;
         else if (a == "--quick") opt.quick = true;
         else if (a == "--json" && i + 1 < argc) opt.json = argv[++i];
+        else if (a == "--csv" && i + 1 < argc) opt.csv = argv[++i];
         else if (a == "--dtype" && i + 1 < argc) {
             const std::string t = argv[++i];
             opt.dtype = t == "fp16" ? DataType::FLOAT16 : t == "bf16" ? DataType::BFLOAT16 : DataType::FLOAT32;
         } else {
-            std::cerr << "usage: ahpc_bench_report [--device] [--dtype fp32|fp16|bf16] [--causal] [--quick] [--json FILE]\n";
+            std::cerr << "usage: ahpc_bench_report [--device] [--dtype fp32|fp16|bf16] [--causal] [--quick] [--json FILE] [--csv FILE]\n";
             return 2;
         }
     }
@@ -227,6 +265,13 @@ int main(int argc, char** argv) {
         return 1;
     }
     std::cout << "Results saved to " << opt.json << "\n";
+    if (!opt.csv.empty()) {
+        if (!save_csv(results, opt.csv)) {
+            std::cerr << "Failed to open file for writing: " << opt.csv << "\n";
+            return 1;
+        }
+        std::cout << "\nResults saved to: " << opt.csv << "\n";
+    }
     for (const Result& r : results)
         if (!r.m.success) return 1;
     return 0;
