@@ -49,6 +49,6 @@ def test_quick_sweep_writes_reference_shaped_results(tmp_path, args):
     assert len(lines) == 1 + len(rows)
     for line, row in zip(lines[1:], rows):
         assert line[0] == "HIP" and [int(x) for x in line[1:5]] == [row[k] for k in ("batch_size", "sequence_length", "num_heads", "head_dimension")]
-        assert float(line[5]) == pytest.approx(row["forward_time_ms"], abs=1e-5) and float(line[6]) == pytest.approx(row["backward_time_ms"], abs=1e-5)
-        assert float(line[7]) == pytest.approx(row["total_time_ms"], abs=1e-5) and float(line[11]) == pytest.approx(row["gflops"], rel=1e-3, abs=1e-3)
+        assert float(line[5]) == pytest.approx(row["forward_time_ms"], rel=1e-4, abs=1e-5) and float(line[6]) == pytest.approx(row["backward_time_ms"], rel=1e-4, abs=1e-5)
+        assert float(line[7]) == pytest.approx(row["total_time_ms"], rel=1e-4, abs=1e-5) and float(line[11]) == pytest.approx(row["gflops"], rel=1e-3, abs=1e-3)
         assert line[12] == "true" and line[13] == ""
