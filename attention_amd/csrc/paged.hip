@@ -519,22 +519,54 @@ __global__ __launch_bounds__(256) void paged_merge_kernel(const DecodeParams p) 
 
 namespace ahpc {
 
-// Waves per decode workgroup (each wave works alone; this only sets how many heads travel together).
-static int decode_waves() { return (int)tuning().decode_waves.load(); }
+// Smallest chunk any launch plan below picks for pages of P tokens (sizes the workspace's upper bound).
+static int64_t smallest_chunk(int64_t P) { return ((128 + P - 1) / P) * P; }
 
-static int64_t pick_chunk_tokens(int64_t B, int64_t H, int64_t max_len, int64_t P, int64_t requested) {
-    int64_t chunk = requested;
-    if (chunk <= 0) chunk = tuning().decode_chunk.load();
-    if (chunk <= 0) {
-        // enough workgroups to keep every CU busy several times over, while the fp32 partials stay
-        // below ~1% of the K/V bytes of a chunk
-        chunk = 256;
-        while (chunk > 128 && B * ((max_len + chunk - 1) / chunk) * ((H + 3) / 4) < 4096) chunk /= 2;
-    }
+static int64_t fit_chunk(int64_t chunk, int64_t P) {
     chunk = ((chunk + P - 1) / P) * P;
     if (chunk < P) chunk = P;
     if (chunk > 64 * P) chunk = 64 * P;  // the decode kernel keeps one page id per lane
     return chunk;
+}
+
+// Tokens per chunk and wavefronts per workgroup of one decode launch.  row_waves = wavefronts that cover the
+// pool heads of one token (each wave works alone; waves only sets how many heads travel together).
+struct DecodePlan { int64_t chunk; int waves; };
+
+static DecodePlan plan_decode(int64_t B, int64_t H_kv, int64_t group, int64_t row_waves, int64_t max_len, int64_t P,
+                              int64_t requested) {
+    DecodePlan plan{requested, (int)tuning().decode_waves.load()};
+    if (plan.waves < 0 || plan.waves > 8) plan.waves = 0;
+    if (plan.chunk <= 0) plan.chunk = tuning().decode_chunk.load();
+    if (plan.chunk > 0) {
+        plan.chunk = fit_chunk(plan.chunk, P);
+        if (!plan.waves) plan.waves = 2;
+        return plan;
+    }
+    if (group == 1) {
+        // One query head per pool head is pure streaming: the longest chunks that still leave about four
+        // wavefronts for every CU (timed on B=1..256, contexts 128..131072: chunks of 1024 tokens win wherever
+        // they leave >= 1024 wavefronts; shorter chunks pay in partials and in part-filled requests).
+        int64_t chunk = 1024;
+        while (chunk > 128 && B * ((max_len + chunk - 1) / chunk) * row_waves < 1024) chunk /= 2;
+        plan.chunk = fit_chunk(chunk, P);
+        if (!plan.waves) {
+            // Whole token rows per workgroup (8 wavefronts read 8 consecutive KiB and more) when such workgroups
+            // still fill the CUs and every sequence spans several of them; single wavefronts otherwise, which
+            // spread a few long sequences over more CUs.
+            const int64_t n_chunks = (max_len + plan.chunk - 1) / plan.chunk;
+            plan.waves = (row_waves >= 8 && n_chunks >= 2 && B * n_chunks >= 256) ? 8 : 1;
+        }
+        return plan;
+    }
+    // Several query heads per pool head: the arithmetic per byte is G times higher and more resident
+    // workgroups hide it better; enough workgroups to keep every CU busy several times over, while the fp32
+    // partials stay below ~1% of the K/V bytes of a chunk.
+    int64_t chunk = 256;
+    while (chunk > 128 && B * ((max_len + chunk - 1) / chunk) * ((H_kv * group + 3) / 4) < 4096) chunk /= 2;
+    plan.chunk = fit_chunk(chunk, P);
+    if (!plan.waves) plan.waves = 2;
+    return plan;
 }
 
 template <typename T, int PT, int G>
@@ -727,7 +759,10 @@ int ahpc_hip_kv_gather(void* k_out, void* v_out, int out_dtype, const void* k_po
 size_t ahpc_hip_paged_decode_workspace_bytes(int64_t B, int64_t H, int64_t d, int64_t max_len, int64_t P,
                                              int64_t chunk_tokens) {
     if (B <= 0 || H <= 0 || d <= 0 || max_len <= 0 || P <= 0) return 0;
-    const int64_t chunk = pick_chunk_tokens(B, H, max_len, P, chunk_tokens);
+    // Without the pool's head count and type the launch plan is not known here: an upper bound, the
+    // smallest chunk a plan picks (a requested or tuned chunk is taken as it is).
+    int64_t chunk = chunk_tokens > 0 ? chunk_tokens : tuning().decode_chunk.load();
+    chunk = fit_chunk(chunk > 0 ? chunk : smallest_chunk(P), P);
     const int64_t n_chunks = (max_len + chunk - 1) / chunk;
     if (n_chunks <= 1) return 0;
     return (size_t)(B * n_chunks * H * (d + 2)) * sizeof(float);
@@ -755,7 +790,11 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
         return AHPC_ERR_BAD_ALIGNMENT;
     if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
 
-    const int64_t chunk = pick_chunk_tokens(B, H, max_len, P, chunk_tokens);
+    const int lph = (int)(d * (pool_dtype == AHPC_F32 ? 4 : 2) / 16);  // lanes that hold one head of a token
+    const int hpw = 64 / lph;
+    const DecodePlan plan = plan_decode(B, H_kv, group, (H_kv + hpw - 1) / hpw, max_len, P, chunk_tokens);
+    const int64_t chunk = plan.chunk;
+    const int waves = plan.waves;
     const int64_t n_chunks = (max_len + chunk - 1) / chunk;
     const size_t need = n_chunks > 1 ? (size_t)(B * n_chunks * H * (d + 2)) * sizeof(float) : 0;
     if (need > 0 && (!workspace || workspace_bytes < need)) return AHPC_ERR_WORKSPACE_TOO_SMALL;
@@ -775,12 +814,6 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     p.scale_log2 = scale * kLog2e;
 
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int elem = pool_dtype == AHPC_F32 ? 4 : 2;
-    const int lph = (int)(d * elem / 16);
-    if (lph < 1 || lph > 64) return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
-    const int hpw = 64 / lph;
-    int waves = decode_waves();
-    if (waves < 1 || waves > 8) waves = 2;
     const int64_t heads_per_wg = (int64_t)hpw * waves;  // pool heads
     const int64_t head_groups = (H_kv + heads_per_wg - 1) / heads_per_wg;
     if (head_groups > 65535) return AHPC_ERR_BAD_SHAPE;
@@ -841,7 +874,7 @@ int ahpc_hip_paged_gather_indices(const int32_t* block_table, const int32_t* seq
     if ((d == 32 || d == 64 || d == 128 || d == 256) && B <= 65535 && H <= 65535) {
         // the decode kernel itself (16-bit pool, one query head per pool head), launched for pool head 0 only,
         // reports the rows it addresses
-        const int64_t chunk = pick_chunk_tokens(B, H, max_len, P, 0);
+        const int64_t chunk = plan_decode(B, H, 1, (H + 3) / 4, max_len, P, 0).chunk;
         const int64_t n_chunks = (max_len + chunk - 1) / chunk;
         if (n_chunks > 65535) return AHPC_ERR_BAD_SHAPE;
         DecodeParams p{};

@@ -268,6 +268,29 @@ def _full_size_decode(gpu, dtype, B, lo, hi, seed, chunk=0):
         assert np.abs(got[b] - want[0]).max() <= 2e-2, f"sequence {b} (len {lens[b]})"
 
 
+@pytest.mark.parametrize("chunk,waves", [(1024, 8), (1024, 1), (512, 4), (128, 2), (0, 0)])
+def test_decode_workgroup_shapes(gpu, chunk, waves):
+    """The launch shapes the plan chooses from (chunk length, wavefronts per workgroup), forced through the tuning
+    values, every sequence against the oracle."""
+    B, H, d, P = 6, 32, 128, 16
+    lens = [2500, 1, 1024, 1025, 300, 4000]
+    q, kp, vp, table, lens, _, _ = build_problem(B, H, d, P, lens, 61, O.F16)
+    scale = 1.0 / np.sqrt(d)
+    want = O.paged_decode(q, kp, vp, table, lens, None, B, H, d, P, scale)
+    kp, vp, table = poison_unused(kp, vp, table, lens, P, H, d)
+    from gpu_util import to_dev
+    before = gpu.get_tuning("decode_chunk"), gpu.get_tuning("decode_waves")
+    gpu.set_tuning("decode_chunk", chunk)
+    gpu.set_tuning("decode_waves", waves)
+    try:
+        got = gpu_decode(gpu, q, to_dev(kp, O.F16), to_dev(vp, O.F16), table, lens, None, B, H, d, P, O.F16, O.F16, scale)
+    finally:
+        gpu.set_tuning("decode_chunk", before[0])
+        gpu.set_tuning("decode_waves", before[1])
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= 2e-2
+
+
 def test_config3_decode_fp16_b64(gpu):
     # fp16, B=64, H=32, d=128, P=16, context lengths U[512, 4096], shuffled block table
     _full_size_decode(gpu, O.F16, 64, 512, 4096, 0xA77E0003)

@@ -179,6 +179,24 @@ def test_decode(emu, dtype, H, d, P):
         assert np.abs(got - want).max() <= TOL[dtype], f"chunk={chunk}"
 
 
+@pytest.mark.parametrize("waves", [1, 2, 4, 8])
+def test_decode_workgroup_shapes(emu, tuned, waves):
+    """Every workgroup width the launch plan can choose (1 to 8 wavefronts: from 4 heads of a token to whole
+    token rows) and its chunk lengths give the result of the oracle; 12 heads leave the last wavefronts of a
+    wide workgroup without a head."""
+    B, H, d, P = 3, 12, 128, 16
+    q, kp, vp, table, lens, _, _ = build_problem(B, H, d, P, [300, 17, 1100], 27, O.F16)
+    scale = 1.0 / np.sqrt(d)
+    want = O.paged_decode(q, kp, vp, table, lens, None, B, H, d, P, scale)
+    kp, vp, table = poison_unused(kp, vp, table, lens, P, H, d, wild_page=1 << 24)
+    tuned("decode_waves", waves)
+    for chunk in (1024, 256, 0):
+        tuned("decode_chunk", chunk)
+        got = decode(emu, q, kp, vp, table, lens, None, B, H, H, d, P, O.F16, O.F16, scale, 0)
+        assert np.isfinite(got).all()
+        assert np.abs(got - want).max() <= 2e-2, f"chunk={chunk}"
+
+
 @pytest.mark.parametrize("G", [2, 4, 8])
 def test_decode_grouped_heads(emu, G):
     B, H_kv, d, P = 3, 2, 128, 16
