@@ -105,6 +105,25 @@ template <> __device__ inline f32x16 mfma_32x32x16<bf16_t>(u32x4 a, u32x4 b, f32
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
 }
 
+// D(16x16) += A(16xK) * B(Kx16), K = 32 or 16.  Lane l supplies A[row l%16][k KPL*(l/16)..] and
+// B[k KPL*(l/16)..][col l%16] (KPL = 8 or 4 values per lane); it receives D[row 4*(l/16) + r][col l%16] in acc[r].
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+template <typename T> __device__ inline f32x4 mfma_16x16x32(u32x4 a, u32x4 b, f32x4 acc);
+template <> __device__ inline f32x4 mfma_16x16x32<f16_t>(u32x4 a, u32x4 b, f32x4 acc) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc, 0, 0, 0);
+}
+template <> __device__ inline f32x4 mfma_16x16x32<bf16_t>(u32x4 a, u32x4 b, f32x4 acc) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+}
+template <typename T> __device__ inline f32x4 mfma_16x16x16(u32x2 a, u32x2 b, f32x4 acc);
+template <> __device__ inline f32x4 mfma_16x16x16<f16_t>(u32x2 a, u32x2 b, f32x4 acc) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), acc, 0, 0, 0);
+}
+template <> __device__ inline f32x4 mfma_16x16x16<bf16_t>(u32x2 a, u32x2 b, f32x4 acc) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), acc, 0, 0, 0);
+}
+
 // ---- wave helpers ----------------------------------------------------------------------------
 // Value held by lane (l ^ 32).
 __device__ inline float swap_halves(float x) {

@@ -353,28 +353,40 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
         const float* const delta = p.delta + ((int64_t)b * p.H + h) * p.rows_padded;
 
         auto dma_both = [&](int i0, unsigned char* dst_q, unsigned char* dst_o) {
-            const int64_t rem = (int64_t)(L - i0 - 1) * sn * 2 + 2 * D;
+            // (a tile that starts at or behind the end of the sequence touches no memory and lands as zeros)
+            const int64_t rem = i0 < L ? (int64_t)(L - i0 - 1) * sn * 2 + 2 * D : 0;
             const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
             dma_tile<D>(gq + (int64_t)i0 * sn, nrec, dma_off, dst_q, wave_u);
             dma_tile<D>(gdo + (int64_t)i0 * sn, nrec, dma_off, dst_o, wave_u);
         };
 
-        auto compute_tile = [&](const unsigned char* tile_q, const unsigned char* tile_o, int i0) {
+        // The rows of statistics of a tile's two blocks of 32 queries (this lane's 16 rows of a block are 4 runs of 4
+        // consecutive rows; the arrays are padded to whole tiles).  They are requested BEFORE the next tile's
+        // direct-to-LDS loads: loads complete in order, so waiting for a load issued behind those would wait for the
+        // whole next tile as well.
+        auto load_stats = [&](f32x4 (&st)[2][2][4], int i0) {
+#pragma unroll
+            for (int ib = 0; ib < 2; ++ib)
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    st[ib][0][g4] = *reinterpret_cast<const f32x4*>(lse2 + i0 + 32 * ib + 8 * g4 + 4 * half);
+                    st[ib][1][g4] = *reinterpret_cast<const f32x4*>(delta + i0 + 32 * ib + 8 * g4 + 4 * half);
+                }
+        };
+
+        auto compute_tile = [&](const unsigned char* tile_q, const unsigned char* tile_o, int i0, const f32x4 (&st)[2][2][4]) {
 #pragma unroll
             for (int ib = 0; ib < 2; ++ib) {
                 const int iblock0 = i0 + 32 * ib;
                 if (iblock0 >= L) continue;                      // nothing but padding
                 if (CAUSAL && iblock0 + 31 < kw) continue;      // every query of the block precedes the keys
-                // the block's rows of statistics: this lane's 16 rows are 4 runs of 4 consecutive rows
                 f32x16 s, dp;
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4) {
-                    const f32x4 a = *reinterpret_cast<const f32x4*>(lse2 + iblock0 + 8 * g4 + 4 * half);
-                    const f32x4 d0 = *reinterpret_cast<const f32x4*>(delta + iblock0 + 8 * g4 + 4 * half);
 #pragma unroll
                     for (int x = 0; x < 4; ++x) {
-                        s[4 * g4 + x] = -a[x];
-                        dp[4 * g4 + x] = -d0[x];
+                        s[4 * g4 + x] = -st[ib][0][g4][x];
+                        dp[4 * g4 + x] = -st[ib][1][g4][x];
                     }
                 }
 #pragma unroll
@@ -417,13 +429,15 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
 
         auto step = [&](unsigned char* cur_q, unsigned char* cur_o, unsigned char* nxt_q, unsigned char* nxt_o, int t) {
             const int i0 = t * kFlashKeys;
-            const bool more = t + 1 < n_tiles;
-            if (more) dma_both(i0 + kFlashKeys, nxt_q, nxt_o);
-            compute_tile(cur_q, cur_o, i0);
-            if (more) {
-                __builtin_amdgcn_s_waitcnt(0);
-                __syncthreads();
-            }
+            f32x4 st[2][2][4];
+            load_stats(st, i0);
+            __builtin_amdgcn_sched_barrier(0);  // the order of the requests is what the comment above is about
+            // Requested even behind the last tile (an empty request): were it conditional, the compiler would
+            // count the loads in flight for the path without it and wait for the statistics as if nothing followed.
+            dma_both(i0 + kFlashKeys, nxt_q, nxt_o);
+            compute_tile(cur_q, cur_o, i0, st);
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
         };
 
         dma_both(t_begin * kFlashKeys, lds_q0, lds_o0);

@@ -516,6 +516,7 @@ __global__ __launch_bounds__(256) void paged_merge_kernel(const DecodeParams p) 
 }  // namespace ahpc
 
 #include "paged_decode_mfma.hpp"  // uses DecodeParams and the q/o vector helpers above
+#include "paged_decode_group.hpp"
 
 namespace ahpc {
 
@@ -534,13 +535,21 @@ static int64_t fit_chunk(int64_t chunk, int64_t P) {
 struct DecodePlan { int64_t chunk; int waves; };
 
 static DecodePlan plan_decode(int64_t B, int64_t H_kv, int64_t group, int64_t row_waves, int64_t max_len, int64_t P,
-                              int64_t requested) {
+                              int64_t requested, bool matrix_kernel = false) {
     DecodePlan plan{requested, (int)tuning().decode_waves.load()};
     if (plan.waves < 0 || plan.waves > 8) plan.waves = 0;
     if (plan.chunk <= 0) plan.chunk = tuning().decode_chunk.load();
     if (plan.chunk > 0) {
         plan.chunk = fit_chunk(plan.chunk, P);
         if (!plan.waves) plan.waves = 2;
+        return plan;
+    }
+    if (matrix_kernel) {
+        // one wavefront per pool head and chunk, bound by the stream like the case below
+        int64_t chunk = 1024;
+        while (chunk > 128 && B * ((max_len + chunk - 1) / chunk) * H_kv < 1024) chunk /= 2;
+        plan.chunk = fit_chunk(chunk, P);
+        if (!plan.waves) plan.waves = 2;  // (unused by those kernels)
         return plan;
     }
     if (group == 1) {
@@ -600,6 +609,28 @@ static int launch_decode_mfma(const DecodeParams& p, hipStream_t st) {
     else if (p.d == 64) hipLaunchKernelGGL((paged_decode_mfma_kernel<T, 64>), grid, block, 0, st, p);
     else return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
     return static_cast<int>(hipGetLastError());
+}
+
+// Matrix-core kernel for groups of up to 16 query heads: a wavefront per (pool head, chunk, batch entry), up to 8
+// pool heads side by side in a workgroup.
+template <typename T, int D>
+static int launch_decode_group_d(const DecodeParams& p, hipStream_t st) {
+    const int w = p.H_kv >= 8 ? 8 : p.H_kv >= 4 ? 4 : p.H_kv >= 2 ? 2 : 1;
+    const dim3 grid((unsigned)((p.H_kv + w - 1) / w), (unsigned)p.n_chunks, (unsigned)p.B), block(64 * w);
+    switch (w) {
+        case 8: hipLaunchKernelGGL((paged_decode_group_kernel<T, D, 8>), grid, block, 0, st, p); break;
+        case 4: hipLaunchKernelGGL((paged_decode_group_kernel<T, D, 4>), grid, block, 0, st, p); break;
+        case 2: hipLaunchKernelGGL((paged_decode_group_kernel<T, D, 2>), grid, block, 0, st, p); break;
+        default: hipLaunchKernelGGL((paged_decode_group_kernel<T, D, 1>), grid, block, 0, st, p); break;
+    }
+    return static_cast<int>(hipGetLastError());
+}
+
+template <typename T>
+static int launch_decode_group(const DecodeParams& p, hipStream_t st) {
+    if (p.d == 128) return launch_decode_group_d<T, 128>(p, st);
+    if (p.d == 64) return launch_decode_group_d<T, 64>(p, st);
+    return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
 }
 
 template <typename T>
@@ -774,9 +805,10 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
                               float scale, int64_t chunk_tokens, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !o || !k_pool || !v_pool || !block_table || !seq_lens) return AHPC_ERR_NULL_POINTER;
     if (H_kv <= 0 || H <= 0 || H % H_kv) return AHPC_ERR_BAD_SHAPE;
-    // Groups of 1, 2, 4, 8 query heads: lane-per-element kernel, any pool type.  Groups of 16 and 32 exist on
-    // the matrix-core kernel only (16-bit pool, d 64 or 128, pages of 16 tokens); the tuning value
-    // decode_matrix_min_group can send groups of 4 and 8 there as well (slightly slower when timed).
+    // Groups of 1 and 2 query heads: lane-per-element kernel, any pool type.  Groups of 4, 8 and 16 (and 2, when the
+    // tuning value decode_matrix_min_group says so): the page-by-page matrix-core kernel; 32: the 32-column one.  Both
+    // need a 16-bit pool, d 64 or 128 and pages of 16 tokens; groups of 4 and 8 on other pools stay on the
+    // lane-per-element kernel, 16 and 32 are refused there.
     const int64_t group = H / H_kv;
     const bool mfma_shape = (pool_dtype == AHPC_F16 || pool_dtype == AHPC_BF16) && (d == 64 || d == 128) && P == 16 && H_kv <= 65535;
     if (group != 1 && group != 2 && group != 4 && group != 8 && !((group == 16 || group == 32) && mfma_shape))
@@ -792,7 +824,10 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
 
     const int lph = (int)(d * (pool_dtype == AHPC_F32 ? 4 : 2) / 16);  // lanes that hold one head of a token
     const int hpw = 64 / lph;
-    const DecodePlan plan = plan_decode(B, H_kv, group, (H_kv + hpw - 1) / hpw, max_len, P, chunk_tokens);
+    // Groups of 4 and more query heads go to the matrix cores (from the tuning value decode_matrix_min_group on).
+    const int64_t matrix_from = tuning().decode_matrix_min_group.load();
+    const bool use_mfma = mfma_shape && (group >= 16 || (group >= 2 && group >= matrix_from));
+    const DecodePlan plan = plan_decode(B, H_kv, group, (H_kv + hpw - 1) / hpw, max_len, P, chunk_tokens, use_mfma);
     const int64_t chunk = plan.chunk;
     const int waves = plan.waves;
     const int64_t n_chunks = (max_len + chunk - 1) / chunk;
@@ -823,9 +858,9 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
 
     dim3 grid((unsigned)head_groups, (unsigned)n_chunks, (unsigned)B), block(64 * waves);
     int rc;
-    const int64_t matrix_from = tuning().decode_matrix_min_group.load();
-    const bool use_mfma = mfma_shape && (group >= 16 || (group >= 4 && group >= matrix_from));
-    if (use_mfma) {
+    if (use_mfma && group <= 16) {
+        rc = pool_dtype == AHPC_F16 ? launch_decode_group<f16_t>(p, st) : launch_decode_group<bf16_t>(p, st);
+    } else if (use_mfma) {
         rc = pool_dtype == AHPC_F16 ? launch_decode_mfma<f16_t>(p, st) : launch_decode_mfma<bf16_t>(p, st);
     } else
     switch (pool_dtype) {

@@ -32,7 +32,7 @@ constexpr int kWaveSize = 64;
 constexpr int kPayload = 64;          // bytes a lane can publish per cross-lane operation
 constexpr size_t kStackBytes = 512 * 1024;
 
-enum Kind : int { K_NONE = 0, K_MFMA, K_TR, K_SWAP, K_BALLOT, K_RFL, K_RL, K_DPP, K_SHFL, K_LDS128 };
+enum Kind : int { K_NONE = 0, K_MFMA, K_TR, K_SWAP, K_BALLOT, K_RFL, K_RL, K_DPP, K_SHFL, K_LDS128, K_WAIT };
 
 struct PendingDma {
     unsigned char* dst;
@@ -194,6 +194,7 @@ void flush_dma(Fiber* f, size_t leave = 0) {
     size_t n = f->dma.size() > leave ? f->dma.size() - leave : 0;
     for (size_t i = 0; i < n; ++i) {
         const PendingDma& d = f->dma[i];
+        if (!d.dst) continue;  // a load to registers: only counted
         if (d.src) std::memcpy(d.dst, d.src, (size_t)d.bytes);
         else std::memset(d.dst, 0, (size_t)d.bytes);
         note_dma_landed(f, d.dst, d.bytes);
@@ -374,6 +375,37 @@ template <typename V> f32x16 mfma_impl(V a, V b, f32x16 c) {
     return d;
 }
 
+// 16x16 matrix instructions: lane l supplies A[row l%16][k KPL*(l/16) ..] and B[k KPL*(l/16) ..][col l%16] and
+// receives D[row 4*(l/16) + r][col l%16] in acc[r].
+template <int KPL, typename V, typename F> f32x4 mfma16_impl(V a, V b, f32x4 c, F to_float) {
+    struct Ops {
+        V a, b;
+    } mine{a, b};
+    const View v = exchange(K_MFMA, &mine, sizeof mine);
+    const Fiber* f = g_cur;
+    const int col = f->lane & 15, rg = f->lane >> 4;
+    f32x4 d = c;
+    for (int r = 0; r < 4; ++r) {
+        const int row = 4 * rg + r;
+        double acc = 0.0;
+        for (int kg = 0; kg < 4; ++kg) {
+            Ops oa, ob;
+            std::memcpy(&oa, v.of(row + 16 * kg), sizeof oa);
+            std::memcpy(&ob, v.of(col + 16 * kg), sizeof ob);
+            for (int e = 0; e < KPL; ++e) acc += (double)to_float(oa.a[e]) * (double)to_float(ob.b[e]);
+        }
+        d[r] = (float)((double)c[r] + acc);
+    }
+    return d;
+}
+
+float bf16_bits_to_f32(short bits) {
+    const uint32_t w = (uint32_t)(uint16_t)bits << 16;
+    float x;
+    std::memcpy(&x, &w, 4);
+    return x;
+}
+
 }  // namespace
 
 // ---- what the shim header declares --------------------------------------------------------------
@@ -400,6 +432,10 @@ void syncthreads() {
 
 f32x16 mfma_32x32x16_f16(f16x8 a, f16x8 b, f32x16 c) { return mfma_impl(a, b, c); }
 f32x16 mfma_32x32x16_bf16(bf16x8 a, bf16x8 b, f32x16 c) { return mfma_impl(a, b, c); }
+f32x4 mfma_16x16x32_f16(f16x8 a, f16x8 b, f32x4 c) { return mfma16_impl<8>(a, b, c, [](_Float16 x) { return (float)x; }); }
+f32x4 mfma_16x16x32_bf16(bf16x8 a, bf16x8 b, f32x4 c) { return mfma16_impl<8>(a, b, c, [](__bf16 x) { return (float)x; }); }
+f32x4 mfma_16x16x16_f16(f16x4 a, f16x4 b, f32x4 c) { return mfma16_impl<4>(a, b, c, [](_Float16 x) { return (float)x; }); }
+f32x4 mfma_16x16x16_bf16(s16x4 a, s16x4 b, f32x4 c) { return mfma16_impl<4>(a, b, c, bf16_bits_to_f32); }
 
 // ds_read_b64_tr_b16: the 16 lanes of a row each address four 16-bit elements; lane j of the row
 // receives element (j % 4) of the lanes 4*r + j/4, r = 0..3 (a 16x4 block handed out transposed).
@@ -542,11 +578,30 @@ void buffer_load_lds(BufferRsrc r, void* lds_base, int size, int voffset, int so
     }
 }
 
+// buffer_load_dwordx4 to registers: the data is taken at once (the compiler waits for registers itself), but
+// the load takes its place in the queue of outstanding loads, so that s_waitcnt vmcnt(n) counts as on hardware.
+u32x4 buffer_load_b128(BufferRsrc r, int voffset, int soffset, int aux) {
+    (void)aux;
+    Fiber* f = g_cur;
+    if (voffset < 0) fail("buffer_load: negative lane offset");
+    const uint64_t off = (uint64_t)(uint32_t)voffset + (uint64_t)(uint32_t)soffset;
+    u32x4 out = {0, 0, 0, 0};
+    if (off + 16 <= (uint64_t)r.num_records) std::memcpy(&out, r.base + off, 16);
+    f->dma.push_back(PendingDma{nullptr, nullptr, 0});
+    if (!g_dma_late) flush_dma(f);
+    return out;
+}
+
 // s_waitcnt with the gfx9 encoding: vmcnt in bits 3:0 and 15:14; the other counters are not modelled
 // (LDS and scalar accesses are synchronous here).
+// The wait belongs to the wavefront: no lane goes on before every lane's loads have landed (a lane may read
+// next what another lane's direct-to-LDS load brought in).
 void waitcnt(int imm) {
     const int vmcnt = (imm & 0xF) | (((imm >> 14) & 3) << 4);
-    if (g_cur) flush_dma(g_cur, (size_t)vmcnt);
+    if (!g_cur) return;
+    flush_dma(g_cur, (size_t)vmcnt);
+    unsigned char nothing[8] = {0};
+    exchange(K_WAIT, nothing, sizeof nothing);
 }
 
 void launch(dim3 grid, dim3 block, const std::function<void()>& body) {

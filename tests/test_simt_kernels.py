@@ -500,7 +500,33 @@ def test_decode_grouped_heads_matrix_core_kernel(emu, G, dtype, d, tuned):
         assert np.all(got[3] == 0.0)
         assert np.abs(got - want).max() <= 2e-2, (chunk, qo)
     reads, read_conflicts, tr, tr_conflicts = S.lds_stats(reset=True)
-    assert reads > 0 and tr > 0 and read_conflicts == 0 and tr_conflicts == 0
+    # groups of up to 16 heads: the page-by-page kernel, whose K rows never pass through LDS
+    assert (reads == 0 if G <= 16 else reads > 0) and tr > 0 and read_conflicts == 0 and tr_conflicts == 0
+
+
+@pytest.mark.parametrize("H_kv,G,d,dtype", [(8, 4, 128, O.F16), (5, 2, 64, O.BF16), (1, 16, 128, O.BF16), (3, 8, 64, O.F16)])
+def test_decode_page_ring_of_the_group_kernel(emu, tuned, H_kv, G, d, dtype):
+    """The page-by-page matrix-core kernel with 8, 4, 2 and 1 pool heads side by side in a workgroup (5 heads leave
+    wavefronts of the second workgroup without a head), chunks long enough for several trips round its ring of
+    page slots and every remainder of pages (0 to 3) behind the last full trip, direct loads landing late."""
+    tuned("decode_matrix_min_group", 2)
+    B, P = 5, 16
+    lens_in = [16 * 4 * 3, 16 * 9 + 1, 16 * 10 + 15, 16 * 7, 3]   # 12, 10, 11, 7 pages and a single short page
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, lens_in, 29, dtype)
+    H = G * H_kv
+    q = O.round_to(O.fill_normal((B, H, d), 29, 1), dtype)
+    scale = 1.0 / np.sqrt(d)
+    rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
+    want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    kp, vp, table = poison_unused(kp, vp, table, lens, P, H_kv, d, wild_page=1 << 24)
+    for chunk, dma_late in ((1024, True), (96, True), (0, False)):
+        S.configure(dma_late, seed=H_kv + chunk)
+        try:
+            got = decode(emu, q, kp, vp, table, lens, None, B, H, H_kv, d, P, dtype, dtype, scale, chunk)
+        finally:
+            S.configure(False, 1)
+        assert np.isfinite(got).all()
+        assert np.abs(got - want).max() <= 2e-2, chunk
 
 
 def test_wide_groups_need_the_matrix_core_shape(emu):

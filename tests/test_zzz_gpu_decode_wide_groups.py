@@ -55,6 +55,30 @@ def test_matrix_core_decode_equals_repeated_heads(gpu, G, dtype, d, matrix_kerne
         assert np.abs(got - want).max() <= 2e-2, (chunk, qo)
 
 
+@pytest.mark.parametrize("H_kv,G,d,dtype", [(8, 4, 128, O.F16), (5, 2, 64, O.BF16), (1, 16, 128, O.BF16), (3, 8, 64, O.F16)])
+def test_page_ring_of_the_group_kernel(gpu, H_kv, G, d, dtype):
+    """8, 4, 2 and 1 pool heads side by side in a workgroup of the page-by-page kernel, chunks of several trips round its
+    ring of page slots with every remainder of pages behind the last full trip."""
+    B, P = 5, 16
+    lens_in = [16 * 4 * 3, 16 * 9 + 1, 16 * 10 + 15, 16 * 7, 3]
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, lens_in, 29, dtype)
+    H = G * H_kv
+    q = O.round_to(O.fill_normal((B, H, d), 29, 1), dtype)
+    scale = 1.0 / np.sqrt(d)
+    rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
+    want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    kp, vp, table = poison_unused(kp, vp, table, lens, P, H_kv, d)
+    before = gpu.get_tuning("decode_matrix_min_group")
+    gpu.set_tuning("decode_matrix_min_group", 2)
+    try:
+        for chunk in (1024, 96, 0):
+            got = run(gpu, q, kp, vp, table, lens, B, H, H_kv, d, P, dtype, dtype, scale, chunk)
+            assert np.isfinite(got).all()
+            assert np.abs(got - want).max() <= 2e-2, chunk
+    finally:
+        gpu.set_tuning("decode_matrix_min_group", before)
+
+
 def test_both_kernels_agree_for_groups_of_four(gpu):
     B, H_kv, d, P, G = 3, 8, 128, 16, 4
     H = G * H_kv
