@@ -160,6 +160,22 @@ static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream
     return static_cast<int>(hipGetLastError());
 }
 
+template <typename T, int D>
+static int launch_mfma_masked(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
+    if (int rc = flash_plan_launch(p, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load(), false)) return rc;
+    dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
+    if (causal) hipLaunchKernelGGL((flash_fwd_mfma_masked_kernel<T, D, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((flash_fwd_mfma_masked_kernel<T, D, false>), grid, block, 0, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
+template <typename T>
+static int dispatch_mfma_masked(const FlashParams& p, int64_t B, int d, bool causal, hipStream_t stream) {
+    if (d == 128) return launch_mfma_masked<T, 128>(p, B, causal, stream);
+    if (d == 64) return launch_mfma_masked<T, 64>(p, B, causal, stream);
+    return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+}
+
 template <typename T, bool VARLEN>
 static int dispatch_mfma(const FlashParams& p, int64_t B, int d, bool causal, hipStream_t stream) {
     if (d == 128) return launch_mfma<T, 128, VARLEN>(p, B, causal, stream);
@@ -210,13 +226,19 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
     if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int32_t group = (int32_t)(H / H_kv);
-    if (!mask && mfma_eligible(dtype, d, q, k, v, o, sq, skv)) {
+    // a mask row is read 16 bytes at a time on the matrix-core kernel: rows of a multiple of 4 floats, aligned base
+    const bool mask_ok = !mask || (N % 4 == 0 && aligned16(mask));
+    if (mask_ok && mfma_eligible(dtype, d, q, k, v, o, sq, skv)) {
         FlashParams p{};
         p.q = q; p.k = k; p.v = v; p.o = o;
+        p.mask = mask;
         p.stride_b = sq.b; p.stride_n = sq.n; p.stride_h = sq.h;
         p.kv_stride_b = skv.b; p.kv_stride_n = skv.n; p.kv_stride_h = skv.h;
         p.N = (int32_t)N; p.H = (int32_t)H; p.kv_group = group;
         p.scale_log2 = scale * kLog2e;
+        if (mask)
+            return dtype == AHPC_F16 ? dispatch_mfma_masked<f16_t>(p, B, (int)d, causal != 0, st)
+                                     : dispatch_mfma_masked<bf16_t>(p, B, (int)d, causal != 0, st);
         return dtype == AHPC_F16 ? dispatch_mfma<f16_t, false>(p, B, (int)d, causal != 0, st)
                                  : dispatch_mfma<bf16_t, false>(p, B, (int)d, causal != 0, st);
     }

@@ -51,6 +51,7 @@ struct FlashParams {
     const void* v;
     void* o;
     const int32_t* cu_seqlens;  // ragged batches only
+    const float* mask;          // masked kernel only: fp32 [B,N,N], shared by all heads; 0.0f removes the key for the query
     int64_t stride_b, stride_n, stride_h;           // Q and O
     int64_t kv_stride_b, kv_stride_n, kv_stride_h;  // K and V
     int32_t N;                  // sequence length (dense) / longest sequence (ragged)
@@ -199,8 +200,14 @@ struct FlashStatsOut {
     int64_t rows_padded;
 };
 
-template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS>
+// MASKED: a dense fp32 mask [B,N,N] removes keys per query (0.0f = removed; FlashAttention::apply_attention_mask,
+// src/algorithms/flash_attention.cpp:596-607).  A lane's 32 scores of a tile are 8 runs of 4 consecutive keys of
+// its query: 8 16-byte loads of the mask row (N is a multiple of 4 then, the host checks).  Any query may then see
+// its first key in any tile, or none at all (zeros come out), so the reference maximum is set per query when its
+// first key shows up.
+template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS, bool MASKED = false>
 __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const FlashStatsOut& st) {
+    static_assert(!(MASKED && (VARLEN || STATS)), "the mask belongs to dense forward launches");
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;  // k-steps of the first product
     constexpr int MB = D / 32;  // 32-row blocks of O^T
@@ -271,7 +278,8 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
     // sequence's last row bound the descriptor, so the rows of a ragged last tile that do not exist
     // read as zeros (their scores are masked; zero V rows keep 0 * x finite).
     auto dma_both = [&](int k0, unsigned char* dst_k, unsigned char* dst_v) {
-        const int64_t rem = (int64_t)(L - k0 - 1) * skv * 2 + 2 * D;
+        // (a tile that starts at or behind the end of the sequence touches no memory and lands as zeros)
+        const int64_t rem = k0 < L ? (int64_t)(L - k0 - 1) * skv * 2 + 2 * D : 0;
         const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
         dma_tile<D>(gk + (int64_t)k0 * skv, nrec, dma_off_k, dst_k, wave_u);
         dma_tile<D>(gv + (int64_t)k0 * skv, nrec, dma_off_v, dst_v, wave_u);
@@ -337,9 +345,23 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
         for (int r = 0; r < 16; ++r) neg_m[r] = 0.0f;
         float l_run = 0.0f;
         bool first = true;
+        bool seen = false;  // masked launches: this lane's query has met a key it may attend to
         constexpr float kRaise = 8.0f;  // raise the reference maximum only when exceeded by 2^8
+        const float* const mrow = MASKED ? p.mask + ((int64_t)b * p.N + (qrow < L ? qrow : L - 1)) * p.N : nullptr;
 
-        auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int k0) {
+        // The mask values of this lane's 32 scores of the tile at k0.  A run that starts behind the row's end reads
+        // the row's last four values instead: its keys do not exist and are removed by the end-of-sequence test.
+        auto load_mask = [&](f32x4 (&mk)[2][4], int k0) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const int key = k0 + 32 * kb + 8 * g4 + 4 * half;
+                    mk[kb][g4] = *reinterpret_cast<const f32x4*>(mrow + (key < p.N - 4 ? key : p.N - 4));
+                }
+        };
+
+        auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int k0, const f32x4 (&mk)[2][4]) {
             // ---- S^T = c*K Q^T - m  (log2 units).  The two 32-key blocks alternate, kAhead operand
             //      pairs are requested before the first product and one more after every two products.
             f32x16 s[2];
@@ -391,15 +413,33 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                         s[kb][r] = off <= lim ? s[kb][r] : -INFINITY;
                     }
             }
+            if constexpr (MASKED) {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) s[kb][r] = mk[kb][r >> 2][r & 3] == 0.0f ? -INFINITY : s[kb][r];
+            }
             // ---- reference maximum: exact on the first tile, afterwards raised only when a score tops
             //      it by more than kRaise (rare, and the only time the accumulators are rescaled) ------
             float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
             for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
-            if (first || __builtin_amdgcn_ballot_w64(mx > kRaise) != 0) {
+            bool adjust;
+            if constexpr (MASKED) adjust = __builtin_amdgcn_ballot_w64(seen ? mx > kRaise : mx > -INFINITY) != 0;
+            else adjust = first || __builtin_amdgcn_ballot_w64(mx > kRaise) != 0;
+            if (adjust) {
                 mx = halves_max(mx);                       // both lanes of a query agree
-                const float delta = first ? mx : fmaxf(mx, 0.0f);
-                const float alpha = fast_exp2(-delta);
+                float delta, alpha;
+                if constexpr (MASKED) {
+                    // a query without a visible key so far has accumulated nothing: its maximum is set exactly,
+                    // nothing is rescaled; one that still sees none stays as it is
+                    delta = seen ? fmaxf(mx, 0.0f) : (mx > -INFINITY ? mx : 0.0f);
+                    alpha = seen ? fast_exp2(-delta) : 1.0f;
+                    seen = seen || mx > -INFINITY;
+                } else {
+                    delta = first ? mx : fmaxf(mx, 0.0f);
+                    alpha = fast_exp2(-delta);
+                }
                 l_run *= alpha;
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
@@ -455,10 +495,20 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
         auto step = [&](unsigned char* cur_k, unsigned char* cur_v, unsigned char* nxt_k, unsigned char* nxt_v, int t) {
             const int k0 = t * kFlashKeys;
             const bool more = t + 1 < n_tiles;
-            if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
+            f32x4 mk[2][4];
+            if constexpr (MASKED) {
+                // The mask is requested BEFORE the next tile (loads complete in order: waiting for a load issued
+                // behind the tile's would wait for the tile), and the tile is requested even behind the last one
+                // (an empty request), so that the compiler counts the same loads in flight on every path.
+                load_mask(mk, k0);
+                __builtin_amdgcn_sched_barrier(0);
+                dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
+            } else {
+                if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
+            }
             // a wavefront whose queries all precede this tile has nothing to add
-            if (!(CAUSAL && k0 > qw + 31)) compute_tile(cur_k, cur_v, k0);
-            if (more) {
+            if (!(CAUSAL && k0 > qw + 31)) compute_tile(cur_k, cur_v, k0, mk);
+            if (MASKED || more) {
                 __builtin_amdgcn_s_waitcnt(0);  // this wave's part of the next tile has landed
                 __syncthreads();                // everyone's has, and everyone is done with the current one
             }
@@ -539,6 +589,12 @@ inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal, int rows_pe
 template <typename T, int D, bool CAUSAL, bool VARLEN>
 __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const FlashParams p) {
     flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, false>(p, FlashStatsOut{});
+}
+
+// Dense launches with a mask [B,N,N].
+template <typename T, int D, bool CAUSAL>
+__global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_masked_kernel(const FlashParams p) {
+    flash_fwd_mfma_body<T, D, CAUSAL, false, false, true>(p, FlashStatsOut{});
 }
 
 // The forward pass with its output kept in registers: writes the softmax statistics the backward needs.

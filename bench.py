@@ -353,6 +353,14 @@ def bench_extras(hip, stream, steps, warmup):
                               gv.data_ptr(), hip.BF16, B, N, H, H, d, st, st, sc, True, wsf.data_ptr(), wsb, stream),
         flops=2.5 * 2.0 * B * H * N * N * d)
 
+    # the headline shape, non-causal, with a dense random mask [B,N,N] (half the keys removed; flops counted as unmasked)
+    dmask = (torch.rand((B, N, N), generator=g, device="cuda") > 0.5).float()
+    run("flash_fwd bf16 non-causal B=4 N=4096 H=32 d=128 with a dense fp32 mask [B,N,N]",
+        lambda: hip.flash_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), hip.BF16, B, N, H, d, st, sc, False, stream,
+                              dmask.data_ptr()),
+        flops=4.0 * B * H * N * N * d)
+    del dmask
+
     # ragged fp16 causal batch: 16 sequences, lengths U[128,8192], H=32, d=64 (sigma 0.5)
     from oracle import oracle as O
     lens = O.fill_lengths(16, 0xA77E0005, 4, 128, 8192)

@@ -122,8 +122,7 @@ int ahpc_hip_flash_fwd(const void* q, const void* k, const void* v, void* o, int
  * AttentionParams::key_value_heads announces (src/api/attention_interface.hpp:61; 0 = H) and the
  * reference never implements (the field is read nowhere; README.md:367-368 lists it as planned).
  * Q and O use (stride_b, stride_n, stride_h), K and V their own strides; with H_kv == H and equal
- * strides this is ahpc_hip_flash_fwd.  mask: NULL, or fp32 [B,N,N] as in the masked entry point
- * (then the fp32-FMA kernel runs). */
+ * strides this is ahpc_hip_flash_fwd.  mask: NULL, or fp32 [B,N,N] as in the masked entry point. */
 int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o, int dtype,
                            int64_t B, int64_t N, int64_t H, int64_t H_kv, int64_t d,
                            int64_t stride_b, int64_t stride_n, int64_t stride_h,
@@ -132,7 +131,10 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
 
 /* Same with a dense fp32 mask [B,N,N] shared by all heads, 0.0f removes the key
  * (FlashAttention::apply_attention_mask, src/algorithms/flash_attention.cpp:596-607;
- * indexing :432-435).  mask may be NULL.  Always runs on the fp32-FMA kernel. */
+ * indexing :432-435).  A query whose keys are all removed gets a zero output row.  fp16/bf16 with d in {64, 128},
+ * N a multiple of 4 and a 16-byte aligned mask run on the matrix-core kernel (the mask row is read 16 bytes at a
+ * time), everything else on the fp32-FMA kernel.  mask may be NULL: then the fp32-FMA kernel runs whatever the
+ * type (the way to ask for it). */
 int ahpc_hip_flash_fwd_masked(const void* q, const void* k, const void* v, void* o, int dtype,
                               int64_t B, int64_t N, int64_t H, int64_t d,
                               int64_t stride_b, int64_t stride_n, int64_t stride_h,

@@ -93,6 +93,67 @@ def test_dense_mask_fp32(gpu):
     assert np.all(got[1, 3] == 0.0)
 
 
+@pytest.mark.parametrize("dtype,d", [(O.F16, 128), (O.BF16, 64), (O.BF16, 128)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("N", [4, 64, 132, 520, 1028, 517])
+def test_dense_mask_16bit(gpu, dtype, d, causal, N):
+    """16-bit inputs with a mask [B,N,N]: the matrix-core kernel when N is a multiple of 4 (517: the fp32-FMA kernel).
+    Rows that see nothing (zeros), a single key, or nothing before the last key tile."""
+    B, H = 2, 3
+    q, k, v = make_qkv((B, N, H, d), 6, dtype)
+    mask = (O.fill_uniform((B, N, N), 6, 6) > 0.3).astype(np.float32)
+    mask[0, N // 2, :] = 0.0
+    mask[1, N - 1, :] = 0.0
+    mask[1, N - 1, N - 1] = 1.0
+    mask[1, 0, :] = 0.0
+    mask[1, 0, 0] = 1.0
+    if N > 70:
+        mask[0, N - 2, :N - 3] = 0.0
+    scale = 1.0 / np.sqrt(d)
+    got = run_dense(gpu, q, k, v, dtype, B, N, H, d, scale, causal, mask=mask)
+    want = O.attention(q, k, v, B, N, H, d, scale, causal, mask=mask)
+    assert np.isfinite(got).all()
+    assert np.all(got[0, N // 2] == 0.0)
+    assert np.abs(got - want).max() <= 2e-2
+
+
+def test_dense_mask_full_size_properties(gpu):
+    """B=2 N=4096 H=8 d=128 bf16 with a mask: (1) an all-ones mask reproduces the unmasked launch bit for bit;
+    (2) a lower-triangular mask reproduces the causal launch within rounding (the same keys, the reference maximum set
+    by another rule); (3) sampled rows of a random mask against the oracle."""
+    import torch
+    from gpu_util import to_dev, to_host, stream_ptr
+    B, N, H, d = 2, 4096, 8, 128
+    g = torch.Generator(device="cuda").manual_seed(606)
+    q, k, v = (torch.randn((B, N, H, d), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16) for _ in range(3))
+    scale = 1.0 / np.sqrt(d)
+    st = (N * H * d, H * d, d)
+
+    def launch(causal, mask):
+        o = torch.full_like(q, float("nan"))
+        gpu.flash_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), O.BF16, B, N, H, d, st, scale, causal, stream_ptr(),
+                      None if mask is None else mask.data_ptr())
+        torch.cuda.synchronize()
+        return o
+
+    plain, causal = launch(False, None), launch(True, None)
+    ones = torch.ones((B, N, N), device="cuda")
+    assert torch.equal(launch(False, ones), plain)
+    tril = torch.tril(torch.ones((N, N), device="cuda")).expand(B, N, N).contiguous()
+    assert (launch(False, tril).float() - causal.float()).abs().max().item() <= 2e-2
+    rnd = (torch.rand((B, N, N), generator=g, device="cuda") > 0.5).float()
+    got = launch(False, rnd)
+    assert torch.isfinite(got.float()).all()
+    rows = [(0, 0, 0), (1, 7, 4095), (0, 3, 2048), (1, 5, 63)]
+    qh, kh, vh, mh = (x.float().cpu().numpy() for x in (q, k, v, rnd))
+    for b, h, n in rows:
+        s = (kh[b, :, h] @ qh[b, n, h]) * scale
+        s[mh[b, n] == 0.0] = -np.inf
+        w = np.exp(s - s.max())
+        want = (w[:, None] * vh[b, :, h]).sum(0) / w.sum()
+        assert np.abs(got[b, n, h].float().cpu().numpy() - want).max() <= 2e-2, (b, h, n)
+
+
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16])
 @pytest.mark.parametrize("d", [64, 128])
 @pytest.mark.parametrize("causal", [False, True])
