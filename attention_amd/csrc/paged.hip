@@ -805,9 +805,9 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
                               float scale, int64_t chunk_tokens, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !o || !k_pool || !v_pool || !block_table || !seq_lens) return AHPC_ERR_NULL_POINTER;
     if (H_kv <= 0 || H <= 0 || H % H_kv) return AHPC_ERR_BAD_SHAPE;
-    // Groups of 1 and 2 query heads: lane-per-element kernel, any pool type.  Groups of 4, 8 and 16 (and 2, when the
-    // tuning value decode_matrix_min_group says so): the page-by-page matrix-core kernel; 32: the 32-column one.  Both
-    // need a 16-bit pool, d 64 or 128 and pages of 16 tokens; groups of 4 and 8 on other pools stay on the
+    // One query head per pool head: lane-per-element kernel, any pool type.  Groups of 2 to 16 (from the tuning
+    // value decode_matrix_min_group on): the page-by-page matrix-core kernel; 32: the 32-column one.  Both need a
+    // 16-bit pool, d 64 or 128 and pages of 16 tokens; groups of 2, 4 and 8 on other pools stay on the
     // lane-per-element kernel, 16 and 32 are refused there.
     const int64_t group = H / H_kv;
     const bool mfma_shape = (pool_dtype == AHPC_F16 || pool_dtype == AHPC_BF16) && (d == 64 || d == 128) && P == 16 && H_kv <= 65535;
@@ -824,9 +824,8 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
 
     const int lph = (int)(d * (pool_dtype == AHPC_F32 ? 4 : 2) / 16);  // lanes that hold one head of a token
     const int hpw = 64 / lph;
-    // Groups of 4 and more query heads go to the matrix cores (from the tuning value decode_matrix_min_group on).
     const int64_t matrix_from = tuning().decode_matrix_min_group.load();
-    const bool use_mfma = mfma_shape && (group >= 16 || (group >= 2 && group >= matrix_from));
+    const bool use_mfma = mfma_shape && (group >= 16 || group >= matrix_from);
     const DecodePlan plan = plan_decode(B, H_kv, group, (H_kv + hpw - 1) / hpw, max_len, P, chunk_tokens, use_mfma);
     const int64_t chunk = plan.chunk;
     const int waves = plan.waves;

@@ -4,22 +4,22 @@
 // A wavefront owns one (batch entry, pool head, chunk of the context); the wavefronts of a workgroup take
 // neighbouring pool heads, so that a workgroup reads whole token rows, and never talk to each other (no barrier).
 // Per page of 16 tokens
-//     S^T = K Q^T        16x16x32 matrix instructions; A = the page's K rows, loaded from global memory straight into
-//                        the operand layout (lane = token, 16 consecutive bytes of its row per instruction),
-//                        B = the group's queries, pre-scaled (columns >= G are zero),
+//     S^T = K Q^T        16x16x32 matrix instructions; A = the page's K rows (lane = token, 16 bytes of its row per
+//                        instruction), B = the group's queries, pre-scaled (columns >= G are zero),
 //     P^T = exp2(S^T - m) online softmax, one query head per lane column, 4 tokens per lane,
 //     O^T += V^T P^T     16x16x16 matrix instructions; A = V^T by transposing LDS reads, B = P^T exactly as the
 //                        registers of S^T hold it.
-// K never touches LDS.  V goes there with direct-to-LDS loads (one instruction per 1 KiB of a page), into a ring of
-// kGroupRing page slots per wavefront; the K rows of the same pages wait in registers.  Three pages per
-// wavefront are on their way while one is consumed: the kernel is bound by the K/V stream and lives on the
-// number of bytes in flight.
+// K and V of a page arrive in LDS by direct-to-LDS loads (one instruction per 1 KiB, whole cache lines), in one of
+// two page slots per wavefront: one page is consumed while the next is on its way.  That is all the depth the
+// memory system can use: a CU keeps about 90 cache-line requests in flight whatever the kernel asks for
+// (counters: requests x latency / time), so what counts is that every request is a whole line asked for once.
+// (Loading K straight into the operand registers - 64 bytes per token and instruction - makes two instructions
+// share every line, and the vector cache asks the L2 for it twice: 3-4 % slower when timed.)
 //
-// The transposing reads are written as asm, with their own wait: the compiler orders every LDS read it knows of
-// behind ALL direct-to-LDS loads in flight once a function holds more than a handful of them, which would
-// serialise the ring.  Direct loads and K loads stay builtins, so the compiler's own counting of outstanding
-// loads (it waits for K registers by itself) stays exact; a page's V loads are issued before its K loads, and
-// loads complete in order, so V has landed when K has - the explicit s_waitcnt states that once more.
+// The LDS reads are written as asm, with their own wait: the compiler orders every LDS read it knows of behind ALL
+// direct-to-LDS loads in flight once a function holds more than a handful of them, which would serialise the two
+// slots.  The direct loads stay builtins and complete in order; the explicit s_waitcnt leaves exactly the next
+// page's loads outstanding.
 //
 // Output: the same (m, l, o) partials per chunk as the lane-per-element kernel, or O itself when the context is a
 // single chunk.  A table entry of -1 inside a sequence ends it there (see paged_decode_kernel).
@@ -33,11 +33,11 @@
 
 namespace ahpc {
 
-constexpr int kGroupRing = 4;  // page slots per wavefront
+constexpr int kGroupRing = 2;  // page slots per wavefront
 #ifndef AHPC_GROUP_AUX
-#define AHPC_GROUP_AUX 0
+#define AHPC_GROUP_AUX 2
 #endif
-constexpr int kStreamAux = AHPC_GROUP_AUX;  // cache policy of the K/V loads: default (non-temporal loads are slower here: two K instructions share every cache line)
+constexpr int kStreamAux = AHPC_GROUP_AUX;  // cache policy of the K/V loads: 2 = non-temporal (every line is used once; worth 10 % when timed)
 
 // ds_read_b64_tr_b16 at lds + IMM without the compiler's knowledge; tr_wait() below completes it.
 template <typename T, int IMM> __device__ inline u32x2 tr_read_async(const unsigned char* lds) {
@@ -64,6 +64,26 @@ template <int N> __device__ inline void tr_wait(u32x2 (&v)[N]) {
 #endif
 }
 
+// ds_read_b128 at lds + IMM, likewise behind the compiler's back (the CPU executor: the traced read).
+template <int IMM> __device__ inline u32x4 lds_read_b128_async(const unsigned char* lds) {
+#if defined(AHPC_TRACED_LDS_READ_B128)
+    return lds_read_b128(lds + IMM);
+#elif defined(__HIP_DEVICE_COMPILE__)
+    u32x4 r;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"((uint32_t)(uintptr_t)lds), "n"(IMM) : "memory");
+    return r;
+#else
+    return u32x4{0u, 0u, 0u, 0u};
+#endif
+}
+template <int N> __device__ inline void b128_wait(u32x4 (&v)[N]) {
+#if !defined(AHPC_TRACED_LDS_READ_B128) && defined(__HIP_DEVICE_COMPILE__)
+    static_assert(N == 2 || N == 4, "one page of d = 64 or 128");
+    if constexpr (N == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
+    else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]));
+#endif
+}
+
 // s_waitcnt immediate that waits until at most N vector-memory loads are outstanding (gfx9 encoding; the other
 // counters stay unconstrained).
 constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
@@ -78,9 +98,10 @@ __global__ __launch_bounds__(64 * W) void paged_decode_group_kernel(const Decode
     constexpr int KS = D / 32;         // matrix instructions of one S^T tile
     constexpr int MB = D / 16;         // 16-row blocks of O^T
     constexpr int R = kGroupRing;
-    constexpr int kSlot = 16 * RB;     // bytes of V of one page and head
+    constexpr int kPart = 16 * RB;     // bytes of V (or K) of one page and head
+    constexpr int kSlot = 2 * kPart;   // a page slot: V, then K
     constexpr int P = 16;
-    constexpr int kOps = NI + KS;      // loads per page and wavefront
+    constexpr int kOps = 2 * NI;       // loads per page and wavefront
     static_assert(D == 64 || D == 128, "head dimensions of this kernel");
 
     __shared__ __attribute__((aligned(1024))) unsigned char lds_v[W * R * kSlot];
@@ -136,7 +157,6 @@ __global__ __launch_bounds__(64 * W) void paged_decode_group_kernel(const Decode
 
     // ---- per-lane byte offsets from the first token row of a page (this head) ---------------------------------
     const int tok_bytes = p.H_kv * RB;
-    const int k_off = col * tok_bytes + 16 * rg;  // + 64*ks: token `col`, the 16 bytes instruction ks wants from this lane
     // V lands row-major in its slot; a row's 16-byte pieces are stored permuted (piece c at position c ^ fv(row)), so
     // that the 8 rows which 32 lanes of a transposing read touch fall into different banks (64 banks of 4 bytes;
     // at d = 64 two rows make up one pass over the banks, and rows of equal parity must differ)
@@ -146,6 +166,14 @@ __global__ __launch_bounds__(64 * W) void paged_decode_group_kernel(const Decode
     for (int i = 0; i < NI; ++i) {
         const int r = i * RPI + lane / CH;
         v_off[i] = r * tok_bytes + (((lane % CH) ^ fv(r)) << 4);
+    }
+    // K: rows are read 16 bytes per lane, 16 rows by 16 lanes at a time: piece c of row r sits at c ^ fk(r)
+    auto fk = [](int r) { return D == 128 ? (r & 15) : ((r >> 1) & 7); };
+    int kd_off[NI];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int r = i * RPI + lane / CH;
+        kd_off[i] = r * tok_bytes + (((lane % CH) ^ fk(r)) << 4);
     }
     unsigned char* const slot0 = lds_v + wave * (R * kSlot);
     // transposing reads: within 16 lanes, lane j asks for token 4*rg + j/4, elements 16*mb + 4*(j%4) .. +3, and
@@ -160,9 +188,13 @@ __global__ __launch_bounds__(64 * W) void paged_decode_group_kernel(const Decode
             v_rd[mb] = slot0 + trow * RB + (((2 * mb) ^ fv(trow)) << 4) + 16 * ((j >> 1) & 1) + 8 * (j & 1);
     }
 
+    // lane (token col, rg) reads piece 4*ks + rg of its token's K row
+    const unsigned char* k_rd[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) k_rd[ks] = slot0 + kPart + col * RB + (((4 * ks + rg) ^ fk(col)) << 4);
+
     const unsigned char* const kpool = static_cast<const unsigned char*>(p.k_pool);
     const unsigned char* const vpool = static_cast<const unsigned char*>(p.v_pool);
-    u32x4 kreg[R][KS];
 
     // Requests page `tt` of the chunk into ring slot S.  Token rows at or beyond the end of the chunk (and whole
     // pages beyond it) lie outside the descriptor: they touch no memory and arrive as zeros.
@@ -180,10 +212,11 @@ __global__ __launch_bounds__(64 * W) void paged_decode_group_kernel(const Decode
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (AHPC_LDS void*)(slot0 + S * kSlot + i * 1024), 16, v_off[i], 0, 0, kStreamAux);
         const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(kpool + byte0), 0, nrec, 0x00020000);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) kreg[S][ks] = __builtin_amdgcn_raw_buffer_load_b128(rk, k_off + 64 * ks, 0, kStreamAux);
+        for (int i = 0; i < NI; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (AHPC_LDS void*)(slot0 + S * kSlot + kPart + i * 1024), 16, kd_off[i], 0, 0, kStreamAux);
 #endif
-        // the loads stay in this order and ahead of the arithmetic that follows: the wait counts below (the
-        // compiler's for K, the explicit one for V) are exact only as long as nothing else slips in between
+        // the requests stay ahead of the arithmetic that follows: the wait count below is exact only as long as
+        // nothing else slips in between
         __builtin_amdgcn_sched_barrier(0);
     };
 
@@ -194,14 +227,18 @@ __global__ __launch_bounds__(64 * W) void paged_decode_group_kernel(const Decode
 
     auto consume = [&](int tt, auto slot_c, auto behind_c) __attribute__((always_inline)) {
         constexpr int S = decltype(slot_c)::value;
-        // V of this page has landed once at most the loads of the pages requested behind it are outstanding
+        // this page has landed once at most the loads of the page requested behind it are outstanding
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(decltype(behind_c)::value * kOps));
         u32x2 vt[MB];
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) vt[mb] = tr_read_async<T, S * kSlot>(v_rd[mb]);
         f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+        u32x4 ka[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) s = mfma_16x16x32<T>(kreg[S][ks], qreg[ks], s);
+        for (int ks = 0; ks < KS; ++ks) ka[ks] = lds_read_b128_async<S * kSlot>(k_rd[ks]);
+        b128_wait(ka);  // (LDS answers in order: V's reads above are done as well)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s = mfma_16x16x32<T>(ka[ks], qreg[ks], s);
         // s[r] belongs to token tt*16 + 4*rg + r, which exists iff it is below n_tok
         const int lim = n_tok - tt * P - 4 * rg;
         float mx = -INFINITY;
@@ -240,35 +277,21 @@ __global__ __launch_bounds__(64 * W) void paged_decode_group_kernel(const Decode
 
     typedef std::integral_constant<int, 0> S0;
     typedef std::integral_constant<int, 1> S1;
-    typedef std::integral_constant<int, 2> S2;
-    typedef std::integral_constant<int, 3> S3;
-    static_assert(R == 4, "the ring below is written out for four slots");
-    // The steady loop has no way out in its middle: the compiler derives its wait counts for the K registers from
-    // every path that reaches an instruction, and a path that leaves early would make it wait for almost everything.
-    issue(0, S0{});
-    issue(1, S1{});
-    issue(2, S2{});
+    static_assert(R == 2, "the ring below is written out for two slots");
+    // The steady loop has no way out in its middle: it requests even behind the last page (empty requests), so the
+    // same number of loads is outstanding at every wait.
     int t = 0;
+    issue(0, S0{});
     for (; t + R <= n_pages; t += R) {
-        issue(t + 3, S3{});
-        consume(t, S0{}, S3{});
-        issue(t + 4, S0{});
-        consume(t + 1, S1{}, S3{});
-        issue(t + 5, S1{});
-        consume(t + 2, S2{}, S3{});
-        issue(t + 6, S2{});
-        consume(t + 3, S3{}, S3{});
+        issue(t + 1, S1{});
+        consume(t, S0{}, S1{});
+        issue(t + 2, S0{});
+        consume(t + 1, S1{}, S1{});
     }
-    // the last one to three pages are in slots 0..2 already, with nothing but empty requests behind them; waiting
-    // for everything also keeps those (zero fills) from outliving the wavefront's LDS
+    // a last odd page is in slot 0 already, with at most an empty request behind it; waiting for everything also keeps
+    // that one (a zero fill) from outliving the wavefront's LDS
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-    if (t < n_pages) {
-        consume(t, S0{}, S0{});
-        if (t + 1 < n_pages) {
-            consume(t + 1, S1{}, S0{});
-            if (t + 2 < n_pages) consume(t + 2, S2{}, S0{});
-        }
-    }
+    if (t < n_pages) consume(t, S0{}, S0{});
 
     float l = l_run + __shfl_xor(l_run, 16, kWave);
     l += __shfl_xor(l, 32, kWave);

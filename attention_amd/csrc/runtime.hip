@@ -18,7 +18,7 @@ Tuning::Tuning()
     : flash_pair_min_tiles(env_value("AHPC_FLASH_PAIR_MIN", 1024)),
       decode_waves(env_value("AHPC_DECODE_WAVES", 0)),
       decode_chunk(env_value("AHPC_DECODE_CHUNK", 0)),
-      decode_matrix_min_group(env_value("AHPC_DECODE_MFMA_MIN_GROUP", 4)) {
+      decode_matrix_min_group(env_value("AHPC_DECODE_MFMA_MIN_GROUP", 2)) {
     if (flash_pair_min_tiles.load() < 1) flash_pair_min_tiles = 1024;
 }
 

@@ -92,7 +92,6 @@ struct BufferRsrc {
     unsigned num_records;
 };
 void buffer_load_lds(BufferRsrc r, void* lds_base, int size, int voffset, int soffset, int imm, int aux);
-u32x4 buffer_load_b128(BufferRsrc r, int voffset, int soffset, int aux);  // to registers; counts as one outstanding load
 void waitcnt(int imm);
 
 inline float fdot2_f16(f16x2 a, f16x2 b, float c) { return (float)a[0] * (float)b[0] + (float)a[1] * (float)b[1] + c; }
@@ -190,7 +189,6 @@ inline hipError_t hipGetLastError() { return ::simt::last_error(); }
 #define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) ::simt::mfma_16x16x32_bf16((a), (b), (c))
 #define __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, x, y, z) ::simt::mfma_16x16x16_f16((a), (b), (c))
 #define __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, x, y, z) ::simt::mfma_16x16x16_bf16((a), (b), (c))
-#define __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, aux) ::simt::buffer_load_b128((r), (voff), (soff), (aux))
 #define __builtin_amdgcn_ds_read_tr16_b64_v4bf16(p) \
     ::simt::bits_to<__attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16>(::simt::ds_read_tr16_b64((const void*)(p)))
 #define __builtin_amdgcn_ds_read_tr16_b64_v4f16(p) \

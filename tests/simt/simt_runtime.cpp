@@ -194,7 +194,6 @@ void flush_dma(Fiber* f, size_t leave = 0) {
     size_t n = f->dma.size() > leave ? f->dma.size() - leave : 0;
     for (size_t i = 0; i < n; ++i) {
         const PendingDma& d = f->dma[i];
-        if (!d.dst) continue;  // a load to registers: only counted
         if (d.src) std::memcpy(d.dst, d.src, (size_t)d.bytes);
         else std::memset(d.dst, 0, (size_t)d.bytes);
         note_dma_landed(f, d.dst, d.bytes);
@@ -576,20 +575,6 @@ void buffer_load_lds(BufferRsrc r, void* lds_base, int size, int voffset, int so
         f->dma.push_back(d);
         flush_dma(f);
     }
-}
-
-// buffer_load_dwordx4 to registers: the data is taken at once (the compiler waits for registers itself), but
-// the load takes its place in the queue of outstanding loads, so that s_waitcnt vmcnt(n) counts as on hardware.
-u32x4 buffer_load_b128(BufferRsrc r, int voffset, int soffset, int aux) {
-    (void)aux;
-    Fiber* f = g_cur;
-    if (voffset < 0) fail("buffer_load: negative lane offset");
-    const uint64_t off = (uint64_t)(uint32_t)voffset + (uint64_t)(uint32_t)soffset;
-    u32x4 out = {0, 0, 0, 0};
-    if (off + 16 <= (uint64_t)r.num_records) std::memcpy(&out, r.base + off, 16);
-    f->dma.push_back(PendingDma{nullptr, nullptr, 0});
-    if (!g_dma_late) flush_dma(f);
-    return out;
 }
 
 // s_waitcnt with the gfx9 encoding: vmcnt in bits 3:0 and 15:14; the other counters are not modelled

@@ -118,9 +118,19 @@ def build_pool(B, Hkv, d, P, lens, seed, dtype):
     return kp, vp, table, lens, n_pages
 
 
+@pytest.fixture(params=[2, 16], ids=["matrix-core-from-2", "lane-per-element-to-8"])
+def kernel_choice(gpu, request):
+    """Groups of 2, 4 and 8 heads on 16-bit pools (d 64/128, pages of 16) exist on both decode kernels: the tuning value
+    decides, and both settings are run."""
+    before = gpu.get_tuning("decode_matrix_min_group")
+    gpu.set_tuning("decode_matrix_min_group", request.param)
+    yield request.param
+    gpu.set_tuning("decode_matrix_min_group", before)
+
+
 @pytest.mark.parametrize("dtype", [O.F32, O.F16, O.BF16])
 @pytest.mark.parametrize("H,Hkv,d,P", [(8, 4, 128, 16), (8, 2, 64, 16), (16, 2, 128, 16), (4, 1, 128, 8), (6, 3, 32, 16)])
-def test_decode_gqa_equals_expanded_pool(gpu, dtype, H, Hkv, d, P):
+def test_decode_gqa_equals_expanded_pool(gpu, dtype, H, Hkv, d, P, kernel_choice):
     import torch
     from gpu_util import to_dev, to_host, stream_ptr, dev_i32, TOL
     g = H // Hkv

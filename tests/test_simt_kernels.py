@@ -229,8 +229,11 @@ def test_decode_workgroup_shapes(emu, tuned, waves):
         assert np.abs(got - want).max() <= 2e-2, f"chunk={chunk}"
 
 
+@pytest.mark.parametrize("matrix_from", [2, 16])
 @pytest.mark.parametrize("G", [2, 4, 8])
-def test_decode_grouped_heads(emu, G):
+def test_decode_grouped_heads(emu, tuned, G, matrix_from):
+    # groups of 2, 4 and 8 exist on the lane-per-element kernel and on the page-by-page matrix-core kernel
+    tuned("decode_matrix_min_group", matrix_from)
     B, H_kv, d, P = 3, 2, 128, 16
     H = G * H_kv
     _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [70, 5, 129], 22, O.F16)
@@ -532,8 +535,7 @@ def test_decode_grouped_heads_matrix_core_kernel(emu, G, dtype, d, tuned):
         assert np.all(got[3] == 0.0)
         assert np.abs(got - want).max() <= 2e-2, (chunk, qo)
     reads, read_conflicts, tr, tr_conflicts = S.lds_stats(reset=True)
-    # groups of up to 16 heads: the page-by-page kernel, whose K rows never pass through LDS
-    assert (reads == 0 if G <= 16 else reads > 0) and tr > 0 and read_conflicts == 0 and tr_conflicts == 0
+    assert reads > 0 and tr > 0 and read_conflicts == 0 and tr_conflicts == 0
 
 
 @pytest.mark.parametrize("H_kv,G,d,dtype", [(8, 4, 128, O.F16), (5, 2, 64, O.BF16), (1, 16, 128, O.BF16), (3, 8, 64, O.F16)])
