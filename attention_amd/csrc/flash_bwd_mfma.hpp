@@ -279,6 +279,9 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
     __shared__ __attribute__((aligned(1024))) unsigned char lds_o0[TL::kBytes];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_q1[TL::kBytes];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_o1[TL::kBytes];
+    // the statistics of a tile's 64 queries travel with it: lse2[64] then delta[64]
+    __shared__ __attribute__((aligned(512))) unsigned char lds_s0[512];
+    __shared__ __attribute__((aligned(512))) unsigned char lds_s1[512];
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
@@ -352,41 +355,36 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
         const float* const lse2 = p.lse2 + ((int64_t)b * p.H + h) * p.rows_padded;
         const float* const delta = p.delta + ((int64_t)b * p.H + h) * p.rows_padded;
 
-        auto dma_both = [&](int i0, unsigned char* dst_q, unsigned char* dst_o) {
+        auto dma_both = [&](int i0, unsigned char* dst_q, unsigned char* dst_o, unsigned char* dst_s) {
             // (a tile that starts at or behind the end of the sequence touches no memory and lands as zeros)
             const int64_t rem = i0 < L ? (int64_t)(L - i0 - 1) * sn * 2 + 2 * D : 0;
             const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
             dma_tile<D>(gq + (int64_t)i0 * sn, nrec, dma_off, dst_q, wave_u);
             dma_tile<D>(gdo + (int64_t)i0 * sn, nrec, dma_off, dst_o, wave_u);
+            // the statistics arrays are padded to whole 128-row tiles: 64 rows from i0 < L on always exist
+            if (wave_u == 0) {
+                const unsigned nst = i0 < L ? 256u : 0u;
+                dma_dword(lse2 + i0, nst, 4 * lane, dst_s);
+                dma_dword(delta + i0, nst, 4 * lane, dst_s + 256);
+            }
         };
 
-        // The rows of statistics of a tile's two blocks of 32 queries (this lane's 16 rows of a block are 4 runs of 4
-        // consecutive rows; the arrays are padded to whole tiles).  They are requested BEFORE the next tile's
-        // direct-to-LDS loads: loads complete in order, so waiting for a load issued behind those would wait for the
-        // whole next tile as well.
-        auto load_stats = [&](f32x4 (&st)[2][2][4], int i0) {
-#pragma unroll
-            for (int ib = 0; ib < 2; ++ib)
-#pragma unroll
-                for (int g4 = 0; g4 < 4; ++g4) {
-                    st[ib][0][g4] = *reinterpret_cast<const f32x4*>(lse2 + i0 + 32 * ib + 8 * g4 + 4 * half);
-                    st[ib][1][g4] = *reinterpret_cast<const f32x4*>(delta + i0 + 32 * ib + 8 * g4 + 4 * half);
-                }
-        };
-
-        auto compute_tile = [&](const unsigned char* tile_q, const unsigned char* tile_o, int i0, const f32x4 (&st)[2][2][4]) {
+        auto compute_tile = [&](const unsigned char* tile_q, const unsigned char* tile_o, const unsigned char* tile_s, int i0) {
 #pragma unroll
             for (int ib = 0; ib < 2; ++ib) {
                 const int iblock0 = i0 + 32 * ib;
                 if (iblock0 >= L) continue;                      // nothing but padding
                 if (CAUSAL && iblock0 + 31 < kw) continue;      // every query of the block precedes the keys
+                // the block's rows of statistics: this lane's 16 rows are 4 runs of 4 consecutive rows
                 f32x16 s, dp;
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4) {
+                    const f32x4 a = *reinterpret_cast<const f32x4*>(tile_s + 4 * (32 * ib + 8 * g4 + 4 * half));
+                    const f32x4 d0 = *reinterpret_cast<const f32x4*>(tile_s + 256 + 4 * (32 * ib + 8 * g4 + 4 * half));
 #pragma unroll
                     for (int x = 0; x < 4; ++x) {
-                        s[4 * g4 + x] = -st[ib][0][g4][x];
-                        dp[4 * g4 + x] = -st[ib][1][g4][x];
+                        s[4 * g4 + x] = -a[x];
+                        dp[4 * g4 + x] = -d0[x];
                     }
                 }
 #pragma unroll
@@ -427,25 +425,24 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
             }
         };
 
-        auto step = [&](unsigned char* cur_q, unsigned char* cur_o, unsigned char* nxt_q, unsigned char* nxt_o, int t) {
+        auto step = [&](unsigned char* cur_q, unsigned char* cur_o, unsigned char* cur_s, unsigned char* nxt_q, unsigned char* nxt_o,
+                        unsigned char* nxt_s, int t) {
             const int i0 = t * kFlashKeys;
-            f32x4 st[2][2][4];
-            load_stats(st, i0);
-            __builtin_amdgcn_sched_barrier(0);  // the order of the requests is what the comment above is about
-            // Requested even behind the last tile (an empty request): were it conditional, the compiler would
-            // count the loads in flight for the path without it and wait for the statistics as if nothing followed.
-            dma_both(i0 + kFlashKeys, nxt_q, nxt_o);
-            compute_tile(cur_q, cur_o, i0, st);
-            __builtin_amdgcn_s_waitcnt(0);
-            __syncthreads();
+            const bool more = t + 1 < n_tiles;
+            if (more) dma_both(i0 + kFlashKeys, nxt_q, nxt_o, nxt_s);
+            compute_tile(cur_q, cur_o, cur_s, i0);
+            if (more) {
+                __builtin_amdgcn_s_waitcnt(0);
+                __syncthreads();
+            }
         };
 
-        dma_both(t_begin * kFlashKeys, lds_q0, lds_o0);
+        dma_both(t_begin * kFlashKeys, lds_q0, lds_o0, lds_s0);
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
         for (int t = t_begin; t < n_tiles; t += 2) {
-            step(lds_q0, lds_o0, lds_q1, lds_o1, t);
-            if (t + 1 < n_tiles) step(lds_q1, lds_o1, lds_q0, lds_o0, t + 1);
+            step(lds_q0, lds_o0, lds_s0, lds_q1, lds_o1, lds_s1, t);
+            if (t + 1 < n_tiles) step(lds_q1, lds_o1, lds_s1, lds_q0, lds_o0, lds_s0, t + 1);
         }
         __syncthreads();  // the next head's first load reuses the buffers
     }
