@@ -119,10 +119,28 @@ __global__ __launch_bounds__(256) void kv_scatter_batch_kernel(const ScatterBatc
         const u32x4* vs = reinterpret_cast<const u32x4*>(static_cast<const TI*>(p.v_src) + src);
         u32x4* kd = reinterpret_cast<u32x4*>(static_cast<TO*>(p.k_pool) + dst);
         u32x4* vd = reinterpret_cast<u32x4*>(static_cast<TO*>(p.v_pool) + dst);
-        for (int i = lane; i < hd / EPV; i += kWave) {
-            const u32x4 kx = ks[i], vx = vs[i];
-            kd[i] = kx;
-            vd[i] = vx;
+        // a token row is moved in rounds of up to 4 KiB of K and 4 KiB of V per wavefront: all of a round's loads are
+        // requested before its first store; nothing is reused, so loads and stores are non-temporal
+        constexpr int kRound = 4;
+        const int n = hd / EPV;
+        for (int i0 = lane; i0 < n; i0 += kWave * kRound) {
+            u32x4 kx[kRound], vx[kRound];
+#pragma unroll
+            for (int u = 0; u < kRound; ++u) {
+                const int i = i0 + kWave * u;
+                if (i < n) {
+                    kx[u] = __builtin_nontemporal_load(ks + i);
+                    vx[u] = __builtin_nontemporal_load(vs + i);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kRound; ++u) {
+                const int i = i0 + kWave * u;
+                if (i < n) {
+                    __builtin_nontemporal_store(kx[u], kd + i);
+                    __builtin_nontemporal_store(vx[u], vd + i);
+                }
+            }
         }
     } else {
         const TI* ks = static_cast<const TI*>(p.k_src) + src;
