@@ -356,6 +356,20 @@ static bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr
 
 static int64_t padded_rows(int64_t N) { return (N + kFlashRows - 1) / kFlashRows * kFlashRows; }
 
+// dK and dV: in one walk over the query tiles where that fits two workgroups on a CU (d = 64), in two walks (dV, then
+// dK) where it does not (d = 128); the tuning value bwd_split (0 = by head dimension, 1 = one walk, 2 = two) overrides.
+template <typename T, int D, bool CAUSAL, bool VARLEN>
+static void launch_dkv(const FlashBwdParams& m, dim3 grid, dim3 block, hipStream_t stream) {
+    const int64_t choice = tuning().bwd_split.load();
+    const bool split = choice == 0 ? D == 128 : choice == 2;
+    if (split) {
+        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, CAUSAL, VARLEN, 1>), grid, block, 0, stream, m);
+        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, CAUSAL, VARLEN, 2>), grid, block, 0, stream, m);
+    } else {
+        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, CAUSAL, VARLEN, 0>), grid, block, 0, stream, m);
+    }
+}
+
 template <typename T, int D, bool VARLEN>
 static int launch_mfma_dv(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool causal, float* lse2, float* delta,
                           hipStream_t stream) {
@@ -381,11 +395,11 @@ static int launch_mfma_dv(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool
     if (causal) {
         hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, true, VARLEN>), grid_stats, block, 0, stream, f, st);
         hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, true, VARLEN>), grid_q, block, 0, stream, m);
-        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, true, VARLEN>), grid_kv, block, 0, stream, m);
+        launch_dkv<T, D, true, VARLEN>(m, grid_kv, block, stream);
     } else {
         hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, false, VARLEN>), grid_stats, block, 0, stream, f, st);
         hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, false, VARLEN>), grid_q, block, 0, stream, m);
-        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, false, VARLEN>), grid_kv, block, 0, stream, m);
+        launch_dkv<T, D, false, VARLEN>(m, grid_kv, block, stream);
     }
     return static_cast<int>(hipGetLastError());
 }

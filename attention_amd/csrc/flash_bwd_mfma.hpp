@@ -268,8 +268,13 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dq_mfma_kernel(const 
 }
 
 // grid: 8 * per_xcd_kv workgroups, see bwd_work_of_block
-template <typename T, int D, bool CAUSAL, bool VARLEN>
-__global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const FlashBwdParams p) {
+// PART: 0 = dK and dV in one walk over the query tiles (four products per tile; at d = 128 that is 324 registers, one
+// wavefront per SIMD), 1 = dV only (S and dV: two products, V and dO.V never touched), 2 = dK only (S, dP, dK).  The
+// two partial walks execute five products between them but each fits two wavefronts per SIMD, which hide each
+// other's softmax arithmetic and LDS waits; at d = 128 they are the faster way (the launcher picks).
+template <typename T, int D, bool CAUSAL, bool VARLEN, int PART>
+__global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_dkv_mfma_kernel(const FlashBwdParams p) {
+    constexpr bool kDoK = PART != 1, kDoV = PART != 2;
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;
     constexpr int MB = D / 32;
@@ -331,7 +336,7 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
     const int krow = key < L ? key : L - 1;
     u32x4 kreg[KS], vreg[KS];
     load_row_operands<T, KS>(kreg, gk + (int64_t)krow * skv, half, p.scale_log2);
-    load_row_operands<T, KS>(vreg, gv + (int64_t)krow * skv, half, 1.0f);
+    if constexpr (kDoK) load_row_operands<T, KS>(vreg, gv + (int64_t)krow * skv, half, 1.0f);
 
     f32x16 acc_k[MB], acc_v[MB];
 #pragma unroll
@@ -380,19 +385,22 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4) {
                     const f32x4 a = *reinterpret_cast<const f32x4*>(tile_s + 4 * (32 * ib + 8 * g4 + 4 * half));
-                    const f32x4 d0 = *reinterpret_cast<const f32x4*>(tile_s + 256 + 4 * (32 * ib + 8 * g4 + 4 * half));
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) {
-                        s[4 * g4 + x] = -a[x];
-                        dp[4 * g4 + x] = -d0[x];
+                    for (int x = 0; x < 4; ++x) s[4 * g4 + x] = -a[x];
+                    if constexpr (kDoK) {
+                        const f32x4 d0 = *reinterpret_cast<const f32x4*>(tile_s + 256 + 4 * (32 * ib + 8 * g4 + 4 * half));
+#pragma unroll
+                        for (int x = 0; x < 4; ++x) dp[4 * g4 + x] = -d0[x];
                     }
                 }
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     const u32x4 aq = lds_read_b128(tile_q + 32 * ib * RB + row_off[ks]);
-                    const u32x4 ao = lds_read_b128(tile_o + 32 * ib * RB + row_off[ks]);
                     s = mfma_32x32x16<T>(aq, kreg[ks], s);
-                    dp = mfma_32x32x16<T>(ao, vreg[ks], dp);
+                    if constexpr (kDoK) {
+                        const u32x4 ao = lds_read_b128(tile_o + 32 * ib * RB + row_off[ks]);
+                        dp = mfma_32x32x16<T>(ao, vreg[ks], dp);
+                    }
                 }
                 // query = iblock0 + 4*half + 8*(r/4) + r%4 contributes iff it exists, the key exists, and
                 // (causal) query >= key
@@ -405,21 +413,28 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
                     const int off = 8 * (r >> 2) + (r & 3);
                     const bool on = off >= first && off < last;
                     pw[r] = on ? fast_exp2(s[r]) : 0.0f;
-                    ds[r] = on ? pw[r] * dp[r] : 0.0f;
+                    if constexpr (kDoK) ds[r] = on ? pw[r] * dp[r] : 0.0f;
                 }
 #pragma unroll
                 for (int g2 = 0; g2 < 2; ++g2) {
-                    const u32x4 bp = pack_operand<T>(pw, 8 * g2);
-                    const u32x4 bs = pack_operand<T>(ds, 8 * g2);
                     const int rows = (32 * ib + 16 * g2) * RB;
+                    if constexpr (kDoV) {
+                        const u32x4 bp = pack_operand<T>(pw, 8 * g2);
 #pragma unroll
-                    for (int mb = 0; mb < MB; ++mb) {
-                        const u32x2 olo = TrRead<T>::load(tile_o + rows + tr_off[mb][0]);
-                        const u32x2 ohi = TrRead<T>::load(tile_o + rows + tr_off[mb][1]);
-                        acc_v[mb] = mfma_32x32x16<T>(u32x4{olo[0], olo[1], ohi[0], ohi[1]}, bp, acc_v[mb]);
-                        const u32x2 qlo = TrRead<T>::load(tile_q + rows + tr_off[mb][0]);
-                        const u32x2 qhi = TrRead<T>::load(tile_q + rows + tr_off[mb][1]);
-                        acc_k[mb] = mfma_32x32x16<T>(u32x4{qlo[0], qlo[1], qhi[0], qhi[1]}, bs, acc_k[mb]);
+                        for (int mb = 0; mb < MB; ++mb) {
+                            const u32x2 olo = TrRead<T>::load(tile_o + rows + tr_off[mb][0]);
+                            const u32x2 ohi = TrRead<T>::load(tile_o + rows + tr_off[mb][1]);
+                            acc_v[mb] = mfma_32x32x16<T>(u32x4{olo[0], olo[1], ohi[0], ohi[1]}, bp, acc_v[mb]);
+                        }
+                    }
+                    if constexpr (kDoK) {
+                        const u32x4 bs = pack_operand<T>(ds, 8 * g2);
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb) {
+                            const u32x2 qlo = TrRead<T>::load(tile_q + rows + tr_off[mb][0]);
+                            const u32x2 qhi = TrRead<T>::load(tile_q + rows + tr_off[mb][1]);
+                            acc_k[mb] = mfma_32x32x16<T>(u32x4{qlo[0], qlo[1], qhi[0], qhi[1]}, bs, acc_k[mb]);
+                        }
                     }
                 }
             }
@@ -447,8 +462,8 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dkv_mfma_kernel(const
         __syncthreads();  // the next head's first load reuses the buffers
     }
     if (key < L) {
-        store_row<T, MB>(static_cast<T*>(p.d_k) + kv_base + (int64_t)key * skv, acc_k, half, p.scale);
-        store_row<T, MB>(static_cast<T*>(p.d_v) + kv_base + (int64_t)key * skv, acc_v, half, 1.0f);
+        if constexpr (kDoK) store_row<T, MB>(static_cast<T*>(p.d_k) + kv_base + (int64_t)key * skv, acc_k, half, p.scale);
+        if constexpr (kDoV) store_row<T, MB>(static_cast<T*>(p.d_v) + kv_base + (int64_t)key * skv, acc_v, half, 1.0f);
     }
 }
 

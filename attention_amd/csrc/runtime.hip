@@ -18,7 +18,8 @@ Tuning::Tuning()
     : flash_pair_min_tiles(env_value("AHPC_FLASH_PAIR_MIN", 1024)),
       decode_waves(env_value("AHPC_DECODE_WAVES", 0)),
       decode_chunk(env_value("AHPC_DECODE_CHUNK", 0)),
-      decode_matrix_min_group(env_value("AHPC_DECODE_MFMA_MIN_GROUP", 2)) {
+      decode_matrix_min_group(env_value("AHPC_DECODE_MFMA_MIN_GROUP", 2)),
+      bwd_split(env_value("AHPC_BWD_SPLIT", 0)) {
     if (flash_pair_min_tiles.load() < 1) flash_pair_min_tiles = 1024;
 }
 
@@ -34,6 +35,7 @@ static std::atomic<int64_t>* tuning_slot(const char* name) {
     if (!std::strcmp(name, "decode_waves")) return &t.decode_waves;
     if (!std::strcmp(name, "decode_chunk")) return &t.decode_chunk;
     if (!std::strcmp(name, "decode_matrix_min_group")) return &t.decode_matrix_min_group;
+    if (!std::strcmp(name, "bwd_split")) return &t.bwd_split;
     return nullptr;
 }
 

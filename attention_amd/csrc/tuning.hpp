@@ -22,6 +22,9 @@ struct Tuning {
     // query head per pool head the lane-per-element kernel stays ahead by 1-2 %.  16 and 32 exist on the
     // matrix-core kernels only.  (AHPC_DECODE_MFMA_MIN_GROUP)
     std::atomic<int64_t> decode_matrix_min_group;
+    // backward: dK and dV in one walk over the query tiles (1), in two (2), or by head dimension (0, the default:
+    // two at d = 128).  (AHPC_BWD_SPLIT)
+    std::atomic<int64_t> bwd_split;
     Tuning();
 };
 

@@ -477,12 +477,14 @@ def test_backward_fp32_kernels_16bit_storage(emu, dtype):
     check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, 0.2, True, H_kv), dtype)
 
 
+@pytest.mark.parametrize("split", [1, 2])
 @pytest.mark.parametrize("dma_late", [False, True])
 @pytest.mark.parametrize("dtype", [O.BF16, O.F16])
 @pytest.mark.parametrize("B,N,H,H_kv,d,causal", [
     (1, 64, 1, 1, 128, False), (2, 129, 2, 2, 128, True), (1, 300, 2, 2, 64, True), (1, 200, 2, 1, 64, False),
     (1, 1, 2, 2, 128, True), (1, 260, 4, 2, 128, True)])
-def test_backward_matrix_core_kernels(emu, dtype, B, N, H, H_kv, d, causal, dma_late):
+def test_backward_matrix_core_kernels(emu, tuned, dtype, B, N, H, H_kv, d, causal, dma_late, split):
+    tuned("bwd_split", split)   # dK and dV in one walk over the query tiles, or in two (the default at d = 128)
     q, k, v, do = bwd_inputs(B, N, H, H_kv, d, 34, dtype)
     scale = 1.0 / np.sqrt(d)
     S.configure(dma_late, seed=N + d)
