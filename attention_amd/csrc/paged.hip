@@ -185,11 +185,24 @@ struct DecodeParams {
     int64_t max_pages;
     int32_t B, H, d, P;       // H = query heads
     int32_t H_kv;             // heads in the pool; H / H_kv consecutive query heads share one
-    int32_t chunk_tokens, n_chunks;
+    int32_t chunk_tokens, n_chunks;  // longest chunk (a multiple of P, at most 64 pages) and how many the longest sequence needs
+    int32_t balanced;         // 1: a sequence cuts itself into equal chunks (see decode_chunk_len); 0: every chunk is chunk_tokens long
     int32_t max_len;
     int32_t qo_dtype;
     float scale_log2;
 };
+
+// Tokens per chunk of a sequence of L tokens.  A sequence needs n = ceil(L / chunk_tokens) chunks; cutting it into n
+// EQUAL page-aligned pieces instead of n - 1 full ones and a remainder gives the launch's workgroups similar amounts of
+// work (contexts U[512,4096] in chunks of up to 1024: 608 to 1024 tokens each instead of 16 to 1024).  Decode kernels
+// and merge evaluate the same function; chunk k of the sequence starts at k * decode_chunk_len and exists iff that is
+// below L.
+__device__ __forceinline__ int decode_chunk_len(const DecodeParams& p, int L, int P) {
+    if (!p.balanced || L <= 0) return p.chunk_tokens;
+    const int n = (L + p.chunk_tokens - 1) / p.chunk_tokens;
+    const int per = (L + n - 1) / n;
+    return ((per + P - 1) / P) * P;  // <= chunk_tokens, which is a multiple of P
+}
 
 __device__ __forceinline__ void store_qo(void* base, int dtype, int64_t i, float x) {
     if (dtype == AHPC_F32) static_cast<float*>(base)[i] = x;
@@ -295,17 +308,17 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     const int P = PT ? PT : p.P;
 
     const int64_t row = p.batch_rows ? p.batch_rows[b] : b;
-    const int t0 = chunk * p.chunk_tokens;
+    const int L = p.seq_lens[row] < p.max_len ? p.seq_lens[row] : p.max_len;
+    const int chunk_len = decode_chunk_len(p, L, P);
+    const int t0 = chunk * chunk_len;
     // page ids of the chunk (at most 64: the host caps chunk_tokens at 64 pages): lane i holds the id of
-    // page (first_page + i).  Requested before the sequence length is known (any entry of the row may
-    // be read), so that this load and the length load are in flight together.
+    // page (first_page + i)
     const int first_page = t0 / P;
     int my_page = 0;
     if (first_page + lane < p.max_pages) my_page = p.table[row * p.max_pages + first_page + lane];
-    const int L = p.seq_lens[row] < p.max_len ? p.seq_lens[row] : p.max_len;
     bool dumps = DUMP && h_raw == 0 && e0 == 0;  // one lane of the launch's first head group
     if constexpr (DUMP) {
-        if (dumps) {
+        if (dumps) {  // (index-dump launches are not balanced: every workgroup clears its own fixed range first)
             const int te = (t0 + p.chunk_tokens) < p.max_len ? (t0 + p.chunk_tokens) : p.max_len;
             for (int t = t0; t < te; ++t) p.dump_offsets[(int64_t)b * p.max_len + t] = -1;
             // what a chunk behind a missing page reads never enters the result (the merge stops in front of it):
@@ -325,7 +338,7 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
         }
         return;
     }
-    int t1 = (t0 + p.chunk_tokens) < L ? (t0 + p.chunk_tokens) : L;
+    int t1 = (t0 + chunk_len) < L ? (t0 + chunk_len) : L;
     // first missing page of the chunk, if any: the chunk ends in front of it
     const unsigned long long missing = __builtin_amdgcn_ballot_w64(lane < (t1 - t0 + P - 1) / P && my_page < 0);
     const bool stopped = missing != 0;
@@ -506,7 +519,8 @@ __global__ __launch_bounds__(256) void paged_merge_kernel(const DecodeParams p) 
     const int e = (int)(he - (int64_t)h * p.d);
     const int64_t row = p.batch_rows ? p.batch_rows[b] : b;
     const int L = p.seq_lens[row] < p.max_len ? p.seq_lens[row] : p.max_len;
-    const int n = (L + p.chunk_tokens - 1) / p.chunk_tokens;
+    const int chunk_len = decode_chunk_len(p, L, p.P);
+    const int n = (L + chunk_len - 1) / chunk_len;
     const float* ml = p.part_ml + ((b * p.n_chunks) * p.H + h) * 2;
     const float* po = p.part_o + ((b * p.n_chunks) * p.H + h) * p.d + e;
     const int64_t ml_step = (int64_t)p.H * 2, po_step = (int64_t)p.H * p.d;
@@ -861,6 +875,7 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     p.B = (int32_t)B; p.H = (int32_t)H; p.d = (int32_t)d; p.P = (int32_t)P;
     p.H_kv = (int32_t)H_kv;
     p.chunk_tokens = (int32_t)chunk; p.n_chunks = (int32_t)n_chunks;
+    p.balanced = 1;
     p.max_len = (int32_t)max_len;
     p.qo_dtype = qo_dtype;
     p.scale_log2 = scale * kLog2e;

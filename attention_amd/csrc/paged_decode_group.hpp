@@ -119,11 +119,12 @@ __global__ __launch_bounds__(64 * W) void paged_decode_group_kernel(const Decode
     const int hq = hk * G + (head_ok ? col : 0);
 
     const int64_t row = p.batch_rows ? p.batch_rows[b] : b;
-    const int t0 = chunk * p.chunk_tokens;
+    const int L = p.seq_lens[row] < p.max_len ? p.seq_lens[row] : p.max_len;
+    const int chunk_len = decode_chunk_len(p, L, P);  // the sequence's own, equal chunks
+    const int t0 = chunk * chunk_len;
     const int first_page = t0 / P;
     int my_page = 0;  // lane i: id of page first_page + i (a chunk has at most 64 pages)
     if (first_page + lane < p.max_pages) my_page = p.table[row * p.max_pages + first_page + lane];
-    const int L = p.seq_lens[row] < p.max_len ? p.seq_lens[row] : p.max_len;
     if (t0 >= L) {
         // an empty sequence still owns an output row: zeros (with several chunks the merge writes it)
         if (chunk == 0 && p.n_chunks == 1 && head_ok) {
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(64 * W) void paged_decode_group_kernel(const Decode
         }
         return;
     }
-    int t1 = (t0 + p.chunk_tokens) < L ? (t0 + p.chunk_tokens) : L;
+    int t1 = (t0 + chunk_len) < L ? (t0 + chunk_len) : L;
     const unsigned long long missing = __builtin_amdgcn_ballot_w64(lane < (t1 - t0 + P - 1) / P && my_page < 0);
     const bool stopped = missing != 0;
     if (stopped) {
