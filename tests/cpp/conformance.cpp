@@ -12,6 +12,7 @@
 #include <cstring>
 #include <functional>
 #include <string>
+#include <atomic>
 #include <thread>
 #include <vector>
 
@@ -981,6 +982,78 @@ CASE(Paged_SequenceLifecycle, true) {  // extend / truncate / reset, src/algorit
     const TensorShape qs = shape4(1, 1, 2, 32);
     pa.forward_batch({ids[39]}, {qs}, {q.data()}, {qs}, {out.data()});
     EXPECT(std::isfinite(out[0]));
+}
+
+CASE(Paged_PoolGrowsWhileOtherThreadsAppendAndDecode, true) {
+    // The pool starts with 4 pages and grows 2 at a time, so the slabs move (device copy, old slabs freed) again and again
+    // while one thread appends to a sequence and reads it back, a second one decodes from it, and a third one creates
+    // and extends other sequences.  Nothing may be lost or read from a slab that has moved.
+    PagedAttention pa;
+    AttentionParams p{};
+    p.batch_size = 1; p.sequence_length = 1; p.num_heads = 2; p.head_dimension = 32; p.max_sequence_length = 512;
+    PagedAttentionConfig c;
+    c.initial_page_pool_size = 4;
+    c.page_pool_growth = 2;
+    pa.configure_paged_attention(c);
+    pa.configure(p);
+    const size_t H = 2, d = 32, P = 16, total = 320, step = 8;
+    const size_t id = pa.create_sequence(512);
+    const auto k = normal(total * H * d, 97, 2), v = normal(total * H * d, 97, 3);
+    std::atomic<size_t> appended{0};
+    std::atomic<bool> stop{false};
+    std::atomic<int> bad{0};
+    std::thread grower([&] {
+        std::vector<size_t> others;
+        const auto x = normal(40 * H * d, 98, 2);
+        for (int i = 0; i < 24 && !stop.load(); ++i) {
+            others.push_back(pa.create_sequence(16));
+            pa.extend_sequence(others.back(), 24);          // 40 tokens = 3 pages pre-allocated: the pool grows
+            pa.append_kv_cache(others.back(), x.data(), x.data(), 40, DataType::FLOAT32);
+            if (i % 3 == 2) {
+                pa.destroy_sequence(others.front());
+                others.erase(others.begin());
+            }
+        }
+    });
+    std::thread decoder([&] {
+        const auto q = normal(H * d, 99, 1);
+        const TensorShape qs = shape4(1, 1, H, d);
+        while (!stop.load()) {
+            // the length is whatever the appending thread has reached by the time the decode launches: the result must
+            // be finite and must equal the oracle for SOME prefix; it is checked exactly once everything is appended
+            std::vector<float> out(H * d, 0.0f);
+            if (appended.load() == 0) continue;
+            pa.forward_batch({id}, {qs}, {q.data()}, {qs}, {out.data()});
+            for (float y : out)
+                if (!std::isfinite(y)) bad.fetch_add(1);
+        }
+    });
+    for (size_t done = 0; done < total; done += step) {
+        pa.append_kv_cache(id, k.data() + done * H * d, v.data() + done * H * d, step, DataType::FLOAT32);
+        appended.store(done + step);
+        if (done % 64 == 0) {
+            std::vector<float> kg((done + step) * H * d), vg(kg.size());
+            pa.get_kv_cache(id, kg.data(), vg.data(), 0, done + step, DataType::FLOAT32);
+            if (!std::equal(kg.begin(), kg.end(), k.begin()) || !std::equal(vg.begin(), vg.end(), v.begin())) bad.fetch_add(1);
+        }
+    }
+    stop.store(true);
+    grower.join();
+    decoder.join();
+    EXPECT(bad.load() == 0);
+    std::vector<float> kg(total * H * d), vg(kg.size());
+    pa.get_kv_cache(id, kg.data(), vg.data(), 0, total, DataType::FLOAT32);
+    EXPECT(kg == k && vg == v);  // bit exact after all the moves
+    const auto q = normal(H * d, 99, 1);
+    const TensorShape qs = shape4(1, 1, H, d);
+    std::vector<float> out(H * d), want(H * d);
+    pa.forward_batch({id}, {qs}, {q.data()}, {qs}, {out.data()});
+    std::vector<int32_t> table(total / P);
+    for (size_t i = 0; i < table.size(); ++i) table[i] = (int32_t)i;
+    const int32_t len = (int32_t)total;
+    ahpc_oracle_paged_decode(q.data(), want.data(), k.data(), v.data(), table.data(), &len, nullptr, 1, H, d, P, table.size(),
+                             1.0f / std::sqrt((float)d), 2);
+    EXPECT(max_abs_diff(out, want) <= 1e-4f);
 }
 
 // ---- main ------------------------------------------------------------------------------------------------------
