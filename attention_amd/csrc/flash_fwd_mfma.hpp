@@ -88,6 +88,58 @@ template <> struct TrRead<f16_t> {
     }
 };
 
+// ---- LDS reads behind the compiler's back ----------------------------------------------------------------------
+// The compiler orders every LDS read it knows of behind ALL direct-to-LDS loads in flight once a function holds more
+// than a handful of them (an s_waitcnt vmcnt(0) in front of reads of a tile that landed long ago), which serialises a
+// pipeline of tiles.  Kernels with such pipelines issue their LDS reads as asm and complete them with the waits below.
+// ds_read_b64_tr_b16 at lds + IMM without the compiler's knowledge; tr_wait() below completes it.
+template <typename T, int IMM> __device__ inline u32x2 tr_read_async(const unsigned char* lds) {
+#if defined(AHPC_TRACED_LDS_READ_B128)  // the CPU executor: an ordinary (modelled) transposing read
+    return TrRead<T>::load(lds + IMM);
+#elif defined(__HIP_DEVICE_COMPILE__)
+    u32x2 r;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"((uint32_t)(uintptr_t)lds), "n"(IMM) : "memory");
+    return r;
+#else
+    return u32x2{0u, 0u};
+#endif
+}
+
+// Waits for the LDS reads issued so far; the values pass through it, so nothing that uses them moves above the wait.
+template <int N> __device__ inline void tr_wait(u32x2 (&v)[N]) {
+#if !defined(AHPC_TRACED_LDS_READ_B128) && defined(__HIP_DEVICE_COMPILE__)
+    static_assert(N == 4 || N == 8, "operand sets of d = 64 or 128");
+    if constexpr (N == 8)
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+    else
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
+#endif
+}
+
+// ds_read_b128 at lds + IMM, likewise behind the compiler's back (the CPU executor: the traced read).
+template <int IMM> __device__ inline u32x4 lds_read_b128_async(const unsigned char* lds) {
+#if defined(AHPC_TRACED_LDS_READ_B128)
+    return lds_read_b128(lds + IMM);
+#elif defined(__HIP_DEVICE_COMPILE__)
+    u32x4 r;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"((uint32_t)(uintptr_t)lds), "n"(IMM) : "memory");
+    return r;
+#else
+    return u32x4{0u, 0u, 0u, 0u};
+#endif
+}
+template <int N> __device__ inline void b128_wait(u32x4 (&v)[N]) {
+#if !defined(AHPC_TRACED_LDS_READ_B128) && defined(__HIP_DEVICE_COMPILE__)
+    static_assert(N == 2 || N == 4 || N == 8, "operand sets of d = 64 or 128");
+    if constexpr (N == 8)
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+    else if constexpr (N == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
+    else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]));
+#endif
+}
+
 // max / sum of x over the two lanes that share a query column (lane and lane ^ 32).
 // v_permlane32_swap(a, b) exchanges the upper 32 lanes of a with the lower 32 lanes of b; with
 // a = b = x the two results hold x's lower half and x's upper half in every lane.

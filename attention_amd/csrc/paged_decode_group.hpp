@@ -39,51 +39,6 @@ constexpr int kGroupRing = 2;  // page slots per wavefront
 #endif
 constexpr int kStreamAux = AHPC_GROUP_AUX;  // cache policy of the K/V loads: 2 = non-temporal (every line is used once; worth 10 % when timed)
 
-// ds_read_b64_tr_b16 at lds + IMM without the compiler's knowledge; tr_wait() below completes it.
-template <typename T, int IMM> __device__ inline u32x2 tr_read_async(const unsigned char* lds) {
-#if defined(AHPC_TRACED_LDS_READ_B128)  // the CPU executor: an ordinary (modelled) transposing read
-    return TrRead<T>::load(lds + IMM);
-#elif defined(__HIP_DEVICE_COMPILE__)
-    u32x2 r;
-    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"((uint32_t)(uintptr_t)lds), "n"(IMM) : "memory");
-    return r;
-#else
-    return u32x2{0u, 0u};
-#endif
-}
-
-// Waits for the LDS reads issued so far; the values pass through it, so nothing that uses them moves above the wait.
-template <int N> __device__ inline void tr_wait(u32x2 (&v)[N]) {
-#if !defined(AHPC_TRACED_LDS_READ_B128) && defined(__HIP_DEVICE_COMPILE__)
-    static_assert(N == 4 || N == 8, "one page of d = 64 or 128");
-    if constexpr (N == 8)
-        asm volatile("s_waitcnt lgkmcnt(0)"
-                     : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
-    else
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
-#endif
-}
-
-// ds_read_b128 at lds + IMM, likewise behind the compiler's back (the CPU executor: the traced read).
-template <int IMM> __device__ inline u32x4 lds_read_b128_async(const unsigned char* lds) {
-#if defined(AHPC_TRACED_LDS_READ_B128)
-    return lds_read_b128(lds + IMM);
-#elif defined(__HIP_DEVICE_COMPILE__)
-    u32x4 r;
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"((uint32_t)(uintptr_t)lds), "n"(IMM) : "memory");
-    return r;
-#else
-    return u32x4{0u, 0u, 0u, 0u};
-#endif
-}
-template <int N> __device__ inline void b128_wait(u32x4 (&v)[N]) {
-#if !defined(AHPC_TRACED_LDS_READ_B128) && defined(__HIP_DEVICE_COMPILE__)
-    static_assert(N == 2 || N == 4, "one page of d = 64 or 128");
-    if constexpr (N == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
-    else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]));
-#endif
-}
-
 // s_waitcnt immediate that waits until at most N vector-memory loads are outstanding (gfx9 encoding; the other
 // counters stay unconstrained).
 constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }

@@ -10,6 +10,9 @@
 // Only G of the 32 result columns carry work; the matrix cores have time to spare, because the kernel is
 // bound by the K/V stream: 16 matrix instructions per 16 KiB of K and V at d = 128.
 //
+// The LDS reads are asm with their own wait (tr_read_async, lds_read_b128_async): the compiler would otherwise put
+// every LDS read behind all direct-to-LDS loads in flight, and the tile on its way could not overlap the tile in hand.
+//
 // The tile is gathered through the block table with direct-to-LDS loads, one instruction per 1 KiB of a page
 // (pages hold 16 tokens): the page id is a lane-uniform readlane, the base address of the instruction a
 // scalar, the per-lane offsets constants.  Two tiles are in flight (one being consumed, one on its way).
@@ -146,8 +149,14 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_kernel(const DecodeParam
         f32x16 s;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+        {
+            u32x4 ka[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) s = mfma_32x32x16<T>(lds_read_b128(tile_k + k_off[ks]), qreg[ks], s);
+            for (int ks = 0; ks < KS; ++ks) ka[ks] = lds_read_b128_async<0>(tile_k + k_off[ks]);
+            b128_wait(ka);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) s = mfma_32x32x16<T>(ka[ks], qreg[ks], s);
+        }
         // token = tile*32 + 4*half + 8*(r/4) + r%4 exists iff it is below n_tok
         const int lim = n_tok - tile * kDecodeTile - 4 * half;
         float mx = -INFINITY;
@@ -182,12 +191,16 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_kernel(const DecodeParam
         for (int g2 = 0; g2 < 2; ++g2) {
             const u32x4 pb = u32x4{pack2<T>(s[8 * g2 + 0], s[8 * g2 + 1]), pack2<T>(s[8 * g2 + 2], s[8 * g2 + 3]),
                                    pack2<T>(s[8 * g2 + 4], s[8 * g2 + 5]), pack2<T>(s[8 * g2 + 6], s[8 * g2 + 7])};
+            u32x2 vt[2 * MB];
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
-                const u32x2 lo = TrRead<T>::load(tile_v + v_off[mb] + (16 * g2) * RB);
-                const u32x2 hi = TrRead<T>::load(tile_v + v_off[mb] + (16 * g2 + 8) * RB);
-                oacc[mb] = mfma_32x32x16<T>(u32x4{lo[0], lo[1], hi[0], hi[1]}, pb, oacc[mb]);
+                vt[2 * mb] = tr_read_async<T, 0>(tile_v + v_off[mb] + (16 * g2) * RB);
+                vt[2 * mb + 1] = tr_read_async<T, 0>(tile_v + v_off[mb] + (16 * g2 + 8) * RB);
             }
+            tr_wait(vt);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+                oacc[mb] = mfma_32x32x16<T>(u32x4{vt[2 * mb][0], vt[2 * mb][1], vt[2 * mb + 1][0], vt[2 * mb + 1][1]}, pb, oacc[mb]);
         }
     };
 
