@@ -115,7 +115,7 @@ __device__ inline void store_row(T* dst_row, const f32x16 (&acc)[MB], int half, 
 
 // grid: 8 * per_xcd_q workgroups, see bwd_work_of_block
 template <typename T, int D, bool CAUSAL, bool VARLEN>
-__global__ __launch_bounds__(kFlashThreads) void flash_bwd_dq_mfma_kernel(const FlashBwdParams p) {
+__global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(const FlashBwdParams p) {
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;
     constexpr int MB = D / 32;
@@ -215,34 +215,72 @@ __global__ __launch_bounds__(kFlashThreads) void flash_bwd_dq_mfma_kernel(const 
             const int kblock0 = k0 + 32 * kb;
             if (kblock0 >= L) continue;                        // nothing but padding
             if (CAUSAL && kblock0 > qw + 31) continue;        // every key of the block is in the future
-            f32x16 s = neg_lse, dp = neg_delta;
+            // K^T operands of the block's first 16 keys: requested now, they arrive while the first two products run
+            u32x2 kt[2][MB][2];
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const u32x4 ak = lds_read_b128(tile_k + 32 * kb * RB + row_off[ks]);
-                const u32x4 av = lds_read_b128(tile_v + 32 * kb * RB + row_off[ks]);
-                s = mfma_32x32x16<T>(ak, qreg[ks], s);
-                dp = mfma_32x32x16<T>(av, doreg[ks], dp);
+            for (int mb = 0; mb < MB; ++mb) {
+                kt[0][mb][0] = TrRead<T>::load(tile_k + (32 * kb) * RB + tr_off[mb][0]);
+                kt[0][mb][1] = TrRead<T>::load(tile_k + (32 * kb) * RB + tr_off[mb][1]);
+            }
+            f32x16 s = neg_lse, dp = neg_delta;
+            {
+                // the operand pairs of the two products are requested kAhead steps ahead of the matrix instructions
+                // that use them (all at once would cost 8 registers per step)
+                u32x4 ak[KS], av[KS];
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    ak[ks] = lds_read_b128(tile_k + 32 * kb * RB + row_off[ks]);
+                    av[ks] = lds_read_b128(tile_v + 32 * kb * RB + row_off[ks]);
+                }
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    s = mfma_32x32x16<T>(ak[ks], qreg[ks], s);
+                    dp = mfma_32x32x16<T>(av[ks], doreg[ks], dp);
+                }
+                constexpr int kAhead = 2;
+                __builtin_amdgcn_sched_group_barrier(0x100, 2 * MB + 2 * kAhead, 0);  // LDS reads (the K^T ones first)
+#pragma unroll
+                for (int i = 0; i < KS - kAhead; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // matrix instructions
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < kAhead; ++i) __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
             }
             // key = kblock0 + 4*half + 8*(r/4) + r%4 is visible iff key <= min(qrow, L-1)
-            int lim = L - 1;
-            if (CAUSAL) lim = qrow < lim ? qrow : lim;
-            lim -= kblock0 + 4 * half;
             f32x16 ds;
+            // the per-element test is needed only where the block meets the diagonal or the end of the sequence
+            // (uniform per wavefront)
+            const bool all_on = kblock0 + 31 < L && (!CAUSAL || kblock0 + 31 <= qw);
+            if (all_on) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int off = 8 * (r >> 2) + (r & 3);
-                ds[r] = off <= lim ? fast_exp2(s[r]) * dp[r] : 0.0f;
+                for (int r = 0; r < 16; ++r) ds[r] = fast_exp2(s[r]) * dp[r];
+            } else {
+                int lim = L - 1;
+                if (CAUSAL) lim = qrow < lim ? qrow : lim;
+                lim -= kblock0 + 4 * half;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int off = 8 * (r >> 2) + (r & 3);
+                    ds[r] = off <= lim ? fast_exp2(s[r]) * dp[r] : 0.0f;
+                }
             }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int g2 = 0; g2 < 2; ++g2) {
                 const u32x4 bop = pack_operand<T>(ds, 8 * g2);
-                const int rows = (32 * kb + 16 * g2) * RB;
+                if (g2 == 0) {
+                    // the second 16 keys' operands travel while the first 16 are multiplied
 #pragma unroll
-                for (int mb = 0; mb < MB; ++mb) {
-                    const u32x2 lo = TrRead<T>::load(tile_k + rows + tr_off[mb][0]);
-                    const u32x2 hi = TrRead<T>::load(tile_k + rows + tr_off[mb][1]);
-                    acc[mb] = mfma_32x32x16<T>(u32x4{lo[0], lo[1], hi[0], hi[1]}, bop, acc[mb]);
+                    for (int mb = 0; mb < MB; ++mb) {
+                        kt[1][mb][0] = TrRead<T>::load(tile_k + (32 * kb + 16) * RB + tr_off[mb][0]);
+                        kt[1][mb][1] = TrRead<T>::load(tile_k + (32 * kb + 16) * RB + tr_off[mb][1]);
+                    }
                 }
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+                    acc[mb] = mfma_32x32x16<T>(u32x4{kt[g2][mb][0][0], kt[g2][mb][0][1], kt[g2][mb][1][0], kt[g2][mb][1][1]}, bop, acc[mb]);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
@@ -393,49 +431,100 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
                         for (int x = 0; x < 4; ++x) dp[4 * g4 + x] = -d0[x];
                     }
                 }
+                __builtin_amdgcn_sched_barrier(0);  // (the statistics reads stay out of the pipeline laid out below)
+                // transposed operands of the block's first 16 queries: requested now, they arrive while the first
+                // products run
+                u32x2 ot[2][MB][2], qt[2][MB][2];
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    const u32x4 aq = lds_read_b128(tile_q + 32 * ib * RB + row_off[ks]);
-                    s = mfma_32x32x16<T>(aq, kreg[ks], s);
-                    if constexpr (kDoK) {
-                        const u32x4 ao = lds_read_b128(tile_o + 32 * ib * RB + row_off[ks]);
-                        dp = mfma_32x32x16<T>(ao, vreg[ks], dp);
+                for (int mb = 0; mb < MB; ++mb) {
+                    if constexpr (kDoV) {
+                        ot[0][mb][0] = TrRead<T>::load(tile_o + (32 * ib) * RB + tr_off[mb][0]);
+                        ot[0][mb][1] = TrRead<T>::load(tile_o + (32 * ib) * RB + tr_off[mb][1]);
                     }
+                    if constexpr (kDoK) {
+                        qt[0][mb][0] = TrRead<T>::load(tile_q + (32 * ib) * RB + tr_off[mb][0]);
+                        qt[0][mb][1] = TrRead<T>::load(tile_q + (32 * ib) * RB + tr_off[mb][1]);
+                    }
+                }
+                {
+                    // the operands of the first products are requested kAhead steps ahead of the matrix
+                    // instructions that use them
+                    constexpr int kPer = kDoK ? 2 : 1;  // products (and operand reads) per step
+                    constexpr int kAhead = 2;
+                    u32x4 aq[KS], ao[KS];
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        aq[ks] = lds_read_b128(tile_q + 32 * ib * RB + row_off[ks]);
+                        if constexpr (kDoK) ao[ks] = lds_read_b128(tile_o + 32 * ib * RB + row_off[ks]);
+                    }
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        s = mfma_32x32x16<T>(aq[ks], kreg[ks], s);
+                        if constexpr (kDoK) dp = mfma_32x32x16<T>(ao[ks], vreg[ks], dp);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2 * MB * (kDoK && kDoV ? 2 : 1) + kPer * kAhead, 0);  // LDS reads
+#pragma unroll
+                    for (int i = 0; i < KS - kAhead; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);  // matrix instructions
+                        __builtin_amdgcn_sched_group_barrier(0x100, kPer, 0);
+                    }
+#pragma unroll
+                    for (int i = 0; i < kAhead; ++i) __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);
                 }
                 // query = iblock0 + 4*half + 8*(r/4) + r%4 contributes iff it exists, the key exists, and
                 // (causal) query >= key
-                int first = 0;
-                if (CAUSAL) first = key - (iblock0 + 4 * half);
-                const int last = (key < L ? L : 0) - (iblock0 + 4 * half);  // off < last
                 f32x16 pw, ds;
+                // the per-element tests are needed only where the block meets the diagonal or an end of the sequence
+                // (uniform per wavefront): everywhere else every (query, key) pair of the block counts
+                const bool all_on = iblock0 + 31 < L && kw + 31 < L && (!CAUSAL || iblock0 >= kw + 31);
+                if (all_on) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int off = 8 * (r >> 2) + (r & 3);
-                    const bool on = off >= first && off < last;
-                    pw[r] = on ? fast_exp2(s[r]) : 0.0f;
-                    if constexpr (kDoK) ds[r] = on ? pw[r] * dp[r] : 0.0f;
+                    for (int r = 0; r < 16; ++r) {
+                        pw[r] = fast_exp2(s[r]);
+                        if constexpr (kDoK) ds[r] = pw[r] * dp[r];
+                    }
+                } else {
+                    int first = 0;
+                    if (CAUSAL) first = key - (iblock0 + 4 * half);
+                    const int last = (key < L ? L : 0) - (iblock0 + 4 * half);  // off < last
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int off = 8 * (r >> 2) + (r & 3);
+                        const bool on = off >= first && off < last;
+                        pw[r] = on ? fast_exp2(s[r]) : 0.0f;
+                        if constexpr (kDoK) ds[r] = on ? pw[r] * dp[r] : 0.0f;
+                    }
                 }
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int g2 = 0; g2 < 2; ++g2) {
-                    const int rows = (32 * ib + 16 * g2) * RB;
+                    if (g2 == 0) {
+                        // the second 16 queries' operands travel while the first 16 are multiplied
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb) {
+                            if constexpr (kDoV) {
+                                ot[1][mb][0] = TrRead<T>::load(tile_o + (32 * ib + 16) * RB + tr_off[mb][0]);
+                                ot[1][mb][1] = TrRead<T>::load(tile_o + (32 * ib + 16) * RB + tr_off[mb][1]);
+                            }
+                            if constexpr (kDoK) {
+                                qt[1][mb][0] = TrRead<T>::load(tile_q + (32 * ib + 16) * RB + tr_off[mb][0]);
+                                qt[1][mb][1] = TrRead<T>::load(tile_q + (32 * ib + 16) * RB + tr_off[mb][1]);
+                            }
+                        }
+                    }
                     if constexpr (kDoV) {
                         const u32x4 bp = pack_operand<T>(pw, 8 * g2);
 #pragma unroll
-                        for (int mb = 0; mb < MB; ++mb) {
-                            const u32x2 olo = TrRead<T>::load(tile_o + rows + tr_off[mb][0]);
-                            const u32x2 ohi = TrRead<T>::load(tile_o + rows + tr_off[mb][1]);
-                            acc_v[mb] = mfma_32x32x16<T>(u32x4{olo[0], olo[1], ohi[0], ohi[1]}, bp, acc_v[mb]);
-                        }
+                        for (int mb = 0; mb < MB; ++mb)
+                            acc_v[mb] = mfma_32x32x16<T>(u32x4{ot[g2][mb][0][0], ot[g2][mb][0][1], ot[g2][mb][1][0], ot[g2][mb][1][1]}, bp, acc_v[mb]);
                     }
                     if constexpr (kDoK) {
                         const u32x4 bs = pack_operand<T>(ds, 8 * g2);
 #pragma unroll
-                        for (int mb = 0; mb < MB; ++mb) {
-                            const u32x2 qlo = TrRead<T>::load(tile_q + rows + tr_off[mb][0]);
-                            const u32x2 qhi = TrRead<T>::load(tile_q + rows + tr_off[mb][1]);
-                            acc_k[mb] = mfma_32x32x16<T>(u32x4{qlo[0], qlo[1], qhi[0], qhi[1]}, bs, acc_k[mb]);
-                        }
+                        for (int mb = 0; mb < MB; ++mb)
+                            acc_k[mb] = mfma_32x32x16<T>(u32x4{qt[g2][mb][0][0], qt[g2][mb][0][1], qt[g2][mb][1][0], qt[g2][mb][1][1]}, bs, acc_k[mb]);
                     }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         };
