@@ -471,7 +471,7 @@ static int flash_bwd_any(const void* d_out, const void* q, const void* k, const 
         FlashBwdParams m{};
         m.q = q; m.k = k; m.v = v; m.d_out = d_out;
         m.d_q = d_q; m.d_k = d_k; m.d_v = d_v;
-        m.lse2 = p.lse; m.delta = p.delta; m.rows_padded = p.rows_padded;
+        m.neg_lse2 = p.lse; m.neg_delta = p.delta; m.rows_padded = p.rows_padded;
         m.cu_seqlens = cu_seqlens;
         m.stride_b = stride_b; m.stride_n = stride_n; m.stride_h = stride_h;
         m.kv_stride_b = kv_stride_b; m.kv_stride_n = kv_stride_n; m.kv_stride_h = kv_stride_h;

@@ -1,7 +1,7 @@
 // FlashAttention backward on the gfx950 matrix cores (fp16 / bf16 storage, fp32 accumulate), dense batches.
 //
 // Input: Q, K, V, dO and the per-row statistics of the forward (lse2 = log2 sum_j exp2(c q.k_j) with
-// c = scale*log2(e), delta = dO.O; written by flash_bwd_stats_mfma_kernel).  With P = exp2(c q.k - lse2):
+// c = scale*log2(e), delta = dO.O; written, negated, by flash_bwd_stats_mfma_kernel).  With P = exp2(c q.k - lse2):
 //
 //   flash_bwd_dq_mfma_kernel    a workgroup owns 128 query rows (32 per wavefront) and walks the keys in
 //       tiles of 64, exactly like the forward:  S^T = K Q^T and dP^T = V dO^T  (A = rows of the K / V tile
@@ -35,8 +35,8 @@ struct FlashBwdParams {
     void* d_q;
     void* d_k;
     void* d_v;
-    const float* lse2;          // [B*H][rows_padded]
-    const float* delta;
+    const float* neg_lse2;      // [B*H][rows_padded]: -lse2 and -delta, what the accumulators start from
+    const float* neg_delta;
     const int32_t* cu_seqlens;  // ragged batches only
     int64_t rows_padded;
     int64_t stride_b, stride_n, stride_h;           // Q, dO, dQ
@@ -196,7 +196,7 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
     const int64_t stat = ((int64_t)b * p.H + h) * p.rows_padded + qrow;  // qrow < rows_padded always
     f32x16 neg_lse, neg_delta;
     {
-        const float a = -p.lse2[stat], d0 = -p.delta[stat];
+        const float a = p.neg_lse2[stat], d0 = p.neg_delta[stat];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             neg_lse[r] = a;
@@ -215,6 +215,8 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
             const int kblock0 = k0 + 32 * kb;
             if (kblock0 >= L) continue;                        // nothing but padding
             if (CAUSAL && kblock0 > qw + 31) continue;        // every key of the block is in the future
+            // (issue priority up while the matrix cores are fed, down for the stretch of exponentials, as in the forward)
+            __builtin_amdgcn_s_setprio(1);
             // K^T operands of the block's first 16 keys: requested now, they arrive while the first two products run
             u32x2 kt[2][MB][2];
 #pragma unroll
@@ -248,6 +250,7 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
                 for (int i = 0; i < kAhead; ++i) __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
             }
             // key = kblock0 + 4*half + 8*(r/4) + r%4 is visible iff key <= min(qrow, L-1)
+            __builtin_amdgcn_s_setprio(0);
             f32x16 ds;
             // the per-element test is needed only where the block meets the diagonal or the end of the sequence
             // (uniform per wavefront)
@@ -265,6 +268,7 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
                     ds[r] = off <= lim ? fast_exp2(s[r]) * dp[r] : 0.0f;
                 }
             }
+            __builtin_amdgcn_s_setprio(1);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int g2 = 0; g2 < 2; ++g2) {
@@ -282,6 +286,7 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
                     acc[mb] = mfma_32x32x16<T>(u32x4{kt[g2][mb][0][0], kt[g2][mb][0][1], kt[g2][mb][1][0], kt[g2][mb][1][1]}, bop, acc[mb]);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            __builtin_amdgcn_s_setprio(0);
         }
     };
 
@@ -322,7 +327,7 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
     __shared__ __attribute__((aligned(1024))) unsigned char lds_o0[TL::kBytes];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_q1[TL::kBytes];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_o1[TL::kBytes];
-    // the statistics of a tile's 64 queries travel with it: lse2[64] then delta[64]
+    // the statistics of a tile's 64 queries travel with it: -lse2[64] then -delta[64]
     __shared__ __attribute__((aligned(512))) unsigned char lds_s0[512];
     __shared__ __attribute__((aligned(512))) unsigned char lds_s1[512];
 
@@ -395,8 +400,8 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
                                     : (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
         const T* const gq = static_cast<const T*>(p.q) + base;
         const T* const gdo = static_cast<const T*>(p.d_out) + base;
-        const float* const lse2 = p.lse2 + ((int64_t)b * p.H + h) * p.rows_padded;
-        const float* const delta = p.delta + ((int64_t)b * p.H + h) * p.rows_padded;
+        const float* const lse2 = p.neg_lse2 + ((int64_t)b * p.H + h) * p.rows_padded;
+        const float* const delta = p.neg_delta + ((int64_t)b * p.H + h) * p.rows_padded;
 
         auto dma_both = [&](int i0, unsigned char* dst_q, unsigned char* dst_o, unsigned char* dst_s) {
             // (a tile that starts at or behind the end of the sequence touches no memory and lands as zeros)
@@ -424,14 +429,15 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
                 for (int g4 = 0; g4 < 4; ++g4) {
                     const f32x4 a = *reinterpret_cast<const f32x4*>(tile_s + 4 * (32 * ib + 8 * g4 + 4 * half));
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) s[4 * g4 + x] = -a[x];
+                    for (int x = 0; x < 4; ++x) s[4 * g4 + x] = a[x];
                     if constexpr (kDoK) {
                         const f32x4 d0 = *reinterpret_cast<const f32x4*>(tile_s + 256 + 4 * (32 * ib + 8 * g4 + 4 * half));
 #pragma unroll
-                        for (int x = 0; x < 4; ++x) dp[4 * g4 + x] = -d0[x];
+                        for (int x = 0; x < 4; ++x) dp[4 * g4 + x] = d0[x];
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);  // (the statistics reads stay out of the pipeline laid out below)
+                __builtin_amdgcn_s_setprio(1);
                 // transposed operands of the block's first 16 queries: requested now, they arrive while the first
                 // products run
                 u32x2 ot[2][MB][2], qt[2][MB][2];
@@ -473,6 +479,7 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
                 }
                 // query = iblock0 + 4*half + 8*(r/4) + r%4 contributes iff it exists, the key exists, and
                 // (causal) query >= key
+                __builtin_amdgcn_s_setprio(0);
                 f32x16 pw, ds;
                 // the per-element tests are needed only where the block meets the diagonal or an end of the sequence
                 // (uniform per wavefront): everywhere else every (query, key) pair of the block counts
@@ -495,6 +502,7 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
                         if constexpr (kDoK) ds[r] = on ? pw[r] * dp[r] : 0.0f;
                     }
                 }
+                __builtin_amdgcn_s_setprio(1);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int g2 = 0; g2 < 2; ++g2) {
@@ -526,6 +534,7 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
+                __builtin_amdgcn_s_setprio(0);
             }
         };
 

@@ -242,13 +242,14 @@ __host__ __device__ inline int flash_qtile_of_part(const FlashParams& p, int n_q
 
 // What the statistics variant of the kernel writes instead of O (first step of the backward):
 // per (sequence, head, query row)  lse2 = log2 sum_j exp2(c q.k_j)  (c = scale*log2(e), the units the kernel
-// works in) and delta = dO . O.  Rows are laid out [B*H][rows_padded], rows_padded a multiple of the
-// 128-row query tile; rows beyond the sequence receive lse2 = +inf (every weight exp2(s - inf) is 0 later
-// on) and delta = 0, so that whole tiles of statistics can be read without a bounds check.
+// works in) and delta = dO . O, both NEGATED: the backward kernels start their accumulators from -lse2 and -delta.
+// Rows are laid out [B*H][rows_padded], rows_padded a multiple of the 128-row query tile; rows beyond the sequence
+// receive -lse2 = -inf (every weight exp2(s - inf) is 0 later on) and -delta = 0, so that whole tiles of statistics
+// can be read without a bounds check.
 struct FlashStatsOut {
     const void* d_out;     // dO, laid out like Q and O
-    float* lse2;
-    float* delta;
+    float* neg_lse2;
+    float* neg_delta;
     int64_t rows_padded;
 };
 
@@ -595,8 +596,8 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
             if (half == 0 && qrow < q_tile0 + kFlashRows) {
                 const int64_t row = (int64_t)bh * st.rows_padded + qrow;
                 const bool live = qrow < L && l > 0.0f;
-                st.lse2[row] = live ? __builtin_log2f(l) - neg_m[0] : INFINITY;
-                st.delta[row] = live ? delta : 0.0f;
+                st.neg_lse2[row] = live ? neg_m[0] - __builtin_log2f(l) : -INFINITY;
+                st.neg_delta[row] = live ? -delta : 0.0f;
             }
         } else if (qrow < L) {
             T* dst = go + (int64_t)qrow * sn + 4 * half;
