@@ -7,7 +7,8 @@
 //   2. dQ          a workgroup owns query rows and walks the keys:  dS_ij = P_ij (dO_i.v_j - delta_i),
 //                  dQ_i = scale * sum_j dS_ij k_j,
 //   3. dK, dV      a workgroup owns key rows and walks the queries: dV_j = sum_i P_ij dO_i,
-//                  dK_j = scale * sum_i dS_ij q_i  (summed over the query heads of a K/V head).
+//                  dK_j = scale * sum_i dS_ij q_i  (summed over the query heads of a K/V head);
+//                  on the matrix cores at d = 128 as one walk for dV and one for dK (launch_dkv).
 // with P_ij = exp(scale q_i.k_j - lse_i).  Nothing is accumulated through atomics, so results do not depend
 // on launch order.  The statistics live in the caller's workspace: two floats per (sequence, head, row).
 #include <hip/hip_runtime.h>
