@@ -132,4 +132,12 @@ __device__ inline float swap_halves(float x) {
 
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Largest of three as ONE instruction (v_maximum3_f32).  fmaxf(a, fmaxf(b, c)) on values the compiler cannot
+// prove canonical (matrix-instruction results) puts a `v_max_f32 x, x, x` per input in front of the maximum
+// itself, three times the instructions in a chain over a tile's scores; the IEEE-754-2019 maximum needs none.
+// It propagates NaN where fmaxf drops it: the scores here are finite or -inf.
+__device__ inline float max3(float a, float b, float c) {
+    return __builtin_elementwise_maximum(__builtin_elementwise_maximum(a, b), c);
+}
+
 }  // namespace ahpc

@@ -476,7 +476,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
             //      it by more than kRaise (rare, and the only time the accumulators are rescaled) ------
             float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
-            for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
+            for (int r = 1; r < 16; ++r) mx = max3(mx, s[0][r], s[1][r]);
             bool adjust;
             if constexpr (MASKED) adjust = __builtin_amdgcn_ballot_w64(seen ? mx > kRaise : mx > -INFINITY) != 0;
             else adjust = first || __builtin_amdgcn_ballot_w64(mx > kRaise) != 0;

@@ -342,8 +342,8 @@ def bench_extras(hip, stream, steps, warmup):
         flops=2.0 * B * H * N * N * d)
 
     # backward at the headline shape.  FLOP by the usual convention: 2.5 x the forward's (five products
-    # against two); the three launches here execute nine, because the interface passes neither the forward
-    # output nor its softmax statistics and they are recomputed.
+    # against two); the four launches here execute ten, because the interface passes neither the forward
+    # output nor its softmax statistics and they are recomputed, and dK and dV each recompute the scores.
     go = randn((B, N, H, d), torch.bfloat16)
     gq, gk, gv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     wsb = hip.flash_bwd_workspace_bytes(B, N, H)
@@ -416,6 +416,26 @@ def bench_extras(hip, stream, steps, warmup):
         lambda: hip.kv_scatter_batch(k.data_ptr(), v.data_ptr(), hip.BF16, N * H * d, H * d, kpool.data_ptr(), vpool.data_ptr(),
                                      hip.BF16, table.data_ptr(), pages_per, rows_.data_ptr(), B, N, H, d, P, stream=stream),
         nbytes=4 * B * N * H * d * 2)
+
+    # Context, not product: what the vendor library's plain bf16 matrix product sustains on this box.  The board holds
+    # its power limit under matrix load and lowers the shader clock, so this, not the 2.4-GHz figure, is what a kernel
+    # that is nothing but matrix instructions reaches here.  Timed with torch's events on torch's stream.
+    M = 8192
+    a, b_ = randn((M, M), torch.bfloat16), randn((M, M), torch.bfloat16)
+    for _ in range(5):
+        torch.matmul(a, b_)
+    torch.cuda.synchronize()
+    reps = max(10, steps)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        torch.matmul(a, b_)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    rows.append({"workload": "context: torch.matmul bf16 8192x8192x8192 (hipBLASLt), not part of the product",
+                 "kernel_ms_mean": round(ms, 4), "TFLOP/s": round(2.0 * M ** 3 / (ms * 1e-3) / 1e12, 1),
+                 "frac_of_2.5_PFLOP/s": round(2.0 * M ** 3 / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)})
     return rows
 
 
