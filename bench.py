@@ -17,6 +17,10 @@ PagedAttention decode result (fp16, B=64, H=32, d=128, page 16, context lengths 
   extras           the other configurations (long-context decode, ragged prefill, backward, grouped heads,
                    batched append), one row each, timed in the same run
 
+`--workload calib` prints yardsticks of the box (device copy, streaming read, the vendor library's bf16 matrix product,
+matrix instructions only); `--workload sensors` prints the shader clock and board power the driver reports while the
+headline forward, that matrix product and a device copy each run back to back for a few seconds.
+
 Inputs of the two headline workloads come from the oracle's seeded generator (splitmix64 + Box-Muller, seeds
 0xA77E0002 / 0xA77E0003, tensor ids 1-5), rounded to the storage type on the host, so that the CPU legs and the
 GPU see the same values; the extras draw theirs with torch.randn on the GPU.
@@ -503,12 +507,85 @@ def run_calibration(steps):
     hip.load().ahpc_hip_stream_destroy(sp.value)
 
 
+def read_sensors():
+    """Shader clock and board power as the amdgpu driver reports them (read-only sysfs files; absent ones are left out)."""
+    import glob
+    out = {}
+    for dev in sorted(glob.glob("/sys/class/drm/card*/device")):
+        card = dev.split("/")[4]
+        try:
+            cur = [l for l in open(dev + "/pp_dpm_sclk").read().split("\n") if l.endswith("*")]
+            if cur:
+                out[card + ".sclk_mhz"] = int("".join(c for c in cur[0].split(":")[1] if c.isdigit()))
+        except (OSError, ValueError, IndexError):
+            pass
+        for hw in glob.glob(dev + "/hwmon/hwmon*"):
+            for name in ("power1_input", "power1_average", "power1_cap"):
+                try:
+                    out[card + "." + name + "_w"] = int(open(os.path.join(hw, name)).read()) / 1e6
+                except (OSError, ValueError):
+                    pass
+    return out
+
+
+def run_sensors(seconds):
+    """Clock and power while a workload runs back to back: the headline forward, the vendor library's bf16 matrix product,
+    a device copy.  One thread launches, this one reads the sensors every 0.3 s (after a second of settling)."""
+    import threading
+    import torch
+    from attention_amd import hip
+    c = FLASH
+    B, N, H, d = c["B"], c["N"], c["H"], c["d"]
+    q = torch.randn((B, N, H, d), device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    k, v, o = torch.randn_like(q), torch.randn_like(q), torch.empty_like(q)
+    a = torch.randn((8192, 8192), device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    b = torch.randn_like(a)
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    st = (N * H * d, H * d, d)
+    work = [
+        ("flash_fwd bf16 causal B=4 N=4096 H=32 d=128",
+         lambda: hip.flash_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), hip.BF16, B, N, H, d, st, 1.0 / np.sqrt(d), True, None)),
+        ("torch.matmul bf16 8192^3", lambda: torch.matmul(a, b)),
+        ("1 GiB device copy", lambda: dst.copy_(src)),
+    ]
+    print(json.dumps({"workload": "idle", "sensors": read_sensors()}))
+    for name, launch in work:
+        done = threading.Event()
+        res = {}
+
+        def loop():
+            launch()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            n = 0
+            while time.perf_counter() - t0 < seconds:
+                for _ in range(50):
+                    launch()
+                torch.cuda.synchronize()
+                n += 50
+            res["ms_per_launch"] = round((time.perf_counter() - t0) / n * 1e3, 4)
+            done.set()
+        th = threading.Thread(target=loop)
+        th.start()
+        time.sleep(1.0)
+        samples = []
+        while not done.is_set():
+            samples.append(read_sensors())
+            time.sleep(0.3)
+        th.join()
+        keys = sorted({kk for smp in samples for kk in smp})
+        print(json.dumps({"workload": name, "ms_per_launch": res.get("ms_per_launch"), "samples": len(samples),
+                          "sensors_min_max": {kk: [min(smp[kk] for smp in samples if kk in smp), max(smp[kk] for smp in samples if kk in smp)]
+                                              for kk in keys}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", choices=["all", "flash", "decode", "calib", "extras"], default="all")
+    ap.add_argument("--workload", choices=["all", "flash", "decode", "calib", "extras", "sensors"], default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline (profiling runs)")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -521,6 +598,9 @@ def main():
         sys.exit("bench.py: no GPU visible")
     if a.workload == "calib":
         run_calibration(a.steps)
+        return
+    if a.workload == "sensors":
+        run_sensors(5.0)
         return
     import ctypes as C
     s = C.c_void_p()
