@@ -8,6 +8,8 @@ PagedAttention decode result (fp16, B=64, H=32, d=128, page 16, context lengths 
 
   value            whole-job throughput: algorithmic FLOP (2*B*H*N^2*d for causal) / wall time of the
                    K timed steps, bracketed by a device synchronize on both sides
+  settle_ms        untimed launches of the same workload for that long in front of the W warm-up steps: the board's
+                   clocks come out of idle over tens of milliseconds, whatever W is (see settle())
   roofline         algorithmic FLOP (or bytes) per launch / mean kernel duration measured with HIP
                    events on the launch stream, against MI355X's dense bf16 MFMA peak (2.5 PFLOP/s)
                    or HBM peak (8 TB/s)
@@ -124,11 +126,31 @@ class Timer:
             self.lib.ahpc_hip_event_destroy(e)
 
 
+SETTLE_MS = 60.0  # untimed launches in front of every workload's warm-up, see settle()
+
+
+def settle(hip, stream, launch):
+    """Untimed launches for SETTLE_MS of wall clock (at most 400), in front of the W warm-up steps.  The board comes out
+    of idle at a low shader clock and its power management needs some tens of milliseconds of load to arrive where it
+    stays: the first 25 launches of the headline forward after idle average 0.61 ms, the next 25 0.58 ms, those after
+    the first 50 0.52 ms, as do those after 1000.  W is the caller's; this phase makes what follows independent of it."""
+    lib = hip.load()
+    t0 = time.perf_counter()
+    n = 0
+    while n < 400 and (time.perf_counter() - t0) * 1e3 < SETTLE_MS:
+        for _ in range(10):
+            launch()
+        assert lib.ahpc_hip_stream_synchronize(stream) == 0
+        n += 10
+    return n
+
+
 def timed_steps(hip, stream, launch, steps, warmup):
-    """W untimed launches, then exactly K timed ones: wall clock around all K (synchronised on both
-    sides) and an event pair around each launch."""
+    """Settling launches (see settle), W untimed launches, then exactly K timed ones: wall clock around all K
+    (synchronised on both sides) and an event pair around each launch."""
     import torch
     lib = hip.load()
+    settle(hip, stream, launch)
     for _ in range(warmup):
         launch()
     assert lib.ahpc_hip_stream_synchronize(stream) == 0
@@ -581,13 +603,17 @@ def run_sensors(seconds):
 
 
 def main():
+    global SETTLE_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", choices=["all", "flash", "decode", "calib", "extras", "sensors"], default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline (profiling runs)")
+    ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
+                    help="untimed launches for this long in front of each workload's warm-up (0: none, for counter runs)")
     a = ap.parse_args()
+    SETTLE_MS = a.settle_ms
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (both paths shard by head or sequence without communication); "
                  f"--gpus {a.gpus} is not supported")
@@ -611,8 +637,8 @@ def main():
         print(json.dumps({"extras": bench_extras(hip, stream, a.steps, a.warmup)}))
         hip.load().ahpc_hip_stream_destroy(stream)
         return
-    out = {"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "higher_is_better": True, "scaling": "weak",
-           "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
+    out = {"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "settle_ms": SETTLE_MS, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
     flash = bench_flash(hip, stream, a.steps, a.warmup, not a.no_cpu) if a.workload in ("all", "flash") else None
     decode = bench_decode(hip, stream, a.steps, a.warmup, not a.no_cpu) if a.workload in ("all", "decode") else None
     head = flash or decode
