@@ -50,6 +50,7 @@ template <> struct Storage<bf16_t> {
 // Bit pattern -> fp32.  Takes the dword BY VALUE on purpose: __builtin_bit_cast applied directly to
 // an element of an ext-vector (v[i]) reads element 0 whatever i is with this compiler.
 __device__ inline float as_f32(uint32_t w) { return __builtin_bit_cast(float, w); }
+__device__ inline uint32_t as_u32(float x) { return __builtin_bit_cast(uint32_t, x); }
 
 // Packs two fp32 into one dword of two 16-bit values (low half = a).
 template <typename T> __device__ inline uint32_t pack2(float a, float b);

@@ -3,6 +3,7 @@
 
 #include <cmath>
 #include <cstdlib>
+#include <mutex>
 
 #include "ahpc_device.hpp"
 #include "flash_fwd_mfma.hpp"
@@ -160,20 +161,112 @@ static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream
     return static_cast<int>(hipGetLastError());
 }
 
-template <typename T, int D>
+template <typename T, int D, int MASK>
 static int launch_mfma_masked(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
     if (int rc = flash_plan_launch(p, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load(), false)) return rc;
     dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
-    if (causal) hipLaunchKernelGGL((flash_fwd_mfma_masked_kernel<T, D, true>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((flash_fwd_mfma_masked_kernel<T, D, false>), grid, block, 0, stream, p);
+    if (causal) hipLaunchKernelGGL((flash_fwd_mfma_masked_kernel<T, D, true, MASK>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((flash_fwd_mfma_masked_kernel<T, D, false, MASK>), grid, block, 0, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 
-template <typename T>
+template <typename T, int MASK>
 static int dispatch_mfma_masked(const FlashParams& p, int64_t B, int d, bool causal, hipStream_t stream) {
-    if (d == 128) return launch_mfma_masked<T, 128>(p, B, causal, stream);
-    if (d == 64) return launch_mfma_masked<T, 64>(p, B, causal, stream);
+    if (d == 128) return launch_mfma_masked<T, 128, MASK>(p, B, causal, stream);
+    if (d == 64) return launch_mfma_masked<T, 64, MASK>(p, B, causal, stream);
     return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+}
+
+// Packs a dense fp32 mask [B,N,N] into one bit per (query, key): word [(b * n_kt + tile) * N + query] holds the 64
+// keys of the tile, bit j set = mask[b][query][64 * tile + j] != 0 (keys at or beyond N: clear).  A wavefront takes
+// 64 queries x 64 keys: per query one coalesced 256-byte read and a ballot; lane r keeps the word of query r, and the
+// 64 words leave as one coalesced 512-byte store.  Consecutive wavefronts take consecutive tiles of the same queries.
+constexpr int kMaskPackThreads = 256;
+__global__ __launch_bounds__(kMaskPackThreads) void flash_mask_pack_kernel(const float* __restrict__ mask, uint64_t* __restrict__ bits,
+                                                                            int N, int n_kt, int n_rb, int64_t n_units) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t unit = (int64_t)blockIdx.x * (kMaskPackThreads / kWave) + (threadIdx.x >> 6);
+    if (unit >= n_units) return;
+    const int kt = (int)(unit % n_kt);
+    const int rb = (int)((unit / n_kt) % n_rb);
+    const int b = (int)(unit / ((int64_t)n_kt * n_rb));
+    const int key = 64 * kt + lane;
+    const float* const src = mask + (int64_t)b * N * N + (key < N ? key : 0);
+    uint64_t mine = 0;
+#pragma unroll 8
+    for (int r = 0; r < 64; ++r) {
+        const int row = 64 * rb + r;
+        const float m = (row < N && key < N) ? src[(int64_t)row * N] : 0.0f;
+        const uint64_t word = __builtin_amdgcn_ballot_w64(m != 0.0f);
+        if (lane == r) mine = word;
+    }
+    const int row = 64 * rb + lane;
+    if (row < N) bits[((int64_t)b * n_kt + kt) * N + row] = mine;
+}
+
+// The packed copy of a mask lives in device memory that the library owns: one buffer per device, grown on demand and kept
+// until the process ends (B * N * ceil(N / 64) * 8 bytes: an eighth of a byte per mask element).  Calls on one device
+// share it: `done` is recorded behind the launch that reads it, and the next call's stream waits for it before the
+// buffer is overwritten; the mutex covers the whole of that.
+struct MaskScratch {
+    std::mutex mu;
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    hipEvent_t done = nullptr;
+};
+constexpr int kMaxDevices = 64;
+constexpr size_t kMaskScratchLimit = size_t(1) << 30;  // larger masks are read in place
+static MaskScratch g_mask_scratch[kMaxDevices];
+
+// Packs `mask` and launches the matrix-core kernel on the packed copy.  AHPC_OK + *launched = false: not possible here
+// (stream under capture, no memory, mask too large), nothing was launched and the caller reads the mask in place.
+template <typename T>
+static int forward_on_packed_mask(FlashParams p, const float* mask, int64_t B, int d, bool causal, hipStream_t stream,
+                                  bool* launched) {
+    *launched = false;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return AHPC_OK;  // allocation and cross-stream waits do not belong into a captured graph
+    }
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return AHPC_OK;
+    const int64_t N = p.N, n_kt = (N + 63) / 64, n_rb = (N + 63) / 64;
+    const size_t need = (size_t)B * (size_t)n_kt * (size_t)N * sizeof(uint64_t);
+    if (need > kMaskScratchLimit) return AHPC_OK;
+    MaskScratch& sc = g_mask_scratch[dev];
+    std::lock_guard<std::mutex> lock(sc.mu);
+    if (!sc.done && hipEventCreateWithFlags(&sc.done, hipEventDisableTiming) != hipSuccess) {
+        sc.done = nullptr;
+        (void)hipGetLastError();
+        return AHPC_OK;
+    }
+    if (need > sc.bytes) {
+        if (hipError_t e = hipEventSynchronize(sc.done); e != hipSuccess) return static_cast<int>(e);  // the old buffer's last reader
+        if (sc.ptr) (void)hipFree(sc.ptr);
+        sc.ptr = nullptr;
+        sc.bytes = 0;
+        if (hipMalloc(&sc.ptr, need) != hipSuccess) {
+            sc.ptr = nullptr;
+            (void)hipGetLastError();
+            return AHPC_OK;
+        }
+        sc.bytes = need;
+    }
+    if (hipError_t e = hipStreamWaitEvent(stream, sc.done, 0); e != hipSuccess) return static_cast<int>(e);
+    const int64_t n_units = B * n_rb * n_kt;
+    const int64_t blocks = (n_units + kMaskPackThreads / kWave - 1) / (kMaskPackThreads / kWave);
+    if (blocks > 0x7FFFFFFFll) return AHPC_OK;
+    hipLaunchKernelGGL(flash_mask_pack_kernel, dim3((unsigned)blocks), dim3(kMaskPackThreads), 0, stream, mask,
+                       static_cast<uint64_t*>(sc.ptr), (int)N, (int)n_kt, (int)n_rb, n_units);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return static_cast<int>(e);
+    p.mask = nullptr;
+    p.mask_bits = static_cast<const uint64_t*>(sc.ptr);
+    p.mask_kt = (int32_t)n_kt;
+    *launched = true;
+    const int rc = dispatch_mfma_masked<T, 2>(p, B, d, causal, stream);
+    const hipError_t e = hipEventRecord(sc.done, stream);
+    return rc != AHPC_OK ? rc : static_cast<int>(e);
 }
 
 template <typename T, bool VARLEN>
@@ -226,9 +319,7 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
     if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int32_t group = (int32_t)(H / H_kv);
-    // a mask row is read 16 bytes at a time on the matrix-core kernel: rows of a multiple of 4 floats, aligned base
-    const bool mask_ok = !mask || (N % 4 == 0 && aligned16(mask));
-    if (mask_ok && mfma_eligible(dtype, d, q, k, v, o, sq, skv)) {
+    if (mfma_eligible(dtype, d, q, k, v, o, sq, skv)) {
         FlashParams p{};
         p.q = q; p.k = k; p.v = v; p.o = o;
         p.mask = mask;
@@ -236,11 +327,21 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
         p.kv_stride_b = skv.b; p.kv_stride_n = skv.n; p.kv_stride_h = skv.h;
         p.N = (int32_t)N; p.H = (int32_t)H; p.kv_group = group;
         p.scale_log2 = scale * kLog2e;
-        if (mask)
-            return dtype == AHPC_F16 ? dispatch_mfma_masked<f16_t>(p, B, (int)d, causal != 0, st)
-                                     : dispatch_mfma_masked<bf16_t>(p, B, (int)d, causal != 0, st);
-        return dtype == AHPC_F16 ? dispatch_mfma<f16_t, false>(p, B, (int)d, causal != 0, st)
-                                 : dispatch_mfma<bf16_t, false>(p, B, (int)d, causal != 0, st);
+        if (!mask)
+            return dtype == AHPC_F16 ? dispatch_mfma<f16_t, false>(p, B, (int)d, causal != 0, st)
+                                     : dispatch_mfma<bf16_t, false>(p, B, (int)d, causal != 0, st);
+        // The mask, by preference, as a packed copy made in front of the launch (every head reads the mask: packed, a
+        // sixteenth of the bytes).  Where that is not possible, or switched off, the kernel reads the mask in place,
+        // 16 bytes at a time: rows of a multiple of 4 floats and an aligned base; everything else takes the kernel below.
+        if (tuning().mask_pack.load() != 0) {
+            bool launched = false;
+            const int rc = dtype == AHPC_F16 ? forward_on_packed_mask<f16_t>(p, mask, B, (int)d, causal != 0, st, &launched)
+                                             : forward_on_packed_mask<bf16_t>(p, mask, B, (int)d, causal != 0, st, &launched);
+            if (launched || rc != AHPC_OK) return rc;
+        }
+        if (N % 4 == 0 && aligned16(mask))
+            return dtype == AHPC_F16 ? dispatch_mfma_masked<f16_t, 1>(p, B, (int)d, causal != 0, st)
+                                     : dispatch_mfma_masked<bf16_t, 1>(p, B, (int)d, causal != 0, st);
     }
     SimpleParams p{q, k, v, o, nullptr, mask, sq.b, sq.n, sq.h, skv.b, skv.n, skv.h, (int32_t)N, (int32_t)H, (int32_t)d, group, scale, causal ? 1 : 0};
     return dispatch_simple<false>(dtype, p, B, st);

@@ -52,6 +52,9 @@ struct FlashParams {
     void* o;
     const int32_t* cu_seqlens;  // ragged batches only
     const float* mask;          // masked kernel only: fp32 [B,N,N], shared by all heads; 0.0f removes the key for the query
+    const uint64_t* mask_bits;  // masked kernel on a packed mask: word [(b * mask_kt + key tile) * N + query] holds the 64 keys
+                                // of the tile, bit j set = key 64 * tile + j stays (flash_mask_pack_kernel writes it)
+    int32_t mask_kt;            // key tiles per row of the packed mask: ceil(N / 64)
     int64_t stride_b, stride_n, stride_h;           // Q and O
     int64_t kv_stride_b, kv_stride_n, kv_stride_h;  // K and V
     int32_t N;                  // sequence length (dense) / longest sequence (ragged)
@@ -253,13 +256,18 @@ struct FlashStatsOut {
     int64_t rows_padded;
 };
 
-// MASKED: a dense fp32 mask [B,N,N] removes keys per query (0.0f = removed; FlashAttention::apply_attention_mask,
-// src/algorithms/flash_attention.cpp:596-607).  A lane's 32 scores of a tile are 8 runs of 4 consecutive keys of
-// its query: 8 16-byte loads of the mask row (N is a multiple of 4 then, the host checks).  Any query may then see
-// its first key in any tile, or none at all (zeros come out), so the reference maximum is set per query when its
-// first key shows up.
-template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS, bool MASKED = false>
+// MASK != 0: a dense fp32 mask [B,N,N] removes keys per query (0.0f = removed; FlashAttention::apply_attention_mask,
+// src/algorithms/flash_attention.cpp:596-607).  Any query may then see its first key in any tile, or none at all
+// (zeros come out), so the reference maximum is set per query when its first key shows up.
+//   MASK == 1: the kernel reads the caller's mask.  A lane's 32 scores of a tile are 8 runs of 4 consecutive keys of
+//              its query: 8 16-byte loads of the mask row (N is a multiple of 4 then, the host checks).  Every head
+//              reads the whole mask again: as many bytes through L2 as K and V together.
+//   MASK == 2: the kernel reads one 64-bit word per query and tile of a packed copy (flash_mask_pack_kernel made it
+//              in front of this launch): a sixteenth of the bytes, one load instead of eight, two registers
+//              instead of 32.
+template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS, int MASK = 0>
 __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const FlashStatsOut& st) {
+    constexpr bool MASKED = MASK != 0;
     static_assert(!(MASKED && (VARLEN || STATS)), "the mask belongs to dense forward launches");
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;  // k-steps of the first product
@@ -400,7 +408,8 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
         bool first = true;
         bool seen = false;  // masked launches: this lane's query has met a key it may attend to
         constexpr float kRaise = 8.0f;  // raise the reference maximum only when exceeded by 2^8
-        const float* const mrow = MASKED ? p.mask + ((int64_t)b * p.N + (qrow < L ? qrow : L - 1)) * p.N : nullptr;
+        const float* const mrow = MASK == 1 ? p.mask + ((int64_t)b * p.N + (qrow < L ? qrow : L - 1)) * p.N : nullptr;
+        const uint64_t* const mword = MASK == 2 ? p.mask_bits + (int64_t)b * p.mask_kt * p.N + (qrow < L ? qrow : L - 1) : nullptr;
 
         // The mask values of this lane's 32 scores of the tile at k0.  A run that starts behind the row's end reads
         // the row's last four values instead: its keys do not exist and are removed by the end-of-sequence test.
@@ -414,7 +423,8 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                 }
         };
 
-        auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int k0, const f32x4 (&mk)[2][4]) {
+        auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int k0, const f32x4 (&mk)[2][4],
+                                uint64_t mw) {
             // ---- S^T = c*K Q^T - m  (log2 units).  The two 32-key blocks alternate, kAhead operand
             //      pairs are requested before the first product and one more after every two products.
             f32x16 s[2];
@@ -466,11 +476,26 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                         s[kb][r] = off <= lim ? s[kb][r] : -INFINITY;
                     }
             }
-            if constexpr (MASKED) {
+            if constexpr (MASK == 1) {
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) s[kb][r] = mk[kb][r >> 2][r & 3] == 0.0f ? -INFINITY : s[kb][r];
+            }
+            if constexpr (MASK == 2) {
+                // the lane's keys of the tile are 4 * half + 32 * kb + 8 * (r / 4) + r % 4: one shift brings them to
+                // fixed places of two 32-bit words; a bit spread over a word (all ones: keep) selects between the
+                // score and -inf
+                const uint64_t w = mw >> (4 * half);
+                const uint32_t word[2] = {(uint32_t)w, (uint32_t)(w >> 32)};
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int pos = 8 * (r >> 2) + (r & 3);
+                        const uint32_t keep = (uint32_t)((int32_t)(word[kb] << (31 - pos)) >> 31);
+                        s[kb][r] = as_f32((as_u32(s[kb][r]) & keep) | (0xFF800000u & ~keep));
+                    }
             }
             // ---- reference maximum: exact on the first tile, afterwards raised only when a score tops
             //      it by more than kRaise (rare, and the only time the accumulators are rescaled) ------
@@ -549,18 +574,20 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
             const int k0 = t * kFlashKeys;
             const bool more = t + 1 < n_tiles;
             f32x4 mk[2][4];
+            uint64_t mw = 0;
             if constexpr (MASKED) {
                 // The mask is requested BEFORE the next tile (loads complete in order: waiting for a load issued
                 // behind the tile's would wait for the tile), and the tile is requested even behind the last one
                 // (an empty request), so that the compiler counts the same loads in flight on every path.
-                load_mask(mk, k0);
+                if constexpr (MASK == 1) load_mask(mk, k0);
+                else mw = mword[(int64_t)t * p.N];
                 __builtin_amdgcn_sched_barrier(0);
                 dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
             } else {
                 if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
             }
             // a wavefront whose queries all precede this tile has nothing to add
-            if (!(CAUSAL && k0 > qw + 31)) compute_tile(cur_k, cur_v, k0, mk);
+            if (!(CAUSAL && k0 > qw + 31)) compute_tile(cur_k, cur_v, k0, mk, mw);
             if (MASKED || more) {
                 __builtin_amdgcn_s_waitcnt(0);  // this wave's part of the next tile has landed
                 __syncthreads();                // everyone's has, and everyone is done with the current one
@@ -644,10 +671,10 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const 
     flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, false>(p, FlashStatsOut{});
 }
 
-// Dense launches with a mask [B,N,N].
-template <typename T, int D, bool CAUSAL>
+// Dense launches with a mask [B,N,N]: MASK 1 reads the caller's fp32 mask, MASK 2 its packed copy.
+template <typename T, int D, bool CAUSAL, int MASK>
 __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_masked_kernel(const FlashParams p) {
-    flash_fwd_mfma_body<T, D, CAUSAL, false, false, true>(p, FlashStatsOut{});
+    flash_fwd_mfma_body<T, D, CAUSAL, false, false, MASK>(p, FlashStatsOut{});
 }
 
 // The forward pass with its output kept in registers: writes the softmax statistics the backward needs.

@@ -25,6 +25,10 @@ struct Tuning {
     // backward: dK and dV in one walk over the query tiles (1), in two (2), or by head dimension (0, the default:
     // two at d = 128).  (AHPC_BWD_SPLIT)
     std::atomic<int64_t> bwd_split;
+    // forward with a dense mask on the matrix-core kernel: 1 (default) = the mask is packed to one bit per element in
+    // front of the launch, into device memory the library keeps; 0 = the kernel reads the caller's fp32 mask in place
+    // (what a stream under graph capture gets in any case).  (AHPC_MASK_PACK)
+    std::atomic<int64_t> mask_pack;
     Tuning();
 };
 

@@ -67,9 +67,9 @@ typedef struct ahpc_device_info {
     int32_t  runtime_version;
 } ahpc_device_info;
 
-/* Launcher tuning values ("flash_pair_min_tiles", "decode_waves", "decode_chunk", "decode_matrix_min_group", "bwd_split"):
- * process-wide, each starts from its environment variable (AHPC_FLASH_PAIR_MIN, AHPC_DECODE_WAVES, AHPC_DECODE_CHUNK,
- * AHPC_DECODE_MFMA_MIN_GROUP, AHPC_BWD_SPLIT), which is read once.  No value
+/* Launcher tuning values ("flash_pair_min_tiles", "decode_waves", "decode_chunk", "decode_matrix_min_group", "bwd_split",
+ * "mask_pack"): process-wide, each starts from its environment variable (AHPC_FLASH_PAIR_MIN, AHPC_DECODE_WAVES,
+ * AHPC_DECODE_CHUNK, AHPC_DECODE_MFMA_MIN_GROUP, AHPC_BWD_SPLIT, AHPC_MASK_PACK), which is read once.  No value
  * changes results; unknown names and negative values are refused.  The reference has no counterpart: its tile sizes
  * sit in PerformanceConfig (src/api/attention_interface.hpp:29-53), which the host classes still honour. */
 int ahpc_hip_set_tuning(const char* name, int64_t value);
@@ -131,10 +131,15 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
 
 /* Same with a dense fp32 mask [B,N,N] shared by all heads, 0.0f removes the key
  * (FlashAttention::apply_attention_mask, src/algorithms/flash_attention.cpp:596-607;
- * indexing :432-435).  A query whose keys are all removed gets a zero output row.  fp16/bf16 with d in {64, 128},
- * N a multiple of 4 and a 16-byte aligned mask run on the matrix-core kernel (the mask row is read 16 bytes at a
- * time), everything else on the fp32-FMA kernel.  mask may be NULL: then the fp32-FMA kernel runs whatever the
- * type (the way to ask for it). */
+ * indexing :432-435).  A query whose keys are all removed gets a zero output row.  fp16/bf16 with d in {64, 128}
+ * run on the matrix-core kernel, everything else on the fp32-FMA kernel.  The matrix-core kernel reads a packed copy
+ * of the mask (one bit per element) that a small kernel writes in front of it, into device memory the LIBRARY owns:
+ * one buffer per device, grown on demand (hipMalloc; B * N * ceil(N / 64) * 8 bytes, at most 1 GiB) and kept until the
+ * process ends; calls on one device share it and are ordered through an event, on whatever streams they run.  A
+ * stream under graph capture, a larger mask, a failed allocation or the tuning value mask_pack = 0 make the kernel read
+ * the mask in place instead (N a multiple of 4 and a 16-byte aligned mask; otherwise the fp32-FMA kernel): no
+ * allocation, more traffic.  mask may be NULL: then the fp32-FMA kernel runs whatever the type (the way to ask for
+ * it). */
 int ahpc_hip_flash_fwd_masked(const void* q, const void* k, const void* v, void* o, int dtype,
                               int64_t B, int64_t N, int64_t H, int64_t d,
                               int64_t stride_b, int64_t stride_n, int64_t stride_h,

@@ -93,12 +93,22 @@ def test_dense_mask_fp32(gpu):
     assert np.all(got[1, 3] == 0.0)
 
 
+@pytest.fixture(params=[1, 0], ids=["packed-copy", "mask-in-place"])
+def mask_path(gpu, request):
+    """The matrix-core kernel takes a dense mask as a packed copy made in front of the launch (any N) or reads it in
+    place (N a multiple of 4; other lengths go to the fp32-FMA kernel then): the tuning value decides, both are run."""
+    before = gpu.get_tuning("mask_pack")
+    gpu.set_tuning("mask_pack", request.param)
+    yield request.param
+    gpu.set_tuning("mask_pack", before)
+
+
 @pytest.mark.parametrize("dtype,d", [(O.F16, 128), (O.BF16, 64), (O.BF16, 128)])
 @pytest.mark.parametrize("causal", [False, True])
-@pytest.mark.parametrize("N", [4, 64, 132, 520, 1028, 517])
-def test_dense_mask_16bit(gpu, dtype, d, causal, N):
-    """16-bit inputs with a mask [B,N,N]: the matrix-core kernel when N is a multiple of 4 (517: the fp32-FMA kernel).
-    Rows that see nothing (zeros), a single key, or nothing before the last key tile."""
+@pytest.mark.parametrize("N", [4, 64, 132, 520, 1028, 517, 63, 129])
+def test_dense_mask_16bit(gpu, dtype, d, causal, N, mask_path):
+    """16-bit inputs with a mask [B,N,N].  Rows that see nothing (zeros), a single key, or nothing before the last key
+    tile; sequence ends inside a 64-bit mask word, on its edge and one behind it."""
     B, H = 2, 3
     q, k, v = make_qkv((B, N, H, d), 6, dtype)
     mask = (O.fill_uniform((B, N, N), 6, 6) > 0.3).astype(np.float32)
@@ -117,7 +127,7 @@ def test_dense_mask_16bit(gpu, dtype, d, causal, N):
     assert np.abs(got - want).max() <= 2e-2
 
 
-def test_dense_mask_full_size_properties(gpu):
+def test_dense_mask_full_size_properties(gpu, mask_path):
     """B=2 N=4096 H=8 d=128 bf16 with a mask: (1) an all-ones mask reproduces the unmasked launch bit for bit;
     (2) a lower-triangular mask reproduces the causal launch within rounding (the same keys, the reference maximum set
     by another rule); (3) sampled rows of a random mask against the oracle."""
@@ -152,6 +162,36 @@ def test_dense_mask_full_size_properties(gpu):
         w = np.exp(s - s.max())
         want = (w[:, None] * vh[b, :, h]).sum(0) / w.sum()
         assert np.abs(got[b, n, h].float().cpu().numpy() - want).max() <= 2e-2, (b, h, n)
+
+
+def test_dense_mask_packed_copy_shared_between_streams_and_sizes(gpu):
+    """The packed copy of the mask is one buffer per device: launches with different masks on two streams, queued without
+    a synchronisation in between and with the sizes growing (the buffer is replaced while earlier launches may still run),
+    each give their own result."""
+    import torch
+    from gpu_util import to_dev, to_host
+    H, d = 2, 128
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    jobs = []
+    for i, N in enumerate([64, 200, 132, 520, 260, 1028]):
+        B = 1 + i % 2
+        q, k, v = make_qkv((B, N, H, d), 70 + i, O.BF16)
+        mask = (O.fill_uniform((B, N, N), 70 + i, 6) > (-0.5 + 0.2 * i)).astype(np.float32)
+        mask[:, np.arange(N), np.arange(N)] = 1.0
+        dq, dk, dv = to_dev(q, O.BF16), to_dev(k, O.BF16), to_dev(v, O.BF16)
+        dm = torch.from_numpy(mask).cuda()
+        do = torch.full_like(dq, float("nan"))
+        jobs.append((B, N, q, k, v, mask, dq, dk, dv, dm, do))
+    torch.cuda.synchronize()
+    for rep in range(3):
+        for i, (B, N, q, k, v, mask, dq, dk, dv, dm, do) in enumerate(jobs):
+            st = streams[(i + rep) % 2]
+            gpu.flash_fwd(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), do.data_ptr(), O.BF16, B, N, H, d, (N * H * d, H * d, d),
+                          1.0 / np.sqrt(d), False, st.cuda_stream, dm.data_ptr())
+    torch.cuda.synchronize()
+    for B, N, q, k, v, mask, dq, dk, dv, dm, do in jobs:
+        want = O.attention(q, k, v, B, N, H, d, 1.0 / np.sqrt(d), False, mask=mask)
+        assert np.abs(to_host(do) - want).max() <= 2e-2, N
 
 
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16])

@@ -65,11 +65,16 @@ def test_fp32_kernel_dense_mask(emu):
 
 
 @pytest.mark.parametrize("dma_late", [False, True])
+@pytest.mark.parametrize("packed", [1, 0], ids=["packed-copy", "mask-in-place"])
 @pytest.mark.parametrize("dtype,N,d,causal,H_kv", [(O.BF16, 64, 128, False, 2), (O.F16, 132, 128, True, 2), (O.F16, 300, 64, False, 1),
-                                                   (O.BF16, 200, 64, True, 2), (O.BF16, 4, 128, False, 2)])
-def test_matrix_core_kernel_dense_mask(emu, dtype, N, d, causal, H_kv, dma_late):
-    """fp16/bf16 with a mask [B,N,N] run on the matrix cores (N a multiple of 4): a row that sees nothing gives zeros, a
-    row whose first visible key lies in the last tile, rows that see a single key, a last tile of 4 to 60 keys."""
+                                                   (O.BF16, 200, 64, True, 2), (O.BF16, 4, 128, False, 2), (O.F16, 131, 128, False, 1),
+                                                   (O.BF16, 65, 64, True, 2)])
+def test_matrix_core_kernel_dense_mask(emu, dtype, N, d, causal, H_kv, dma_late, packed):
+    """fp16/bf16 with a mask [B,N,N] run on the matrix cores, on a packed copy of the mask (any N) or on the mask in place
+    (N a multiple of 4): a row that sees nothing gives zeros, a row whose first visible key lies in the last tile, rows
+    that see a single key, a last tile of 1 to 60 keys."""
+    if not packed and N % 4:
+        pytest.skip("the mask is read in place 16 bytes at a time: other lengths take the fp32 kernel")
     B, H = 2, 2
     q, k, v = qkv((B, N, H, d), 17, dtype)
     k, v = k[:, :, :H_kv].copy(), v[:, :, :H_kv].copy()
@@ -83,10 +88,13 @@ def test_matrix_core_kernel_dense_mask(emu, dtype, N, d, causal, H_kv, dma_late)
         mask[0, N - 2, :N - 3] = 0.0  # nothing before the last tile
     scale = 1.0 / np.sqrt(d)
     S.configure(dma_late, seed=N + d)
+    before = emu.get_tuning("mask_pack")
+    emu.set_tuning("mask_pack", packed)
     try:
         got = flash(emu, q, k, v, dtype, B, N, H, d, scale, causal, H_kv=H_kv, mask=mask, front=dma_late)
     finally:
         S.configure(False, 1)
+        emu.set_tuning("mask_pack", before)
     rep = H // H_kv   # grouped heads = the same K/V head repeated
     want = O.attention(q, np.repeat(k, rep, axis=2), np.repeat(v, rep, axis=2), B, N, H, d, scale, causal, mask=mask)
     assert np.isfinite(got).all()
