@@ -7,6 +7,7 @@
 
 #include "ahpc_device.hpp"
 #include "flash_fwd_mfma.hpp"
+#include "flash_fwd_f32_mfma.hpp"
 #include "tuning.hpp"
 
 namespace ahpc {
@@ -218,11 +219,11 @@ constexpr int kMaxDevices = 64;
 constexpr size_t kMaskScratchLimit = size_t(1) << 30;  // larger masks are read in place
 static MaskScratch g_mask_scratch[kMaxDevices];
 
-// Packs `mask` and launches the matrix-core kernel on the packed copy.  AHPC_OK + *launched = false: not possible here
+// Packs `mask` and launches a matrix-core kernel (launch_on_bits) on the packed copy.  AHPC_OK + *launched = false: not possible here
 // (stream under capture, no memory, mask too large), nothing was launched and the caller reads the mask in place.
-template <typename T>
-static int forward_on_packed_mask(FlashParams p, const float* mask, int64_t B, int d, bool causal, hipStream_t stream,
-                                  bool* launched) {
+template <typename Launch>
+static int forward_on_packed_mask(FlashParams p, const float* mask, int64_t B, hipStream_t stream, bool* launched,
+                                  Launch launch_on_bits) {
     *launched = false;
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
@@ -264,7 +265,7 @@ static int forward_on_packed_mask(FlashParams p, const float* mask, int64_t B, i
     p.mask_bits = static_cast<const uint64_t*>(sc.ptr);
     p.mask_kt = (int32_t)n_kt;
     *launched = true;
-    const int rc = dispatch_mfma_masked<T, 2>(p, B, d, causal, stream);
+    const int rc = launch_on_bits(p);
     const hipError_t e = hipEventRecord(sc.done, stream);
     return rc != AHPC_OK ? rc : static_cast<int>(e);
 }
@@ -290,6 +291,30 @@ static bool mfma_eligible(int dtype, int64_t d, const void* q, const void* k, co
     if ((sq.b % 8) || (sq.n % 8) || (sq.h % 8) || (skv.b % 8) || (skv.n % 8) || (skv.h % 8)) return false;
     // a key tile is addressed with 32-bit byte offsets from its first row, and rows must not overlap
     return sq.n >= d && skv.n >= d && skv.n < (int64_t(1) << 24);
+}
+
+// fp32 tensors on the matrix cores: d 64 or 128, 16-byte aligned rows, no dense mask.
+static bool f32_mfma_eligible(int dtype, int64_t d, const void* q, const void* k, const void* v, const void* o,
+                              const Strides& sq, const Strides& skv) {
+    if (dtype != AHPC_F32 || (d != 64 && d != 128)) return false;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return false;
+    if ((sq.b % 4) || (sq.n % 4) || (sq.h % 4) || (skv.b % 4) || (skv.n % 4) || (skv.h % 4)) return false;
+    // a key tile is addressed with 32-bit byte offsets from its first row, and rows must not overlap
+    return sq.n >= d && skv.n >= d && skv.n < (int64_t(1) << 24);
+}
+
+template <bool VARLEN, bool MASKED>
+static int launch_f32_mfma(FlashParams p, int64_t B, int d, bool causal, hipStream_t stream) {
+    if (int rc = flash_plan_launch(p, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load(), VARLEN)) return rc;
+    dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
+    if (d == 128) {
+        if (causal) hipLaunchKernelGGL((flash_fwd_f32_mfma_kernel<128, true, VARLEN, MASKED>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((flash_fwd_f32_mfma_kernel<128, false, VARLEN, MASKED>), grid, block, 0, stream, p);
+    } else {
+        if (causal) hipLaunchKernelGGL((flash_fwd_f32_mfma_kernel<64, true, VARLEN, MASKED>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((flash_fwd_f32_mfma_kernel<64, false, VARLEN, MASKED>), grid, block, 0, stream, p);
+    }
+    return static_cast<int>(hipGetLastError());
 }
 
 static int check_dense(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N, int64_t H,
@@ -335,13 +360,32 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
         // 16 bytes at a time: rows of a multiple of 4 floats and an aligned base; everything else takes the kernel below.
         if (tuning().mask_pack.load() != 0) {
             bool launched = false;
-            const int rc = dtype == AHPC_F16 ? forward_on_packed_mask<f16_t>(p, mask, B, (int)d, causal != 0, st, &launched)
-                                             : forward_on_packed_mask<bf16_t>(p, mask, B, (int)d, causal != 0, st, &launched);
+            const int rc = forward_on_packed_mask(p, mask, B, st, &launched, [&](const FlashParams& pb) {
+                return dtype == AHPC_F16 ? dispatch_mfma_masked<f16_t, 2>(pb, B, (int)d, causal != 0, st)
+                                         : dispatch_mfma_masked<bf16_t, 2>(pb, B, (int)d, causal != 0, st);
+            });
             if (launched || rc != AHPC_OK) return rc;
         }
         if (N % 4 == 0 && aligned16(mask))
             return dtype == AHPC_F16 ? dispatch_mfma_masked<f16_t, 1>(p, B, (int)d, causal != 0, st)
                                      : dispatch_mfma_masked<bf16_t, 1>(p, B, (int)d, causal != 0, st);
+    }
+    if (f32_mfma_eligible(dtype, d, q, k, v, o, sq, skv)) {
+        FlashParams p{};
+        p.q = q; p.k = k; p.v = v; p.o = o;
+        p.stride_b = sq.b; p.stride_n = sq.n; p.stride_h = sq.h;
+        p.kv_stride_b = skv.b; p.kv_stride_n = skv.n; p.kv_stride_h = skv.h;
+        p.N = (int32_t)N; p.H = (int32_t)H; p.kv_group = group;
+        p.scale_log2 = scale * kLog2e;
+        if (!mask) return launch_f32_mfma<false, false>(p, B, (int)d, causal != 0, st);
+        // with a mask: on its packed copy, or not on the matrix cores at all
+        if (tuning().mask_pack.load() != 0) {
+            bool launched = false;
+            const int rc = forward_on_packed_mask(p, mask, B, st, &launched, [&](const FlashParams& pb) {
+                return launch_f32_mfma<false, true>(pb, B, (int)d, causal != 0, st);
+            });
+            if (launched || rc != AHPC_OK) return rc;
+        }
     }
     SimpleParams p{q, k, v, o, nullptr, mask, sq.b, sq.n, sq.h, skv.b, skv.n, skv.h, (int32_t)N, (int32_t)H, (int32_t)d, group, scale, causal ? 1 : 0};
     return dispatch_simple<false>(dtype, p, B, st);
@@ -409,6 +453,16 @@ int ahpc_hip_flash_fwd_varlen_gqa(const void* q, const void* k, const void* v, v
         p.scale_log2 = scale * kLog2e;
         return dtype == AHPC_F16 ? dispatch_mfma<f16_t, true>(p, n_seqs, (int)d, causal != 0, st)
                                  : dispatch_mfma<bf16_t, true>(p, n_seqs, (int)d, causal != 0, st);
+    }
+    if (f32_mfma_eligible(dtype, d, q, k, v, o, sq, skv)) {
+        FlashParams p{};
+        p.q = q; p.k = k; p.v = v; p.o = o;
+        p.cu_seqlens = cu_seqlens;
+        p.stride_b = 0; p.stride_n = sq.n; p.stride_h = sq.h;
+        p.kv_stride_b = 0; p.kv_stride_n = skv.n; p.kv_stride_h = skv.h;
+        p.N = (int32_t)max_len; p.H = (int32_t)H; p.kv_group = group;
+        p.scale_log2 = scale * kLog2e;
+        return launch_f32_mfma<true, false>(p, n_seqs, (int)d, causal != 0, st);
     }
     SimpleParams p{q, k, v, o, cu_seqlens, nullptr, 0, sq.n, sq.h, 0, skv.n, skv.h, (int32_t)max_len, (int32_t)H, (int32_t)d, group, scale, causal ? 1 : 0};
     return dispatch_simple<true>(dtype, p, n_seqs, st);

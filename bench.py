@@ -335,13 +335,16 @@ def bench_extras(hip, stream, steps, warmup):
     def randn(shape, dtype):
         return torch.randn(shape, generator=g, device="cuda", dtype=torch.float32).to(dtype)
 
-    def run(name, launch, flops=None, nbytes=None):
+    def run(name, launch, flops=None, nbytes=None, fp32=False):
         wall, per = timed_steps(hip, stream, launch, steps, warmup)
         ms = float(np.mean(per))
         row = {"workload": name, "kernel_ms_mean": round(ms, 4), "kernel_ms_min": round(float(np.min(per)), 4)}
         if flops:
             row["TFLOP/s"] = round(flops / (ms * 1e-3) / 1e12, 1)
-            row["frac_of_2.5_PFLOP/s"] = round(flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)
+            if fp32:  # fp32 matrix instructions: MI355X's published dense fp32 peak
+                row["frac_of_157.3_TFLOP/s_fp32"] = round(flops / (ms * 1e-3) / 1e12 / 157.3, 4)
+            else:
+                row["frac_of_2.5_PFLOP/s"] = round(flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)
         if nbytes:
             row["GB/s"] = round(nbytes / (ms * 1e-3) / 1e9, 1)
             row["frac_of_8_TB/s"] = round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
@@ -366,6 +369,14 @@ def bench_extras(hip, stream, steps, warmup):
         lambda: hip.flash_fwd_gqa(q.data_ptr(), kg.data_ptr(), vg.data_ptr(), o.data_ptr(), hip.BF16, B, N, H, Hkv, d, st,
                                   (N * Hkv * d, Hkv * d, d), sc, True, stream),
         flops=2.0 * B * H * N * N * d)
+
+    # the headline shape in fp32, the reference's default data type: the fp32 matrix-core kernel
+    qf, kf, vf = randn((B, N, H, d), torch.float32), randn((B, N, H, d), torch.float32), randn((B, N, H, d), torch.float32)
+    of = torch.empty_like(qf)
+    run("flash_fwd fp32 causal B=4 N=4096 H=32 d=128",
+        lambda: hip.flash_fwd(qf.data_ptr(), kf.data_ptr(), vf.data_ptr(), of.data_ptr(), hip.F32, B, N, H, d, st, sc, True, stream),
+        flops=2.0 * B * H * N * N * d, fp32=True)
+    del qf, kf, vf, of
 
     # backward at the headline shape.  FLOP by the usual convention: 2.5 x the forward's (five products
     # against two); the four launches here execute ten, because the interface passes neither the forward

@@ -106,9 +106,10 @@ int ahpc_hip_event_elapsed_ms(void* start, void* stop, float* ms);
  * src/algorithms/flash_attention.cpp:238-275) is stride_b = N*H*d, stride_n = H*d,
  * stride_h = d; [B,H,N,d] is stride_b = H*N*d, stride_h = N*d, stride_n = d, so no transpose
  * pass (src/backends/cuda/cuda_kernels.cu:668-687) is ever needed.  Q, K, V and O share one
- * dtype and one set of strides.  fp16/bf16 with d in {64, 128} run on the MFMA kernel; every
- * other case (fp32, other d <= 256) runs on the fp32-FMA kernel.  Accumulation is fp32
- * throughout.  A row with no visible key yields zeros
+ * dtype and one set of strides.  d in {64, 128} with 16-byte aligned rows runs on the matrix cores:
+ * fp16/bf16 on 16-bit matrix instructions, fp32 (the reference's default, DataType::FLOAT32) on fp32 ones
+ * (fp32 products and sums: same accuracy as the fp32-FMA kernel); every other case (other d <= 256,
+ * unaligned tensors) runs on the fp32-FMA kernel.  Accumulation is fp32 throughout.  A row with no visible key yields zeros
  * (OnlineSoftmaxState::get_normalizer, src/algorithms/flash_attention.hpp:59-61).
  * scale <= 0 means 1/sqrt(d) (AttentionParams::scale_factor,
  * src/api/attention_interface.hpp:64). */
@@ -131,14 +132,14 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
 
 /* Same with a dense fp32 mask [B,N,N] shared by all heads, 0.0f removes the key
  * (FlashAttention::apply_attention_mask, src/algorithms/flash_attention.cpp:596-607;
- * indexing :432-435).  A query whose keys are all removed gets a zero output row.  fp16/bf16 with d in {64, 128}
- * run on the matrix-core kernel, everything else on the fp32-FMA kernel.  The matrix-core kernel reads a packed copy
+ * indexing :432-435).  A query whose keys are all removed gets a zero output row.  Tensors that qualify for the
+ * matrix cores (see ahpc_hip_flash_fwd) stay there, everything else runs on the fp32-FMA kernel.  The matrix-core kernels read a packed copy
  * of the mask (one bit per element) that a small kernel writes in front of it, into device memory the LIBRARY owns:
  * one buffer per device, grown on demand (hipMalloc; B * N * ceil(N / 64) * 8 bytes, at most 1 GiB) and kept until the
  * process ends; calls on one device share it and are ordered through an event, on whatever streams they run.  A
- * stream under graph capture, a larger mask, a failed allocation or the tuning value mask_pack = 0 make the kernel read
- * the mask in place instead (N a multiple of 4 and a 16-byte aligned mask; otherwise the fp32-FMA kernel): no
- * allocation, more traffic.  mask may be NULL: then the fp32-FMA kernel runs whatever the type (the way to ask for
+ * stream under graph capture, a larger mask, a failed allocation or the tuning value mask_pack = 0 make the 16-bit
+ * kernel read the mask in place instead (N a multiple of 4 and a 16-byte aligned mask; otherwise, and for fp32
+ * tensors, the fp32-FMA kernel): no allocation, more traffic.  mask may be NULL: then the fp32-FMA kernel runs whatever the type (the way to ask for
  * it). */
 int ahpc_hip_flash_fwd_masked(const void* q, const void* k, const void* v, void* o, int dtype,
                               int64_t B, int64_t N, int64_t H, int64_t d,

@@ -71,6 +71,7 @@ int lane_id();
 
 f32x16 mfma_32x32x16_f16(f16x8 a, f16x8 b, f32x16 c);
 f32x16 mfma_32x32x16_bf16(bf16x8 a, bf16x8 b, f32x16 c);
+f32x16 mfma_32x32x2_f32(float a, float b, f32x16 c);
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -190,6 +191,7 @@ inline hipError_t hipGetLastError() { return ::simt::last_error(); }
 
 #define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) ::simt::mfma_32x32x16_f16((a), (b), (c))
 #define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) ::simt::mfma_32x32x16_bf16((a), (b), (c))
+#define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, x, y, z) ::simt::mfma_32x32x2_f32((a), (b), (c))
 #define __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, x, y, z) ::simt::mfma_16x16x32_f16((a), (b), (c))
 #define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) ::simt::mfma_16x16x32_bf16((a), (b), (c))
 #define __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, x, y, z) ::simt::mfma_16x16x16_f16((a), (b), (c))

@@ -431,6 +431,29 @@ void syncthreads() {
 
 f32x16 mfma_32x32x16_f16(f16x8 a, f16x8 b, f32x16 c) { return mfma_impl(a, b, c); }
 f32x16 mfma_32x32x16_bf16(bf16x8 a, bf16x8 b, f32x16 c) { return mfma_impl(a, b, c); }
+
+// v_mfma_f32_32x32x2_f32: lane l supplies A[row l%32][k l/32] and B[k l/32][col l%32]; results laid out as above.
+f32x16 mfma_32x32x2_f32(float a, float b, f32x16 c) {
+    struct Ops {
+        float a, b;
+    } mine{a, b};
+    const View v = exchange(K_MFMA, &mine, sizeof mine);
+    const Fiber* f = g_cur;
+    const int col = f->lane & 31, half = f->lane >> 5;
+    f32x16 d = c;
+    for (int r = 0; r < 16; ++r) {
+        const int row = 8 * (r / 4) + 4 * half + (r % 4);
+        double acc = 0.0;
+        for (int kh = 0; kh < 2; ++kh) {
+            Ops oa, ob;
+            std::memcpy(&oa, v.of(row + 32 * kh), sizeof oa);
+            std::memcpy(&ob, v.of(col + 32 * kh), sizeof ob);
+            acc += (double)oa.a * (double)ob.b;
+        }
+        d[r] = (float)((double)c[r] + acc);
+    }
+    return d;
+}
 f32x4 mfma_16x16x32_f16(f16x8 a, f16x8 b, f32x4 c) { return mfma16_impl<8>(a, b, c, [](_Float16 x) { return (float)x; }); }
 f32x4 mfma_16x16x32_bf16(bf16x8 a, bf16x8 b, f32x4 c) { return mfma16_impl<8>(a, b, c, [](__bf16 x) { return (float)x; }); }
 f32x4 mfma_16x16x16_f16(f16x4 a, f16x4 b, f32x4 c) { return mfma16_impl<4>(a, b, c, [](_Float16 x) { return (float)x; }); }

@@ -273,6 +273,36 @@ def test_config2_shape_bf16_causal_sampled_rows(gpu):
     assert np.abs(got - want).max() <= 2e-2
 
 
+@pytest.mark.parametrize("d,causal", [(128, True), (64, False)])
+def test_headline_shape_fp32_sampled_rows(gpu, d, causal):
+    """fp32 at the headline shape (B=4 N=4096 H=32), the fp32 matrix-core kernel at its real size: a seeded sample of
+    rows against the oracle within 1e-4, and what holds for every output row (finite, inside the range of V)."""
+    import torch
+    from gpu_util import stream_ptr
+    B, N, H = 4, 4096, 32
+    g = torch.Generator(device="cuda").manual_seed(0xA77E0012)
+    dq, dk, dv = (torch.randn((B, N, H, d), generator=g, device="cuda", dtype=torch.float32) for _ in range(3))
+    do = torch.full_like(dq, float("nan"))
+    scale = 1.0 / np.sqrt(d)
+    gpu.flash_fwd(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), do.data_ptr(), O.F32, B, N, H, d, (N * H * d, H * d, d),
+                  scale, causal, stream_ptr())
+    torch.cuda.synchronize()
+    assert torch.isfinite(do).all()
+    if causal:
+        assert torch.equal(do[:, 0], dv[:, 0])   # row 0 sees only key 0
+        vmax, vmin = torch.cummax(dv, dim=1).values, torch.cummin(dv, dim=1).values
+    else:
+        vmax, vmin = dv.amax(dim=1, keepdim=True), dv.amin(dim=1, keepdim=True)
+    assert (do <= vmax + 1e-4).all() and (do >= vmin - 1e-4).all()
+    rng = np.random.default_rng(12)
+    rows = np.unique(np.concatenate([rng.integers(0, B * H * N, 256), [N - 1, B * H * N - 1, 127, 128, 4095]])).astype(np.int64)
+    q, k, v = (t.cpu().numpy() for t in (dq, dk, dv))
+    want = O.attention_rows(q, k, v, B, N, H, d, scale, rows, causal)
+    out = do.cpu().numpy()
+    got = np.stack([out[r // (N * H), r % N, (r // N) % H] for r in rows])
+    assert np.abs(got - want).max() <= 1e-4
+
+
 @pytest.mark.parametrize("dtype,d", [(O.F16, 64), (O.BF16, 128), (O.F32, 64), (O.F16, 32)])
 @pytest.mark.parametrize("causal", [True, False])
 def test_varlen_small(gpu, dtype, d, causal):
