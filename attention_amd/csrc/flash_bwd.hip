@@ -18,6 +18,7 @@
 
 #include "ahpc_device.hpp"
 #include "flash_bwd_mfma.hpp"
+#include "flash_bwd_f32_mfma.hpp"
 #include "tuning.hpp"
 
 namespace ahpc {
@@ -418,6 +419,54 @@ static int launch_mfma(const FlashBwdParams& p, int64_t B, int64_t H_kv, int d, 
     return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
 }
 
+// fp32 tensors: the same three steps on the fp32 matrix instructions (flash_bwd_f32_mfma.hpp), dK and dV always in two walks
+template <int D, bool VARLEN>
+static int launch_f32_mfma_dv(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool causal, float* lse2, float* delta,
+                              hipStream_t stream) {
+    FlashParams f{};
+    f.q = p.q; f.k = p.k; f.v = p.v; f.o = nullptr;
+    f.stride_b = p.stride_b; f.stride_n = p.stride_n; f.stride_h = p.stride_h;
+    f.kv_stride_b = p.kv_stride_b; f.kv_stride_n = p.kv_stride_n; f.kv_stride_h = p.kv_stride_h;
+    f.N = p.N; f.H = p.H; f.kv_group = p.kv_group;
+    f.cu_seqlens = p.cu_seqlens;
+    f.scale_log2 = p.scale_log2;
+    if (int rc = flash_plan_launch(f, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load(), VARLEN)) return rc;
+    const FlashStatsOut st{p.d_out, lse2, delta, p.rows_padded};
+    const dim3 block(kFlashThreads);
+    const dim3 grid_stats((unsigned)(f.blocks_per_xcd * 8));
+    FlashBwdParams m = p;
+    m.n_tiles = (p.N + kFlashRows - 1) / kFlashRows;
+    const int64_t total_q = B * p.H * (int64_t)m.n_tiles, total_kv = B * H_kv * (int64_t)m.n_tiles;
+    if (total_q > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
+    m.total_q = (int32_t)total_q; m.per_xcd_q = (int32_t)((total_q + 7) / 8);
+    m.total_kv = (int32_t)total_kv; m.per_xcd_kv = (int32_t)((total_kv + 7) / 8);
+    const dim3 grid_q((unsigned)(m.per_xcd_q * 8)), grid_kv((unsigned)(m.per_xcd_kv * 8));
+    if (causal) {
+        hipLaunchKernelGGL((flash_bwd_stats_f32_mfma_kernel<D, true, VARLEN>), grid_stats, block, 0, stream, f, st);
+        hipLaunchKernelGGL((flash_bwd_dq_f32_mfma_kernel<D, true, VARLEN>), grid_q, block, 0, stream, m);
+        hipLaunchKernelGGL((flash_bwd_dkv_f32_mfma_kernel<D, true, VARLEN, 1>), grid_kv, block, 0, stream, m);
+        hipLaunchKernelGGL((flash_bwd_dkv_f32_mfma_kernel<D, true, VARLEN, 2>), grid_kv, block, 0, stream, m);
+    } else {
+        hipLaunchKernelGGL((flash_bwd_stats_f32_mfma_kernel<D, false, VARLEN>), grid_stats, block, 0, stream, f, st);
+        hipLaunchKernelGGL((flash_bwd_dq_f32_mfma_kernel<D, false, VARLEN>), grid_q, block, 0, stream, m);
+        hipLaunchKernelGGL((flash_bwd_dkv_f32_mfma_kernel<D, false, VARLEN, 1>), grid_kv, block, 0, stream, m);
+        hipLaunchKernelGGL((flash_bwd_dkv_f32_mfma_kernel<D, false, VARLEN, 2>), grid_kv, block, 0, stream, m);
+    }
+    return static_cast<int>(hipGetLastError());
+}
+
+static int launch_f32_mfma(const FlashBwdParams& p, int64_t B, int64_t H_kv, int d, bool causal, float* lse2, float* delta,
+                           hipStream_t stream) {
+    if (p.cu_seqlens) {
+        if (d == 128) return launch_f32_mfma_dv<128, true>(p, B, H_kv, causal, lse2, delta, stream);
+        if (d == 64) return launch_f32_mfma_dv<64, true>(p, B, H_kv, causal, lse2, delta, stream);
+    } else {
+        if (d == 128) return launch_f32_mfma_dv<128, false>(p, B, H_kv, causal, lse2, delta, stream);
+        if (d == 64) return launch_f32_mfma_dv<64, false>(p, B, H_kv, causal, lse2, delta, stream);
+    }
+    return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+}
+
 }  // namespace ahpc
 
 using namespace ahpc;
@@ -467,7 +516,11 @@ static int flash_bwd_any(const void* d_out, const void* q, const void* k, const 
     // fp16 / bf16 with d in {64, 128}, 16-byte aligned rows and no dense mask: the matrix-core kernels
     const bool strides_ok = !(stride_b % 8) && !(stride_n % 8) && !(stride_h % 8) && !(kv_stride_b % 8) && !(kv_stride_n % 8) &&
                             !(kv_stride_h % 8) && stride_n < (int64_t(1) << 24) && kv_stride_n < (int64_t(1) << 24);
-    if (!mask && (dtype == AHPC_F16 || dtype == AHPC_BF16) && (d == 64 || d == 128) && strides_ok && aligned16(q) &&
+    // fp32 with d in {64, 128} likewise (rows of whole 16-byte pieces): the fp32 matrix-core kernels
+    const bool strides4_ok = !(stride_b % 4) && !(stride_n % 4) && !(stride_h % 4) && !(kv_stride_b % 4) && !(kv_stride_n % 4) &&
+                             !(kv_stride_h % 4) && stride_n < (int64_t(1) << 24) && kv_stride_n < (int64_t(1) << 24);
+    const bool is16 = dtype == AHPC_F16 || dtype == AHPC_BF16;
+    if (!mask && (d == 64 || d == 128) && (is16 ? strides_ok : strides4_ok) && aligned16(q) &&
         aligned16(k) && aligned16(v) && aligned16(d_out) && aligned16(d_q) && aligned16(d_k) && aligned16(d_v)) {
         FlashBwdParams m{};
         m.q = q; m.k = k; m.v = v; m.d_out = d_out;
@@ -479,6 +532,7 @@ static int flash_bwd_any(const void* d_out, const void* q, const void* k, const 
         m.N = (int32_t)N; m.H = (int32_t)H; m.kv_group = p.kv_group;
         m.scale = scale;
         m.scale_log2 = scale * kLog2e;
+        if (dtype == AHPC_F32) return launch_f32_mfma(m, B, H_kv, (int)d, causal != 0, p.lse, p.delta, st);
         return dtype == AHPC_F16 ? launch_mfma<f16_t>(m, B, H_kv, (int)d, causal != 0, p.lse, p.delta, st)
                                  : launch_mfma<bf16_t>(m, B, H_kv, (int)d, causal != 0, p.lse, p.delta, st);
     }

@@ -40,10 +40,12 @@ __device__ inline f32x16 mfma_32x32x2_f32(float a, float b, f32x16 c) {
 // one XCD, long tiles first, causal launches with a late and an early query tile per workgroup.
 // MASKED: a dense mask [B,N,N] in its packed form (FlashParams::mask_bits, see flash_fwd_mfma.hpp: one 64-bit word per
 // query and 64 keys) removes keys per query; the reference maximum is then set per query when its first key shows up.
-template <int D, bool CAUSAL, bool VARLEN, bool MASKED = false>
-__global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_f32_mfma_kernel(const FlashParams p) {
+// STATS: the first step of the backward.  The output stays in registers; per query row the kernel writes what
+// FlashStatsOut describes (flash_fwd_mfma.hpp): -lse2 and -(dO . O), padding rows -inf and 0.
+template <int D, bool CAUSAL, bool VARLEN, bool MASKED, bool STATS>
+__device__ __forceinline__ void flash_fwd_f32_mfma_body(const FlashParams& p, const FlashStatsOut& st) {
     static_assert(D == 64 || D == 128, "head dimensions of the fp32 matrix-core kernel");
-    static_assert(!(MASKED && VARLEN), "the mask belongs to dense launches");
+    static_assert(!(MASKED && (VARLEN || STATS)), "the mask belongs to dense forward launches");
     constexpr int RB = 4 * D;                 // row bytes
     constexpr int CH = D / 4;                 // 16-byte chunks per row
     constexpr int RPI = 1024 / RB;            // rows one load instruction covers
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_f32_mfma_kernel(co
     const float* const gq = static_cast<const float*>(p.q) + base;
     const float* const gk = static_cast<const float*>(p.k) + kv_base;
     const float* const gv = static_cast<const float*>(p.v) + kv_base;
-    float* const go = static_cast<float*>(p.o) + base;
+    float* const go = STATS ? nullptr : static_cast<float*>(p.o) + base;  // the statistics pass has no output tensor
     const int64_t sn = p.stride_n;
     const int64_t skv = p.kv_stride_n;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
@@ -300,7 +302,28 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_f32_mfma_kernel(co
         // ---- normalise and store: per 32-row block a lane holds 4 runs of 4 consecutive d of its query
         const float l = halves_sum(l_run);
         const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-        if (qrow < L) {
+        if constexpr (STATS) {
+            // delta = dO . O over the elements this lane holds, then over the two lanes of the query
+            float part = 0.0f;
+            if (qrow < L) {
+                const float* src = static_cast<const float*>(st.d_out) + base + (int64_t)qrow * sn + 4 * half;
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        const f32x4 w = *reinterpret_cast<const f32x4*>(src + 32 * mb + 8 * g4);
+                        part += oacc[mb][4 * g4] * w[0] + oacc[mb][4 * g4 + 1] * w[1] + oacc[mb][4 * g4 + 2] * w[2] +
+                                oacc[mb][4 * g4 + 3] * w[3];
+                    }
+            }
+            const float delta = halves_sum(part) * inv;
+            if (half == 0) {  // every row of the 128-row tile gets a value: the statistics arrays are padded to whole tiles
+                const int64_t row = (int64_t)work.bh * st.rows_padded + qrow;
+                const bool live = qrow < L && l > 0.0f;
+                st.neg_lse2[row] = live ? neg_m[0] - __builtin_log2f(l) : -INFINITY;
+                st.neg_delta[row] = live ? -delta : 0.0f;
+            }
+        } else if (qrow < L) {
             float* dst = go + (int64_t)qrow * sn + 4 * half;
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
@@ -310,6 +333,16 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_f32_mfma_kernel(co
                         f32x4{oacc[mb][4 * g4] * inv, oacc[mb][4 * g4 + 1] * inv, oacc[mb][4 * g4 + 2] * inv, oacc[mb][4 * g4 + 3] * inv};
         }
     }
+}
+
+template <int D, bool CAUSAL, bool VARLEN, bool MASKED = false>
+__global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_f32_mfma_kernel(const FlashParams p) {
+    flash_fwd_f32_mfma_body<D, CAUSAL, VARLEN, MASKED, false>(p, FlashStatsOut{});
+}
+
+template <int D, bool CAUSAL, bool VARLEN>
+__global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_stats_f32_mfma_kernel(const FlashParams p, const FlashStatsOut st) {
+    flash_fwd_f32_mfma_body<D, CAUSAL, VARLEN, false, true>(p, st);
 }
 
 }  // namespace ahpc

@@ -390,6 +390,15 @@ def bench_extras(hip, stream, steps, warmup):
                               gv.data_ptr(), hip.BF16, B, N, H, H, d, st, st, sc, True, wsf.data_ptr(), wsb, stream),
         flops=2.5 * 2.0 * B * H * N * N * d)
 
+    # the same backward in fp32 (fp32 matrix-core kernels; dK and dV always in two walks)
+    qf, kf, vf, gof = (randn((B, N, H, d), torch.float32) for _ in range(4))
+    gqf, gkf, gvf = torch.empty_like(qf), torch.empty_like(kf), torch.empty_like(vf)
+    run("flash_bwd fp32 causal B=4 N=4096 H=32 d=128",
+        lambda: hip.flash_bwd(gof.data_ptr(), qf.data_ptr(), kf.data_ptr(), vf.data_ptr(), gqf.data_ptr(), gkf.data_ptr(),
+                              gvf.data_ptr(), hip.F32, B, N, H, H, d, st, st, sc, True, wsf.data_ptr(), wsb, stream),
+        flops=2.5 * 2.0 * B * H * N * N * d, fp32=True)
+    del qf, kf, vf, gof, gqf, gkf, gvf
+
     # the headline shape, non-causal, with a dense random mask [B,N,N] (half the keys removed; flops counted as unmasked)
     dmask = (torch.rand((B, N, N), generator=g, device="cuda") > 0.5).float()
     run("flash_fwd bf16 non-causal B=4 N=4096 H=32 d=128 with a dense fp32 mask [B,N,N]",

@@ -596,6 +596,25 @@ def test_backward_matrix_core_kernels(emu, tuned, dtype, B, N, H, H_kv, d, causa
     check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), dtype)
 
 
+@pytest.mark.parametrize("dma_late", [False, True])
+@pytest.mark.parametrize("B,N,H,H_kv,d,causal", [
+    (1, 64, 1, 1, 128, False), (2, 129, 2, 2, 128, True), (1, 300, 2, 2, 64, True), (1, 200, 2, 1, 64, False),
+    (1, 1, 2, 2, 128, True), (1, 260, 4, 2, 128, True), (1, 33, 2, 2, 64, True), (1, 31, 1, 1, 128, False)])
+def test_backward_fp32_matrix_core_kernels(emu, B, N, H, H_kv, d, causal, dma_late):
+    """fp32 tensors with d 64 or 128: statistics, dQ, and the dV and dK walks on the fp32 matrix instructions."""
+    q, k, v, do = bwd_inputs(B, N, H, H_kv, d, 38, O.F32)
+    scale = 1.0 / np.sqrt(d)
+    S.configure(dma_late, seed=N + d)
+    S.lds_stats(reset=True)
+    try:
+        got = backward(emu, q, k, v, do, O.F32, B, N, H, H_kv, d, scale, causal, front=dma_late)
+    finally:
+        S.configure(False, 1)
+    check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), O.F32)
+    reads, read_conflicts, _, _ = S.lds_stats(reset=True)
+    assert reads > 0 and read_conflicts == 0   # the matrix-core kernels ran (the FMA kernels make no traced reads)
+
+
 # ---- LDS bank conflicts (model: 64 banks of 4 bytes) --------------------------------------------------------
 @pytest.mark.parametrize("dtype,d", [(O.BF16, 128), (O.F16, 64)])
 def test_operand_reads_are_free_of_bank_conflicts(emu, dtype, d):
@@ -675,7 +694,7 @@ def test_wide_groups_need_the_matrix_core_shape(emu):
         decode(emu, q, kp, vp, table, lens, None, B, G * H_kv, H_kv, d, P, O.F32, O.F32, 0.125)
 
 
-@pytest.mark.parametrize("dtype,d,H,H_kv", [(O.F16, 64, 2, 2), (O.BF16, 128, 4, 2), (O.F32, 32, 2, 1)])
+@pytest.mark.parametrize("dtype,d,H,H_kv", [(O.F16, 64, 2, 2), (O.BF16, 128, 4, 2), (O.F32, 32, 2, 1), (O.F32, 128, 2, 1), (O.F32, 64, 2, 2)])
 @pytest.mark.parametrize("causal", [False, True])
 def test_backward_ragged_batch(emu, dtype, d, H, H_kv, causal):
     """Packed sequences of different lengths: every sequence's gradients equal the dense oracle's on that sequence."""
