@@ -194,6 +194,37 @@ def test_dense_mask_packed_copy_shared_between_streams_and_sizes(gpu):
         assert np.abs(to_host(do) - want).max() <= 2e-2, N
 
 
+def test_dense_mask_under_graph_capture_allocates_nothing(gpu):
+    """A stream under graph capture gets the kernel that reads the mask in place (the packed copy would need an allocation
+    and a wait on another stream's event): the captured graph replays correctly, with new inputs between the replays."""
+    import torch
+    from gpu_util import to_dev, to_host
+    B, N, H, d = 2, 260, 2, 128
+    q, k, v = make_qkv((B, N, H, d), 81, O.BF16)
+    mask = (O.fill_uniform((B, N, N), 81, 6) > -0.2).astype(np.float32)
+    mask[:, np.arange(N), np.arange(N)] = 1.0
+    dq, dk, dv, dm = to_dev(q, O.BF16), to_dev(k, O.BF16), to_dev(v, O.BF16), torch.from_numpy(mask).cuda()
+    do = torch.full_like(dq, float("nan"))
+    scale = 1.0 / np.sqrt(d)
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        gpu.flash_fwd(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), do.data_ptr(), O.BF16, B, N, H, d, (N * H * d, H * d, d),
+                      scale, False, torch.cuda.current_stream().cuda_stream, dm.data_ptr())
+    for rep in range(3):
+        if rep:
+            q, k, v = make_qkv((B, N, H, d), 81 + rep, O.BF16)
+            mask = (O.fill_uniform((B, N, N), 81 + rep, 6) > 0.1 * rep).astype(np.float32)
+            mask[:, np.arange(N), np.arange(N)] = 1.0
+            dq.copy_(to_dev(q, O.BF16)); dk.copy_(to_dev(k, O.BF16)); dv.copy_(to_dev(v, O.BF16)); dm.copy_(torch.from_numpy(mask).cuda())
+        do.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = O.attention(q, k, v, B, N, H, d, scale, False, mask=mask)
+        assert np.abs(to_host(do) - want).max() <= 2e-2, rep
+
+
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16])
 @pytest.mark.parametrize("d", [64, 128])
 @pytest.mark.parametrize("causal", [False, True])
