@@ -389,7 +389,10 @@ static int launch_mfma_dv(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool
     const dim3 grid_stats((unsigned)(f.blocks_per_xcd * 8));
     FlashBwdParams m = p;
     m.n_tiles = (p.N + kFlashRows - 1) / kFlashRows;
-    const int64_t total_q = B * p.H * (int64_t)m.n_tiles, total_kv = B * H_kv * (int64_t)m.n_tiles;
+    // causal dense launches: a workgroup takes a long and a short tile of its head, so that all do the same work
+    m.paired = (causal && !VARLEN && m.n_tiles >= 2 && tuning().bwd_pair.load() != 0) ? 1 : 0;
+    const int64_t units = bwd_units(m);
+    const int64_t total_q = B * p.H * units, total_kv = B * H_kv * units;
     if (total_q > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
     m.total_q = (int32_t)total_q; m.per_xcd_q = (int32_t)((total_q + 7) / 8);
     m.total_kv = (int32_t)total_kv; m.per_xcd_kv = (int32_t)((total_kv + 7) / 8);
@@ -436,7 +439,10 @@ static int launch_f32_mfma_dv(const FlashBwdParams& p, int64_t B, int64_t H_kv, 
     const dim3 grid_stats((unsigned)(f.blocks_per_xcd * 8));
     FlashBwdParams m = p;
     m.n_tiles = (p.N + kFlashRows - 1) / kFlashRows;
-    const int64_t total_q = B * p.H * (int64_t)m.n_tiles, total_kv = B * H_kv * (int64_t)m.n_tiles;
+    // causal dense launches: a workgroup takes a long and a short tile of its head, so that all do the same work
+    m.paired = (causal && !VARLEN && m.n_tiles >= 2 && tuning().bwd_pair.load() != 0) ? 1 : 0;
+    const int64_t units = bwd_units(m);
+    const int64_t total_q = B * p.H * units, total_kv = B * H_kv * units;
     if (total_q > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
     m.total_q = (int32_t)total_q; m.per_xcd_q = (int32_t)((total_q + 7) / 8);
     m.total_kv = (int32_t)total_kv; m.per_xcd_kv = (int32_t)((total_kv + 7) / 8);

@@ -45,6 +45,9 @@ struct FlashBwdParams {
     int32_t H;                  // query heads
     int32_t kv_group;           // query heads per key/value head
     int32_t n_tiles;            // 128-row tiles per sequence
+    int32_t paired;             // 1: a workgroup takes two tiles of a head, a long walk and a short one (causal dense launches:
+                                // tile i sees i + 1 tiles' worth of the other side, so i and n_tiles - 1 - i together are the
+                                // same work for every workgroup); total_q / total_kv count workgroups accordingly
     int32_t total_q, per_xcd_q;     // dQ kernel: workgroups (B * H * n_tiles) and ceil(that / 8)
     int32_t total_kv, per_xcd_kv;   // dK/dV kernel: workgroups (B * H_kv * n_tiles) and ceil(that / 8)
     float scale;
@@ -58,6 +61,8 @@ struct BwdWork {
     int bh, tile;
     bool valid;
 };
+// work units per head: tiles, or pairs of them
+__host__ __device__ inline int bwd_units(const FlashBwdParams& p) { return p.paired ? (p.n_tiles + 1) >> 1 : p.n_tiles; }
 __host__ __device__ inline BwdWork bwd_work_of_block(unsigned block_id, int total, int per_xcd, int n_tiles) {
     const int logical = (int)(block_id & 7u) * per_xcd + (int)(block_id >> 3);
     if (logical >= total) return BwdWork{0, 0, false};
@@ -131,7 +136,7 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
     const int lane = tid & 63;
     const int col = lane & 31;
     const int half = lane >> 5;
-    const BwdWork work = bwd_work_of_block(blockIdx.x, p.total_q, p.per_xcd_q, p.n_tiles);
+    const BwdWork work = bwd_work_of_block(blockIdx.x, p.total_q, p.per_xcd_q, bwd_units(p));
     if (!work.valid) return;
     const int b = work.bh / p.H, h = work.bh - b * p.H;
     const int hk = h / p.kv_group;
@@ -147,10 +152,6 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
         base = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
         kv_base = (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
     }
-    // long tiles first: under a causal mask the late query tiles walk the most keys
-    const int q_tile0 = (p.n_tiles - 1 - work.tile) * kFlashRows;
-    if (q_tile0 >= L) return;  // ragged batches: a sequence shorter than the longest one
-
     const T* const gq = static_cast<const T*>(p.q) + base;
     const T* const gdo = static_cast<const T*>(p.d_out) + base;
     const T* const gk = static_cast<const T*>(p.k) + kv_base;
@@ -182,132 +183,141 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
 #pragma unroll
         for (int a = 0; a < 2; ++a) tr_off[mb][a] = tr_offset_rowswizzled<D>(lane, mb, a);
 
-    int k_end = L;
-    if (CAUSAL) k_end = (q_tile0 + kFlashRows) < L ? (q_tile0 + kFlashRows) : L;
-    const int n_tiles = (k_end + kFlashKeys - 1) / kFlashKeys;
-    dma_both(0, lds_k0, lds_v0);
+    for (int part = 0; part < 2; ++part) {
+        // long tiles first: under a causal mask the late query tiles walk the most keys; a paired workgroup then takes the
+        // early tile that completes its share
+        const int tile = part == 0 ? work.tile : p.n_tiles - 1 - work.tile;
+        if (part == 1 && (!p.paired || tile == work.tile)) break;
+        const int q_tile0 = (p.n_tiles - 1 - tile) * kFlashRows;
+        if (q_tile0 >= L) continue;  // ragged batches: a sequence shorter than the longest one
+        if (part == 1) __syncthreads();  // every wavefront is done with the first pass's last tile
+        int k_end = L;
+        if (CAUSAL) k_end = (q_tile0 + kFlashRows) < L ? (q_tile0 + kFlashRows) : L;
+        const int n_tiles = (k_end + kFlashKeys - 1) / kFlashKeys;
+        dma_both(0, lds_k0, lds_v0);
 
-    const int qw = q_tile0 + wave * 32;
-    const int qrow = qw + col;
-    const int row = qrow < L ? qrow : L - 1;
-    u32x4 qreg[KS], doreg[KS];
-    load_row_operands<T, KS>(qreg, gq + (int64_t)row * sn, half, p.scale_log2);
-    load_row_operands<T, KS>(doreg, gdo + (int64_t)row * sn, half, 1.0f);
-    const int64_t stat = ((int64_t)b * p.H + h) * p.rows_padded + qrow;  // qrow < rows_padded always
-    f32x16 neg_lse, neg_delta;
-    {
-        const float a = p.neg_lse2[stat], d0 = p.neg_delta[stat];
+        const int qw = q_tile0 + wave * 32;
+        const int qrow = qw + col;
+        const int row = qrow < L ? qrow : L - 1;
+        u32x4 qreg[KS], doreg[KS];
+        load_row_operands<T, KS>(qreg, gq + (int64_t)row * sn, half, p.scale_log2);
+        load_row_operands<T, KS>(doreg, gdo + (int64_t)row * sn, half, 1.0f);
+        const int64_t stat = ((int64_t)b * p.H + h) * p.rows_padded + qrow;  // qrow < rows_padded always
+        f32x16 neg_lse, neg_delta;
+        {
+            const float a = p.neg_lse2[stat], d0 = p.neg_delta[stat];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            neg_lse[r] = a;
-            neg_delta[r] = d0;
+            for (int r = 0; r < 16; ++r) {
+                neg_lse[r] = a;
+                neg_delta[r] = d0;
+            }
         }
-    }
-    f32x16 acc[MB];
+        f32x16 acc[MB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+        for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[mb][r] = 0.0f;
+            for (int r = 0; r < 16; ++r) acc[mb][r] = 0.0f;
 
-    auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int k0) {
+        auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int k0) {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-            const int kblock0 = k0 + 32 * kb;
-            if (kblock0 >= L) continue;                        // nothing but padding
-            if (CAUSAL && kblock0 > qw + 31) continue;        // every key of the block is in the future
-            // (issue priority up while the matrix cores are fed, down for the stretch of exponentials, as in the forward)
-            __builtin_amdgcn_s_setprio(1);
-            // K^T operands of the block's first 16 keys: requested now, they arrive while the first two products run
-            u32x2 kt[2][MB][2];
+            for (int kb = 0; kb < 2; ++kb) {
+                const int kblock0 = k0 + 32 * kb;
+                if (kblock0 >= L) continue;                        // nothing but padding
+                if (CAUSAL && kblock0 > qw + 31) continue;        // every key of the block is in the future
+                // (issue priority up while the matrix cores are fed, down for the stretch of exponentials, as in the forward)
+                __builtin_amdgcn_s_setprio(1);
+                // K^T operands of the block's first 16 keys: requested now, they arrive while the first two products run
+                u32x2 kt[2][MB][2];
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) {
-                kt[0][mb][0] = TrRead<T>::load(tile_k + (32 * kb) * RB + tr_off[mb][0]);
-                kt[0][mb][1] = TrRead<T>::load(tile_k + (32 * kb) * RB + tr_off[mb][1]);
-            }
-            f32x16 s = neg_lse, dp = neg_delta;
-            {
-                // the operand pairs of the two products are requested kAhead steps ahead of the matrix instructions
-                // that use them (all at once would cost 8 registers per step)
-                u32x4 ak[KS], av[KS];
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    ak[ks] = lds_read_b128(tile_k + 32 * kb * RB + row_off[ks]);
-                    av[ks] = lds_read_b128(tile_v + 32 * kb * RB + row_off[ks]);
+                for (int mb = 0; mb < MB; ++mb) {
+                    kt[0][mb][0] = TrRead<T>::load(tile_k + (32 * kb) * RB + tr_off[mb][0]);
+                    kt[0][mb][1] = TrRead<T>::load(tile_k + (32 * kb) * RB + tr_off[mb][1]);
                 }
+                f32x16 s = neg_lse, dp = neg_delta;
+                {
+                    // the operand pairs of the two products are requested kAhead steps ahead of the matrix instructions
+                    // that use them (all at once would cost 8 registers per step)
+                    u32x4 ak[KS], av[KS];
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    s = mfma_32x32x16<T>(ak[ks], qreg[ks], s);
-                    dp = mfma_32x32x16<T>(av[ks], doreg[ks], dp);
+                    for (int ks = 0; ks < KS; ++ks) {
+                        ak[ks] = lds_read_b128(tile_k + 32 * kb * RB + row_off[ks]);
+                        av[ks] = lds_read_b128(tile_v + 32 * kb * RB + row_off[ks]);
+                    }
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        s = mfma_32x32x16<T>(ak[ks], qreg[ks], s);
+                        dp = mfma_32x32x16<T>(av[ks], doreg[ks], dp);
+                    }
+                    constexpr int kAhead = 2;
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2 * MB + 2 * kAhead, 0);  // LDS reads (the K^T ones first)
+#pragma unroll
+                    for (int i = 0; i < KS - kAhead; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // matrix instructions
+                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    }
+#pragma unroll
+                    for (int i = 0; i < kAhead; ++i) __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
                 }
-                constexpr int kAhead = 2;
-                __builtin_amdgcn_sched_group_barrier(0x100, 2 * MB + 2 * kAhead, 0);  // LDS reads (the K^T ones first)
+                // key = kblock0 + 4*half + 8*(r/4) + r%4 is visible iff key <= min(qrow, L-1)
+                __builtin_amdgcn_s_setprio(0);
+                f32x16 ds;
+                // the per-element test is needed only where the block meets the diagonal or the end of the sequence
+                // (uniform per wavefront)
+                const bool all_on = kblock0 + 31 < L && (!CAUSAL || kblock0 + 31 <= qw);
+                if (all_on) {
 #pragma unroll
-                for (int i = 0; i < KS - kAhead; ++i) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // matrix instructions
-                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                }
+                    for (int r = 0; r < 16; ++r) ds[r] = fast_exp2(s[r]) * dp[r];
+                } else {
+                    int lim = L - 1;
+                    if (CAUSAL) lim = qrow < lim ? qrow : lim;
+                    lim -= kblock0 + 4 * half;
 #pragma unroll
-                for (int i = 0; i < kAhead; ++i) __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            }
-            // key = kblock0 + 4*half + 8*(r/4) + r%4 is visible iff key <= min(qrow, L-1)
-            __builtin_amdgcn_s_setprio(0);
-            f32x16 ds;
-            // the per-element test is needed only where the block meets the diagonal or the end of the sequence
-            // (uniform per wavefront)
-            const bool all_on = kblock0 + 31 < L && (!CAUSAL || kblock0 + 31 <= qw);
-            if (all_on) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) ds[r] = fast_exp2(s[r]) * dp[r];
-            } else {
-                int lim = L - 1;
-                if (CAUSAL) lim = qrow < lim ? qrow : lim;
-                lim -= kblock0 + 4 * half;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int off = 8 * (r >> 2) + (r & 3);
-                    ds[r] = off <= lim ? fast_exp2(s[r]) * dp[r] : 0.0f;
-                }
-            }
-            __builtin_amdgcn_s_setprio(1);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int g2 = 0; g2 < 2; ++g2) {
-                const u32x4 bop = pack_operand<T>(ds, 8 * g2);
-                if (g2 == 0) {
-                    // the second 16 keys' operands travel while the first 16 are multiplied
-#pragma unroll
-                    for (int mb = 0; mb < MB; ++mb) {
-                        kt[1][mb][0] = TrRead<T>::load(tile_k + (32 * kb + 16) * RB + tr_off[mb][0]);
-                        kt[1][mb][1] = TrRead<T>::load(tile_k + (32 * kb + 16) * RB + tr_off[mb][1]);
+                    for (int r = 0; r < 16; ++r) {
+                        const int off = 8 * (r >> 2) + (r & 3);
+                        ds[r] = off <= lim ? fast_exp2(s[r]) * dp[r] : 0.0f;
                     }
                 }
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
-                    acc[mb] = mfma_32x32x16<T>(u32x4{kt[g2][mb][0][0], kt[g2][mb][0][1], kt[g2][mb][1][0], kt[g2][mb][1][1]}, bop, acc[mb]);
+                __builtin_amdgcn_s_setprio(1);
                 __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int g2 = 0; g2 < 2; ++g2) {
+                    const u32x4 bop = pack_operand<T>(ds, 8 * g2);
+                    if (g2 == 0) {
+                        // the second 16 keys' operands travel while the first 16 are multiplied
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb) {
+                            kt[1][mb][0] = TrRead<T>::load(tile_k + (32 * kb + 16) * RB + tr_off[mb][0]);
+                            kt[1][mb][1] = TrRead<T>::load(tile_k + (32 * kb + 16) * RB + tr_off[mb][1]);
+                        }
+                    }
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+                        acc[mb] = mfma_32x32x16<T>(u32x4{kt[g2][mb][0][0], kt[g2][mb][0][1], kt[g2][mb][1][0], kt[g2][mb][1][1]}, bop, acc[mb]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                __builtin_amdgcn_s_setprio(0);
             }
-            __builtin_amdgcn_s_setprio(0);
-        }
-    };
+        };
 
-    auto step = [&](unsigned char* cur_k, unsigned char* cur_v, unsigned char* nxt_k, unsigned char* nxt_v, int t) {
-        const int k0 = t * kFlashKeys;
-        const bool more = t + 1 < n_tiles;
-        if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
-        compute_tile(cur_k, cur_v, k0);
-        if (more) {
-            __builtin_amdgcn_s_waitcnt(0);
-            __syncthreads();
-        }
-    };
+        auto step = [&](unsigned char* cur_k, unsigned char* cur_v, unsigned char* nxt_k, unsigned char* nxt_v, int t) {
+            const int k0 = t * kFlashKeys;
+            const bool more = t + 1 < n_tiles;
+            if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
+            compute_tile(cur_k, cur_v, k0);
+            if (more) {
+                __builtin_amdgcn_s_waitcnt(0);
+                __syncthreads();
+            }
+        };
 
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    for (int t = 0; t < n_tiles; t += 2) {
-        step(lds_k0, lds_v0, lds_k1, lds_v1, t);
-        if (t + 1 < n_tiles) step(lds_k1, lds_v1, lds_k0, lds_v0, t + 1);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        for (int t = 0; t < n_tiles; t += 2) {
+            step(lds_k0, lds_v0, lds_k1, lds_v1, t);
+            if (t + 1 < n_tiles) step(lds_k1, lds_v1, lds_k0, lds_v0, t + 1);
+        }
+        if (qrow < L) store_row<T, MB>(static_cast<T*>(p.d_q) + base + (int64_t)qrow * sn, acc, half, p.scale);
     }
-    if (qrow < L) store_row<T, MB>(static_cast<T*>(p.d_q) + base + (int64_t)qrow * sn, acc, half, p.scale);
 }
 
 // grid: 8 * per_xcd_kv workgroups, see bwd_work_of_block
@@ -336,7 +346,7 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
     const int lane = tid & 63;
     const int col = lane & 31;
     const int half = lane >> 5;
-    const BwdWork work = bwd_work_of_block(blockIdx.x, p.total_kv, p.per_xcd_kv, p.n_tiles);
+    const BwdWork work = bwd_work_of_block(blockIdx.x, p.total_kv, p.per_xcd_kv, bwd_units(p));
     if (!work.valid) return;
     const int heads_kv = p.H / p.kv_group;
     const int b = work.bh / heads_kv, hk = work.bh - b * heads_kv;
@@ -346,10 +356,6 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
         seq0 = p.cu_seqlens[b];
         L = p.cu_seqlens[b + 1] - seq0;
     }
-    // under a causal mask the early key tiles see the most queries: they go first
-    const int k_tile0 = work.tile * kFlashRows;
-    if (k_tile0 >= L) return;  // ragged batches: a sequence shorter than the longest one
-
     const int64_t kv_base = VARLEN ? (int64_t)seq0 * p.kv_stride_n + (int64_t)hk * p.kv_stride_h
                                    : (int64_t)b * p.kv_stride_b + (int64_t)hk * p.kv_stride_h;
     const T* const gk = static_cast<const T*>(p.k) + kv_base;
@@ -374,194 +380,202 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
 #pragma unroll
         for (int a = 0; a < 2; ++a) tr_off[mb][a] = tr_offset_rowswizzled<D>(lane, mb, a);
 
-    const int kw = k_tile0 + wave * 32;  // first key of this wavefront
-    const int key = kw + col;
-    const int krow = key < L ? key : L - 1;
-    u32x4 kreg[KS], vreg[KS];
-    load_row_operands<T, KS>(kreg, gk + (int64_t)krow * skv, half, p.scale_log2);
-    if constexpr (kDoK) load_row_operands<T, KS>(vreg, gv + (int64_t)krow * skv, half, 1.0f);
+    for (int part = 0; part < 2; ++part) {
+        // under a causal mask the early key tiles see the most queries: they go first; a paired workgroup then takes the
+        // late tile that completes its share
+        const int tile = part == 0 ? work.tile : p.n_tiles - 1 - work.tile;
+        if (part == 1 && (!p.paired || tile == work.tile)) break;
+        const int k_tile0 = tile * kFlashRows;
+        if (k_tile0 >= L) continue;  // ragged batches: a sequence shorter than the longest one
+        const int kw = k_tile0 + wave * 32;  // first key of this wavefront
+        const int key = kw + col;
+        const int krow = key < L ? key : L - 1;
+        u32x4 kreg[KS], vreg[KS];
+        load_row_operands<T, KS>(kreg, gk + (int64_t)krow * skv, half, p.scale_log2);
+        if constexpr (kDoK) load_row_operands<T, KS>(vreg, gv + (int64_t)krow * skv, half, 1.0f);
 
-    f32x16 acc_k[MB], acc_v[MB];
+        f32x16 acc_k[MB], acc_v[MB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+        for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            acc_k[mb][r] = 0.0f;
-            acc_v[mb][r] = 0.0f;
-        }
-
-    // queries before the first key of the workgroup see none of its keys under a causal mask
-    const int t_begin = CAUSAL ? k_tile0 / kFlashKeys : 0;
-    const int n_tiles = (L + kFlashKeys - 1) / kFlashKeys;
-
-    for (int g = 0; g < p.kv_group; ++g) {
-        const int h = hk * p.kv_group + g;
-        const int64_t base = VARLEN ? (int64_t)seq0 * p.stride_n + (int64_t)h * p.stride_h
-                                    : (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
-        const T* const gq = static_cast<const T*>(p.q) + base;
-        const T* const gdo = static_cast<const T*>(p.d_out) + base;
-        const float* const lse2 = p.neg_lse2 + ((int64_t)b * p.H + h) * p.rows_padded;
-        const float* const delta = p.neg_delta + ((int64_t)b * p.H + h) * p.rows_padded;
-
-        auto dma_both = [&](int i0, unsigned char* dst_q, unsigned char* dst_o, unsigned char* dst_s) {
-            // (a tile that starts at or behind the end of the sequence touches no memory and lands as zeros)
-            const int64_t rem = i0 < L ? (int64_t)(L - i0 - 1) * sn * 2 + 2 * D : 0;
-            const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
-            dma_tile<D>(gq + (int64_t)i0 * sn, nrec, dma_off, dst_q, wave_u);
-            dma_tile<D>(gdo + (int64_t)i0 * sn, nrec, dma_off, dst_o, wave_u);
-            // the statistics arrays are padded to whole 128-row tiles: 64 rows from i0 < L on always exist
-            if (wave_u == 0) {
-                const unsigned nst = i0 < L ? 256u : 0u;
-                dma_dword(lse2 + i0, nst, 4 * lane, dst_s);
-                dma_dword(delta + i0, nst, 4 * lane, dst_s + 256);
+            for (int r = 0; r < 16; ++r) {
+                acc_k[mb][r] = 0.0f;
+                acc_v[mb][r] = 0.0f;
             }
-        };
 
-        auto compute_tile = [&](const unsigned char* tile_q, const unsigned char* tile_o, const unsigned char* tile_s, int i0) {
-#pragma unroll
-            for (int ib = 0; ib < 2; ++ib) {
-                const int iblock0 = i0 + 32 * ib;
-                if (iblock0 >= L) continue;                      // nothing but padding
-                if (CAUSAL && iblock0 + 31 < kw) continue;      // every query of the block precedes the keys
-                // the block's rows of statistics: this lane's 16 rows are 4 runs of 4 consecutive rows
-                f32x16 s, dp;
-#pragma unroll
-                for (int g4 = 0; g4 < 4; ++g4) {
-                    const f32x4 a = *reinterpret_cast<const f32x4*>(tile_s + 4 * (32 * ib + 8 * g4 + 4 * half));
-#pragma unroll
-                    for (int x = 0; x < 4; ++x) s[4 * g4 + x] = a[x];
-                    if constexpr (kDoK) {
-                        const f32x4 d0 = *reinterpret_cast<const f32x4*>(tile_s + 256 + 4 * (32 * ib + 8 * g4 + 4 * half));
-#pragma unroll
-                        for (int x = 0; x < 4; ++x) dp[4 * g4 + x] = d0[x];
-                    }
+        // queries before the first key of the workgroup see none of its keys under a causal mask
+        const int t_begin = CAUSAL ? k_tile0 / kFlashKeys : 0;
+        const int n_tiles = (L + kFlashKeys - 1) / kFlashKeys;
+
+        for (int g = 0; g < p.kv_group; ++g) {
+            const int h = hk * p.kv_group + g;
+            const int64_t base = VARLEN ? (int64_t)seq0 * p.stride_n + (int64_t)h * p.stride_h
+                                        : (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+            const T* const gq = static_cast<const T*>(p.q) + base;
+            const T* const gdo = static_cast<const T*>(p.d_out) + base;
+            const float* const lse2 = p.neg_lse2 + ((int64_t)b * p.H + h) * p.rows_padded;
+            const float* const delta = p.neg_delta + ((int64_t)b * p.H + h) * p.rows_padded;
+
+            auto dma_both = [&](int i0, unsigned char* dst_q, unsigned char* dst_o, unsigned char* dst_s) {
+                // (a tile that starts at or behind the end of the sequence touches no memory and lands as zeros)
+                const int64_t rem = i0 < L ? (int64_t)(L - i0 - 1) * sn * 2 + 2 * D : 0;
+                const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
+                dma_tile<D>(gq + (int64_t)i0 * sn, nrec, dma_off, dst_q, wave_u);
+                dma_tile<D>(gdo + (int64_t)i0 * sn, nrec, dma_off, dst_o, wave_u);
+                // the statistics arrays are padded to whole 128-row tiles: 64 rows from i0 < L on always exist
+                if (wave_u == 0) {
+                    const unsigned nst = i0 < L ? 256u : 0u;
+                    dma_dword(lse2 + i0, nst, 4 * lane, dst_s);
+                    dma_dword(delta + i0, nst, 4 * lane, dst_s + 256);
                 }
-                __builtin_amdgcn_sched_barrier(0);  // (the statistics reads stay out of the pipeline laid out below)
-                __builtin_amdgcn_s_setprio(1);
-                // transposed operands of the block's first 16 queries: requested now, they arrive while the first
-                // products run
-                u32x2 ot[2][MB][2], qt[2][MB][2];
+            };
+
+            auto compute_tile = [&](const unsigned char* tile_q, const unsigned char* tile_o, const unsigned char* tile_s, int i0) {
 #pragma unroll
-                for (int mb = 0; mb < MB; ++mb) {
-                    if constexpr (kDoV) {
-                        ot[0][mb][0] = TrRead<T>::load(tile_o + (32 * ib) * RB + tr_off[mb][0]);
-                        ot[0][mb][1] = TrRead<T>::load(tile_o + (32 * ib) * RB + tr_off[mb][1]);
-                    }
-                    if constexpr (kDoK) {
-                        qt[0][mb][0] = TrRead<T>::load(tile_q + (32 * ib) * RB + tr_off[mb][0]);
-                        qt[0][mb][1] = TrRead<T>::load(tile_q + (32 * ib) * RB + tr_off[mb][1]);
-                    }
-                }
-                {
-                    // the operands of the first products are requested kAhead steps ahead of the matrix
-                    // instructions that use them
-                    constexpr int kPer = kDoK ? 2 : 1;  // products (and operand reads) per step
-                    constexpr int kAhead = 2;
-                    u32x4 aq[KS], ao[KS];
+                for (int ib = 0; ib < 2; ++ib) {
+                    const int iblock0 = i0 + 32 * ib;
+                    if (iblock0 >= L) continue;                      // nothing but padding
+                    if (CAUSAL && iblock0 + 31 < kw) continue;      // every query of the block precedes the keys
+                    // the block's rows of statistics: this lane's 16 rows are 4 runs of 4 consecutive rows
+                    f32x16 s, dp;
 #pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) {
-                        aq[ks] = lds_read_b128(tile_q + 32 * ib * RB + row_off[ks]);
-                        if constexpr (kDoK) ao[ks] = lds_read_b128(tile_o + 32 * ib * RB + row_off[ks]);
-                    }
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        const f32x4 a = *reinterpret_cast<const f32x4*>(tile_s + 4 * (32 * ib + 8 * g4 + 4 * half));
 #pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) {
-                        s = mfma_32x32x16<T>(aq[ks], kreg[ks], s);
-                        if constexpr (kDoK) dp = mfma_32x32x16<T>(ao[ks], vreg[ks], dp);
-                    }
-                    __builtin_amdgcn_sched_group_barrier(0x100, 2 * MB * (kDoK && kDoV ? 2 : 1) + kPer * kAhead, 0);  // LDS reads
+                        for (int x = 0; x < 4; ++x) s[4 * g4 + x] = a[x];
+                        if constexpr (kDoK) {
+                            const f32x4 d0 = *reinterpret_cast<const f32x4*>(tile_s + 256 + 4 * (32 * ib + 8 * g4 + 4 * half));
 #pragma unroll
-                    for (int i = 0; i < KS - kAhead; ++i) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);  // matrix instructions
-                        __builtin_amdgcn_sched_group_barrier(0x100, kPer, 0);
-                    }
-#pragma unroll
-                    for (int i = 0; i < kAhead; ++i) __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);
-                }
-                // query = iblock0 + 4*half + 8*(r/4) + r%4 contributes iff it exists, the key exists, and
-                // (causal) query >= key
-                __builtin_amdgcn_s_setprio(0);
-                f32x16 pw, ds;
-                // the per-element tests are needed only where the block meets the diagonal or an end of the sequence
-                // (uniform per wavefront): everywhere else every (query, key) pair of the block counts
-                const bool all_on = iblock0 + 31 < L && kw + 31 < L && (!CAUSAL || iblock0 >= kw + 31);
-                if (all_on) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        pw[r] = fast_exp2(s[r]);
-                        if constexpr (kDoK) ds[r] = pw[r] * dp[r];
-                    }
-                } else {
-                    int first = 0;
-                    if (CAUSAL) first = key - (iblock0 + 4 * half);
-                    const int last = (key < L ? L : 0) - (iblock0 + 4 * half);  // off < last
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int off = 8 * (r >> 2) + (r & 3);
-                        const bool on = off >= first && off < last;
-                        pw[r] = on ? fast_exp2(s[r]) : 0.0f;
-                        if constexpr (kDoK) ds[r] = on ? pw[r] * dp[r] : 0.0f;
-                    }
-                }
-                __builtin_amdgcn_s_setprio(1);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int g2 = 0; g2 < 2; ++g2) {
-                    if (g2 == 0) {
-                        // the second 16 queries' operands travel while the first 16 are multiplied
-#pragma unroll
-                        for (int mb = 0; mb < MB; ++mb) {
-                            if constexpr (kDoV) {
-                                ot[1][mb][0] = TrRead<T>::load(tile_o + (32 * ib + 16) * RB + tr_off[mb][0]);
-                                ot[1][mb][1] = TrRead<T>::load(tile_o + (32 * ib + 16) * RB + tr_off[mb][1]);
-                            }
-                            if constexpr (kDoK) {
-                                qt[1][mb][0] = TrRead<T>::load(tile_q + (32 * ib + 16) * RB + tr_off[mb][0]);
-                                qt[1][mb][1] = TrRead<T>::load(tile_q + (32 * ib + 16) * RB + tr_off[mb][1]);
-                            }
+                            for (int x = 0; x < 4; ++x) dp[4 * g4 + x] = d0[x];
                         }
                     }
-                    if constexpr (kDoV) {
-                        const u32x4 bp = pack_operand<T>(pw, 8 * g2);
+                    __builtin_amdgcn_sched_barrier(0);  // (the statistics reads stay out of the pipeline laid out below)
+                    __builtin_amdgcn_s_setprio(1);
+                    // transposed operands of the block's first 16 queries: requested now, they arrive while the first
+                    // products run
+                    u32x2 ot[2][MB][2], qt[2][MB][2];
 #pragma unroll
-                        for (int mb = 0; mb < MB; ++mb)
-                            acc_v[mb] = mfma_32x32x16<T>(u32x4{ot[g2][mb][0][0], ot[g2][mb][0][1], ot[g2][mb][1][0], ot[g2][mb][1][1]}, bp, acc_v[mb]);
+                    for (int mb = 0; mb < MB; ++mb) {
+                        if constexpr (kDoV) {
+                            ot[0][mb][0] = TrRead<T>::load(tile_o + (32 * ib) * RB + tr_off[mb][0]);
+                            ot[0][mb][1] = TrRead<T>::load(tile_o + (32 * ib) * RB + tr_off[mb][1]);
+                        }
+                        if constexpr (kDoK) {
+                            qt[0][mb][0] = TrRead<T>::load(tile_q + (32 * ib) * RB + tr_off[mb][0]);
+                            qt[0][mb][1] = TrRead<T>::load(tile_q + (32 * ib) * RB + tr_off[mb][1]);
+                        }
                     }
-                    if constexpr (kDoK) {
-                        const u32x4 bs = pack_operand<T>(ds, 8 * g2);
+                    {
+                        // the operands of the first products are requested kAhead steps ahead of the matrix
+                        // instructions that use them
+                        constexpr int kPer = kDoK ? 2 : 1;  // products (and operand reads) per step
+                        constexpr int kAhead = 2;
+                        u32x4 aq[KS], ao[KS];
 #pragma unroll
-                        for (int mb = 0; mb < MB; ++mb)
-                            acc_k[mb] = mfma_32x32x16<T>(u32x4{qt[g2][mb][0][0], qt[g2][mb][0][1], qt[g2][mb][1][0], qt[g2][mb][1][1]}, bs, acc_k[mb]);
+                        for (int ks = 0; ks < KS; ++ks) {
+                            aq[ks] = lds_read_b128(tile_q + 32 * ib * RB + row_off[ks]);
+                            if constexpr (kDoK) ao[ks] = lds_read_b128(tile_o + 32 * ib * RB + row_off[ks]);
+                        }
+#pragma unroll
+                        for (int ks = 0; ks < KS; ++ks) {
+                            s = mfma_32x32x16<T>(aq[ks], kreg[ks], s);
+                            if constexpr (kDoK) dp = mfma_32x32x16<T>(ao[ks], vreg[ks], dp);
+                        }
+                        __builtin_amdgcn_sched_group_barrier(0x100, 2 * MB * (kDoK && kDoV ? 2 : 1) + kPer * kAhead, 0);  // LDS reads
+#pragma unroll
+                        for (int i = 0; i < KS - kAhead; ++i) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);  // matrix instructions
+                            __builtin_amdgcn_sched_group_barrier(0x100, kPer, 0);
+                        }
+#pragma unroll
+                        for (int i = 0; i < kAhead; ++i) __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);
                     }
+                    // query = iblock0 + 4*half + 8*(r/4) + r%4 contributes iff it exists, the key exists, and
+                    // (causal) query >= key
+                    __builtin_amdgcn_s_setprio(0);
+                    f32x16 pw, ds;
+                    // the per-element tests are needed only where the block meets the diagonal or an end of the sequence
+                    // (uniform per wavefront): everywhere else every (query, key) pair of the block counts
+                    const bool all_on = iblock0 + 31 < L && kw + 31 < L && (!CAUSAL || iblock0 >= kw + 31);
+                    if (all_on) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            pw[r] = fast_exp2(s[r]);
+                            if constexpr (kDoK) ds[r] = pw[r] * dp[r];
+                        }
+                    } else {
+                        int first = 0;
+                        if (CAUSAL) first = key - (iblock0 + 4 * half);
+                        const int last = (key < L ? L : 0) - (iblock0 + 4 * half);  // off < last
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const int off = 8 * (r >> 2) + (r & 3);
+                            const bool on = off >= first && off < last;
+                            pw[r] = on ? fast_exp2(s[r]) : 0.0f;
+                            if constexpr (kDoK) ds[r] = on ? pw[r] * dp[r] : 0.0f;
+                        }
+                    }
+                    __builtin_amdgcn_s_setprio(1);
                     __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int g2 = 0; g2 < 2; ++g2) {
+                        if (g2 == 0) {
+                            // the second 16 queries' operands travel while the first 16 are multiplied
+#pragma unroll
+                            for (int mb = 0; mb < MB; ++mb) {
+                                if constexpr (kDoV) {
+                                    ot[1][mb][0] = TrRead<T>::load(tile_o + (32 * ib + 16) * RB + tr_off[mb][0]);
+                                    ot[1][mb][1] = TrRead<T>::load(tile_o + (32 * ib + 16) * RB + tr_off[mb][1]);
+                                }
+                                if constexpr (kDoK) {
+                                    qt[1][mb][0] = TrRead<T>::load(tile_q + (32 * ib + 16) * RB + tr_off[mb][0]);
+                                    qt[1][mb][1] = TrRead<T>::load(tile_q + (32 * ib + 16) * RB + tr_off[mb][1]);
+                                }
+                            }
+                        }
+                        if constexpr (kDoV) {
+                            const u32x4 bp = pack_operand<T>(pw, 8 * g2);
+#pragma unroll
+                            for (int mb = 0; mb < MB; ++mb)
+                                acc_v[mb] = mfma_32x32x16<T>(u32x4{ot[g2][mb][0][0], ot[g2][mb][0][1], ot[g2][mb][1][0], ot[g2][mb][1][1]}, bp, acc_v[mb]);
+                        }
+                        if constexpr (kDoK) {
+                            const u32x4 bs = pack_operand<T>(ds, 8 * g2);
+#pragma unroll
+                            for (int mb = 0; mb < MB; ++mb)
+                                acc_k[mb] = mfma_32x32x16<T>(u32x4{qt[g2][mb][0][0], qt[g2][mb][0][1], qt[g2][mb][1][0], qt[g2][mb][1][1]}, bs, acc_k[mb]);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    __builtin_amdgcn_s_setprio(0);
                 }
-                __builtin_amdgcn_s_setprio(0);
-            }
-        };
+            };
 
-        auto step = [&](unsigned char* cur_q, unsigned char* cur_o, unsigned char* cur_s, unsigned char* nxt_q, unsigned char* nxt_o,
-                        unsigned char* nxt_s, int t) {
-            const int i0 = t * kFlashKeys;
-            const bool more = t + 1 < n_tiles;
-            if (more) dma_both(i0 + kFlashKeys, nxt_q, nxt_o, nxt_s);
-            compute_tile(cur_q, cur_o, cur_s, i0);
-            if (more) {
-                __builtin_amdgcn_s_waitcnt(0);
-                __syncthreads();
-            }
-        };
+            auto step = [&](unsigned char* cur_q, unsigned char* cur_o, unsigned char* cur_s, unsigned char* nxt_q, unsigned char* nxt_o,
+                            unsigned char* nxt_s, int t) {
+                const int i0 = t * kFlashKeys;
+                const bool more = t + 1 < n_tiles;
+                if (more) dma_both(i0 + kFlashKeys, nxt_q, nxt_o, nxt_s);
+                compute_tile(cur_q, cur_o, cur_s, i0);
+                if (more) {
+                    __builtin_amdgcn_s_waitcnt(0);
+                    __syncthreads();
+                }
+            };
 
-        dma_both(t_begin * kFlashKeys, lds_q0, lds_o0, lds_s0);
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        for (int t = t_begin; t < n_tiles; t += 2) {
-            step(lds_q0, lds_o0, lds_s0, lds_q1, lds_o1, lds_s1, t);
-            if (t + 1 < n_tiles) step(lds_q1, lds_o1, lds_s1, lds_q0, lds_o0, lds_s0, t + 1);
+            dma_both(t_begin * kFlashKeys, lds_q0, lds_o0, lds_s0);
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+            for (int t = t_begin; t < n_tiles; t += 2) {
+                step(lds_q0, lds_o0, lds_s0, lds_q1, lds_o1, lds_s1, t);
+                if (t + 1 < n_tiles) step(lds_q1, lds_o1, lds_s1, lds_q0, lds_o0, lds_s0, t + 1);
+            }
+            __syncthreads();  // the next head's first load reuses the buffers
         }
-        __syncthreads();  // the next head's first load reuses the buffers
-    }
-    if (key < L) {
-        if constexpr (kDoK) store_row<T, MB>(static_cast<T*>(p.d_k) + kv_base + (int64_t)key * skv, acc_k, half, p.scale);
-        if constexpr (kDoV) store_row<T, MB>(static_cast<T*>(p.d_v) + kv_base + (int64_t)key * skv, acc_v, half, 1.0f);
+        if (key < L) {
+            if constexpr (kDoK) store_row<T, MB>(static_cast<T*>(p.d_k) + kv_base + (int64_t)key * skv, acc_k, half, p.scale);
+            if constexpr (kDoV) store_row<T, MB>(static_cast<T*>(p.d_v) + kv_base + (int64_t)key * skv, acc_v, half, 1.0f);
+        }
     }
 }
 

@@ -20,7 +20,8 @@ Tuning::Tuning()
       decode_chunk(env_value("AHPC_DECODE_CHUNK", 0)),
       decode_matrix_min_group(env_value("AHPC_DECODE_MFMA_MIN_GROUP", 2)),
       bwd_split(env_value("AHPC_BWD_SPLIT", 0)),
-      mask_pack(env_value("AHPC_MASK_PACK", 1)) {
+      mask_pack(env_value("AHPC_MASK_PACK", 1)),
+      bwd_pair(env_value("AHPC_BWD_PAIR", 1)) {
     if (flash_pair_min_tiles.load() < 1) flash_pair_min_tiles = 1024;
 }
 
@@ -38,6 +39,7 @@ static std::atomic<int64_t>* tuning_slot(const char* name) {
     if (!std::strcmp(name, "decode_matrix_min_group")) return &t.decode_matrix_min_group;
     if (!std::strcmp(name, "bwd_split")) return &t.bwd_split;
     if (!std::strcmp(name, "mask_pack")) return &t.mask_pack;
+    if (!std::strcmp(name, "bwd_pair")) return &t.bwd_pair;
     return nullptr;
 }
 

@@ -29,6 +29,9 @@ struct Tuning {
     // front of the launch, into device memory the library keeps; 0 = the kernel reads the caller's fp32 mask in place
     // (what a stream under graph capture gets in any case).  (AHPC_MASK_PACK)
     std::atomic<int64_t> mask_pack;
+    // backward, causal dense launches: 1 (default) = the dQ and dK/dV workgroups take a long and a short tile of their
+    // head each (equal work for all), 0 = one tile per workgroup, long tiles first.  (AHPC_BWD_PAIR)
+    std::atomic<int64_t> bwd_pair;
     Tuning();
 };
 

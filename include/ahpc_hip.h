@@ -68,8 +68,8 @@ typedef struct ahpc_device_info {
 } ahpc_device_info;
 
 /* Launcher tuning values ("flash_pair_min_tiles", "decode_waves", "decode_chunk", "decode_matrix_min_group", "bwd_split",
- * "mask_pack"): process-wide, each starts from its environment variable (AHPC_FLASH_PAIR_MIN, AHPC_DECODE_WAVES,
- * AHPC_DECODE_CHUNK, AHPC_DECODE_MFMA_MIN_GROUP, AHPC_BWD_SPLIT, AHPC_MASK_PACK), which is read once.  No value
+ * "bwd_pair", "mask_pack"): process-wide, each starts from its environment variable (AHPC_FLASH_PAIR_MIN, AHPC_DECODE_WAVES,
+ * AHPC_DECODE_CHUNK, AHPC_DECODE_MFMA_MIN_GROUP, AHPC_BWD_SPLIT, AHPC_BWD_PAIR, AHPC_MASK_PACK), which is read once.  No value
  * changes results; unknown names and negative values are refused.  The reference has no counterpart: its tile sizes
  * sit in PerformanceConfig (src/api/attention_interface.hpp:29-53), which the host classes still honour. */
 int ahpc_hip_set_tuning(const char* name, int64_t value);

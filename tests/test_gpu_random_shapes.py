@@ -140,7 +140,9 @@ def test_backward_random_shapes(gpu, dtype, B, N, H, Hkv, d, causal, split, seed
     wsb = gpu.flash_bwd_workspace_bytes(B, N, H)
     ws = torch.empty(max(wsb, 4) // 4, dtype=torch.float32, device="cuda")
     before = gpu.get_tuning("bwd_split")
+    before_pair = gpu.get_tuning("bwd_pair")
     gpu.set_tuning("bwd_split", split)
+    gpu.set_tuning("bwd_pair", seed % 2)   # causal launches: one tile per workgroup, or a long and a short one
     try:
         gpu.flash_bwd(dgo.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), gq.data_ptr(), gk.data_ptr(), gv.data_ptr(),
                       dtype, B, N, H, Hkv, d, (N * H * d, H * d, d), (N * Hkv * d, Hkv * d, d), scale, causal,
@@ -148,6 +150,7 @@ def test_backward_random_shapes(gpu, dtype, B, N, H, Hkv, d, causal, split, seed
         torch.cuda.synchronize()
     finally:
         gpu.set_tuning("bwd_split", before)
+        gpu.set_tuning("bwd_pair", before_pair)
     bar = 1e-4 if dtype == O.F32 else 2e-2
     for name, got, ref in zip(("dq", "dk", "dv"), (gq, gk, gv), want):
         got = to_host(got)

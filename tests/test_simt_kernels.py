@@ -586,6 +586,7 @@ def test_backward_fp32_kernels_16bit_storage(emu, dtype):
     (1, 1, 2, 2, 128, True), (1, 260, 4, 2, 128, True)])
 def test_backward_matrix_core_kernels(emu, tuned, dtype, B, N, H, H_kv, d, causal, dma_late, split):
     tuned("bwd_split", split)   # dK and dV in one walk over the query tiles, or in two (the default at d = 128)
+    tuned("bwd_pair", split - 1)  # causal launches: one tile per workgroup (with one walk), a long and a short one (with two)
     q, k, v, do = bwd_inputs(B, N, H, H_kv, d, 34, dtype)
     scale = 1.0 / np.sqrt(d)
     S.configure(dma_late, seed=N + d)
@@ -600,8 +601,10 @@ def test_backward_matrix_core_kernels(emu, tuned, dtype, B, N, H, H_kv, d, causa
 @pytest.mark.parametrize("B,N,H,H_kv,d,causal", [
     (1, 64, 1, 1, 128, False), (2, 129, 2, 2, 128, True), (1, 300, 2, 2, 64, True), (1, 200, 2, 1, 64, False),
     (1, 1, 2, 2, 128, True), (1, 260, 4, 2, 128, True), (1, 33, 2, 2, 64, True), (1, 31, 1, 1, 128, False)])
-def test_backward_fp32_matrix_core_kernels(emu, B, N, H, H_kv, d, causal, dma_late):
-    """fp32 tensors with d 64 or 128: statistics, dQ, and the dV and dK walks on the fp32 matrix instructions."""
+def test_backward_fp32_matrix_core_kernels(emu, tuned, B, N, H, H_kv, d, causal, dma_late):
+    """fp32 tensors with d 64 or 128: statistics, dQ, and the dV and dK walks on the fp32 matrix instructions.  Causal launches
+    with one tile per workgroup (tile requests on time) and with a long and a short one (requests late)."""
+    tuned("bwd_pair", 1 if dma_late else 0)
     q, k, v, do = bwd_inputs(B, N, H, H_kv, d, 38, O.F32)
     scale = 1.0 / np.sqrt(d)
     S.configure(dma_late, seed=N + d)
