@@ -283,10 +283,14 @@ struct Strides {
     int64_t b, n, h;
 };
 
+// The head dimension a matrix-core kernel is instantiated for: 64 or 128, the tensors' own or the next larger one (the
+// kernels then compute with columns that contribute nothing, FlashParams::d_real).
+static int kernel_head_dim(int64_t d) { return d <= 64 ? 64 : 128; }
+
 static bool mfma_eligible(int dtype, int64_t d, const void* q, const void* k, const void* v, const void* o,
                           const Strides& sq, const Strides& skv) {
     if (dtype != AHPC_F16 && dtype != AHPC_BF16) return false;
-    if (d != 64 && d != 128) return false;
+    if (d < 8 || d > 128 || (d % 8)) return false;  // rows of whole 16-byte pieces
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return false;
     if ((sq.b % 8) || (sq.n % 8) || (sq.h % 8) || (skv.b % 8) || (skv.n % 8) || (skv.h % 8)) return false;
     // a key tile is addressed with 32-bit byte offsets from its first row, and rows must not overlap
@@ -296,7 +300,7 @@ static bool mfma_eligible(int dtype, int64_t d, const void* q, const void* k, co
 // fp32 tensors on the matrix cores: d 64 or 128, 16-byte aligned rows, no dense mask.
 static bool f32_mfma_eligible(int dtype, int64_t d, const void* q, const void* k, const void* v, const void* o,
                               const Strides& sq, const Strides& skv) {
-    if (dtype != AHPC_F32 || (d != 64 && d != 128)) return false;
+    if (dtype != AHPC_F32 || d < 4 || d > 128 || (d % 4)) return false;  // rows of whole 16-byte pieces
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return false;
     if ((sq.b % 4) || (sq.n % 4) || (sq.h % 4) || (skv.b % 4) || (skv.n % 4) || (skv.h % 4)) return false;
     // a key tile is addressed with 32-bit byte offsets from its first row, and rows must not overlap
@@ -352,23 +356,24 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
         p.kv_stride_b = skv.b; p.kv_stride_n = skv.n; p.kv_stride_h = skv.h;
         p.N = (int32_t)N; p.H = (int32_t)H; p.kv_group = group;
         p.scale_log2 = scale * kLog2e;
+        p.d_real = (int32_t)d;
         if (!mask)
-            return dtype == AHPC_F16 ? dispatch_mfma<f16_t, false>(p, B, (int)d, causal != 0, st)
-                                     : dispatch_mfma<bf16_t, false>(p, B, (int)d, causal != 0, st);
+            return dtype == AHPC_F16 ? dispatch_mfma<f16_t, false>(p, B, kernel_head_dim(d), causal != 0, st)
+                                     : dispatch_mfma<bf16_t, false>(p, B, kernel_head_dim(d), causal != 0, st);
         // The mask, by preference, as a packed copy made in front of the launch (every head reads the mask: packed, a
         // sixteenth of the bytes).  Where that is not possible, or switched off, the kernel reads the mask in place,
         // 16 bytes at a time: rows of a multiple of 4 floats and an aligned base; everything else takes the kernel below.
         if (tuning().mask_pack.load() != 0) {
             bool launched = false;
             const int rc = forward_on_packed_mask(p, mask, B, st, &launched, [&](const FlashParams& pb) {
-                return dtype == AHPC_F16 ? dispatch_mfma_masked<f16_t, 2>(pb, B, (int)d, causal != 0, st)
-                                         : dispatch_mfma_masked<bf16_t, 2>(pb, B, (int)d, causal != 0, st);
+                return dtype == AHPC_F16 ? dispatch_mfma_masked<f16_t, 2>(pb, B, kernel_head_dim(d), causal != 0, st)
+                                         : dispatch_mfma_masked<bf16_t, 2>(pb, B, kernel_head_dim(d), causal != 0, st);
             });
             if (launched || rc != AHPC_OK) return rc;
         }
         if (N % 4 == 0 && aligned16(mask))
-            return dtype == AHPC_F16 ? dispatch_mfma_masked<f16_t, 1>(p, B, (int)d, causal != 0, st)
-                                     : dispatch_mfma_masked<bf16_t, 1>(p, B, (int)d, causal != 0, st);
+            return dtype == AHPC_F16 ? dispatch_mfma_masked<f16_t, 1>(p, B, kernel_head_dim(d), causal != 0, st)
+                                     : dispatch_mfma_masked<bf16_t, 1>(p, B, kernel_head_dim(d), causal != 0, st);
     }
     if (f32_mfma_eligible(dtype, d, q, k, v, o, sq, skv)) {
         FlashParams p{};
@@ -377,12 +382,13 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
         p.kv_stride_b = skv.b; p.kv_stride_n = skv.n; p.kv_stride_h = skv.h;
         p.N = (int32_t)N; p.H = (int32_t)H; p.kv_group = group;
         p.scale_log2 = scale * kLog2e;
-        if (!mask) return launch_f32_mfma<false, false>(p, B, (int)d, causal != 0, st);
+        p.d_real = (int32_t)d;
+        if (!mask) return launch_f32_mfma<false, false>(p, B, kernel_head_dim(d), causal != 0, st);
         // with a mask: on its packed copy, or not on the matrix cores at all
         if (tuning().mask_pack.load() != 0) {
             bool launched = false;
             const int rc = forward_on_packed_mask(p, mask, B, st, &launched, [&](const FlashParams& pb) {
-                return launch_f32_mfma<false, true>(pb, B, (int)d, causal != 0, st);
+                return launch_f32_mfma<false, true>(pb, B, kernel_head_dim(d), causal != 0, st);
             });
             if (launched || rc != AHPC_OK) return rc;
         }
@@ -451,8 +457,9 @@ int ahpc_hip_flash_fwd_varlen_gqa(const void* q, const void* k, const void* v, v
         p.kv_stride_b = 0; p.kv_stride_n = skv.n; p.kv_stride_h = skv.h;
         p.N = (int32_t)max_len; p.H = (int32_t)H; p.kv_group = group;
         p.scale_log2 = scale * kLog2e;
-        return dtype == AHPC_F16 ? dispatch_mfma<f16_t, true>(p, n_seqs, (int)d, causal != 0, st)
-                                 : dispatch_mfma<bf16_t, true>(p, n_seqs, (int)d, causal != 0, st);
+        p.d_real = (int32_t)d;
+        return dtype == AHPC_F16 ? dispatch_mfma<f16_t, true>(p, n_seqs, kernel_head_dim(d), causal != 0, st)
+                                 : dispatch_mfma<bf16_t, true>(p, n_seqs, kernel_head_dim(d), causal != 0, st);
     }
     if (f32_mfma_eligible(dtype, d, q, k, v, o, sq, skv)) {
         FlashParams p{};
@@ -462,7 +469,8 @@ int ahpc_hip_flash_fwd_varlen_gqa(const void* q, const void* k, const void* v, v
         p.kv_stride_b = 0; p.kv_stride_n = skv.n; p.kv_stride_h = skv.h;
         p.N = (int32_t)max_len; p.H = (int32_t)H; p.kv_group = group;
         p.scale_log2 = scale * kLog2e;
-        return launch_f32_mfma<true, false>(p, n_seqs, (int)d, causal != 0, st);
+        p.d_real = (int32_t)d;
+        return launch_f32_mfma<true, false>(p, n_seqs, kernel_head_dim(d), causal != 0, st);
     }
     SimpleParams p{q, k, v, o, cu_seqlens, nullptr, 0, sq.n, sq.h, 0, skv.n, skv.h, (int32_t)max_len, (int32_t)H, (int32_t)d, group, scale, causal ? 1 : 0};
     return dispatch_simple<true>(dtype, p, n_seqs, st);

@@ -96,6 +96,7 @@ __device__ __forceinline__ void flash_fwd_f32_mfma_body(const FlashParams& p, co
     const int64_t sn = p.stride_n;
     const int64_t skv = p.kv_stride_n;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int d_real = (p.d_real > 0 && p.d_real < D) ? p.d_real : D;
 
     auto fk = [](int r) { return r & (CH - 1); };
     auto fv = [](int r) { return 8 * ((r >> 2) & 1); };  // exchanges the 128-byte blocks 2j and 2j + 1 of a row
@@ -107,13 +108,15 @@ __device__ __forceinline__ void flash_fwd_f32_mfma_body(const FlashParams& p, co
     for (int i = 0; i < IPW; ++i) {
         const int r = (wave * IPW + i) * RPI + lane / CH;
         const int pc = lane % CH;
-        dma_off_k[i] = (int)(r * skv * 4) + ((pc ^ fk(r)) << 4);
-        dma_off_v[i] = (int)(r * skv * 4) + ((pc ^ fv(r)) << 4);
+        const int ck = pc ^ fk(r), cv = pc ^ fv(r);  // the 4-float chunk of the row that belongs at this lane's place
+        // a head dimension below D (FlashParams::d_real): columns from d_real on fetch the row's first chunk again
+        dma_off_k[i] = (int)(r * skv * 4) + ((4 * ck < d_real ? ck : 0) << 4);
+        dma_off_v[i] = (int)(r * skv * 4) + ((4 * cv < d_real ? cv : 0) << 4);
     }
     // Bytes from the tile's first row to the end of the sequence's last row bound the descriptor: rows of a ragged last
     // tile that do not exist read as zeros (their scores are masked; zero V rows keep 0 * x finite).
     auto dma_both = [&](int k0, unsigned char* dst_k, unsigned char* dst_v) {
-        const int64_t rem = k0 < L ? (int64_t)(L - k0 - 1) * skv * 4 + RB : 0;
+        const int64_t rem = k0 < L ? (int64_t)(L - k0 - 1) * skv * 4 + 4 * d_real : 0;  // the last row ends with its own d
         const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
 #pragma unroll
         for (int i = 0; i < IPW; ++i) {
@@ -146,7 +149,7 @@ __device__ __forceinline__ void flash_fwd_f32_mfma_body(const FlashParams& p, co
             const float* src = gq + (int64_t)(qrow < L ? qrow : L - 1) * sn + 4 * half;
 #pragma unroll
             for (int m = 0; m < MS; ++m) {
-                const f32x4 raw = *reinterpret_cast<const f32x4*>(src + 8 * m);
+                const f32x4 raw = 8 * m + 4 * half < d_real ? *reinterpret_cast<const f32x4*>(src + 8 * m) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
                 qreg[m] = f32x4{raw[0] * c, raw[1] * c, raw[2] * c, raw[3] * c};
             }
         }
@@ -329,8 +332,9 @@ __device__ __forceinline__ void flash_fwd_f32_mfma_body(const FlashParams& p, co
             for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4)
-                    *reinterpret_cast<f32x4*>(dst + 32 * mb + 8 * g4) =
-                        f32x4{oacc[mb][4 * g4] * inv, oacc[mb][4 * g4 + 1] * inv, oacc[mb][4 * g4 + 2] * inv, oacc[mb][4 * g4 + 3] * inv};
+                    if (32 * mb + 8 * g4 + 4 * half < d_real)
+                        *reinterpret_cast<f32x4*>(dst + 32 * mb + 8 * g4) =
+                            f32x4{oacc[mb][4 * g4] * inv, oacc[mb][4 * g4 + 1] * inv, oacc[mb][4 * g4 + 2] * inv, oacc[mb][4 * g4 + 3] * inv};
         }
     }
 }

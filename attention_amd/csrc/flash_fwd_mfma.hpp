@@ -55,6 +55,11 @@ struct FlashParams {
     const uint64_t* mask_bits;  // masked kernel on a packed mask: word [(b * mask_kt + key tile) * N + query] holds the 64 keys
                                 // of the tile, bit j set = key 64 * tile + j stays (flash_mask_pack_kernel writes it)
     int32_t mask_kt;            // key tiles per row of the packed mask: ceil(N / 64)
+    int32_t d_real;             // head dimension of the tensors when it is smaller than the kernel's D (a multiple of 8 for
+                                // 16-bit tensors, of 4 for fp32), 0 = D.  The kernel then computes with D columns of which the
+                                // last D - d_real contribute nothing: Q's are zero, so whatever K holds there is multiplied
+                                // by zero (the tile requests of those columns fetch the row's first chunk again, never
+                                // memory behind the row), and V's produce output columns that are not stored.
     int64_t stride_b, stride_n, stride_h;           // Q and O
     int64_t kv_stride_b, kv_stride_n, kv_stride_h;  // K and V
     int32_t N;                  // sequence length (dense) / longest sequence (ragged)
@@ -325,6 +330,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
     const int64_t sn = p.stride_n;
     const int64_t skv = p.kv_stride_n;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int d_real = (p.d_real > 0 && p.d_real < D) ? p.d_real : D;
 
     // ---- per-lane DMA offsets (bytes from the first row of a tile), fixed for the whole kernel ------
     int dma_off_k[TL::kInstrPerWave], dma_off_v[TL::kInstrPerWave];
@@ -332,15 +338,16 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
     for (int i = 0; i < TL::kInstrPerWave; ++i) {
         const int r = (wave * TL::kInstrPerWave + i) * TL::kRowsPerInstr + lane / TL::kChunks;
         const int pc = lane % TL::kChunks;
-        dma_off_k[i] = (int)(r * skv * 2) + ((pc ^ TL::fk(r)) << 4);
-        dma_off_v[i] = (int)(r * skv * 2) + ((pc ^ TL::fv(r)) << 4);
+        const int ck = pc ^ TL::fk(r), cv = pc ^ TL::fv(r);  // the 8-element chunk of the row that belongs at this lane's place
+        dma_off_k[i] = (int)(r * skv * 2) + ((8 * ck < d_real ? ck : 0) << 4);
+        dma_off_v[i] = (int)(r * skv * 2) + ((8 * cv < d_real ? cv : 0) << 4);
     }
     // Keys k0.. of this head into a buffer pair.  Bytes from the tile's first row to the end of the
     // sequence's last row bound the descriptor, so the rows of a ragged last tile that do not exist
     // read as zeros (their scores are masked; zero V rows keep 0 * x finite).
     auto dma_both = [&](int k0, unsigned char* dst_k, unsigned char* dst_v) {
         // (a tile that starts at or behind the end of the sequence touches no memory and lands as zeros)
-        const int64_t rem = k0 < L ? (int64_t)(L - k0 - 1) * skv * 2 + 2 * D : 0;
+        const int64_t rem = k0 < L ? (int64_t)(L - k0 - 1) * skv * 2 + 2 * d_real : 0;  // the last row ends with its own d
         const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
         dma_tile<D>(gk + (int64_t)k0 * skv, nrec, dma_off_k, dst_k, wave_u);
         dma_tile<D>(gv + (int64_t)k0 * skv, nrec, dma_off_v, dst_v, wave_u);
@@ -385,7 +392,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
             const float c = p.scale_log2;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const u32x4 raw = *reinterpret_cast<const u32x4*>(src + 16 * ks);
+                const u32x4 raw = 16 * ks + 8 * half < d_real ? *reinterpret_cast<const u32x4*>(src + 16 * ks) : u32x4{0u, 0u, 0u, 0u};
                 u32x4 sc;
 #pragma unroll
                 for (int w = 0; w < 4; ++w) sc[w] = pack2<T>(lo_f32<T>(raw[w]) * c, hi_f32<T>(raw[w]) * c);
@@ -635,7 +642,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                     const f32x16& a = oacc[mb];
                     const u32x2 w = u32x2{pack2<T>(a[4 * g4 + 0] * inv, a[4 * g4 + 1] * inv),
                                           pack2<T>(a[4 * g4 + 2] * inv, a[4 * g4 + 3] * inv)};
-                    *reinterpret_cast<u32x2*>(dst + 32 * mb + 8 * g4) = w;
+                    if (32 * mb + 8 * g4 + 4 * half < d_real) *reinterpret_cast<u32x2*>(dst + 32 * mb + 8 * g4) = w;
                 }
         }
         __syncthreads();  // the next query tile's first DMA reuses the buffers

@@ -225,6 +225,31 @@ def test_dense_mask_under_graph_capture_allocates_nothing(gpu):
         assert np.abs(to_host(do) - want).max() <= 2e-2, rep
 
 
+@pytest.mark.parametrize("dtype,d", [(O.BF16, 32), (O.F16, 96), (O.BF16, 8), (O.F16, 120), (O.BF16, 80), (O.F32, 32), (O.F32, 100),
+                                     (O.F32, 4), (O.F32, 72)])
+@pytest.mark.parametrize("N,causal,H,H_kv", [(150, True, 2, 1), (64, False, 3, 3), (517, True, 4, 2)])
+def test_smaller_head_dimensions_on_the_matrix_cores(gpu, dtype, d, N, causal, H, H_kv):
+    """Head dimensions below 64 / 128 (multiples of 8 for 16-bit tensors, of 4 for fp32) run on the matrix-core kernels with
+    columns that contribute nothing; the output tensor is pre-filled with NaN, every element must have been written."""
+    import torch
+    from gpu_util import to_dev, to_host, stream_ptr, TOL
+    B = 2
+    q = O.round_to(O.fill_normal((B, N, H, d), 91, 1), dtype)
+    k = O.round_to(O.fill_normal((B, N, H_kv, d), 91, 2), dtype)
+    v = O.round_to(O.fill_normal((B, N, H_kv, d), 91, 3), dtype)
+    scale = 1.0 / np.sqrt(d)
+    rep = H // H_kv
+    want = O.attention(q, np.repeat(k, rep, axis=2), np.repeat(v, rep, axis=2), B, N, H, d, scale, causal)
+    dq, dk, dv = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype)
+    do = torch.full_like(dq, float("nan"))
+    gpu.flash_fwd_gqa(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), do.data_ptr(), dtype, B, N, H, H_kv, d,
+                      (N * H * d, H * d, d), (N * H_kv * d, H_kv * d, d), scale, causal, stream_ptr())
+    torch.cuda.synchronize()
+    got = to_host(do)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16])
 @pytest.mark.parametrize("d", [64, 128])
 @pytest.mark.parametrize("causal", [False, True])

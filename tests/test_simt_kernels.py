@@ -109,6 +109,56 @@ def test_fp32_matrix_core_kernel_dense_mask(emu, N, d, causal, H_kv, dma_late):
     assert S.lds_stats(reset=True)[0] > 0
 
 
+@pytest.mark.parametrize("dma_late", [False, True])
+@pytest.mark.parametrize("dtype,d", [(O.BF16, 32), (O.F16, 96), (O.BF16, 8), (O.F16, 120), (O.F32, 32), (O.F32, 100), (O.F32, 4), (O.F32, 72)])
+@pytest.mark.parametrize("N,causal,H,H_kv", [(150, True, 2, 1), (64, False, 3, 3)])
+def test_matrix_core_kernels_smaller_head_dimensions(emu, dtype, d, N, causal, H, H_kv, dma_late):
+    """Head dimensions below the kernels' 64 / 128 (multiples of 8 for 16-bit tensors, of 4 for fp32) run on the matrix-core
+    kernels with columns that contribute nothing.  Tensors sit at the very end (or start) of guarded buffers: nothing behind
+    a row's own d elements may be read, in particular not behind the last row of the last head."""
+    B = 2
+    q = O.round_to(O.fill_normal((B, N, H, d), 25, 1), dtype)
+    k = O.round_to(O.fill_normal((B, N, H_kv, d), 25, 2), dtype)
+    v = O.round_to(O.fill_normal((B, N, H_kv, d), 25, 3), dtype)
+    scale = 1.0 / np.sqrt(d)
+    S.configure(dma_late, seed=N + d)
+    S.lds_stats(reset=True)
+    try:
+        got = flash(emu, q, k, v, dtype, B, N, H, d, scale, causal, H_kv=H_kv, front=dma_late)
+    finally:
+        S.configure(False, 1)
+    rep = H // H_kv
+    want = O.attention(q, np.repeat(k, rep, axis=2), np.repeat(v, rep, axis=2), B, N, H, d, scale, causal)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= TOL[dtype]
+    assert S.lds_stats(reset=True)[0] > 0   # a matrix-core kernel ran (the FMA kernel makes no traced LDS reads)
+
+
+def test_matrix_core_kernels_smaller_head_dimensions_ragged_and_masked(emu):
+    H, d = 2, 40
+    lens = np.array([1, 130, 0, 64, 33], np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    for dtype in (O.BF16, O.F32):
+        q, k, v = qkv((T, H, d), 26, dtype)
+        dq, dk, dv = dev(q, dtype), dev(k, dtype), dev(v, dtype)
+        do = S.guarded(S.empty_storage((T, H, d), dtype))
+        dcu = S.guarded(cu)
+        S.lds_stats(reset=True)
+        emu.flash_fwd_varlen(S.ptr(dq), S.ptr(dk), S.ptr(dv), S.ptr(do), dtype, S.ptr(dcu), len(lens), int(lens.max()), H, d,
+                             H * d, d, 0.2, True)
+        want = O.attention_varlen(q, k, v, cu, H, d, 0.2, True)
+        assert np.abs(S.from_storage(do, dtype) - want).max() <= TOL[dtype]
+        assert S.lds_stats(reset=True)[0] > 0
+        B, N = 2, 70
+        q, k, v = qkv((B, N, H, d), 27, dtype)
+        mask = (O.fill_uniform((B, N, N), 27, 6) > 0.0).astype(np.float32)
+        mask[:, np.arange(N), np.arange(N)] = 1.0
+        got = flash(emu, q, k, v, dtype, B, N, H, d, 0.2, False, mask=mask)
+        assert np.abs(got - O.attention(q, k, v, B, N, H, d, 0.2, False, mask=mask)).max() <= TOL[dtype]
+        assert S.lds_stats(reset=True)[0] > 0
+
+
 def test_fp32_matrix_core_kernel_large_scores_and_strides(emu):
     """Scores that grow along the sequence (the reference maximum is raised again and again), head-major strides."""
     B, N, H, d = 1, 200, 2, 64
