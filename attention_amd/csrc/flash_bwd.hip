@@ -383,6 +383,7 @@ static int launch_mfma_dv(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool
     f.N = p.N; f.H = p.H; f.kv_group = p.kv_group;
     f.cu_seqlens = p.cu_seqlens;
     f.scale_log2 = p.scale_log2;
+    f.d_real = p.d_real;
     if (int rc = flash_plan_launch(f, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load(), VARLEN)) return rc;
     const FlashStatsOut st{p.d_out, lse2, delta, p.rows_padded};
     const dim3 block(kFlashThreads);
@@ -433,6 +434,7 @@ static int launch_f32_mfma_dv(const FlashBwdParams& p, int64_t B, int64_t H_kv, 
     f.N = p.N; f.H = p.H; f.kv_group = p.kv_group;
     f.cu_seqlens = p.cu_seqlens;
     f.scale_log2 = p.scale_log2;
+    f.d_real = p.d_real;
     if (int rc = flash_plan_launch(f, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load(), VARLEN)) return rc;
     const FlashStatsOut st{p.d_out, lse2, delta, p.rows_padded};
     const dim3 block(kFlashThreads);
@@ -526,7 +528,10 @@ static int flash_bwd_any(const void* d_out, const void* q, const void* k, const 
     const bool strides4_ok = !(stride_b % 4) && !(stride_n % 4) && !(stride_h % 4) && !(kv_stride_b % 4) && !(kv_stride_n % 4) &&
                              !(kv_stride_h % 4) && stride_n < (int64_t(1) << 24) && kv_stride_n < (int64_t(1) << 24);
     const bool is16 = dtype == AHPC_F16 || dtype == AHPC_BF16;
-    if (!mask && (d == 64 || d == 128) && (is16 ? strides_ok : strides4_ok) && aligned16(q) &&
+    // head dimensions up to 128 in whole 16-byte pieces; one below 64 or 128 runs on the next kernel (FlashParams::d_real)
+    const bool d_ok = d <= 128 && d >= (is16 ? 8 : 4) && d % (is16 ? 8 : 4) == 0;
+    const int kernel_d = d <= 64 ? 64 : 128;
+    if (!mask && d_ok && (is16 ? strides_ok : strides4_ok) && aligned16(q) &&
         aligned16(k) && aligned16(v) && aligned16(d_out) && aligned16(d_q) && aligned16(d_k) && aligned16(d_v)) {
         FlashBwdParams m{};
         m.q = q; m.k = k; m.v = v; m.d_out = d_out;
@@ -538,9 +543,10 @@ static int flash_bwd_any(const void* d_out, const void* q, const void* k, const 
         m.N = (int32_t)N; m.H = (int32_t)H; m.kv_group = p.kv_group;
         m.scale = scale;
         m.scale_log2 = scale * kLog2e;
-        if (dtype == AHPC_F32) return launch_f32_mfma(m, B, H_kv, (int)d, causal != 0, p.lse, p.delta, st);
-        return dtype == AHPC_F16 ? launch_mfma<f16_t>(m, B, H_kv, (int)d, causal != 0, p.lse, p.delta, st)
-                                 : launch_mfma<bf16_t>(m, B, H_kv, (int)d, causal != 0, p.lse, p.delta, st);
+        m.d_real = (int32_t)d;
+        if (dtype == AHPC_F32) return launch_f32_mfma(m, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st);
+        return dtype == AHPC_F16 ? launch_mfma<f16_t>(m, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st)
+                                 : launch_mfma<bf16_t>(m, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st);
     }
     switch (dtype) {
         case AHPC_F32: return launch_simple<float>(p, B, H_kv, st);

@@ -38,10 +38,11 @@ template <int D> struct F32Tile {
     static constexpr int kBytes = kF32Keys * RB;
     __device__ static int f(int r) { return r & (CH - 1); }
     // byte offset of the load instruction i of this wavefront: row, and the chunk that belongs at the lane's place
-    __device__ static int dma_off(int wave, int lane, int i, int64_t stride_elems) {
+    // (a head dimension d below D: the columns from d on fetch the row's first chunk again, FlashParams::d_real)
+    __device__ static int dma_off(int wave, int lane, int i, int64_t stride_elems, int d) {
         const int r = (wave * IPW + i) * RPI + lane / CH;
-        const int pc = lane % CH;
-        return (int)(r * stride_elems * 4) + ((pc ^ f(r)) << 4);
+        const int ch = (lane % CH) ^ f(r);
+        return (int)(r * stride_elems * 4) + ((4 * ch < d ? ch : 0) << 4);
     }
     // 16 bytes of row `col`: logical chunk 2m + half
     __device__ static int row_off(int col, int half, int m) { return col * RB + (((2 * m + half) ^ f(col)) << 4); }
@@ -99,12 +100,13 @@ __global__ __launch_bounds__(kFlashThreads, (D == 128 ? 1 : 2)) void flash_bwd_d
     const int64_t sn = p.stride_n;
     const int64_t skv = p.kv_stride_n;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int d_real = (p.d_real > 0 && p.d_real < D) ? p.d_real : D;
 
     int dma_off[TL::IPW];
 #pragma unroll
-    for (int i = 0; i < TL::IPW; ++i) dma_off[i] = TL::dma_off(wave, lane, i, skv);
+    for (int i = 0; i < TL::IPW; ++i) dma_off[i] = TL::dma_off(wave, lane, i, skv, d_real);
     auto dma_both = [&](int k0, unsigned char* dst_k, unsigned char* dst_v) {
-        const int64_t rem = k0 < L ? (int64_t)(L - k0 - 1) * skv * 4 + RB : 0;
+        const int64_t rem = k0 < L ? (int64_t)(L - k0 - 1) * skv * 4 + 4 * d_real : 0;
         const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
         f32_dma_tile<D>(gk + (int64_t)k0 * skv, nrec, dma_off, dst_k, wave_u);
         f32_dma_tile<D>(gv + (int64_t)k0 * skv, nrec, dma_off, dst_v, wave_u);
@@ -139,9 +141,10 @@ __global__ __launch_bounds__(kFlashThreads, (D == 128 ? 1 : 2)) void flash_bwd_d
             const float* sd = gdo + (int64_t)row * sn + 4 * half;
 #pragma unroll
             for (int m = 0; m < MS; ++m) {
-                const f32x4 raw = *reinterpret_cast<const f32x4*>(sq + 8 * m);
+                const bool there = 8 * m + 4 * half < d_real;  // columns the tensors have
+                const f32x4 raw = there ? *reinterpret_cast<const f32x4*>(sq + 8 * m) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
                 qreg[m] = f32x4{raw[0] * c, raw[1] * c, raw[2] * c, raw[3] * c};
-                doreg[m] = *reinterpret_cast<const f32x4*>(sd + 8 * m);
+                doreg[m] = there ? *reinterpret_cast<const f32x4*>(sd + 8 * m) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             }
         }
         f32x16 neg_lse, neg_delta, zero;
@@ -243,8 +246,9 @@ __global__ __launch_bounds__(kFlashThreads, (D == 128 ? 1 : 2)) void flash_bwd_d
             for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4)
-                    *reinterpret_cast<f32x4*>(dst + 32 * mb + 8 * g4) =
-                        f32x4{acc[mb][4 * g4] * sc, acc[mb][4 * g4 + 1] * sc, acc[mb][4 * g4 + 2] * sc, acc[mb][4 * g4 + 3] * sc};
+                    if (32 * mb + 8 * g4 + 4 * half < d_real)
+                        *reinterpret_cast<f32x4*>(dst + 32 * mb + 8 * g4) =
+                            f32x4{acc[mb][4 * g4] * sc, acc[mb][4 * g4 + 1] * sc, acc[mb][4 * g4 + 2] * sc, acc[mb][4 * g4 + 3] * sc};
         }
     }
 }
@@ -284,10 +288,11 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 2 ? 1 : 2)) void flash_bwd_
     const int64_t sn = p.stride_n;
     const int64_t skv = p.kv_stride_n;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int d_real = (p.d_real > 0 && p.d_real < D) ? p.d_real : D;
 
     int dma_off[TL::IPW];
 #pragma unroll
-    for (int i = 0; i < TL::IPW; ++i) dma_off[i] = TL::dma_off(wave, lane, i, sn);
+    for (int i = 0; i < TL::IPW; ++i) dma_off[i] = TL::dma_off(wave, lane, i, sn, d_real);
     int row_off[MS];
 #pragma unroll
     for (int m = 0; m < MS; ++m) row_off[m] = TL::row_off(col, half, m);
@@ -312,9 +317,10 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 2 ? 1 : 2)) void flash_bwd_
             const float* sv = gv + (int64_t)krow * skv + 4 * half;
 #pragma unroll
             for (int m = 0; m < MS; ++m) {
-                const f32x4 raw = *reinterpret_cast<const f32x4*>(sk + 8 * m);
+                const bool there = 8 * m + 4 * half < d_real;  // columns the tensors have
+                const f32x4 raw = there ? *reinterpret_cast<const f32x4*>(sk + 8 * m) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
                 kreg[m] = f32x4{raw[0] * c, raw[1] * c, raw[2] * c, raw[3] * c};
-                if constexpr (kDoK) vreg[m] = *reinterpret_cast<const f32x4*>(sv + 8 * m);
+                if constexpr (kDoK) vreg[m] = there ? *reinterpret_cast<const f32x4*>(sv + 8 * m) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             }
         }
         f32x16 zero;
@@ -338,7 +344,7 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 2 ? 1 : 2)) void flash_bwd_
             const float* const delta = p.neg_delta + ((int64_t)b * p.H + h) * p.rows_padded;
 
             auto dma_both = [&](int i0, unsigned char* dst_q, unsigned char* dst_o) {
-                const int64_t rem = i0 < L ? (int64_t)(L - i0 - 1) * sn * 4 + RB : 0;
+                const int64_t rem = i0 < L ? (int64_t)(L - i0 - 1) * sn * 4 + 4 * d_real : 0;
                 const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
                 f32_dma_tile<D>(gq + (int64_t)i0 * sn, nrec, dma_off, dst_q, wave_u);
                 f32_dma_tile<D>(gdo + (int64_t)i0 * sn, nrec, dma_off, dst_o, wave_u);
@@ -449,8 +455,9 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 2 ? 1 : 2)) void flash_bwd_
             for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4)
-                    *reinterpret_cast<f32x4*>(dst + 32 * mb + 8 * g4) =
-                        f32x4{acc[mb][4 * g4] * sc, acc[mb][4 * g4 + 1] * sc, acc[mb][4 * g4 + 2] * sc, acc[mb][4 * g4 + 3] * sc};
+                    if (32 * mb + 8 * g4 + 4 * half < d_real)
+                        *reinterpret_cast<f32x4*>(dst + 32 * mb + 8 * g4) =
+                            f32x4{acc[mb][4 * g4] * sc, acc[mb][4 * g4 + 1] * sc, acc[mb][4 * g4 + 2] * sc, acc[mb][4 * g4 + 3] * sc};
         }
     }
 }

@@ -52,6 +52,7 @@ struct FlashBwdParams {
     int32_t total_kv, per_xcd_kv;   // dK/dV kernel: workgroups (B * H_kv * n_tiles) and ceil(that / 8)
     float scale;
     float scale_log2;           // scale * log2(e)
+    int32_t d_real;             // head dimension of the tensors when smaller than the kernels' D, 0 = D (FlashParams::d_real)
 };
 
 // Workgroup id -> (sequence * heads + head, tile).  Both kernels are launched on a 1-D grid of 8 * per_xcd
@@ -89,13 +90,14 @@ __device__ inline u32x4 pack_operand(const f32x16& x, int r0) {
                  pack2<T>(x[r0 + 6], x[r0 + 7])};
 }
 
-// Loads the row `row` of a [rows][D] tensor as B operands (8 consecutive elements per k-step), scaled by c.
+// Loads the row `row` of a [rows][d] tensor as B operands (8 consecutive elements per k-step), scaled by c; elements from
+// d on (a head dimension below the kernel's) are zero and not read.
 template <typename T, int KS>
-__device__ inline void load_row_operands(u32x4 (&reg)[KS], const T* row_ptr, int half, float c) {
+__device__ inline void load_row_operands(u32x4 (&reg)[KS], const T* row_ptr, int half, float c, int d) {
     const T* src = row_ptr + 8 * half;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-        const u32x4 raw = *reinterpret_cast<const u32x4*>(src + 16 * ks);
+        const u32x4 raw = 16 * ks + 8 * half < d ? *reinterpret_cast<const u32x4*>(src + 16 * ks) : u32x4{0u, 0u, 0u, 0u};
         u32x4 sc;
 #pragma unroll
         for (int w = 0; w < 4; ++w) sc[w] = pack2<T>(lo_f32<T>(raw[w]) * c, hi_f32<T>(raw[w]) * c);
@@ -104,9 +106,9 @@ __device__ inline void load_row_operands(u32x4 (&reg)[KS], const T* row_ptr, int
 }
 
 // Stores the transposed accumulators of one output row (a lane holds 4 runs of 4 consecutive elements per
-// 32-element block), scaled by f.
+// 32-element block), scaled by f; elements from d on do not exist.
 template <typename T, int MB>
-__device__ inline void store_row(T* dst_row, const f32x16 (&acc)[MB], int half, float f) {
+__device__ inline void store_row(T* dst_row, const f32x16 (&acc)[MB], int half, float f, int d) {
     T* dst = dst_row + 4 * half;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -114,7 +116,7 @@ __device__ inline void store_row(T* dst_row, const f32x16 (&acc)[MB], int half, 
         for (int g4 = 0; g4 < 4; ++g4) {
             const f32x16& a = acc[mb];
             const u32x2 w = u32x2{pack2<T>(a[4 * g4 + 0] * f, a[4 * g4 + 1] * f), pack2<T>(a[4 * g4 + 2] * f, a[4 * g4 + 3] * f)};
-            *reinterpret_cast<u32x2*>(dst + 32 * mb + 8 * g4) = w;
+            if (32 * mb + 8 * g4 + 4 * half < d) *reinterpret_cast<u32x2*>(dst + 32 * mb + 8 * g4) = w;
         }
 }
 
@@ -159,16 +161,18 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
     const int64_t sn = p.stride_n;
     const int64_t skv = p.kv_stride_n;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int d_real = (p.d_real > 0 && p.d_real < D) ? p.d_real : D;
 
     int dma_off[TL::kInstrPerWave];
 #pragma unroll
     for (int i = 0; i < TL::kInstrPerWave; ++i) {
         const int r = (wave * TL::kInstrPerWave + i) * TL::kRowsPerInstr + lane / TL::kChunks;
         const int pc = lane % TL::kChunks;
-        dma_off[i] = (int)(r * skv * 2) + ((pc ^ TL::fb(r)) << 4);
+        const int ch = pc ^ TL::fb(r);  // the row's chunk that belongs here; columns from d_real on fetch the first chunk again
+        dma_off[i] = (int)(r * skv * 2) + ((8 * ch < d_real ? ch : 0) << 4);
     }
     auto dma_both = [&](int k0, unsigned char* dst_k, unsigned char* dst_v) {
-        const int64_t rem = (int64_t)(L - k0 - 1) * skv * 2 + 2 * D;
+        const int64_t rem = (int64_t)(L - k0 - 1) * skv * 2 + 2 * d_real;
         const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
         dma_tile<D>(gk + (int64_t)k0 * skv, nrec, dma_off, dst_k, wave_u);
         dma_tile<D>(gv + (int64_t)k0 * skv, nrec, dma_off, dst_v, wave_u);
@@ -200,8 +204,8 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
         const int qrow = qw + col;
         const int row = qrow < L ? qrow : L - 1;
         u32x4 qreg[KS], doreg[KS];
-        load_row_operands<T, KS>(qreg, gq + (int64_t)row * sn, half, p.scale_log2);
-        load_row_operands<T, KS>(doreg, gdo + (int64_t)row * sn, half, 1.0f);
+        load_row_operands<T, KS>(qreg, gq + (int64_t)row * sn, half, p.scale_log2, d_real);
+        load_row_operands<T, KS>(doreg, gdo + (int64_t)row * sn, half, 1.0f, d_real);
         const int64_t stat = ((int64_t)b * p.H + h) * p.rows_padded + qrow;  // qrow < rows_padded always
         f32x16 neg_lse, neg_delta;
         {
@@ -316,7 +320,7 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
             step(lds_k0, lds_v0, lds_k1, lds_v1, t);
             if (t + 1 < n_tiles) step(lds_k1, lds_v1, lds_k0, lds_v0, t + 1);
         }
-        if (qrow < L) store_row<T, MB>(static_cast<T*>(p.d_q) + base + (int64_t)qrow * sn, acc, half, p.scale);
+        if (qrow < L) store_row<T, MB>(static_cast<T*>(p.d_q) + base + (int64_t)qrow * sn, acc, half, p.scale, d_real);
     }
 }
 
@@ -363,13 +367,15 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
     const int64_t sn = p.stride_n;
     const int64_t skv = p.kv_stride_n;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int d_real = (p.d_real > 0 && p.d_real < D) ? p.d_real : D;
 
     int dma_off[TL::kInstrPerWave];
 #pragma unroll
     for (int i = 0; i < TL::kInstrPerWave; ++i) {
         const int r = (wave * TL::kInstrPerWave + i) * TL::kRowsPerInstr + lane / TL::kChunks;
         const int pc = lane % TL::kChunks;
-        dma_off[i] = (int)(r * sn * 2) + ((pc ^ TL::fb(r)) << 4);
+        const int ch = pc ^ TL::fb(r);
+        dma_off[i] = (int)(r * sn * 2) + ((8 * ch < d_real ? ch : 0) << 4);
     }
     int row_off[KS];
 #pragma unroll
@@ -391,8 +397,8 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
         const int key = kw + col;
         const int krow = key < L ? key : L - 1;
         u32x4 kreg[KS], vreg[KS];
-        load_row_operands<T, KS>(kreg, gk + (int64_t)krow * skv, half, p.scale_log2);
-        if constexpr (kDoK) load_row_operands<T, KS>(vreg, gv + (int64_t)krow * skv, half, 1.0f);
+        load_row_operands<T, KS>(kreg, gk + (int64_t)krow * skv, half, p.scale_log2, d_real);
+        if constexpr (kDoK) load_row_operands<T, KS>(vreg, gv + (int64_t)krow * skv, half, 1.0f, d_real);
 
         f32x16 acc_k[MB], acc_v[MB];
 #pragma unroll
@@ -418,7 +424,7 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
 
             auto dma_both = [&](int i0, unsigned char* dst_q, unsigned char* dst_o, unsigned char* dst_s) {
                 // (a tile that starts at or behind the end of the sequence touches no memory and lands as zeros)
-                const int64_t rem = i0 < L ? (int64_t)(L - i0 - 1) * sn * 2 + 2 * D : 0;
+                const int64_t rem = i0 < L ? (int64_t)(L - i0 - 1) * sn * 2 + 2 * d_real : 0;
                 const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
                 dma_tile<D>(gq + (int64_t)i0 * sn, nrec, dma_off, dst_q, wave_u);
                 dma_tile<D>(gdo + (int64_t)i0 * sn, nrec, dma_off, dst_o, wave_u);
@@ -573,8 +579,8 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
             __syncthreads();  // the next head's first load reuses the buffers
         }
         if (key < L) {
-            if constexpr (kDoK) store_row<T, MB>(static_cast<T*>(p.d_k) + kv_base + (int64_t)key * skv, acc_k, half, p.scale);
-            if constexpr (kDoV) store_row<T, MB>(static_cast<T*>(p.d_v) + kv_base + (int64_t)key * skv, acc_v, half, 1.0f);
+            if constexpr (kDoK) store_row<T, MB>(static_cast<T*>(p.d_k) + kv_base + (int64_t)key * skv, acc_k, half, p.scale, d_real);
+            if constexpr (kDoV) store_row<T, MB>(static_cast<T*>(p.d_v) + kv_base + (int64_t)key * skv, acc_v, half, 1.0f, d_real);
         }
     }
 }

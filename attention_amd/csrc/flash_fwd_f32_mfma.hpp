@@ -314,6 +314,7 @@ __device__ __forceinline__ void flash_fwd_f32_mfma_body(const FlashParams& p, co
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                     for (int g4 = 0; g4 < 4; ++g4) {
+                        if (32 * mb + 8 * g4 + 4 * half >= d_real) continue;  // columns the tensors do not have
                         const f32x4 w = *reinterpret_cast<const f32x4*>(src + 32 * mb + 8 * g4);
                         part += oacc[mb][4 * g4] * w[0] + oacc[mb][4 * g4 + 1] * w[1] + oacc[mb][4 * g4 + 2] * w[2] +
                                 oacc[mb][4 * g4 + 3] * w[3];

@@ -620,6 +620,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                     for (int g4 = 0; g4 < 4; ++g4) {
+                        if (32 * mb + 8 * g4 + 4 * half >= d_real) continue;  // columns the tensors do not have
                         const u32x2 w = *reinterpret_cast<const u32x2*>(src + 32 * mb + 8 * g4);
                         const f32x16& a = oacc[mb];
                         part += a[4 * g4 + 0] * lo_f32<T>(w[0]) + a[4 * g4 + 1] * hi_f32<T>(w[0]) +

@@ -668,6 +668,25 @@ def test_backward_fp32_matrix_core_kernels(emu, tuned, B, N, H, H_kv, d, causal,
     assert reads > 0 and read_conflicts == 0   # the matrix-core kernels ran (the FMA kernels make no traced reads)
 
 
+@pytest.mark.parametrize("dma_late", [False, True])
+@pytest.mark.parametrize("dtype,d", [(O.BF16, 32), (O.F16, 96), (O.BF16, 8), (O.F32, 32), (O.F32, 100), (O.F32, 4)])
+@pytest.mark.parametrize("N,causal,H,H_kv", [(150, True, 2, 1), (64, False, 2, 2)])
+def test_backward_smaller_head_dimensions(emu, dtype, d, N, causal, H, H_kv, dma_late):
+    """Head dimensions below the kernels' 64 / 128 in the backward: the matrix-core kernels with columns that contribute
+    nothing, tensors at either end of guarded buffers."""
+    B = 1
+    q, k, v, do = bwd_inputs(B, N, H, H_kv, d, 39, dtype)
+    scale = 1.0 / np.sqrt(d)
+    S.configure(dma_late, seed=N + d)
+    S.lds_stats(reset=True)
+    try:
+        got = backward(emu, q, k, v, do, dtype, B, N, H, H_kv, d, scale, causal, front=dma_late)
+    finally:
+        S.configure(False, 1)
+    check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), dtype)
+    assert S.lds_stats(reset=True)[0] > 0   # the matrix-core kernels ran
+
+
 # ---- LDS bank conflicts (model: 64 banks of 4 bytes) --------------------------------------------------------
 @pytest.mark.parametrize("dtype,d", [(O.BF16, 128), (O.F16, 64)])
 def test_operand_reads_are_free_of_bank_conflicts(emu, dtype, d):

@@ -55,6 +55,18 @@ def test_fp32_tensors(gpu, B, N, H, H_kv, d, causal):
     check(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), O.F32)
 
 
+@pytest.mark.parametrize("dtype,d", [(O.BF16, 32), (O.F16, 96), (O.BF16, 8), (O.F16, 120), (O.F32, 100), (O.F32, 4), (O.F32, 72)])
+@pytest.mark.parametrize("N,causal,H,H_kv", [(150, True, 2, 1), (64, False, 3, 3), (517, True, 4, 2)])
+def test_smaller_head_dimensions_on_the_matrix_cores(gpu, dtype, d, N, causal, H, H_kv):
+    """Head dimensions below 64 / 128 (multiples of 8 for 16-bit tensors, of 4 for fp32): the matrix-core kernels with
+    columns that contribute nothing; gradients are pre-filled with NaN, every element must have been written."""
+    B = 2
+    q, k, v, do = inputs(B, N, H, H_kv, d, 33, dtype)
+    scale = 1.0 / np.sqrt(d)
+    got = run_backward(gpu, q, k, v, do, dtype, B, N, H, H_kv, d, scale, causal)
+    check(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), dtype)
+
+
 def test_dense_mask(gpu):
     B, N, H, d = 2, 37, 2, 64
     q, k, v, do = inputs(B, N, H, H, d, 32, O.F32)
