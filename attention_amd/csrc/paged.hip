@@ -183,7 +183,10 @@ struct DecodeParams {
     float* part_ml;   // [B][n_chunks][H][2]  (m in log2 units, l; l carries a minus sign when the chunk met a missing page)
     int64_t* dump_offsets;  // index-dump launches only: [B][max_len] element offsets of the token rows the kernel addresses
     int64_t max_pages;
-    int32_t B, H, d, P;       // H = query heads
+    int32_t B, H, d, P;       // H = query heads; d = head dimension of the tensors
+    int32_t d_kernel;         // head dimension the lane-per-element kernel is instantiated for: 32, 64, 128 or 256, the
+                              // smallest that holds d.  The lanes of a head whose 16-byte piece lies at or beyond d
+                              // carry a zero query, re-read the row's first piece and store nothing.
     int32_t H_kv;             // heads in the pool; H / H_kv consecutive query heads share one
     int32_t chunk_tokens, n_chunks;  // longest chunk (a multiple of P, at most 64 pages) and how many the longest sequence needs
     int32_t balanced;         // 1: a sequence cuts itself into equal chunks (see decode_chunk_len); 0: every chunk is chunk_tokens long
@@ -305,6 +308,9 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     const bool head_ok = h_raw < p.H_kv;
     const int h = head_ok ? h_raw : p.H_kv - 1;
     const int e0 = (lane % LPH) * EPL;
+    const int d = p.d;                    // the tensors' head dimension, D or less
+    const bool piece_ok = e0 < d;         // this lane's 16-byte piece exists
+    const int e_ld = piece_ok ? e0 : 0;   // where it reads K and V from
     const int P = PT ? PT : p.P;
 
     const int64_t row = p.batch_rows ? p.batch_rows[b] : b;
@@ -334,7 +340,8 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
 #pragma unroll
             for (int e = 0; e < EPL; ++e) zero[e] = 0.0f;
 #pragma unroll
-            for (int g = 0; g < G; ++g) store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + h * G + g) * D + e0, zero);
+            for (int g = 0; g < G; ++g)
+                if (piece_ok) store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + h * G + g) * d + e0, zero);
         }
         return;
     }
@@ -353,7 +360,12 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     if constexpr (!DUMP) {
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            load_qo_vec<EPL>(p.q, p.qo_dtype, ((int64_t)b * p.H + h * G + g) * D + e0, qf[g]);
+            if (piece_ok) {
+                load_qo_vec<EPL>(p.q, p.qo_dtype, ((int64_t)b * p.H + h * G + g) * d + e0, qf[g]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) qf[g][e] = 0.0f;
+            }
             if (kPacked) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) qp[g][i] = pack2<TP>(qf[g][2 * i], qf[g][2 * i + 1]);
@@ -362,8 +374,8 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     }
 
     // byte offset of this lane's piece inside a token row; token rows are tok_bytes apart
-    const uint32_t lane_off = (uint32_t)((h * D + e0) * (int)sizeof(T));
-    const int64_t tok_bytes = (int64_t)p.H_kv * D * (int64_t)sizeof(T);
+    const uint32_t lane_off = (uint32_t)((h * d + e_ld) * (int)sizeof(T));
+    const int64_t tok_bytes = (int64_t)p.H_kv * d * (int64_t)sizeof(T);
     const char* const kbase = static_cast<const char*>(p.k_pool);
     const char* const vbase = static_cast<const char*>(p.v_pool);
 
@@ -492,12 +504,14 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
             float res[EPL];
 #pragma unroll
             for (int e = 0; e < EPL; ++e) res[e] = acc[g][e] * inv;
-            store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + hq) * D + e0, res);
+            if (piece_ok) store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + hq) * d + e0, res);
         } else {
             const int64_t slot = ((int64_t)b * p.n_chunks + chunk) * p.H + hq;
-            f32x4* dst = reinterpret_cast<f32x4*>(p.part_o + slot * D + e0);
+            f32x4* dst = reinterpret_cast<f32x4*>(p.part_o + slot * d + e_ld);
+            if (piece_ok) {
 #pragma unroll
-            for (int e = 0; e < EPL; e += 4) dst[e / 4] = f32x4{acc[g][e], acc[g][e + 1], acc[g][e + 2], acc[g][e + 3]};
+                for (int e = 0; e < EPL; e += 4) dst[e / 4] = f32x4{acc[g][e], acc[g][e + 1], acc[g][e + 2], acc[g][e + 3]};
+            }
             if (lane % LPH == 0) {
                 p.part_ml[slot * 2] = m[g];
                 p.part_ml[slot * 2 + 1] = stopped ? -l[g] : l[g];  // l >= 0, and -(0.0f) still carries the sign
@@ -612,7 +626,7 @@ static DecodePlan plan_decode(int64_t B, int64_t H_kv, int64_t group, int64_t ro
 
 template <typename T, int PT, int G>
 static int launch_decode_dpg(const DecodeParams& p, dim3 grid, dim3 block, hipStream_t st) {
-    switch (p.d) {
+    switch (p.d_kernel) {
         case 32: hipLaunchKernelGGL((paged_decode_kernel<T, 32, PT, G>), grid, block, 0, st, p); break;
         case 64: hipLaunchKernelGGL((paged_decode_kernel<T, 64, PT, G>), grid, block, 0, st, p); break;
         case 128: hipLaunchKernelGGL((paged_decode_kernel<T, 128, PT, G>), grid, block, 0, st, p); break;
@@ -848,13 +862,17 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     if (qo_dtype < AHPC_F32 || qo_dtype > AHPC_BF16 || pool_dtype < AHPC_F32 || pool_dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
     if (B <= 0 || B > 65535 || max_len <= 0 || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;
     if ((max_len + P - 1) / P > max_pages) return AHPC_ERR_BAD_SHAPE;
-    if (d != 32 && d != 64 && d != 128 && d != 256) return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+    // head dimensions up to 256 in whole 16-byte pieces of the pool's type; the lane-per-element kernel is instantiated
+    // for 32, 64, 128 and 256 and takes the smallest that holds d (DecodeParams::d_kernel)
+    const int64_t piece = pool_dtype == AHPC_F32 ? 4 : 8;
+    if (d > 256 || d < piece || (d % piece)) return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+    const int64_t d_kernel = d <= 32 ? 32 : d <= 64 ? 64 : d <= 128 ? 128 : 256;
     if ((reinterpret_cast<uintptr_t>(k_pool) & 15u) || (reinterpret_cast<uintptr_t>(v_pool) & 15u) ||
         (reinterpret_cast<uintptr_t>(q) & 15u) || (reinterpret_cast<uintptr_t>(o) & 15u))
         return AHPC_ERR_BAD_ALIGNMENT;
     if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
 
-    const int lph = (int)(d * (pool_dtype == AHPC_F32 ? 4 : 2) / 16);  // lanes that hold one head of a token
+    const int lph = (int)(d_kernel * (pool_dtype == AHPC_F32 ? 4 : 2) / 16);  // lanes that hold one head of a token
     const int hpw = 64 / lph;
     const int64_t matrix_from = tuning().decode_matrix_min_group.load();
     const bool use_mfma = mfma_shape && (group >= 16 || group >= matrix_from);
@@ -873,6 +891,7 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     p.part_ml = p.part_o ? p.part_o + B * n_chunks * H * d : nullptr;
     p.max_pages = max_pages;
     p.B = (int32_t)B; p.H = (int32_t)H; p.d = (int32_t)d; p.P = (int32_t)P;
+    p.d_kernel = (int32_t)d_kernel;
     p.H_kv = (int32_t)H_kv;
     p.chunk_tokens = (int32_t)chunk; p.n_chunks = (int32_t)n_chunks;
     p.balanced = 1;
@@ -949,6 +968,7 @@ int ahpc_hip_paged_gather_indices(const int32_t* block_table, const int32_t* seq
         p.dump_offsets = offsets;
         p.max_pages = max_pages;
         p.B = (int32_t)B; p.H = (int32_t)H; p.H_kv = (int32_t)H; p.d = (int32_t)d; p.P = (int32_t)P;
+        p.d_kernel = (int32_t)d;
         p.chunk_tokens = (int32_t)chunk; p.n_chunks = (int32_t)n_chunks;
         p.max_len = (int32_t)max_len;
         const dim3 grid(1, (unsigned)n_chunks, (unsigned)B), block(64);

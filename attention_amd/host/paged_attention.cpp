@@ -142,8 +142,11 @@ void PagedAttention::configure(const AttentionParams& params, const PerformanceC
     }
     if (params.page_size == 0) throw AttentionException(AttentionError::INVALID_PARAMETERS, "page_size must be positive");
     const size_t d = params.head_dimension;
-    if (d != 32 && d != 64 && d != 128 && d != 256)
-        throw AttentionException(AttentionError::UNSUPPORTED_OPERATION, "paged decode supports head_dimension 32, 64, 128, 256");
+    // whole 16-byte pieces of the cache's type, which is known at the first append only: a multiple of 4 passes here,
+    // a 16-bit cache then needs a multiple of 8 (the decode call reports it otherwise)
+    if (d > 256 || d % 4)
+        throw AttentionException(AttentionError::UNSUPPORTED_OPERATION,
+                                 "paged decode supports head_dimension up to 256 in whole 16-byte pieces");
     int n = 0;
     ahpc_hip_device_count(&n);
     if (n < 1) throw AttentionException(AttentionError::BACKEND_NOT_AVAILABLE, "no HIP device");

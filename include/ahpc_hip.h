@@ -291,7 +291,9 @@ int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype,
  * gather_indices calls take H = H_kv), q and o hold H = g * H_kv heads, g in {1, 2, 4, 8}; query
  * head h reads pool head h / g.  Every K/V byte is still read once and serves g query heads.
  * g = 16 and 32 (up to multi-query attention with 32 heads) are served by a matrix-core kernel that needs
- * an fp16/bf16 pool, d in {64, 128} and P = 16; other combinations return AHPC_ERR_UNSUPPORTED_GROUP.
+ * an fp16/bf16 pool, d in {64, 128} and P = 16; other combinations return AHPC_ERR_UNSUPPORTED_GROUP.  The head dimension
+ * may be anything up to 256 in whole 16-byte pieces of the pool's type (a multiple of 8 for fp16/bf16 pools, of 4 for
+ * fp32 ones); AHPC_ERR_UNSUPPORTED_HEAD_DIM otherwise.
  * Workspace size: ahpc_hip_paged_decode_workspace_bytes with the QUERY head count. */
 int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype,
                               const void* k_pool, const void* v_pool, int pool_dtype,
@@ -318,7 +320,7 @@ int ahpc_hip_paged_decode_noalloc(const void* q, void* o, int qo_dtype,
 
 /* What the decode kernel gathers: offsets[b*max_len + t] = the element offset in the pool of (token t, head 0,
  * element 0) of batch entry b, or -1 for a token the decode does not attend to (t >= seq_lens[row], or at and behind
- * the first negative table entry of the row).  For the head dimensions the decode kernel takes (32, 64, 128, 256) the
+ * the first negative table entry of the row).  For the head dimensions the decode kernel is instantiated for (32, 64, 128, 256) the
  * values are written by that kernel itself, launched in a reporting mode in which the expression that addresses a
  * token row feeds a store instead of the loads; for other head dimensions by the index function of append and
  * read-back.  Lets a test hold the GPU's gather indices bit for bit against the index math of the reference

@@ -75,7 +75,7 @@ def test_paged_decode_argument_checks(lib):
     assert decode(lib, qo=5) == BAD_DTYPE and decode(lib, pool=-2) == BAD_DTYPE
     assert decode(lib, B=0) == BAD_SHAPE and decode(lib, max_len=0) == BAD_SHAPE
     assert decode(lib, max_len=65, max_pages=4) == BAD_SHAPE           # the table row cannot hold that many tokens
-    assert decode(lib, d=48) == HEAD_DIM
+    assert decode(lib, d=44) == HEAD_DIM and decode(lib, d=264) == HEAD_DIM   # whole 16-byte pieces of an fp16 row, up to 256
     assert decode(lib, kp=P + 8) == BAD_ALIGNMENT and decode(lib, o=P + 2) == BAD_ALIGNMENT
     assert decode(lib, H=6, Hkv=2) == BAD_GROUP                        # 3 query heads per K/V head
     assert decode(lib, H=6, Hkv=4) == BAD_SHAPE                        # does not divide

@@ -83,6 +83,24 @@ def test_decode_small(gpu, dtype, H, d, P):
         assert np.abs(got - want).max() <= tol, f"chunk={chunk}"
 
 
+@pytest.mark.parametrize("dtype,H,d,P", [(O.BF16, 4, 96, 16), (O.F16, 8, 80, 16), (O.F32, 3, 100, 8), (O.BF16, 2, 8, 16), (O.F32, 4, 4, 16),
+                                        (O.F16, 6, 200, 4), (O.BF16, 32, 112, 16)])
+def test_decode_other_head_dimensions(gpu, dtype, H, d, P):
+    """Head dimensions in whole 16-byte pieces that are not 32, 64, 128 or 256 run on the kernel of the next size; unused
+    slots and pages of the pool are NaN."""
+    from gpu_util import to_dev
+    B = 5
+    q, kp, vp, table, lens, _, _ = build_problem(B, H, d, P, [33, 1, 16, 150, 700], 43, dtype)
+    scale = 1.0 / np.sqrt(d)
+    want = O.paged_decode(q, kp, vp, table, lens, None, B, H, d, P, scale)
+    kp_n, vp_n, _ = poison_unused(kp, vp, table, lens, P, H, d)
+    kd, vd = to_dev(kp_n, dtype), to_dev(vp_n, dtype)
+    for chunk in (0, 2 * P, 16 * P):
+        got = gpu_decode(gpu, q, kd, vd, table, lens, None, B, H, d, P, dtype, dtype, scale, chunk)
+        assert np.isfinite(got).all()
+        assert np.abs(got - want).max() <= (1e-4 if dtype == O.F32 else 2e-2), f"chunk={chunk}"
+
+
 def test_decode_split_count_invariance_and_fp32_query_on_fp16_pool(gpu):
     from gpu_util import to_dev
     B, H, d, P = 3, 8, 128, 16
@@ -306,7 +324,7 @@ def test_bad_arguments_are_rejected_without_launch(gpu):
     x = torch.zeros(4096, device="cuda")
     p = x.data_ptr()
     with pytest.raises(gpu.HipError):
-        gpu.paged_decode(p, p, O.F32, p, p, O.F32, p, p, None, 1, 4, 48, 16, 4, 64, 0.1)  # head dim
+        gpu.paged_decode(p, p, O.F32, p, p, O.F32, p, p, None, 1, 4, 50, 16, 4, 64, 0.1)  # head dim: not whole 16-byte pieces
     with pytest.raises(gpu.HipError):
         gpu.paged_decode(p, p, O.F32, p, p, O.F32, p, p, None, 1, 4, 64, 16, 4, 6400, 0.1)  # max_len needs more pages than the table has
     with pytest.raises(gpu.HipError):

@@ -359,6 +359,28 @@ def test_decode(emu, dtype, H, d, P):
         assert np.abs(got - want).max() <= TOL[dtype], f"chunk={chunk}"
 
 
+@pytest.mark.parametrize("dtype,H,H_kv,d,P", [(O.BF16, 4, 4, 96, 16), (O.F16, 8, 2, 80, 16), (O.F32, 3, 3, 100, 8), (O.BF16, 2, 1, 8, 16),
+                                             (O.F32, 4, 4, 4, 16), (O.F16, 6, 6, 200, 4), (O.BF16, 8, 8, 40, 16)])
+def test_decode_other_head_dimensions(emu, dtype, H, H_kv, d, P):
+    """Head dimensions in whole 16-byte pieces that are not 32, 64, 128 or 256: the lane-per-element kernel of the next
+    size, whose surplus lanes carry a zero query, re-read a row's first piece and store nothing (the pool sits at the end
+    of a guarded buffer, unused slots and pages are NaN)."""
+    B = 4
+    q, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [33, 1, 16, 150], 23, dtype)
+    q = O.round_to(O.fill_normal((B, H, d), 23, 1), dtype)
+    scale = 1.0 / np.sqrt(d)
+    g = H // H_kv
+    n_slots = kp.size // (H_kv * d)
+    kx = np.repeat(kp.reshape(n_slots, H_kv, d), g, axis=1).reshape(-1)
+    vx = np.repeat(vp.reshape(n_slots, H_kv, d), g, axis=1).reshape(-1)
+    want = O.paged_decode(q, kx, vx, table, lens, None, B, H, d, P, scale)
+    kp, vp, table = poison_unused(kp, vp, table, lens, P, H_kv, d, wild_page=1 << 24)
+    for chunk in (0, 2 * P):
+        got = decode(emu, q, kp, vp, table, lens, None, B, H, H_kv, d, P, dtype, dtype, scale, chunk)
+        assert np.isfinite(got).all()
+        assert np.abs(got - want).max() <= TOL[dtype], f"chunk={chunk}"
+
+
 @pytest.mark.parametrize("waves", [1, 2, 4, 8])
 def test_decode_workgroup_shapes(emu, tuned, waves):
     """Every workgroup width the launch plan can choose (1 to 8 wavefronts: from 4 heads of a token to whole
