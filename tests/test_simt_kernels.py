@@ -109,9 +109,8 @@ def test_fp32_matrix_core_kernel_dense_mask(emu, N, d, causal, H_kv, dma_late):
     assert S.lds_stats(reset=True)[0] > 0
 
 
-@pytest.mark.parametrize("dma_late", [False, True])
 @pytest.mark.parametrize("dtype,d", [(O.BF16, 32), (O.F16, 96), (O.BF16, 8), (O.F16, 120), (O.F32, 32), (O.F32, 100), (O.F32, 4), (O.F32, 72)])
-@pytest.mark.parametrize("N,causal,H,H_kv", [(150, True, 2, 1), (64, False, 3, 3)])
+@pytest.mark.parametrize("N,causal,H,H_kv,dma_late", [(150, True, 2, 1, True), (64, False, 3, 3, False)])
 def test_matrix_core_kernels_smaller_head_dimensions(emu, dtype, d, N, causal, H, H_kv, dma_late):
     """Head dimensions below the kernels' 64 / 128 (multiples of 8 for 16-bit tensors, of 4 for fp32) run on the matrix-core
     kernels with columns that contribute nothing.  Tensors sit at the very end (or start) of guarded buffers: nothing behind
@@ -204,8 +203,7 @@ def test_fp32_kernel_dense_mask(emu):
     assert np.abs(got - want).max() <= 1e-4
 
 
-@pytest.mark.parametrize("dma_late", [False, True])
-@pytest.mark.parametrize("packed", [1, 0], ids=["packed-copy", "mask-in-place"])
+@pytest.mark.parametrize("packed,dma_late", [(1, True), (0, False)], ids=["packed-copy", "mask-in-place"])
 @pytest.mark.parametrize("dtype,N,d,causal,H_kv", [(O.BF16, 64, 128, False, 2), (O.F16, 132, 128, True, 2), (O.F16, 300, 64, False, 1),
                                                    (O.BF16, 200, 64, True, 2), (O.BF16, 4, 128, False, 2), (O.F16, 131, 128, False, 1),
                                                    (O.BF16, 65, 64, True, 2)])
@@ -650,8 +648,7 @@ def test_backward_fp32_kernels_16bit_storage(emu, dtype):
     check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, 0.2, True, H_kv), dtype)
 
 
-@pytest.mark.parametrize("split", [1, 2])
-@pytest.mark.parametrize("dma_late", [False, True])
+@pytest.mark.parametrize("split,dma_late", [(1, False), (2, True)])
 @pytest.mark.parametrize("dtype", [O.BF16, O.F16])
 @pytest.mark.parametrize("B,N,H,H_kv,d,causal", [
     (1, 64, 1, 1, 128, False), (2, 129, 2, 2, 128, True), (1, 300, 2, 2, 64, True), (1, 200, 2, 1, 64, False),
@@ -690,9 +687,8 @@ def test_backward_fp32_matrix_core_kernels(emu, tuned, B, N, H, H_kv, d, causal,
     assert reads > 0 and read_conflicts == 0   # the matrix-core kernels ran (the FMA kernels make no traced reads)
 
 
-@pytest.mark.parametrize("dma_late", [False, True])
 @pytest.mark.parametrize("dtype,d", [(O.BF16, 32), (O.F16, 96), (O.BF16, 8), (O.F32, 32), (O.F32, 100), (O.F32, 4)])
-@pytest.mark.parametrize("N,causal,H,H_kv", [(150, True, 2, 1), (64, False, 2, 2)])
+@pytest.mark.parametrize("N,causal,H,H_kv,dma_late", [(150, True, 2, 1, True), (64, False, 2, 2, False)])
 def test_backward_smaller_head_dimensions(emu, dtype, d, N, causal, H, H_kv, dma_late):
     """Head dimensions below the kernels' 64 / 128 in the backward: the matrix-core kernels with columns that contribute
     nothing, tensors at either end of guarded buffers."""
