@@ -194,10 +194,10 @@ __global__ __launch_bounds__(kMaskPackThreads) void flash_mask_pack_kernel(const
     const int key = 64 * kt + lane;
     const float* const src = mask + (int64_t)b * N * N + (key < N ? key : 0);
     uint64_t mine = 0;
-#pragma unroll 8
+#pragma unroll 16
     for (int r = 0; r < 64; ++r) {
         const int row = 64 * rb + r;
-        const float m = (row < N && key < N) ? src[(int64_t)row * N] : 0.0f;
+        const float m = (row < N && key < N) ? __builtin_nontemporal_load(src + (int64_t)row * N) : 0.0f;  // read once
         const uint64_t word = __builtin_amdgcn_ballot_w64(m != 0.0f);
         if (lane == r) mine = word;
     }
