@@ -482,6 +482,25 @@ def bench_extras(hip, stream, steps, warmup):
     rows.append({"workload": "context: torch.matmul bf16 8192x8192x8192 (hipBLASLt), not part of the product",
                  "kernel_ms_mean": round(ms, 4), "TFLOP/s": round(2.0 * M ** 3 / (ms * 1e-3) / 1e12, 1),
                  "frac_of_2.5_PFLOP/s": round(2.0 * M ** 3 / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+    del a, b_
+
+    # Context for the copy-shaped rows (scatter into the pool): torch's device-to-device copy of 1 GiB,
+    # counted as bytes read plus bytes written, on the same box.
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(5):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        dst.copy_(src)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    rows.append({"workload": "context: torch device-to-device copy of 1 GiB (read + write), not part of the product",
+                 "kernel_ms_mean": round(ms, 4), "GB/s": round(2.0 * n / (ms * 1e-3) / 1e9, 1),
+                 "frac_of_8_TB/s": round(2.0 * n / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
     return rows
 
 
