@@ -309,6 +309,8 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     const int h = head_ok ? h_raw : p.H_kv - 1;
     const int e0 = (lane % LPH) * EPL;
     const int d = p.d;                    // the tensors' head dimension, D or less
+    const int gr = G == 1 ? 1 : p.H / p.H_kv;  // query heads per pool head that exist, G or fewer: the others carry a
+                                               // zero query, are computed along and stored nowhere
     const bool piece_ok = e0 < d;         // this lane's 16-byte piece exists
     const int e_ld = piece_ok ? e0 : 0;   // where it reads K and V from
     const int P = PT ? PT : p.P;
@@ -341,7 +343,7 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
             for (int e = 0; e < EPL; ++e) zero[e] = 0.0f;
 #pragma unroll
             for (int g = 0; g < G; ++g)
-                if (piece_ok) store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + h * G + g) * d + e0, zero);
+                if (piece_ok && g < gr) store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + h * gr + g) * d + e0, zero);
         }
         return;
     }
@@ -360,8 +362,8 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     if constexpr (!DUMP) {
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            if (piece_ok) {
-                load_qo_vec<EPL>(p.q, p.qo_dtype, ((int64_t)b * p.H + h * G + g) * d + e0, qf[g]);
+            if (piece_ok && g < gr) {
+                load_qo_vec<EPL>(p.q, p.qo_dtype, ((int64_t)b * p.H + h * gr + g) * d + e0, qf[g]);
             } else {
 #pragma unroll
                 for (int e = 0; e < EPL; ++e) qf[g][e] = 0.0f;
@@ -498,7 +500,8 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     if (!head_ok) return;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        const int hq = h * G + g;
+        if (g >= gr) break;
+        const int hq = h * gr + g;
         if (p.n_chunks == 1) {
             const float inv = l[g] > 0.0f ? 1.0f / l[g] : 0.0f;
             float res[EPL];
@@ -638,11 +641,12 @@ static int launch_decode_dpg(const DecodeParams& p, dim3 grid, dim3 block, hipSt
 
 template <typename T, int PT>
 static int launch_decode_dp(const DecodeParams& p, dim3 grid, dim3 block, hipStream_t st) {
+    // instantiated for groups of 1, 2, 4 and 8 query heads; a group in between runs on the next size
     switch (p.H / p.H_kv) {
         case 1: return launch_decode_dpg<T, PT, 1>(p, grid, block, st);
         case 2: return launch_decode_dpg<T, PT, 2>(p, grid, block, st);
-        case 4: return launch_decode_dpg<T, PT, 4>(p, grid, block, st);
-        case 8: return launch_decode_dpg<T, PT, 8>(p, grid, block, st);
+        case 3: case 4: return launch_decode_dpg<T, PT, 4>(p, grid, block, st);
+        case 5: case 6: case 7: case 8: return launch_decode_dpg<T, PT, 8>(p, grid, block, st);
         default: return AHPC_ERR_UNSUPPORTED_GROUP;
     }
 }
@@ -851,14 +855,14 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
                               float scale, int64_t chunk_tokens, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !o || !k_pool || !v_pool || !block_table || !seq_lens) return AHPC_ERR_NULL_POINTER;
     if (H_kv <= 0 || H <= 0 || H % H_kv) return AHPC_ERR_BAD_SHAPE;
-    // One query head per pool head: lane-per-element kernel, any pool type.  Groups of 2 to 16 (from the tuning
-    // value decode_matrix_min_group on): the page-by-page matrix-core kernel; 32: the 32-column one.  Both need a
-    // 16-bit pool, d 64 or 128 and pages of 16 tokens; groups of 2, 4 and 8 on other pools stay on the
-    // lane-per-element kernel, 16 and 32 are refused there.
+    // Up to 8 query heads per pool head: lane-per-element kernel, any pool type (from the tuning value
+    // decode_matrix_min_group on: the page-by-page matrix-core kernel, where the pool allows it).  9 to 16: the
+    // page-by-page matrix-core kernel; 17 to 32: the 32-column one.  Both need a 16-bit pool, d 64 or 128 and pages
+    // of 16 tokens; on other pools groups beyond 8 are refused.  The matrix-core kernels take the group size as it
+    // is (idle result columns), the lane-per-element kernel runs a group of 3 as 4 and 5 to 7 as 8.
     const int64_t group = H / H_kv;
     const bool mfma_shape = (pool_dtype == AHPC_F16 || pool_dtype == AHPC_BF16) && (d == 64 || d == 128) && P == 16 && H_kv <= 65535;
-    if (group != 1 && group != 2 && group != 4 && group != 8 && !((group == 16 || group == 32) && mfma_shape))
-        return AHPC_ERR_UNSUPPORTED_GROUP;
+    if (group > 32 || (group > 8 && !mfma_shape)) return AHPC_ERR_UNSUPPORTED_GROUP;
     if (qo_dtype < AHPC_F32 || qo_dtype > AHPC_BF16 || pool_dtype < AHPC_F32 || pool_dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
     if (B <= 0 || B > 65535 || max_len <= 0 || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;
     if ((max_len + P - 1) / P > max_pages) return AHPC_ERR_BAD_SHAPE;
@@ -875,7 +879,7 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     const int lph = (int)(d_kernel * (pool_dtype == AHPC_F32 ? 4 : 2) / 16);  // lanes that hold one head of a token
     const int hpw = 64 / lph;
     const int64_t matrix_from = tuning().decode_matrix_min_group.load();
-    const bool use_mfma = mfma_shape && (group >= 16 || group >= matrix_from);
+    const bool use_mfma = mfma_shape && (group > 8 || group >= matrix_from);
     const DecodePlan plan = plan_decode(B, H_kv, group, (H_kv + hpw - 1) / hpw, max_len, P, chunk_tokens, use_mfma);
     const int64_t chunk = plan.chunk;
     const int waves = plan.waves;

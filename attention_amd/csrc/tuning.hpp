@@ -19,7 +19,7 @@ struct Tuning {
     // decode: query heads per K/V head from which on the matrix-core kernels are taken where they apply (16-bit pool,
     // d 64/128, pages of 16).  Default 2: timed on 8 pool heads, the page-by-page matrix-core kernel reaches 0.65-0.72
     // of 8 TB/s for groups of 2, 4 and 8 where the lane-per-element kernel reaches 0.58, 0.55 and 0.36; with one
-    // query head per pool head the lane-per-element kernel stays ahead by 1-2 %.  16 and 32 exist on the
+    // query head per pool head the lane-per-element kernel stays ahead by 1-2 %.  Groups of 9 to 32 exist on the
     // matrix-core kernels only.  (AHPC_DECODE_MFMA_MIN_GROUP)
     std::atomic<int64_t> decode_matrix_min_group;
     // backward: dK and dV in one walk over the query tiles (1), in two (2), or by head dimension (0, the default:

@@ -832,32 +832,43 @@ CASE(Gqa_FlashForwardEqualsRepeatedHeads, true) {
     EXPECT_THROWS(fa.configure(p), AttentionError::INVALID_PARAMETERS);
 }
 CASE(Gqa_PagedDecodeEqualsRepeatedHeads, true) {
-    const size_t H = 8, Hkv = 2, d = 128, P = 16, g = H / Hkv, L = 300;
+    // groups of 4, 3 and 7 query heads per cached head on the reference's default fp32 cache
+    for (const size_t H : {size_t(8), size_t(6), size_t(14)}) {
+        const size_t Hkv = 2, d = 128, P = 16, g = H / Hkv, L = 300;
+        AttentionParams p{};
+        p.batch_size = 1; p.sequence_length = 1; p.num_heads = H; p.key_value_heads = Hkv; p.head_dimension = d; p.max_sequence_length = 512;
+        PagedAttention pa;
+        pa.configure(p);
+        const size_t id = pa.create_sequence(512);
+        auto k = normal(L * Hkv * d, 96, 2), v = normal(L * Hkv * d, 96, 3), q = normal(H * d, 96, 1);
+        pa.append_kv_cache(id, k.data(), v.data(), L, DataType::FLOAT32);   // [n, key_value_heads, d]
+        std::vector<float> out(H * d, 7.0f);
+        const TensorShape s({1, 1, H, d}, DataType::FLOAT32);
+        pa.forward_batch({id}, {s}, {q.data()}, {s}, {out.data()});
+        std::vector<int32_t> table((L + P - 1) / P);
+        for (size_t i = 0; i < table.size(); ++i) table[i] = (int32_t)i;
+        auto kx = repeat_heads(k, L, Hkv, g, d), vx = repeat_heads(v, L, Hkv, g, d);
+        kx.resize(table.size() * P * H * d, 0.0f);
+        vx.resize(kx.size(), 0.0f);
+        std::vector<float> want(H * d, 0.0f);
+        const int32_t len = (int32_t)L;
+        ahpc_oracle_paged_decode(q.data(), want.data(), kx.data(), vx.data(), table.data(), &len, nullptr, 1, H, d, P, table.size(),
+                                 1.0f / std::sqrt((float)d), 1);
+        EXPECT(max_abs_diff(out, want) <= 1e-4f);
+    }
+    const size_t H = 8, Hkv = 2, d = 128, L = 300;
     AttentionParams p{};
     p.batch_size = 1; p.sequence_length = 1; p.num_heads = H; p.key_value_heads = Hkv; p.head_dimension = d; p.max_sequence_length = 512;
     PagedAttention pa;
     pa.configure(p);
     const size_t id = pa.create_sequence(512);
-    auto k = normal(L * Hkv * d, 96, 2), v = normal(L * Hkv * d, 96, 3), q = normal(H * d, 96, 1);
-    pa.append_kv_cache(id, k.data(), v.data(), L, DataType::FLOAT32);   // [n, key_value_heads, d]
-    std::vector<float> out(H * d, 7.0f);
-    const TensorShape s({1, 1, H, d}, DataType::FLOAT32);
-    pa.forward_batch({id}, {s}, {q.data()}, {s}, {out.data()});
-    std::vector<int32_t> table((L + P - 1) / P);
-    for (size_t i = 0; i < table.size(); ++i) table[i] = (int32_t)i;
-    auto kx = repeat_heads(k, L, Hkv, g, d), vx = repeat_heads(v, L, Hkv, g, d);
-    kx.resize(table.size() * P * H * d, 0.0f);
-    vx.resize(kx.size(), 0.0f);
-    std::vector<float> want(H * d, 0.0f);
-    const int32_t len = (int32_t)L;
-    ahpc_oracle_paged_decode(q.data(), want.data(), kx.data(), vx.data(), table.data(), &len, nullptr, 1, H, d, P, table.size(),
-                             1.0f / std::sqrt((float)d), 1);
-    EXPECT(max_abs_diff(out, want) <= 1e-4f);
+    auto k = normal(L * Hkv * d, 96, 2), v = normal(L * Hkv * d, 96, 3);
+    pa.append_kv_cache(id, k.data(), v.data(), L, DataType::FLOAT32);
     // read-back returns what was appended, in the pool's own head count
     std::vector<float> kb(L * Hkv * d), vb(L * Hkv * d);
     pa.get_kv_cache(id, kb.data(), vb.data(), 0, L, DataType::FLOAT32);
     EXPECT(kb == k && vb == v);
-    p.key_value_heads = 1; p.num_heads = 3;  // three query heads per K/V head: refused by the decode kernel
+    p.key_value_heads = 1; p.num_heads = 33;  // 33 query heads per K/V head: more than any decode kernel takes
     EXPECT_THROWS(pa.configure(p), AttentionError::UNSUPPORTED_OPERATION);
 }
 

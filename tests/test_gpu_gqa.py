@@ -129,7 +129,8 @@ def kernel_choice(gpu, request):
 
 
 @pytest.mark.parametrize("dtype", [O.F32, O.F16, O.BF16])
-@pytest.mark.parametrize("H,Hkv,d,P", [(8, 4, 128, 16), (8, 2, 64, 16), (16, 2, 128, 16), (4, 1, 128, 8), (6, 3, 32, 16)])
+@pytest.mark.parametrize("H,Hkv,d,P", [(8, 4, 128, 16), (8, 2, 64, 16), (16, 2, 128, 16), (4, 1, 128, 8), (6, 3, 32, 16),
+                                       (9, 3, 64, 16), (10, 2, 128, 16), (14, 2, 128, 16), (6, 1, 96, 8), (21, 3, 128, 16)])
 def test_decode_gqa_equals_expanded_pool(gpu, dtype, H, Hkv, d, P, kernel_choice):
     import torch
     from gpu_util import to_dev, to_host, stream_ptr, dev_i32, TOL
@@ -160,12 +161,12 @@ def test_decode_gqa_equals_expanded_pool(gpu, dtype, H, Hkv, d, P, kernel_choice
         assert np.abs(got - want).max() <= TOL[dtype], f"chunk={chunk}"
 
 
-def test_decode_gqa_rejects_group_of_three(gpu):
+def test_decode_gqa_rejects_group_of_33(gpu):
     import torch
     from attention_amd.hip import HipError
     x = torch.zeros(4096, dtype=torch.float16, device="cuda")
     t = torch.zeros(4, dtype=torch.int32, device="cuda")
     with pytest.raises(HipError) as e:
         gpu.paged_decode_gqa(x.data_ptr(), x.data_ptr(), O.F16, x.data_ptr(), x.data_ptr(), O.F16, t.data_ptr(), t.data_ptr(),
-                             None, 1, 6, 2, 64, 16, 1, 16, 0.0, 0, None, 0, None)
+                             None, 1, 66, 2, 64, 16, 1, 16, 0.0, 0, None, 0, None)
     assert e.value.code == -8

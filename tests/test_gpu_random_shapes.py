@@ -167,7 +167,7 @@ def decode_cases(n, seed):
         P = 16 if rng.random() < 0.75 else pick(rng, [4, 8, 32])
         Hkv = int(rng.integers(1, 4))
         matrix_ok = dtype != O.F32 and d in (64, 128) and P == 16
-        g = pick(rng, [1, 2, 4, 8, 16, 32] if matrix_ok else [1, 2, 4, 8])
+        g = pick(rng, list(range(1, 33)) if matrix_ok else list(range(1, 9)))
         B = int(rng.integers(1, 6))
         lens = []
         for _ in range(B):

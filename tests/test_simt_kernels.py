@@ -775,6 +775,31 @@ def test_decode_page_ring_of_the_group_kernel(emu, tuned, H_kv, G, d, dtype):
         assert np.abs(got - want).max() <= 2e-2, chunk
 
 
+@pytest.mark.parametrize("G,dtype,d,P,matrix_from", [
+    (3, O.F32, 64, 16, 2), (5, O.F32, 128, 8, 2), (7, O.F16, 96, 16, 2), (6, O.BF16, 128, 16, 16), (3, O.F16, 64, 16, 16),  # lane per element
+    (3, O.F16, 128, 16, 2), (7, O.BF16, 64, 16, 2), (12, O.F16, 128, 16, 2), (9, O.BF16, 64, 16, 16),                       # page by page
+    (17, O.F16, 64, 16, 2), (24, O.BF16, 128, 16, 2), (31, O.F16, 128, 16, 16)])                                            # 32 columns
+def test_decode_group_sizes_in_between(emu, tuned, G, dtype, d, P, matrix_from):
+    """Group sizes the kernels are not instantiated for: the lane-per-element kernel of the next size with surplus query
+    heads that hold zeros and store nothing, the matrix-core kernels with idle result columns.  The output sits
+    directly against an inaccessible page, so a store for a head that does not exist faults."""
+    tuned("decode_matrix_min_group", matrix_from)
+    B, H_kv = 4, 3
+    H = G * H_kv
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [70, 5, 129, 32], 26, dtype)
+    lens = lens.copy()
+    lens[3] = 0                                     # an empty sequence: zeros
+    q = O.round_to(O.fill_normal((B, H, d), 26, 1), dtype)
+    scale = 1.0 / np.sqrt(d)
+    rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
+    want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    kp, vp, table = poison_unused(kp, vp, table, lens, P, H_kv, d, wild_page=1 << 24)
+    for chunk in (0, 2 * P, 64 * P):
+        got = decode(emu, q, kp, vp, table, lens, None, B, H, H_kv, d, P, dtype, dtype, scale, chunk)
+        assert np.all(got[3] == 0.0)
+        assert np.abs(got - want).max() <= TOL[dtype], chunk
+
+
 def test_wide_groups_need_the_matrix_core_shape(emu):
     # 16 query heads per pool head on an fp32 pool: refused
     B, H_kv, d, P, G = 1, 1, 64, 16, 16
@@ -782,6 +807,12 @@ def test_wide_groups_need_the_matrix_core_shape(emu):
     q = O.fill_normal((B, G * H_kv, d), 24, 1)
     with pytest.raises(emu.HipError):
         decode(emu, q, kp, vp, table, lens, None, B, G * H_kv, H_kv, d, P, O.F32, O.F32, 0.125)
+    # 9 on pages of 8 tokens, 33 on any pool: refused as well
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, 8, [20], 24, O.F16)
+    for G in (9, 33):
+        q = O.round_to(O.fill_normal((B, G * H_kv, d), 24, 1), O.F16)
+        with pytest.raises(emu.HipError):
+            decode(emu, q, kp, vp, table, lens, None, B, G * H_kv, H_kv, d, 8 if G == 9 else 16, O.F16, O.F16, 0.125)
 
 
 @pytest.mark.parametrize("dtype,d,H,H_kv", [(O.F16, 64, 2, 2), (O.BF16, 128, 4, 2), (O.F32, 32, 2, 1), (O.F32, 128, 2, 1), (O.F32, 64, 2, 2)])
