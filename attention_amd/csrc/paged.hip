@@ -188,6 +188,8 @@ struct DecodeParams {
                               // smallest that holds d.  The lanes of a head whose 16-byte piece lies at or beyond d
                               // carry a zero query, re-read the row's first piece and store nothing.
     int32_t H_kv;             // heads in the pool; H / H_kv consecutive query heads share one
+    int32_t g0;               // lane-per-element kernel: first query head (within its group) that this launch serves; a group
+                              // wider than the kernel is instantiated for is served in several launches
     int32_t chunk_tokens, n_chunks;  // longest chunk (a multiple of P, at most 64 pages) and how many the longest sequence needs
     int32_t balanced;         // 1: a sequence cuts itself into equal chunks (see decode_chunk_len); 0: every chunk is chunk_tokens long
     int32_t max_len;
@@ -309,8 +311,10 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     const int h = head_ok ? h_raw : p.H_kv - 1;
     const int e0 = (lane % LPH) * EPL;
     const int d = p.d;                    // the tensors' head dimension, D or less
-    const int gr = G == 1 ? 1 : p.H / p.H_kv;  // query heads per pool head that exist, G or fewer: the others carry a
-                                               // zero query, are computed along and stored nowhere
+    const int group = G == 1 ? 1 : p.H / p.H_kv;  // query heads per pool head
+    const int g0 = G == 1 ? 0 : p.g0;             // the first of them that this launch serves
+    const int gr = group - g0 < G ? group - g0 : G;  // how many it serves, G or fewer: the others of the G carry a zero
+                                                     // query, are computed along and stored nowhere
     const bool piece_ok = e0 < d;         // this lane's 16-byte piece exists
     const int e_ld = piece_ok ? e0 : 0;   // where it reads K and V from
     const int P = PT ? PT : p.P;
@@ -343,7 +347,7 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
             for (int e = 0; e < EPL; ++e) zero[e] = 0.0f;
 #pragma unroll
             for (int g = 0; g < G; ++g)
-                if (piece_ok && g < gr) store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + h * gr + g) * d + e0, zero);
+                if (piece_ok && g < gr) store_qo_vec<EPL>(p.o, p.qo_dtype, ((int64_t)b * p.H + h * group + g0 + g) * d + e0, zero);
         }
         return;
     }
@@ -363,7 +367,7 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             if (piece_ok && g < gr) {
-                load_qo_vec<EPL>(p.q, p.qo_dtype, ((int64_t)b * p.H + h * gr + g) * d + e0, qf[g]);
+                load_qo_vec<EPL>(p.q, p.qo_dtype, ((int64_t)b * p.H + h * group + g0 + g) * d + e0, qf[g]);
             } else {
 #pragma unroll
                 for (int e = 0; e < EPL; ++e) qf[g][e] = 0.0f;
@@ -501,7 +505,7 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         if (g >= gr) break;
-        const int hq = h * gr + g;
+        const int hq = h * group + g0 + g;
         if (p.n_chunks == 1) {
             const float inv = l[g] > 0.0f ? 1.0f / l[g] : 0.0f;
             float res[EPL];
@@ -640,15 +644,22 @@ static int launch_decode_dpg(const DecodeParams& p, dim3 grid, dim3 block, hipSt
 }
 
 template <typename T, int PT>
-static int launch_decode_dp(const DecodeParams& p, dim3 grid, dim3 block, hipStream_t st) {
-    // instantiated for groups of 1, 2, 4 and 8 query heads; a group in between runs on the next size
-    switch (p.H / p.H_kv) {
-        case 1: return launch_decode_dpg<T, PT, 1>(p, grid, block, st);
-        case 2: return launch_decode_dpg<T, PT, 2>(p, grid, block, st);
-        case 3: case 4: return launch_decode_dpg<T, PT, 4>(p, grid, block, st);
-        case 5: case 6: case 7: case 8: return launch_decode_dpg<T, PT, 8>(p, grid, block, st);
-        default: return AHPC_ERR_UNSUPPORTED_GROUP;
+static int launch_decode_dp(const DecodeParams& base, dim3 grid, dim3 block, hipStream_t st) {
+    // Instantiated for 1, 2, 4 and 8 query heads per pool head.  A group in between runs on the next size; a wider one
+    // in slices of 8 query heads, one launch each (every slice reads the K/V stream again), the last slice on the
+    // size that holds it.
+    const int group = base.H / base.H_kv;
+    if (group == 1) return launch_decode_dpg<T, PT, 1>(base, grid, block, st);
+    DecodeParams p = base;
+    for (int g0 = 0; g0 < group; g0 += 8) {
+        p.g0 = g0;
+        const int slice = group - g0 < 8 ? group - g0 : 8;
+        const int rc = slice <= 2 ? launch_decode_dpg<T, PT, 2>(p, grid, block, st)
+                     : slice <= 4 ? launch_decode_dpg<T, PT, 4>(p, grid, block, st)
+                                  : launch_decode_dpg<T, PT, 8>(p, grid, block, st);
+        if (rc) return rc;
     }
+    return AHPC_OK;
 }
 
 // Matrix-core kernel for grouped heads: one wavefront per (pool head, chunk, batch entry).
@@ -858,11 +869,12 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     // Up to 8 query heads per pool head: lane-per-element kernel, any pool type (from the tuning value
     // decode_matrix_min_group on: the page-by-page matrix-core kernel, where the pool allows it).  9 to 16: the
     // page-by-page matrix-core kernel; 17 to 32: the 32-column one.  Both need a 16-bit pool, d 64 or 128 and pages
-    // of 16 tokens; on other pools groups beyond 8 are refused.  The matrix-core kernels take the group size as it
-    // is (idle result columns), the lane-per-element kernel runs a group of 3 as 4 and 5 to 7 as 8.
+    // of 16 tokens; other pools, and groups beyond 32, go through the lane-per-element kernel in slices of 8 query
+    // heads.  The matrix-core kernels take the group size as it is (idle result columns), the lane-per-element
+    // kernel runs a group or slice of 3 as 4 and 5 to 7 as 8.
     const int64_t group = H / H_kv;
-    const bool mfma_shape = (pool_dtype == AHPC_F16 || pool_dtype == AHPC_BF16) && (d == 64 || d == 128) && P == 16 && H_kv <= 65535;
-    if (group > 32 || (group > 8 && !mfma_shape)) return AHPC_ERR_UNSUPPORTED_GROUP;
+    const bool mfma_shape = (pool_dtype == AHPC_F16 || pool_dtype == AHPC_BF16) && (d == 64 || d == 128) && P == 16 && H_kv <= 65535 &&
+                            group <= 32;
     if (qo_dtype < AHPC_F32 || qo_dtype > AHPC_BF16 || pool_dtype < AHPC_F32 || pool_dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
     if (B <= 0 || B > 65535 || max_len <= 0 || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;
     if ((max_len + P - 1) / P > max_pages) return AHPC_ERR_BAD_SHAPE;
@@ -880,7 +892,7 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     const int hpw = 64 / lph;
     const int64_t matrix_from = tuning().decode_matrix_min_group.load();
     const bool use_mfma = mfma_shape && (group > 8 || group >= matrix_from);
-    const DecodePlan plan = plan_decode(B, H_kv, group, (H_kv + hpw - 1) / hpw, max_len, P, chunk_tokens, use_mfma);
+    const DecodePlan plan = plan_decode(B, H_kv, group < 8 ? group : 8, (H_kv + hpw - 1) / hpw, max_len, P, chunk_tokens, use_mfma);
     const int64_t chunk = plan.chunk;
     const int waves = plan.waves;
     const int64_t n_chunks = (max_len + chunk - 1) / chunk;

@@ -73,7 +73,7 @@ const char* ahpc_hip_error_string(int code) {
         case AHPC_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";
         case AHPC_ERR_NO_DEVICE: return "no HIP device available";
         case AHPC_ERR_BAD_ALIGNMENT: return "pointer or stride not aligned for 16-byte access";
-        case AHPC_ERR_UNSUPPORTED_GROUP: return "query heads per key/value head not supported (decode: up to 8; up to 32 with a 16-bit pool, d 64/128, pages of 16)";
+        case AHPC_ERR_UNSUPPORTED_GROUP: return "query heads per key/value head not supported";
         case AHPC_ERR_SCRATCH_LIMIT: return "the call needs more scratch than ahpc_hip_paged_decode_noalloc has built in (16 MiB): use ahpc_hip_paged_decode_gqa with a workspace";
         default: break;
     }

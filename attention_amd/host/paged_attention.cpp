@@ -127,17 +127,11 @@ void PagedAttention::configure(const AttentionParams& params, const PerformanceC
     if (params.batch_size == 0 || params.sequence_length == 0 || params.num_heads == 0 || params.head_dimension == 0)
         throw AttentionException(AttentionError::INVALID_PARAMETERS, "Invalid attention parameters: dimensions must be positive");
     // Grouped key/value heads: the pool stores key_value_heads heads per token and every one of them serves
-    // num_heads / key_value_heads consecutive query heads (the decode kernels take groups of up to 8, and up to 32
-    // on the matrix-core kernels, which need a 16-bit cache: that is known at the first append only).
+    // num_heads / key_value_heads consecutive query heads (any number of them; see ahpc_hip_paged_decode_gqa for the
+    // kernel a group size runs on).
     if (params.key_value_heads != 0) {
         if (params.key_value_heads > params.num_heads || params.num_heads % params.key_value_heads)
             throw AttentionException(AttentionError::INVALID_PARAMETERS, "key_value_heads must divide num_heads");
-        const size_t g = params.num_heads / params.key_value_heads;
-        const bool wide_ok = g <= 32 && params.page_size == 16 && (params.head_dimension == 64 || params.head_dimension == 128);
-        if (g > 8 && !wide_ok)
-            throw AttentionException(AttentionError::UNSUPPORTED_OPERATION,
-                                     "paged decode supports up to 8 query heads per key/value head, and up to 32 with "
-                                     "pages of 16 tokens, head_dimension 64 or 128 and a 16-bit cache");
     }
     if (params.page_size == 0) throw AttentionException(AttentionError::INVALID_PARAMETERS, "page_size must be positive");
     const size_t d = params.head_dimension;

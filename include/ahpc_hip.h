@@ -43,7 +43,7 @@ typedef enum ahpc_status {
     AHPC_ERR_WORKSPACE_TOO_SMALL = -5,
     AHPC_ERR_NO_DEVICE = -6,
     AHPC_ERR_BAD_ALIGNMENT = -7,   /* pointers/strides must allow 16-byte vector access */
-    AHPC_ERR_UNSUPPORTED_GROUP = -8, /* query heads per K/V head: decode takes up to 8 (up to 32: see paged_decode_gqa) */
+    AHPC_ERR_UNSUPPORTED_GROUP = -8, /* query heads per K/V head not supported (kept for callers that test for it: decode takes any group size now) */
     AHPC_ERR_SCRATCH_LIMIT = -9     /* ahpc_hip_paged_decode_noalloc: the call needs more than AHPC_NOALLOC_SCRATCH_BYTES */
 } ahpc_status;
 
@@ -288,10 +288,10 @@ int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype,
                           void* workspace, size_t workspace_bytes, void* stream);
 
 /* Decode with grouped K/V heads: the pool holds H_kv heads per token (its kv_scatter / kv_gather /
- * gather_indices calls take H = H_kv), q and o hold H = g * H_kv heads, g from 1 to 8; query
- * head h reads pool head h / g.  Every K/V byte is still read once and serves g query heads.
- * g from 9 to 32 (up to multi-query attention with 32 heads) is served by matrix-core kernels that need
- * an fp16/bf16 pool, d in {64, 128} and P = 16; other combinations return AHPC_ERR_UNSUPPORTED_GROUP.  The head dimension
+ * gather_indices calls take H = H_kv), q and o hold H = g * H_kv heads, any g; query head h reads pool head h / g.
+ * Up to g = 8 every K/V byte is read once and serves the g query heads.  g from 9 to 32 (up to multi-query attention
+ * with 32 heads) does the same on matrix-core kernels when the pool is fp16/bf16, d is 64 or 128 and P = 16; on other
+ * pools, and beyond 32, the group is served in slices of 8 query heads that each read the K/V stream.  The head dimension
  * may be anything up to 256 in whole 16-byte pieces of the pool's type (a multiple of 8 for fp16/bf16 pools, of 4 for
  * fp32 ones); AHPC_ERR_UNSUPPORTED_HEAD_DIM otherwise.
  * Workspace size: ahpc_hip_paged_decode_workspace_bytes with the QUERY head count. */

@@ -77,9 +77,6 @@ def test_paged_decode_argument_checks(lib):
     assert decode(lib, max_len=65, max_pages=4) == BAD_SHAPE           # the table row cannot hold that many tokens
     assert decode(lib, d=44) == HEAD_DIM and decode(lib, d=264) == HEAD_DIM   # whole 16-byte pieces of an fp16 row, up to 256
     assert decode(lib, kp=P + 8) == BAD_ALIGNMENT and decode(lib, o=P + 2) == BAD_ALIGNMENT
-    assert decode(lib, H=66, Hkv=2) == BAD_GROUP                       # 33 query heads per K/V head
-    assert decode(lib, H=18, Hkv=2, pool=0) == BAD_GROUP               # 9 on an fp32 pool: the matrix-core kernels need 16 bits
-    assert decode(lib, H=18, Hkv=2, Pg=8) == BAD_GROUP                 # ... and pages of 16 tokens
     assert decode(lib, H=6, Hkv=4) == BAD_SHAPE                        # does not divide
     # several chunks need the workspace the size query reports
     need = lib.ahpc_hip_paged_decode_workspace_bytes(2, 8, 128, 64, 16, 16)

@@ -161,12 +161,32 @@ def test_decode_gqa_equals_expanded_pool(gpu, dtype, H, Hkv, d, P, kernel_choice
         assert np.abs(got - want).max() <= TOL[dtype], f"chunk={chunk}"
 
 
-def test_decode_gqa_rejects_group_of_33(gpu):
+@pytest.mark.parametrize("dtype,H,Hkv,d,P", [(O.F16, 66, 2, 64, 16), (O.F32, 32, 2, 128, 16), (O.BF16, 18, 2, 64, 8), (O.F32, 71, 1, 64, 16)])
+def test_decode_gqa_wide_groups_in_slices(gpu, dtype, H, Hkv, d, P):
+    """More than 8 query heads per cached head where the matrix-core kernels do not apply (more than 32, an fp32 pool,
+    pages of 8 tokens): slices of 8 query heads on the lane-per-element kernel."""
     import torch
-    from attention_amd.hip import HipError
-    x = torch.zeros(4096, dtype=torch.float16, device="cuda")
-    t = torch.zeros(4, dtype=torch.int32, device="cuda")
-    with pytest.raises(HipError) as e:
-        gpu.paged_decode_gqa(x.data_ptr(), x.data_ptr(), O.F16, x.data_ptr(), x.data_ptr(), O.F16, t.data_ptr(), t.data_ptr(),
-                             None, 1, 66, 2, 64, 16, 1, 16, 0.0, 0, None, 0, None)
-    assert e.value.code == -8
+    from gpu_util import to_dev, to_host, stream_ptr, dev_i32, TOL
+    g = H // Hkv
+    B = 3
+    kp, vp, table, lens, n_pages = build_pool(B, Hkv, d, P, [45, 0, 260], 43, dtype)
+    q = O.round_to(O.fill_normal((B, H, d), 43, 1), dtype)
+    scale = 1.0 / np.sqrt(d)
+    kx = expand_heads(kp.reshape(n_pages * P, Hkv, d), g, 1).reshape(-1)
+    vx = expand_heads(vp.reshape(n_pages * P, Hkv, d), g, 1).reshape(-1)
+    want = O.paged_decode(q, kx, vx, table, lens, None, B, H, d, P, scale)
+    kd, vd = to_dev(kp, dtype), to_dev(vp, dtype)
+    dt, dl = dev_i32(table), dev_i32(lens)
+    max_len = int(lens.max())
+    for chunk in (0, 4 * P):
+        dq = to_dev(q, dtype)
+        do = torch.full_like(dq, float("nan"))
+        ws_bytes = gpu.paged_decode_workspace_bytes(B, H, d, max_len, P, chunk)
+        ws = torch.empty(max(ws_bytes, 4) // 4, dtype=torch.float32, device="cuda")
+        gpu.paged_decode_gqa(dq.data_ptr(), do.data_ptr(), dtype, kd.data_ptr(), vd.data_ptr(), dtype, dt.data_ptr(),
+                             dl.data_ptr(), None, B, H, Hkv, d, P, table.shape[1], max_len, scale, chunk, ws.data_ptr(),
+                             ws_bytes, stream_ptr())
+        torch.cuda.synchronize()
+        got = to_host(do)
+        assert np.all(got[1] == 0.0)
+        assert np.abs(got - want).max() <= TOL[dtype], f"chunk={chunk}"

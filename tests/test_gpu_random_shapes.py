@@ -166,8 +166,7 @@ def decode_cases(n, seed):
         d = pick(rng, [64, 128]) if rng.random() < 0.8 else pick(rng, [32, 256])
         P = 16 if rng.random() < 0.75 else pick(rng, [4, 8, 32])
         Hkv = int(rng.integers(1, 4))
-        matrix_ok = dtype != O.F32 and d in (64, 128) and P == 16
-        g = pick(rng, list(range(1, 33)) if matrix_ok else list(range(1, 9)))
+        g = pick(rng, list(range(1, 33)) + [40, 71]) if rng.random() < 0.85 else 1
         B = int(rng.integers(1, 6))
         lens = []
         for _ in range(B):

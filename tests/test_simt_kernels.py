@@ -800,19 +800,23 @@ def test_decode_group_sizes_in_between(emu, tuned, G, dtype, d, P, matrix_from):
         assert np.abs(got - want).max() <= TOL[dtype], chunk
 
 
-def test_wide_groups_need_the_matrix_core_shape(emu):
-    # 16 query heads per pool head on an fp32 pool: refused
-    B, H_kv, d, P, G = 1, 1, 64, 16, 16
-    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [20], 24, O.F32)
-    q = O.fill_normal((B, G * H_kv, d), 24, 1)
-    with pytest.raises(emu.HipError):
-        decode(emu, q, kp, vp, table, lens, None, B, G * H_kv, H_kv, d, P, O.F32, O.F32, 0.125)
-    # 9 on pages of 8 tokens, 33 on any pool: refused as well
-    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, 8, [20], 24, O.F16)
-    for G in (9, 33):
-        q = O.round_to(O.fill_normal((B, G * H_kv, d), 24, 1), O.F16)
-        with pytest.raises(emu.HipError):
-            decode(emu, q, kp, vp, table, lens, None, B, G * H_kv, H_kv, d, 8 if G == 9 else 16, O.F16, O.F16, 0.125)
+@pytest.mark.parametrize("G,dtype,d,P", [(16, O.F32, 64, 16), (9, O.F16, 64, 8), (33, O.F16, 128, 16), (12, O.BF16, 96, 16), (20, O.F32, 128, 4),
+                                        (71, O.BF16, 64, 16)])
+def test_wide_groups_off_the_matrix_core_shape(emu, G, dtype, d, P):
+    """More than 8 query heads per pool head where the matrix-core kernels do not apply (fp32 pool, other page sizes or
+    head dimensions, more than 32 heads): the lane-per-element kernel serves the group in slices of 8 query heads."""
+    B, H_kv = 3, 2
+    H = G * H_kv
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [70, 0, 33], 24, dtype)
+    q = O.round_to(O.fill_normal((B, H, d), 24, 1), dtype)
+    scale = 1.0 / np.sqrt(d)
+    rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
+    want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    kp, vp, table = poison_unused(kp, vp, table, lens, P, H_kv, d, wild_page=1 << 24)
+    for chunk in (0, 2 * P):
+        got = decode(emu, q, kp, vp, table, lens, None, B, H, H_kv, d, P, dtype, dtype, scale, chunk)
+        assert np.all(got[1] == 0.0)
+        assert np.abs(got - want).max() <= TOL[dtype], chunk
 
 
 @pytest.mark.parametrize("dtype,d,H,H_kv,causal", [(O.F16, 64, 2, 2, False), (O.F16, 64, 2, 2, True), (O.BF16, 128, 4, 2, True),

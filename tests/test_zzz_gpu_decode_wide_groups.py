@@ -94,14 +94,3 @@ def test_both_kernels_agree_for_groups_of_four(gpu):
     finally:
         gpu.set_tuning("decode_matrix_min_group", before)
     assert np.abs(a - b).max() <= 5e-3   # same inputs, fp32 outputs: only P's rounding to 16 bits differs
-
-
-def test_wide_groups_on_other_pools_are_refused(gpu):
-    import torch
-    x = torch.zeros(1 << 16, device="cuda")
-    p = x.data_ptr()
-    with pytest.raises(gpu.HipError):   # fp32 pool
-        gpu.paged_decode_gqa(p, p, O.F32, p, p, O.F32, p, p, None, 1, 16, 1, 64, 16, 4, 64, 0.1, 0, None, 0, None)
-    with pytest.raises(gpu.HipError):   # pages of 8 tokens
-        gpu.paged_decode_gqa(p, p, O.F16, p, p, O.F16, p, p, None, 1, 32, 1, 64, 8, 8, 64, 0.1, 0, None, 0, None)
-    torch.cuda.synchronize()
