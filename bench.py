@@ -215,7 +215,7 @@ def bench_flash(hip, stream, steps, warmup, cpu):
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": flash_traffic, "traffic_source": flash_traffic_src,
                      "kernel": "flash_fwd_mfma_kernel<bf16,128,causal>", "kernel_ms_mean": round(kern_ms, 4),
-                     "kernel_ms_min": round(float(np.min(per)), 4), "flop_per_launch": flops},
+                     "kernel_ms_median": round(float(np.median(per)), 4), "kernel_ms_min": round(float(np.min(per)), 4), "flop_per_launch": flops},
         "config": {"workload": "flash_fwd bf16 causal B=4 N=4096 H=32 d=128 layout [B,N,H,d], fp32 accumulate, bf16 out"},
     }
     if cpu:
@@ -284,7 +284,7 @@ def bench_decode(hip, stream, steps, warmup, cpu):
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": decode_traffic, "traffic_source": decode_traffic_src,
                      "kernel": "paged_decode_kernel<f16,128> + paged_merge_kernel", "kernel_ms_mean": round(kern_ms, 4),
-                     "kernel_ms_min": round(float(np.min(per)), 4), "bytes_per_launch": nbytes},
+                     "kernel_ms_median": round(float(np.median(per)), 4), "kernel_ms_min": round(float(np.min(per)), 4), "bytes_per_launch": nbytes},
         "config": {"workload": f"paged_decode fp16 B=64 H=32 d=128 page=16 context U[512,4096] (sum {int(lens.sum())} tokens), "
                                f"shuffled block table, pool {n_pages} pages"},
     }
@@ -338,7 +338,8 @@ def bench_extras(hip, stream, steps, warmup):
     def run(name, launch, flops=None, nbytes=None, fp32=False):
         wall, per = timed_steps(hip, stream, launch, steps, warmup)
         ms = float(np.mean(per))
-        row = {"workload": name, "kernel_ms_mean": round(ms, 4), "kernel_ms_min": round(float(np.min(per)), 4)}
+        row = {"workload": name, "kernel_ms_mean": round(ms, 4), "kernel_ms_median": round(float(np.median(per)), 4),
+               "kernel_ms_min": round(float(np.min(per)), 4)}
         if flops:
             row["TFLOP/s"] = round(flops / (ms * 1e-3) / 1e12, 1)
             if fp32:  # fp32 matrix instructions: MI355X's published dense fp32 peak
