@@ -371,6 +371,17 @@ def bench_extras(hip, stream, steps, warmup):
                                   (N * Hkv * d, Hkv * d, d), sc, True, stream),
         flops=2.0 * B * H * N * N * d)
 
+    # one long sequence (1 x 32768 tokens, 16 times the headline's work): a workgroup walks 8 times as many key tiles
+    # per query tile, so what a query tile and a launch cost at their start and end weighs less
+    Nl = 32768
+    ql, kl, vl = (randn((1, Nl, H, d), torch.bfloat16) for _ in range(3))
+    ol = torch.empty_like(ql)
+    stl = (Nl * H * d, H * d, d)
+    run("flash_fwd bf16 causal B=1 N=32768 H=32 d=128 (one long sequence)",
+        lambda: hip.flash_fwd(ql.data_ptr(), kl.data_ptr(), vl.data_ptr(), ol.data_ptr(), hip.BF16, 1, Nl, H, d, stl, sc, True, stream),
+        flops=2.0 * H * Nl * Nl * d)
+    del ql, kl, vl, ol
+
     # the headline shape in fp32, the reference's default data type: the fp32 matrix-core kernel
     qf, kf, vf = randn((B, N, H, d), torch.float32), randn((B, N, H, d), torch.float32), randn((B, N, H, d), torch.float32)
     of = torch.empty_like(qf)
