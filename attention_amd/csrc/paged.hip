@@ -527,43 +527,91 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     }
 }
 
-// One thread per output element: folds the chunk partials of its (batch entry, head) with the rule
-// m' = max(m, m2), l' = l*2^(m-m') + l2*2^(m2-m'), accumulators scaled by the same factors.  Done in
-// two passes (global maximum first) so that the loads of the second pass do not wait on one another.
-__global__ __launch_bounds__(256) void paged_merge_kernel(const DecodeParams p) {
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t hd = (int64_t)p.H * p.d;
-    if (idx >= p.B * hd) return;
-    const int64_t b = idx / hd;
-    const int64_t he = idx - b * hd;
-    const int h = (int)(he / p.d);
-    const int e = (int)(he - (int64_t)h * p.d);
+// One wavefront per (batch entry, head): folds the chunk partials with the rule
+// m' = max(m, m2), l' = l*2^(m-m') + l2*2^(m2-m'), accumulators scaled by the same factors.  The round trips to
+// memory are what this kernel takes (a long context has 32 chunks and more), so it makes few of them: the (m, l)
+// pairs of up to 64 chunks arrive in one, a lane each, and the accumulators in batches of 16 chunks, every load of a
+// batch issued before the first is used (a lane holds four consecutive elements of d).
+constexpr int kMergeWaves = 4;   // (batch entry, head) pairs per workgroup
+constexpr int kMergeBatch = 16;  // chunks whose accumulators are in flight together
+__global__ __launch_bounds__(64 * kMergeWaves) void paged_merge_kernel(const DecodeParams p) {
+    const int lane = threadIdx.x & 63;
+    const int64_t pair = (int64_t)blockIdx.x * kMergeWaves + (threadIdx.x >> 6);
+    if (pair >= (int64_t)p.B * p.H) return;  // (uniform per wavefront)
+    const int64_t b = pair / p.H;
+    const int h = (int)(pair - b * p.H);
     const int64_t row = p.batch_rows ? p.batch_rows[b] : b;
     const int L = p.seq_lens[row] < p.max_len ? p.seq_lens[row] : p.max_len;
     const int chunk_len = decode_chunk_len(p, L, p.P);
     const int n = (L + chunk_len - 1) / chunk_len;
     const float* ml = p.part_ml + ((b * p.n_chunks) * p.H + h) * 2;
-    const float* po = p.part_o + ((b * p.n_chunks) * p.H + h) * p.d + e;
+    const float* po = p.part_o + ((b * p.n_chunks) * p.H + h) * p.d;
     const int64_t ml_step = (int64_t)p.H * 2, po_step = (int64_t)p.H * p.d;
-    // a chunk whose l carries a minus sign met a missing page: it is the last one that counts
+    const int e0 = 4 * lane;
+    const bool active = e0 < p.d;  // d is a multiple of 4
+
+    // A chunk whose l carries a minus sign met a missing page: it is the last one that counts.  Every chunk of the
+    // sequence has written its (m, l) pair.  First walk: where the sequence ends, and the largest m up to there.
     float m = -INFINITY;
     int n_used = n;
-    for (int ci = 0; ci < n; ++ci) {
-        m = fmaxf(m, ml[ci * ml_step]);
-        if (__builtin_bit_cast(uint32_t, ml[ci * ml_step + 1]) >> 31) {
-            n_used = ci + 1;
-            break;
+    for (int c0 = 0; c0 < n; c0 += kWave) {
+        const int c = c0 + lane;
+        float mc = -INFINITY;
+        bool stops = false;
+        if (c < n) {
+            mc = ml[c * ml_step];
+            stops = (__builtin_bit_cast(uint32_t, ml[c * ml_step + 1]) >> 31) != 0;
+        }
+        const unsigned long long stop = __builtin_amdgcn_ballot_w64(stops);
+        if (stop != 0) {
+            const int first = c0 + (int)__builtin_ctzll(stop);
+            n_used = first + 1;
+            if (c > first) mc = -INFINITY;
+        }
+        m = fmaxf(m, mc);
+        if (stop != 0) break;  // (uniform)
+    }
+#pragma unroll
+    for (int s = 1; s < kWave; s <<= 1) m = fmaxf(m, __shfl_xor(m, s, kWave));
+
+    // Second walk: weights 2^(m_c - m), a lane per chunk; the accumulators of a batch of chunks, then their sum.
+    float l = 0.0f;
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int c0 = 0; c0 < n_used; c0 += kWave) {
+        const int c = c0 + lane;
+        float f = 0.0f;
+        if (c < n_used) {
+            f = fast_exp2(ml[c * ml_step] - m);  // (m is -inf only when every m_c is: then l stays 0 below)
+            l = __builtin_fmaf(__builtin_fabsf(ml[c * ml_step + 1]), f, l);
+        }
+        const int cnt = n_used - c0 < kWave ? n_used - c0 : kWave;
+        for (int ci = 0; ci < cnt; ci += kMergeBatch) {
+            f32x4 v[kMergeBatch];
+#pragma unroll
+            for (int u = 0; u < kMergeBatch; ++u) {
+                v[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                if (ci + u < cnt && active) v[u] = *reinterpret_cast<const f32x4*>(po + (int64_t)(c0 + ci + u) * po_step + e0);
+            }
+#pragma unroll
+            for (int u = 0; u < kMergeBatch; ++u) {
+                // (a lane index beyond the batch's chunks is never used: v[u] is zero there)
+                const float fc = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(f), (ci + u) & (kWave - 1)));
+                if (ci + u < cnt) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[i] = __builtin_fmaf(v[u][i], fc, acc[i]);
+                }
+            }
         }
     }
-    float l = 0.0f, acc = 0.0f;
-#pragma unroll 4
-    for (int ci = 0; ci < n_used; ++ci) {
-        const float f = fast_exp2(ml[ci * ml_step] - m);
-        l = __builtin_fmaf(__builtin_fabsf(ml[ci * ml_step + 1]), f, l);
-        acc = __builtin_fmaf(po[ci * po_step], f, acc);
-    }
+#pragma unroll
+    for (int s = 1; s < kWave; s <<= 1) l += __shfl_xor(l, s, kWave);
     // nothing attended to (empty sequence, or its first page missing): l is 0, or NaN from (-inf) - (-inf)
-    store_qo(p.o, p.qo_dtype, idx, l > 0.0f ? acc / l : 0.0f);
+    if (active) {
+        const bool live = l > 0.0f;
+        const float inv = live ? 1.0f / l : 0.0f;
+        const float res[4] = {live ? acc[0] * inv : 0.0f, live ? acc[1] * inv : 0.0f, live ? acc[2] * inv : 0.0f, live ? acc[3] * inv : 0.0f};
+        store_qo_vec<4>(p.o, p.qo_dtype, pair * p.d + e0, res);
+    }
 }
 
 }  // namespace ahpc
@@ -898,6 +946,7 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     const int64_t n_chunks = (max_len + chunk - 1) / chunk;
     const size_t need = n_chunks > 1 ? (size_t)(B * n_chunks * H * (d + 2)) * sizeof(float) : 0;
     if (need > 0 && (!workspace || workspace_bytes < need)) return AHPC_ERR_WORKSPACE_TOO_SMALL;
+    if (need > 0 && (reinterpret_cast<uintptr_t>(workspace) & 15u)) return AHPC_ERR_BAD_ALIGNMENT;  // partials move in 16-byte pieces
     if (n_chunks > 65535) return AHPC_ERR_BAD_SHAPE;
 
     DecodeParams p{};
@@ -920,8 +969,7 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     const int64_t head_groups = (H_kv + heads_per_wg - 1) / heads_per_wg;
     if (head_groups > 65535) return AHPC_ERR_BAD_SHAPE;
 
-    const int64_t total = B * H * d;
-    dim3 eblock(256), egrid((unsigned)((total + 255) / 256));
+    dim3 eblock(64 * kMergeWaves), egrid((unsigned)((B * H + kMergeWaves - 1) / kMergeWaves));  // the merge: a wavefront per (b, h)
 
     dim3 grid((unsigned)head_groups, (unsigned)n_chunks, (unsigned)B), block(64 * waves);
     int rc;

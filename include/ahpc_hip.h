@@ -277,7 +277,8 @@ int ahpc_hip_kv_gather(void* k_out, void* v_out, int out_dtype,
  * merged with the rule of OnlineSoftmaxState::update, src/algorithms/flash_attention.hpp:50-57.
  * `max_len` bounds seq_lens (it sizes the grid; tokens beyond it are not read).
  * workspace must hold ahpc_hip_paged_decode_workspace_bytes() bytes: with chunk_tokens = 0 that is an upper
- * bound over the chunk lengths the launch may choose (128 to 1024 tokens, by batch, context and head count). */
+ * bound over the chunk lengths the launch may choose (128 to 1024 tokens, by batch, context and head count); 16-byte
+ * aligned (AHPC_ERR_BAD_ALIGNMENT otherwise). */
 size_t ahpc_hip_paged_decode_workspace_bytes(int64_t B, int64_t H, int64_t d, int64_t max_len,
                                              int64_t P, int64_t chunk_tokens);
 int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype,
