@@ -43,7 +43,7 @@ def forward_cases(n, seed):
     return out
 
 
-@pytest.mark.parametrize("dtype,B,N,H,Hkv,d,causal,masked,seed", forward_cases(48, 20261))
+@pytest.mark.parametrize("dtype,B,N,H,Hkv,d,causal,masked,seed", forward_cases(96, 20261))
 def test_forward_random_shapes(gpu, dtype, B, N, H, Hkv, d, causal, masked, seed):
     import torch
     from gpu_util import to_dev, to_host, stream_ptr, TOL
@@ -86,7 +86,7 @@ def varlen_cases(n, seed):
     return out
 
 
-@pytest.mark.parametrize("dtype,lens,H,Hkv,d,causal,seed", varlen_cases(24, 20262))
+@pytest.mark.parametrize("dtype,lens,H,Hkv,d,causal,seed", varlen_cases(48, 20262))
 def test_ragged_forward_random_batches(gpu, dtype, lens, H, Hkv, d, causal, seed):
     import torch
     from gpu_util import to_dev, to_host, stream_ptr, dev_i32, TOL
@@ -125,7 +125,7 @@ def backward_cases(n, seed):
     return out
 
 
-@pytest.mark.parametrize("dtype,B,N,H,Hkv,d,causal,split,seed", backward_cases(24, 20263))
+@pytest.mark.parametrize("dtype,B,N,H,Hkv,d,causal,split,seed", backward_cases(48, 20263))
 def test_backward_random_shapes(gpu, dtype, B, N, H, Hkv, d, causal, split, seed):
     import torch
     from gpu_util import to_dev, to_host, stream_ptr
@@ -184,7 +184,7 @@ def decode_cases(n, seed):
     return out
 
 
-@pytest.mark.parametrize("dtype,B,lens,H,Hkv,d,P,chunk,waves,matrix_from,seed", decode_cases(64, 20264))
+@pytest.mark.parametrize("dtype,B,lens,H,Hkv,d,P,chunk,waves,matrix_from,seed", decode_cases(128, 20264))
 def test_decode_random_shapes(gpu, dtype, B, lens, H, Hkv, d, P, chunk, waves, matrix_from, seed):
     import torch
     from gpu_util import to_dev, to_host, stream_ptr, dev_i32, TOL
