@@ -274,6 +274,7 @@ template <typename T, bool VARLEN>
 static int dispatch_mfma(const FlashParams& p, int64_t B, int d, bool causal, hipStream_t stream) {
     if (d == 128) return launch_mfma<T, 128, VARLEN>(p, B, causal, stream);
     if (d == 64) return launch_mfma<T, 64, VARLEN>(p, B, causal, stream);
+    if (d == 256) return launch_mfma<T, 256, VARLEN>(p, B, causal, stream);
     return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
 }
 
@@ -283,14 +284,17 @@ struct Strides {
     int64_t b, n, h;
 };
 
-// The head dimension a matrix-core kernel is instantiated for: 64 or 128, the tensors' own or the next larger one (the
-// kernels then compute with columns that contribute nothing, FlashParams::d_real).
-static int kernel_head_dim(int64_t d) { return d <= 64 ? 64 : 128; }
+// The head dimension a matrix-core kernel is instantiated for: 64 or 128 (the 16-bit forward without a mask: also 256),
+// the tensors' own or the next larger one (the kernels then compute with columns that contribute nothing,
+// FlashParams::d_real).
+static int kernel_head_dim(int64_t d) { return d <= 64 ? 64 : d <= 128 ? 128 : 256; }
 
+// max_d: 128 wherever a dense mask is involved; 256 for the plain forward, whose instantiation for 256 keeps one workgroup
+// per CU (its operands need the accumulation registers as a second register file, and 128 KiB of LDS).
 static bool mfma_eligible(int dtype, int64_t d, const void* q, const void* k, const void* v, const void* o,
-                          const Strides& sq, const Strides& skv) {
+                          const Strides& sq, const Strides& skv, int64_t max_d = 128) {
     if (dtype != AHPC_F16 && dtype != AHPC_BF16) return false;
-    if (d < 8 || d > 128 || (d % 8)) return false;  // rows of whole 16-byte pieces
+    if (d < 8 || d > max_d || (d % 8)) return false;  // rows of whole 16-byte pieces
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return false;
     if ((sq.b % 8) || (sq.n % 8) || (sq.h % 8) || (skv.b % 8) || (skv.n % 8) || (skv.h % 8)) return false;
     // a key tile is addressed with 32-bit byte offsets from its first row, and rows must not overlap
@@ -348,7 +352,7 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
     if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int32_t group = (int32_t)(H / H_kv);
-    if (mfma_eligible(dtype, d, q, k, v, o, sq, skv)) {
+    if (mfma_eligible(dtype, d, q, k, v, o, sq, skv, mask ? 128 : 256)) {
         FlashParams p{};
         p.q = q; p.k = k; p.v = v; p.o = o;
         p.mask = mask;
@@ -449,7 +453,7 @@ int ahpc_hip_flash_fwd_varlen_gqa(const void* q, const void* k, const void* v, v
     if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int32_t group = (int32_t)(H / H_kv);
-    if (mfma_eligible(dtype, d, q, k, v, o, sq, skv)) {
+    if (mfma_eligible(dtype, d, q, k, v, o, sq, skv, 256)) {
         FlashParams p{};
         p.q = q; p.k = k; p.v = v; p.o = o;
         p.cu_seqlens = cu_seqlens;

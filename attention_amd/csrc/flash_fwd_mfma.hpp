@@ -167,8 +167,8 @@ template <int D> struct FlashTile {
     static constexpr int kInstrPerWave = kFlashKeys / (4 * kRowsPerInstr);
     static constexpr int kBytes = kFlashKeys * kRowBytes;
     // swizzles (XOR on the 16-byte chunk index)
-    __device__ static int fk(int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); }
-    __device__ static int fv(int row) { return D == 128 ? 4 * (row & 3) : 4 * ((row >> 1) & 1); }
+    __device__ static int fk(int row) { return D >= 128 ? (row & 15) : ((row >> 1) & 7); }
+    __device__ static int fv(int row) { return D >= 128 ? 4 * (row & 3) : 4 * ((row >> 1) & 1); }
     // for tiles that are read both ways (backward): 16 consecutive rows get 16 different chunks (row reads),
     // and the 4 rows of a transposing read get chunk quads that do not overlap
     __device__ static int fb(int row) {
@@ -675,7 +675,7 @@ inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal, int rows_pe
 }
 
 template <typename T, int D, bool CAUSAL, bool VARLEN>
-__global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_kernel(const FlashParams p) {
+__global__ __launch_bounds__(kFlashThreads, D == 256 ? 1 : 2) void flash_fwd_mfma_kernel(const FlashParams p) {
     flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, false>(p, FlashStatsOut{});
 }
 

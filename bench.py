@@ -382,6 +382,17 @@ def bench_extras(hip, stream, steps, warmup):
         flops=2.0 * H * Nl * Nl * d)
     del ql, kl, vl, ol
 
+    # head dimension 256 (half the heads, the same tensor sizes): the 16-bit kernel's instantiation with one workgroup per CU
+    Hw, dw = 16, 256
+    qw, kw, vw = (randn((B, N, Hw, dw), torch.bfloat16) for _ in range(3))
+    ow = torch.empty_like(qw)
+    stw = (N * Hw * dw, Hw * dw, dw)
+    run("flash_fwd bf16 causal B=4 N=4096 H=16 d=256",
+        lambda: hip.flash_fwd(qw.data_ptr(), kw.data_ptr(), vw.data_ptr(), ow.data_ptr(), hip.BF16, B, N, Hw, dw, stw, 1.0 / np.sqrt(dw), True,
+                              stream),
+        flops=2.0 * B * Hw * N * N * dw)
+    del qw, kw, vw, ow
+
     # the headline shape in fp32, the reference's default data type: the fp32 matrix-core kernel
     qf, kf, vf = randn((B, N, H, d), torch.float32), randn((B, N, H, d), torch.float32), randn((B, N, H, d), torch.float32)
     of = torch.empty_like(qf)

@@ -133,6 +133,40 @@ def test_matrix_core_kernels_smaller_head_dimensions(emu, dtype, d, N, causal, H
     assert S.lds_stats(reset=True)[0] > 0   # a matrix-core kernel ran (the FMA kernel makes no traced LDS reads)
 
 
+@pytest.mark.parametrize("dtype,d", [(O.BF16, 256), (O.F16, 200), (O.BF16, 136), (O.F16, 256)])
+@pytest.mark.parametrize("N,causal,H,H_kv,dma_late", [(150, True, 2, 1, True), (70, False, 2, 2, False)])
+def test_matrix_core_forward_head_dimensions_to_256(emu, dtype, d, N, causal, H, H_kv, dma_late):
+    """Head dimensions above 128 (to 256, in multiples of 8): the 16-bit forward's instantiation for 256, dense and ragged,
+    with its conflict counts (the swizzles are the ones of 128)."""
+    B = 2
+    q = O.round_to(O.fill_normal((B, N, H, d), 27, 1), dtype)
+    k = O.round_to(O.fill_normal((B, N, H_kv, d), 27, 2), dtype)
+    v = O.round_to(O.fill_normal((B, N, H_kv, d), 27, 3), dtype)
+    scale = 1.0 / np.sqrt(d)
+    S.configure(dma_late, seed=N + d)
+    S.lds_stats(reset=True)
+    try:
+        got = flash(emu, q, k, v, dtype, B, N, H, d, scale, causal, H_kv=H_kv, front=dma_late)
+    finally:
+        S.configure(False, 1)
+    rep = H // H_kv
+    kx, vx = np.repeat(k, rep, axis=2), np.repeat(v, rep, axis=2)
+    want = O.attention(q, kx, vx, B, N, H, d, scale, causal)
+    assert np.abs(got - want).max() <= TOL[dtype]
+    reads, read_conflicts, tr, tr_conflicts = S.lds_stats(reset=True)
+    assert reads > 0 and tr > 0   # the matrix-core kernel ran
+    print(f"d={d}: operand reads {reads} (conflicts {read_conflicts}), transposing reads {tr} (conflicts {tr_conflicts})")
+    # the same tensors as a ragged batch of B sequences
+    T = B * N
+    cu = np.arange(B + 1, dtype=np.int32) * N
+    dq, dk, dv = dev(q.reshape(T, H, d), dtype), dev(k.reshape(T, H_kv, d), dtype), dev(v.reshape(T, H_kv, d), dtype)
+    do = S.guarded(S.empty_storage((T, H, d), dtype))
+    dcu = S.guarded(cu)
+    emu.flash_fwd_varlen_gqa(S.ptr(dq), S.ptr(dk), S.ptr(dv), S.ptr(do), dtype, S.ptr(dcu), B, N, H, H_kv, d, H * d, d, H_kv * d, d,
+                             scale, causal)
+    assert np.abs(S.from_storage(do, dtype).reshape(B, N, H, d) - want).max() <= TOL[dtype]
+
+
 def test_matrix_core_kernels_smaller_head_dimensions_ragged_and_masked(emu):
     H, d = 2, 40
     lens = np.array([1, 130, 0, 64, 33], np.int32)
