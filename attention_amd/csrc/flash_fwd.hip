@@ -175,6 +175,9 @@ template <typename T, int MASK>
 static int dispatch_mfma_masked(const FlashParams& p, int64_t B, int d, bool causal, hipStream_t stream) {
     if (d == 128) return launch_mfma_masked<T, 128, MASK>(p, B, causal, stream);
     if (d == 64) return launch_mfma_masked<T, 64, MASK>(p, B, causal, stream);
+    if constexpr (MASK == 2) {  // the packed mask only: the in-place mask's 32 registers do not fit beside d = 256
+        if (d == 256) return launch_mfma_masked<T, 256, MASK>(p, B, causal, stream);
+    }
     return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
 }
 
@@ -289,8 +292,8 @@ struct Strides {
 // FlashParams::d_real).
 static int kernel_head_dim(int64_t d) { return d <= 64 ? 64 : d <= 128 ? 128 : 256; }
 
-// max_d: 128 wherever a dense mask is involved; 256 for the plain forward, whose instantiation for 256 keeps one workgroup
-// per CU (its operands need the accumulation registers as a second register file, and 128 KiB of LDS).
+// max_d: 256 for the forward, whose instantiation for 256 keeps one workgroup per CU (its operands need the accumulation
+// registers as a second register file, and 128 KiB of LDS); 128 otherwise.
 static bool mfma_eligible(int dtype, int64_t d, const void* q, const void* k, const void* v, const void* o,
                           const Strides& sq, const Strides& skv, int64_t max_d = 128) {
     if (dtype != AHPC_F16 && dtype != AHPC_BF16) return false;
@@ -352,7 +355,7 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
     if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int32_t group = (int32_t)(H / H_kv);
-    if (mfma_eligible(dtype, d, q, k, v, o, sq, skv, mask ? 128 : 256)) {
+    if (mfma_eligible(dtype, d, q, k, v, o, sq, skv, 256)) {
         FlashParams p{};
         p.q = q; p.k = k; p.v = v; p.o = o;
         p.mask = mask;
@@ -375,7 +378,7 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
             });
             if (launched || rc != AHPC_OK) return rc;
         }
-        if (N % 4 == 0 && aligned16(mask))
+        if (d <= 128 && N % 4 == 0 && aligned16(mask))  // (beyond 128 only the packed mask has a kernel)
             return dtype == AHPC_F16 ? dispatch_mfma_masked<f16_t, 1>(p, B, kernel_head_dim(d), causal != 0, st)
                                      : dispatch_mfma_masked<bf16_t, 1>(p, B, kernel_head_dim(d), causal != 0, st);
     }

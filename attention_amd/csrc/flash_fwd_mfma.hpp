@@ -681,7 +681,7 @@ __global__ __launch_bounds__(kFlashThreads, D == 256 ? 1 : 2) void flash_fwd_mfm
 
 // Dense launches with a mask [B,N,N]: MASK 1 reads the caller's fp32 mask, MASK 2 its packed copy.
 template <typename T, int D, bool CAUSAL, int MASK>
-__global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_mfma_masked_kernel(const FlashParams p) {
+__global__ __launch_bounds__(kFlashThreads, D == 256 ? 1 : 2) void flash_fwd_mfma_masked_kernel(const FlashParams p) {
     flash_fwd_mfma_body<T, D, CAUSAL, false, false, MASK>(p, FlashStatsOut{});
 }
 

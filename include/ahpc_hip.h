@@ -110,7 +110,7 @@ int ahpc_hip_event_elapsed_ms(void* start, void* stop, float* ms);
  * runs on the matrix cores: fp16/bf16 on 16-bit matrix instructions, fp32 (the reference's default,
  * DataType::FLOAT32) on fp32 ones (fp32 products and sums: same accuracy as the fp32-FMA kernel).  The kernels are
  * built for d = 64 and 128; a smaller d runs on the next one with columns that contribute nothing.  fp16/bf16 tensors
- * without a dense mask also have a kernel built for d = 256 (d from 136 to 256 in multiples of 8).  Every other
+ * also have a kernel built for d = 256 (d from 136 to 256 in multiples of 8; with a dense mask: on its packed copy).  Every other
  * case (d up to 256, unaligned tensors) runs on the fp32-FMA kernel.  Accumulation is fp32 throughout.  A row with no visible key yields zeros
  * (OnlineSoftmaxState::get_normalizer, src/algorithms/flash_attention.hpp:59-61).
  * scale <= 0 means 1/sqrt(d) (AttentionParams::scale_factor,

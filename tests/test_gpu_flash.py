@@ -103,7 +103,7 @@ def mask_path(gpu, request):
     gpu.set_tuning("mask_pack", before)
 
 
-@pytest.mark.parametrize("dtype,d", [(O.F16, 128), (O.BF16, 64), (O.BF16, 128)])
+@pytest.mark.parametrize("dtype,d", [(O.F16, 128), (O.BF16, 64), (O.BF16, 128), (O.BF16, 256), (O.F16, 200)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("N", [4, 64, 132, 520, 1028, 517, 63, 129])
 def test_dense_mask_16bit(gpu, dtype, d, causal, N, mask_path):

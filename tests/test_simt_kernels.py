@@ -135,7 +135,7 @@ def test_matrix_core_kernels_smaller_head_dimensions(emu, dtype, d, N, causal, H
 
 @pytest.mark.parametrize("dtype,d", [(O.BF16, 256), (O.F16, 200), (O.BF16, 136), (O.F16, 256)])
 @pytest.mark.parametrize("N,causal,H,H_kv,dma_late", [(150, True, 2, 1, True), (70, False, 2, 2, False)])
-def test_matrix_core_forward_head_dimensions_to_256(emu, dtype, d, N, causal, H, H_kv, dma_late):
+def test_matrix_core_forward_head_dimensions_to_256(emu, tuned, dtype, d, N, causal, H, H_kv, dma_late):
     """Head dimensions above 128 (to 256, in multiples of 8): the 16-bit forward's instantiation for 256, dense and ragged,
     with its conflict counts (the swizzles are the ones of 128)."""
     B = 2
@@ -165,6 +165,16 @@ def test_matrix_core_forward_head_dimensions_to_256(emu, dtype, d, N, causal, H,
     emu.flash_fwd_varlen_gqa(S.ptr(dq), S.ptr(dk), S.ptr(dv), S.ptr(do), dtype, S.ptr(dcu), B, N, H, H_kv, d, H * d, d, H_kv * d, d,
                              scale, causal)
     assert np.abs(S.from_storage(do, dtype).reshape(B, N, H, d) - want).max() <= TOL[dtype]
+    # and under a dense mask: the packed copy has a kernel of this size, the mask read in place has none (fp32-FMA kernel)
+    mask = (O.fill_normal((B, N, N), 28, 9) > -0.3).astype(np.float32)
+    mask[0, 3, :] = 0.0   # a query that sees nothing: zeros
+    want_m = O.attention(q, kx, vx, B, N, H, d, scale, causal, mask=mask)
+    for packed in (1, 0):
+        tuned("mask_pack", packed)
+        S.lds_stats(reset=True)
+        got_m = flash(emu, q, k, v, dtype, B, N, H, d, scale, causal, H_kv=H_kv, mask=mask)
+        assert np.abs(got_m - want_m).max() <= TOL[dtype], packed
+        assert (S.lds_stats(reset=True)[0] > 0) == (packed == 1)
 
 
 def test_matrix_core_kernels_smaller_head_dimensions_ragged_and_masked(emu):
