@@ -304,10 +304,10 @@ static bool mfma_eligible(int dtype, int64_t d, const void* q, const void* k, co
     return sq.n >= d && skv.n >= d && skv.n < (int64_t(1) << 24);
 }
 
-// fp32 tensors on the matrix cores: d 64 or 128, 16-byte aligned rows, no dense mask.
+// fp32 tensors on the matrix cores: kernels for d = 64, 128 and 256, 16-byte aligned rows.
 static bool f32_mfma_eligible(int dtype, int64_t d, const void* q, const void* k, const void* v, const void* o,
                               const Strides& sq, const Strides& skv) {
-    if (dtype != AHPC_F32 || d < 4 || d > 128 || (d % 4)) return false;  // rows of whole 16-byte pieces
+    if (dtype != AHPC_F32 || d < 4 || d > 256 || (d % 4)) return false;  // rows of whole 16-byte pieces
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return false;
     if ((sq.b % 4) || (sq.n % 4) || (sq.h % 4) || (skv.b % 4) || (skv.n % 4) || (skv.h % 4)) return false;
     // a key tile is addressed with 32-bit byte offsets from its first row, and rows must not overlap
@@ -318,7 +318,10 @@ template <bool VARLEN, bool MASKED>
 static int launch_f32_mfma(FlashParams p, int64_t B, int d, bool causal, hipStream_t stream) {
     if (int rc = flash_plan_launch(p, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load(), VARLEN)) return rc;
     dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
-    if (d == 128) {
+    if (d == 256) {  // (one workgroup per CU: registers and LDS of twice the size)
+        if (causal) hipLaunchKernelGGL((flash_fwd_f32_mfma_kernel<256, true, VARLEN, MASKED>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((flash_fwd_f32_mfma_kernel<256, false, VARLEN, MASKED>), grid, block, 0, stream, p);
+    } else if (d == 128) {
         if (causal) hipLaunchKernelGGL((flash_fwd_f32_mfma_kernel<128, true, VARLEN, MASKED>), grid, block, 0, stream, p);
         else hipLaunchKernelGGL((flash_fwd_f32_mfma_kernel<128, false, VARLEN, MASKED>), grid, block, 0, stream, p);
     } else {

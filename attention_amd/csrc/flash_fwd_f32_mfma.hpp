@@ -44,7 +44,7 @@ __device__ inline f32x16 mfma_32x32x2_f32(float a, float b, f32x16 c) {
 // FlashStatsOut describes (flash_fwd_mfma.hpp): -lse2 and -(dO . O), padding rows -inf and 0.
 template <int D, bool CAUSAL, bool VARLEN, bool MASKED, bool STATS>
 __device__ __forceinline__ void flash_fwd_f32_mfma_body(const FlashParams& p, const FlashStatsOut& st) {
-    static_assert(D == 64 || D == 128, "head dimensions of the fp32 matrix-core kernel");
+    static_assert(D == 64 || D == 128 || D == 256, "head dimensions of the fp32 matrix-core kernel");
     static_assert(!(MASKED && (VARLEN || STATS)), "the mask belongs to dense forward launches");
     constexpr int RB = 4 * D;                 // row bytes
     constexpr int CH = D / 4;                 // 16-byte chunks per row
@@ -341,7 +341,7 @@ __device__ __forceinline__ void flash_fwd_f32_mfma_body(const FlashParams& p, co
 }
 
 template <int D, bool CAUSAL, bool VARLEN, bool MASKED = false>
-__global__ __launch_bounds__(kFlashThreads, 2) void flash_fwd_f32_mfma_kernel(const FlashParams p) {
+__global__ __launch_bounds__(kFlashThreads, D == 256 ? 1 : 2) void flash_fwd_f32_mfma_kernel(const FlashParams p) {
     flash_fwd_f32_mfma_body<D, CAUSAL, VARLEN, MASKED, false>(p, FlashStatsOut{});
 }
 

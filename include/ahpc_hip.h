@@ -106,11 +106,11 @@ int ahpc_hip_event_elapsed_ms(void* start, void* stop, float* ms);
  * src/algorithms/flash_attention.cpp:238-275) is stride_b = N*H*d, stride_n = H*d,
  * stride_h = d; [B,H,N,d] is stride_b = H*N*d, stride_h = N*d, stride_n = d, so no transpose
  * pass (src/backends/cuda/cuda_kernels.cu:668-687) is ever needed.  Q, K, V and O share one
- * dtype and one set of strides.  d <= 128 with 16-byte aligned rows (d a multiple of 8 for fp16/bf16, of 4 for fp32)
+ * dtype and one set of strides.  d <= 256 with 16-byte aligned rows (d a multiple of 8 for fp16/bf16, of 4 for fp32)
  * runs on the matrix cores: fp16/bf16 on 16-bit matrix instructions, fp32 (the reference's default,
  * DataType::FLOAT32) on fp32 ones (fp32 products and sums: same accuracy as the fp32-FMA kernel).  The kernels are
- * built for d = 64 and 128; a smaller d runs on the next one with columns that contribute nothing.  fp16/bf16 tensors
- * also have a kernel built for d = 256 (d from 136 to 256 in multiples of 8; with a dense mask: on its packed copy).  Every other
+ * built for d = 64, 128 and 256 (the last at one workgroup per CU); any other d runs on the next one with columns that
+ * contribute nothing (beyond 128 with a dense mask: on its packed copy only).  Every other
  * case (d up to 256, unaligned tensors) runs on the fp32-FMA kernel.  Accumulation is fp32 throughout.  A row with no visible key yields zeros
  * (OnlineSoftmaxState::get_normalizer, src/algorithms/flash_attention.hpp:59-61).
  * scale <= 0 means 1/sqrt(d) (AttentionParams::scale_factor,

@@ -226,10 +226,10 @@ def test_dense_mask_under_graph_capture_allocates_nothing(gpu):
 
 
 @pytest.mark.parametrize("dtype,d", [(O.BF16, 32), (O.F16, 96), (O.BF16, 8), (O.F16, 120), (O.BF16, 80), (O.F32, 32), (O.F32, 100),
-                                     (O.F32, 4), (O.F32, 72), (O.BF16, 256), (O.F16, 200), (O.BF16, 136), (O.F16, 256)])
+                                     (O.F32, 4), (O.F32, 72), (O.BF16, 256), (O.F16, 200), (O.BF16, 136), (O.F16, 256), (O.F32, 256), (O.F32, 132)])
 @pytest.mark.parametrize("N,causal,H,H_kv", [(150, True, 2, 1), (64, False, 3, 3), (517, True, 4, 2)])
 def test_smaller_head_dimensions_on_the_matrix_cores(gpu, dtype, d, N, causal, H, H_kv):
-    """Head dimensions other than 64 / 128 (multiples of 8 for 16-bit tensors, of 4 for fp32; 16-bit tensors up to 256) run
+    """Head dimensions other than 64 / 128 (multiples of 8 for 16-bit tensors, of 4 for fp32; up to 256) run
     on the matrix-core kernels of the next size with columns that contribute nothing; the output tensor is pre-filled with
     NaN, every element must have been written."""
     import torch
