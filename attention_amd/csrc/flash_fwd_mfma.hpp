@@ -116,8 +116,13 @@ template <typename T, int IMM> __device__ inline u32x2 tr_read_async(const unsig
 // Waits for the LDS reads issued so far; the values pass through it, so nothing that uses them moves above the wait.
 template <int N> __device__ inline void tr_wait(u32x2 (&v)[N]) {
 #if !defined(AHPC_TRACED_LDS_READ_B128) && defined(__HIP_DEVICE_COMPILE__)
-    static_assert(N == 4 || N == 8, "operand sets of d = 64 or 128");
-    if constexpr (N == 8)
+    static_assert(N == 4 || N == 8 || N == 16, "operand sets of d = 64, 128 or 256");
+    if constexpr (N == 16) {
+        // (an asm statement takes 30 operands at most: the second half passes through an empty one right behind the wait)
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+        asm volatile("" : "+v"(v[8]), "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]), "+v"(v[14]), "+v"(v[15]));
+    } else if constexpr (N == 8)
         asm volatile("s_waitcnt lgkmcnt(0)"
                      : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
     else
@@ -139,8 +144,12 @@ template <int IMM> __device__ inline u32x4 lds_read_b128_async(const unsigned ch
 }
 template <int N> __device__ inline void b128_wait(u32x4 (&v)[N]) {
 #if !defined(AHPC_TRACED_LDS_READ_B128) && defined(__HIP_DEVICE_COMPILE__)
-    static_assert(N == 2 || N == 4 || N == 8, "operand sets of d = 64 or 128");
-    if constexpr (N == 8)
+    static_assert(N == 2 || N == 4 || N == 8 || N == 16, "operand sets of d = 64, 128 or 256");
+    if constexpr (N == 16) {
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+        asm volatile("" : "+v"(v[8]), "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]), "+v"(v[14]), "+v"(v[15]));
+    } else if constexpr (N == 8)
         asm volatile("s_waitcnt lgkmcnt(0)"
                      : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
     else if constexpr (N == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));

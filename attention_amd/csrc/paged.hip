@@ -716,6 +716,7 @@ static int launch_decode_mfma(const DecodeParams& p, hipStream_t st) {
     const dim3 grid((unsigned)p.H_kv, (unsigned)p.n_chunks, (unsigned)p.B), block(64);
     if (p.d == 128) hipLaunchKernelGGL((paged_decode_mfma_kernel<T, 128>), grid, block, 0, st, p);
     else if (p.d == 64) hipLaunchKernelGGL((paged_decode_mfma_kernel<T, 64>), grid, block, 0, st, p);
+    else if (p.d == 256) hipLaunchKernelGGL((paged_decode_mfma_kernel<T, 256>), grid, block, 0, st, p);
     else return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
     return static_cast<int>(hipGetLastError());
 }
@@ -724,10 +725,13 @@ static int launch_decode_mfma(const DecodeParams& p, hipStream_t st) {
 // pool heads side by side in a workgroup.
 template <typename T, int D>
 static int launch_decode_group_d(const DecodeParams& p, hipStream_t st) {
-    const int w = p.H_kv >= 8 ? 8 : p.H_kv >= 4 ? 4 : p.H_kv >= 2 ? 2 : 1;
+    // (at d = 256 a wavefront's two page slots take 32 KiB of LDS: four wavefronts at most)
+    const int w = (p.H_kv >= 8 && D <= 128) ? 8 : p.H_kv >= 4 ? 4 : p.H_kv >= 2 ? 2 : 1;
     const dim3 grid((unsigned)((p.H_kv + w - 1) / w), (unsigned)p.n_chunks, (unsigned)p.B), block(64 * w);
     switch (w) {
-        case 8: hipLaunchKernelGGL((paged_decode_group_kernel<T, D, 8>), grid, block, 0, st, p); break;
+        case 8:
+            if constexpr (D <= 128) hipLaunchKernelGGL((paged_decode_group_kernel<T, D, 8>), grid, block, 0, st, p);
+            break;
         case 4: hipLaunchKernelGGL((paged_decode_group_kernel<T, D, 4>), grid, block, 0, st, p); break;
         case 2: hipLaunchKernelGGL((paged_decode_group_kernel<T, D, 2>), grid, block, 0, st, p); break;
         default: hipLaunchKernelGGL((paged_decode_group_kernel<T, D, 1>), grid, block, 0, st, p); break;
@@ -739,6 +743,7 @@ template <typename T>
 static int launch_decode_group(const DecodeParams& p, hipStream_t st) {
     if (p.d == 128) return launch_decode_group_d<T, 128>(p, st);
     if (p.d == 64) return launch_decode_group_d<T, 64>(p, st);
+    if (p.d == 256) return launch_decode_group_d<T, 256>(p, st);
     return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
 }
 
@@ -921,7 +926,7 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     // heads.  The matrix-core kernels take the group size as it is (idle result columns), the lane-per-element
     // kernel runs a group or slice of 3 as 4 and 5 to 7 as 8.
     const int64_t group = H / H_kv;
-    const bool mfma_shape = (pool_dtype == AHPC_F16 || pool_dtype == AHPC_BF16) && (d == 64 || d == 128) && P == 16 && H_kv <= 65535 &&
+    const bool mfma_shape = (pool_dtype == AHPC_F16 || pool_dtype == AHPC_BF16) && (d == 64 || d == 128 || d == 256) && P == 16 && H_kv <= 65535 &&
                             group <= 32;
     if (qo_dtype < AHPC_F32 || qo_dtype > AHPC_BF16 || pool_dtype < AHPC_F32 || pool_dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
     if (B <= 0 || B > 65535 || max_len <= 0 || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;

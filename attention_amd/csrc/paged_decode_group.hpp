@@ -57,7 +57,8 @@ __global__ __launch_bounds__(64 * W) void paged_decode_group_kernel(const Decode
     constexpr int kSlot = 2 * kPart;   // a page slot: V, then K
     constexpr int P = 16;
     constexpr int kOps = 2 * NI;       // loads per page and wavefront
-    static_assert(D == 64 || D == 128, "head dimensions of this kernel");
+    static_assert(D == 64 || D == 128 || D == 256, "head dimensions of this kernel");
+    static_assert(W * R * kSlot <= 160 * 1024, "page slots of all wavefronts in LDS");
 
     __shared__ __attribute__((aligned(1024))) unsigned char lds_v[W * R * kSlot];
 
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(64 * W) void paged_decode_group_kernel(const Decode
     // V lands row-major in its slot; a row's 16-byte pieces are stored permuted (piece c at position c ^ fv(row)), so
     // that the 8 rows which 32 lanes of a transposing read touch fall into different banks (64 banks of 4 bytes;
     // at d = 64 two rows make up one pass over the banks, and rows of equal parity must differ)
-    auto fv = [](int r) { return D == 128 ? 2 * (r & 3) + 8 * ((r >> 2) & 1) : 2 * ((r >> 1) & 3); };
+    auto fv = [](int r) { return D >= 128 ? 2 * (r & 3) + 8 * ((r >> 2) & 1) : 2 * ((r >> 1) & 3); };
     int v_off[NI];
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
@@ -124,7 +125,7 @@ __global__ __launch_bounds__(64 * W) void paged_decode_group_kernel(const Decode
         v_off[i] = r * tok_bytes + (((lane % CH) ^ fv(r)) << 4);
     }
     // K: rows are read 16 bytes per lane, 16 rows by 16 lanes at a time: piece c of row r sits at c ^ fk(r)
-    auto fk = [](int r) { return D == 128 ? (r & 15) : ((r >> 1) & 7); };
+    auto fk = [](int r) { return D >= 128 ? (r & 15) : ((r >> 1) & 7); };
     int kd_off[NI];
 #pragma unroll
     for (int i = 0; i < NI; ++i) {

@@ -292,7 +292,7 @@ int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype,
 /* Decode with grouped K/V heads: the pool holds H_kv heads per token (its kv_scatter / kv_gather /
  * gather_indices calls take H = H_kv), q and o hold H = g * H_kv heads, any g; query head h reads pool head h / g.
  * Up to g = 8 every K/V byte is read once and serves the g query heads.  g from 9 to 32 (up to multi-query attention
- * with 32 heads) does the same on matrix-core kernels when the pool is fp16/bf16, d is 64 or 128 and P = 16; on other
+ * with 32 heads) does the same on matrix-core kernels when the pool is fp16/bf16, d is 64, 128 or 256 and P = 16; on other
  * pools, and beyond 32, the group is served in slices of 8 query heads that each read the K/V stream.  The head dimension
  * may be anything up to 256 in whole 16-byte pieces of the pool's type (a multiple of 8 for fp16/bf16 pools, of 4 for
  * fp32 ones); AHPC_ERR_UNSUPPORTED_HEAD_DIM otherwise.

@@ -794,6 +794,35 @@ def test_decode_grouped_heads_matrix_core_kernel(emu, G, dtype, d, tuned):
     assert reads > 0 and tr > 0 and read_conflicts == 0 and tr_conflicts == 0
 
 
+@pytest.mark.parametrize("H_kv,G,dtype", [(2, 4, O.F16), (8, 7, O.BF16), (5, 16, O.F16), (1, 32, O.BF16), (3, 20, O.F16)])
+def test_decode_grouped_heads_matrix_core_kernels_head_dimension_256(emu, tuned, H_kv, G, dtype):
+    """Both matrix-core decode kernels instantiated for d = 256 (the page-by-page one with at most four wavefronts in a
+    workgroup: its page slots take twice the LDS), chunks of several trips round the page ring, loads landing late."""
+    tuned("decode_matrix_min_group", 2)
+    B, P, d = 4, 16, 256
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [16 * 9 + 1, 5, 129, 32], 33, dtype)
+    lens = lens.copy()
+    lens[3] = 0
+    H = G * H_kv
+    q = O.round_to(O.fill_normal((B, H, d), 33, 1), dtype)
+    scale = 1.0 / np.sqrt(d)
+    rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
+    want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    kp, vp, table = poison_unused(kp, vp, table, lens, P, H_kv, d, wild_page=1 << 24)
+    S.lds_stats(reset=True)
+    for chunk, dma_late in ((0, False), (48, True), (1024, True)):
+        S.configure(dma_late, seed=G + chunk)
+        try:
+            got = decode(emu, q, kp, vp, table, lens, None, B, H, H_kv, d, P, dtype, dtype, scale, chunk)
+        finally:
+            S.configure(False, 1)
+        assert np.all(got[3] == 0.0)
+        assert np.abs(got - want).max() <= 2e-2, chunk
+    reads, read_conflicts, tr, tr_conflicts = S.lds_stats(reset=True)
+    assert reads > 0 and tr > 0   # a matrix-core kernel ran
+    print(f"G={G}: operand reads {reads} (conflicts {read_conflicts}), transposing reads {tr} (conflicts {tr_conflicts})")
+
+
 @pytest.mark.parametrize("H_kv,G,d,dtype", [(8, 4, 128, O.F16), (5, 2, 64, O.BF16), (1, 16, 128, O.BF16), (3, 8, 64, O.F16)])
 def test_decode_page_ring_of_the_group_kernel(emu, tuned, H_kv, G, d, dtype):
     """The page-by-page matrix-core kernel with 8, 4, 2 and 1 pool heads side by side in a workgroup (5 heads leave

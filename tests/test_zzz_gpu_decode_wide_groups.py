@@ -35,7 +35,7 @@ def matrix_kernel_from_four(gpu):
     gpu.set_tuning("decode_matrix_min_group", before)
 
 
-@pytest.mark.parametrize("dtype,d", [(O.F16, 128), (O.BF16, 64), (O.BF16, 128)])
+@pytest.mark.parametrize("dtype,d", [(O.F16, 128), (O.BF16, 64), (O.BF16, 128), (O.F16, 256), (O.BF16, 256)])
 @pytest.mark.parametrize("G", [4, 5, 7, 8, 12, 16, 17, 24, 31, 32])
 def test_matrix_core_decode_equals_repeated_heads(gpu, G, dtype, d, matrix_kernel_from_four):
     B, H_kv, P = 5, 2, 16
