@@ -153,8 +153,25 @@ static int dispatch_simple(int dtype, const SimpleParams& p, int64_t B, hipStrea
 }
 
 // ---------------------------------------------------------------------------------------------
+// Query rows per workgroup of the 16-bit forward: the tuning value when it names one, else by shape.
+static int flash_rows_for(int D) {
+    const int64_t t = tuning().flash_rows.load();
+    if (D == 256) return kFlashRows;  // (one wavefront per SIMD already)
+    if (t == kFlashRows || t == kFlashWideRows) return (int)t;
+    return kFlashRows;
+}
+
 template <typename T, int D, bool VARLEN>
 static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
+    if constexpr (D != 256) {
+        if (flash_rows_for(D) == kFlashWideRows) {
+            if (int rc = flash_plan_launch(p, B, causal, kFlashWideRows, tuning().flash_pair_min_tiles.load(), VARLEN)) return rc;
+            dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(64 * kFlashWideWaves);
+            if (causal) hipLaunchKernelGGL((flash_fwd_mfma_wide_kernel<T, D, true, VARLEN>), grid, block, 0, stream, p);
+            else hipLaunchKernelGGL((flash_fwd_mfma_wide_kernel<T, D, false, VARLEN>), grid, block, 0, stream, p);
+            return static_cast<int>(hipGetLastError());
+        }
+    }
     if (int rc = flash_plan_launch(p, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load(), VARLEN)) return rc;
     dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(kFlashThreads);
     if (causal) hipLaunchKernelGGL((flash_fwd_mfma_kernel<T, D, true, VARLEN>), grid, block, 0, stream, p);

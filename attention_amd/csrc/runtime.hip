@@ -21,7 +21,8 @@ Tuning::Tuning()
       decode_matrix_min_group(env_value("AHPC_DECODE_MFMA_MIN_GROUP", 2)),
       bwd_split(env_value("AHPC_BWD_SPLIT", 0)),
       mask_pack(env_value("AHPC_MASK_PACK", 1)),
-      bwd_pair(env_value("AHPC_BWD_PAIR", 1)) {
+      bwd_pair(env_value("AHPC_BWD_PAIR", 1)),
+      flash_rows(env_value("AHPC_FLASH_ROWS", 0)) {
     if (flash_pair_min_tiles.load() < 1) flash_pair_min_tiles = 1024;
 }
 
@@ -40,6 +41,7 @@ static std::atomic<int64_t>* tuning_slot(const char* name) {
     if (!std::strcmp(name, "bwd_split")) return &t.bwd_split;
     if (!std::strcmp(name, "mask_pack")) return &t.mask_pack;
     if (!std::strcmp(name, "bwd_pair")) return &t.bwd_pair;
+    if (!std::strcmp(name, "flash_rows")) return &t.flash_rows;
     return nullptr;
 }
 

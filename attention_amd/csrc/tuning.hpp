@@ -32,6 +32,10 @@ struct Tuning {
     // backward, causal dense launches: 1 (default) = the dQ and dK/dV workgroups take a long and a short tile of their
     // head each (equal work for all), 0 = one tile per workgroup, long tiles first.  (AHPC_BWD_PAIR)
     std::atomic<int64_t> bwd_pair;
+    // forward on the 16-bit matrix-core kernel: query rows per workgroup, 128 (4 wavefronts, two workgroups per CU) or
+    // 256 (8 wavefronts, one workgroup per CU: one stream of K/V tiles feeds twice the rows); 0 (default) = by shape.
+    // (AHPC_FLASH_ROWS)
+    std::atomic<int64_t> flash_rows;
     Tuning();
 };
 
