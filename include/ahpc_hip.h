@@ -67,9 +67,10 @@ typedef struct ahpc_device_info {
     int32_t  runtime_version;
 } ahpc_device_info;
 
-/* Launcher tuning values ("flash_pair_min_tiles", "decode_waves", "decode_chunk", "decode_matrix_min_group", "bwd_split",
- * "bwd_pair", "mask_pack"): process-wide, each starts from its environment variable (AHPC_FLASH_PAIR_MIN, AHPC_DECODE_WAVES,
- * AHPC_DECODE_CHUNK, AHPC_DECODE_MFMA_MIN_GROUP, AHPC_BWD_SPLIT, AHPC_BWD_PAIR, AHPC_MASK_PACK), which is read once.  No value
+/* Launcher tuning values ("flash_pair_min_tiles", "flash_rows", "decode_waves", "decode_chunk", "decode_matrix_min_group",
+ * "bwd_split", "bwd_pair", "mask_pack"): process-wide, each starts from its environment variable (AHPC_FLASH_PAIR_MIN,
+ * AHPC_FLASH_ROWS, AHPC_DECODE_WAVES, AHPC_DECODE_CHUNK, AHPC_DECODE_MFMA_MIN_GROUP, AHPC_BWD_SPLIT, AHPC_BWD_PAIR,
+ * AHPC_MASK_PACK), which is read once.  No value
  * changes results; unknown names and negative values are refused.  The reference has no counterpart: its tile sizes
  * sit in PerformanceConfig (src/api/attention_interface.hpp:29-53), which the host classes still honour. */
 int ahpc_hip_set_tuning(const char* name, int64_t value);
@@ -169,8 +170,9 @@ int ahpc_hip_flash_fwd_varlen_gqa(const void* q, const void* k, const void* v, v
 /* Debug twin of the MFMA kernel's launch geometry, evaluated on the HOST by the very function the kernel
  * uses (no GPU needed): for a dense fp16/bf16 launch of B sequences, N tokens, H heads it reports the grid
  * size in *n_blocks and, when the three arrays (capacity entries each) are given, for every workgroup id
- * its (sequence * H + head), the query tile (of 128 rows) it handles first and the one it handles second
- * (-1 = none; all -1 for padding workgroups).  Lets a test check that every query tile of every head is
+ * its (sequence * H + head), the query tile it handles first and the one it handles second (-1 = none; all -1
+ * for padding workgroups).  Tiles are 128 query rows, or 256 while the tuning value "flash_rows" is 256 (the
+ * launcher itself takes 256 rows at d = 128 for dense launches of at least 2048 tokens that fill the chip).  Lets a test check that every query tile of every head is
  * handled exactly once, whatever the pairing and interleaving in force.  No counterpart in the reference
  * (its kernels are launched one tile per block, src/backends/cuda/cuda_kernels.cu:125-127). */
 int ahpc_hip_flash_block_map(int64_t B, int64_t N, int64_t H, int causal, int64_t capacity, int64_t* n_blocks,

@@ -5,10 +5,10 @@ attention; one that names a head that does not exist reads outside the tensors."
 import numpy as np
 import pytest
 
-ROWS = 128  # query rows per workgroup pass
+ROWS = 128  # query rows per workgroup pass (256 while the tuning value flash_rows says so)
 
 
-def check_exact_cover(B, N, H, causal):
+def check_exact_cover(B, N, H, causal, ROWS=ROWS):
     from attention_amd import hip
     bh, t0, t1 = hip.flash_block_map(B, N, H, causal)
     n_tiles = (N + ROWS - 1) // ROWS
@@ -44,6 +44,18 @@ def test_default_map_covers_every_tile_once_and_keeps_its_order(B, N, H, causal)
         assert bh[block] == logical // per_head and t0[block] == n_tiles - 1 - slot
         want_second = slot if paired and 2 * slot != n_tiles - 1 else -1
         assert t1[block] == want_second
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,N,H", SHAPES)
+def test_map_of_256_row_workgroups_covers_every_tile_once(B, N, H, causal):
+    from attention_amd import hip
+    before = hip.get_tuning("flash_rows")
+    hip.set_tuning("flash_rows", 256)
+    try:
+        check_exact_cover(B, N, H, causal, ROWS=256)
+    finally:
+        hip.set_tuning("flash_rows", before)
 
 
 def test_rejects_bad_shapes_without_a_gpu():

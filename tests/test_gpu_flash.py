@@ -265,6 +265,58 @@ def test_mfma_small(gpu, dtype, d, causal, N):
     assert np.abs(got - want).max() <= 2e-2
 
 
+@pytest.fixture
+def flash_rows(gpu):
+    """flash_rows(n) pins the query rows per workgroup of the 16-bit forward (128 or 256) for the rest of the test."""
+    before = gpu.get_tuning("flash_rows")
+    yield lambda n: gpu.set_tuning("flash_rows", n)
+    gpu.set_tuning("flash_rows", before)
+
+
+@pytest.mark.parametrize("dtype,d", [(O.BF16, 128), (O.F16, 128), (O.F16, 64), (O.BF16, 96)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("N", [1, 64, 255, 256, 257, 517, 1300])
+def test_256_row_workgroups_against_oracle_and_128_row_form(gpu, flash_rows, dtype, d, causal, N):
+    """The forward with 8 wavefronts per workgroup (256 query rows share one stream of K/V tiles): against the oracle,
+    and bit-identical with the 4-wavefront form (a wavefront does the same arithmetic on the same keys in both)."""
+    from gpu_util import TOL
+    B, H = 2, 3
+    q, k, v = make_qkv((B, N, H, d), 300 + N, dtype)
+    scale = 1.0 / np.sqrt(d)
+    flash_rows(256)
+    wide = run_dense(gpu, q, k, v, dtype, B, N, H, d, scale, causal)
+    flash_rows(128)
+    narrow = run_dense(gpu, q, k, v, dtype, B, N, H, d, scale, causal)
+    assert np.isfinite(wide).all()
+    assert np.abs(wide - O.attention(q, k, v, B, N, H, d, scale, causal)).max() <= TOL[dtype]
+    assert np.array_equal(wide, narrow)
+
+
+def test_256_row_workgroups_ragged_and_grouped_heads(gpu, flash_rows):
+    import torch
+    from gpu_util import stream_ptr, to_dev, to_host, dev_i32, TOL
+    flash_rows(256)
+    gpu.set_tuning("flash_pair_min_tiles", 1)
+    try:
+        dtype, H, H_kv, d = O.BF16, 4, 2, 128
+        lens = np.array([700, 1, 256, 1029, 64], np.int32)
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        T = int(cu[-1])
+        q = O.round_to(O.fill_normal((T, H, d), 77, 1), dtype)
+        k = O.round_to(O.fill_normal((T, H_kv, d), 77, 2), dtype)
+        v = O.round_to(O.fill_normal((T, H_kv, d), 77, 3), dtype)
+        dq, dk, dv = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype)
+        do = torch.full_like(dq, float("nan"))
+        gpu.flash_fwd_varlen_gqa(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), do.data_ptr(), dtype, dev_i32(cu).data_ptr(), len(lens),
+                                 int(lens.max()), H, H_kv, d, H * d, d, H_kv * d, d, 0.1, True, stream_ptr())
+        torch.cuda.synchronize()
+        kr, vr = np.repeat(k, H // H_kv, axis=1), np.repeat(v, H // H_kv, axis=1)
+        want = O.attention_varlen(q, kr, vr, cu, H, d, 0.1, True)
+        assert np.abs(to_host(do) - want).max() <= TOL[dtype]
+    finally:
+        gpu.set_tuning("flash_pair_min_tiles", 1024)
+
+
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16])
 def test_mfma_closed_forms(gpu, dtype):
     B, N, H, d = 1, 256, 2, 128
