@@ -3,6 +3,9 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <vector>
 
 #include "ahpc_hip.h"
 #include "tuning.hpp"
@@ -22,7 +25,8 @@ Tuning::Tuning()
       bwd_split(env_value("AHPC_BWD_SPLIT", 0)),
       mask_pack(env_value("AHPC_MASK_PACK", 1)),
       bwd_pair(env_value("AHPC_BWD_PAIR", 1)),
-      flash_rows(env_value("AHPC_FLASH_ROWS", 0)) {
+      flash_rows(env_value("AHPC_FLASH_ROWS", 0)),
+      pool_in_place(env_value("AHPC_POOL_IN_PLACE", 1)) {
     if (flash_pair_min_tiles.load() < 1) flash_pair_min_tiles = 1024;
 }
 
@@ -42,6 +46,7 @@ static std::atomic<int64_t>* tuning_slot(const char* name) {
     if (!std::strcmp(name, "mask_pack")) return &t.mask_pack;
     if (!std::strcmp(name, "bwd_pair")) return &t.bwd_pair;
     if (!std::strcmp(name, "flash_rows")) return &t.flash_rows;
+    if (!std::strcmp(name, "pool_in_place")) return &t.pool_in_place;
     return nullptr;
 }
 
@@ -121,19 +126,149 @@ int ahpc_hip_device_info(int device, ahpc_device_info* out) {
     return AHPC_OK;
 }
 
+// A failed allocation must not be reported again by whatever asks for the last error next (every kernel launcher
+// does): the error is read here, where it is returned.
 int ahpc_hip_malloc(void** ptr, size_t bytes) {
     if (!ptr) return AHPC_ERR_NULL_POINTER;
-    return static_cast<int>(hipMalloc(ptr, bytes ? bytes : 1));
+    const hipError_t e = hipMalloc(ptr, bytes ? bytes : 1);
+    if (e != hipSuccess) {
+        *ptr = nullptr;
+        (void)hipGetLastError();
+    }
+    return static_cast<int>(e);
 }
 
 int ahpc_hip_free(void* ptr) { return ptr ? static_cast<int>(hipFree(ptr)) : AHPC_OK; }
 
 int ahpc_hip_host_malloc(void** ptr, size_t bytes) {
     if (!ptr) return AHPC_ERR_NULL_POINTER;
-    return static_cast<int>(hipHostMalloc(ptr, bytes ? bytes : 1, hipHostMallocDefault));
+    const hipError_t e = hipHostMalloc(ptr, bytes ? bytes : 1, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        *ptr = nullptr;
+        (void)hipGetLastError();
+    }
+    return static_cast<int>(e);
 }
 
 int ahpc_hip_host_free(void* ptr) { return ptr ? static_cast<int>(hipHostFree(ptr)) : AHPC_OK; }
+
+// ---- address ranges that grow in place ------------------------------------------------------------------------
+// A range of device addresses is reserved once; physical memory is mapped behind its front part on demand
+// (hipMemAddressReserve / hipMemCreate / hipMemMap / hipMemSetAccess), in chunks of ONE size per range: on this
+// runtime hipMemSetAccess refuses a mapping whose size differs from that of the range's earlier mappings.  Pointers
+// into the range stay valid while it grows, nothing is copied and no stream is synchronised.  The library keeps the
+// physical handles of every range.
+namespace {
+struct VmemRange {
+    size_t reserved = 0;
+    size_t chunk = 0;
+    size_t committed = 0;
+    int device = 0;
+    std::vector<hipMemGenericAllocationHandle_t> chunks;
+};
+std::mutex g_vmem_mu;
+std::map<void*, VmemRange> g_vmem;
+constexpr size_t kVmemAlign = size_t(2) << 20;  // chunks are multiples of 2 MiB
+size_t round_up(size_t n, size_t to) { return (n + to - 1) / to * to; }
+}  // namespace
+
+int ahpc_hip_vmem_granularity(size_t* bytes) {
+    if (!bytes) return AHPC_ERR_NULL_POINTER;
+    *bytes = 0;
+    int dev = 0, sup = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&sup, hipDeviceAttributeVirtualMemoryManagementSupported, dev) != hipSuccess || !sup) {
+        (void)hipGetLastError();
+        return AHPC_OK;
+    }
+    *bytes = kVmemAlign;
+    return AHPC_OK;
+}
+
+int ahpc_hip_vmem_reserve(void** base, size_t bytes, size_t chunk_bytes) {
+    if (!base) return AHPC_ERR_NULL_POINTER;
+    *base = nullptr;
+    if (!bytes || !chunk_bytes) return AHPC_ERR_BAD_SHAPE;
+    size_t gran = 0;
+    ahpc_hip_vmem_granularity(&gran);
+    if (!gran) return AHPC_ERR_NO_DEVICE;
+    VmemRange r;
+    r.chunk = round_up(chunk_bytes, kVmemAlign);
+    r.reserved = round_up(bytes, r.chunk);
+    if (hipGetDevice(&r.device) != hipSuccess) return AHPC_ERR_NO_DEVICE;
+    void* p = nullptr;
+    const hipError_t e = hipMemAddressReserve(&p, r.reserved, 0, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return static_cast<int>(e);
+    }
+    std::lock_guard<std::mutex> lock(g_vmem_mu);
+    g_vmem[p] = r;
+    *base = p;
+    return AHPC_OK;
+}
+
+int ahpc_hip_vmem_commit(void* base, size_t bytes, size_t* committed) {
+    std::lock_guard<std::mutex> lock(g_vmem_mu);
+    auto it = g_vmem.find(base);
+    if (it == g_vmem.end()) return AHPC_ERR_NULL_POINTER;
+    VmemRange& r = it->second;
+    if (committed) *committed = r.committed;
+    const size_t want = round_up(bytes, r.chunk);
+    if (want > r.reserved) return AHPC_ERR_BAD_SHAPE;
+    hipMemAllocationProp prop = {};
+    prop.type = hipMemAllocationTypePinned;
+    prop.location.type = hipMemLocationTypeDevice;
+    prop.location.id = r.device;
+    hipMemAccessDesc acc = {};
+    acc.location.type = hipMemLocationTypeDevice;
+    acc.location.id = r.device;
+    acc.flags = hipMemAccessFlagsProtReadWrite;
+    while (r.committed < want) {
+        // one chunk at a time: whatever fails, the chunks mapped so far stay usable and nothing half-mapped is left
+        hipMemGenericAllocationHandle_t h;
+        hipError_t e = hipMemCreate(&h, r.chunk, &prop, 0);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return static_cast<int>(e);  // (out of memory)
+        }
+        char* at = static_cast<char*>(base) + r.committed;
+        e = hipMemMap(at, r.chunk, 0, h, 0);
+        if (e == hipSuccess) {
+            e = hipMemSetAccess(at, r.chunk, &acc, 1);
+            if (e != hipSuccess) (void)hipMemUnmap(at, r.chunk);
+        }
+        if (e != hipSuccess) {
+            (void)hipMemRelease(h);
+            (void)hipGetLastError();
+            return static_cast<int>(e);
+        }
+        r.chunks.push_back(h);
+        r.committed += r.chunk;
+        if (committed) *committed = r.committed;
+    }
+    return AHPC_OK;
+}
+
+int ahpc_hip_vmem_release(void* base) {
+    if (!base) return AHPC_OK;
+    std::lock_guard<std::mutex> lock(g_vmem_mu);
+    auto it = g_vmem.find(base);
+    if (it == g_vmem.end()) return AHPC_ERR_NULL_POINTER;
+    VmemRange& r = it->second;
+    hipError_t first = hipSuccess;
+    for (size_t i = 0; i < r.chunks.size(); ++i) {
+        hipError_t e = hipMemUnmap(static_cast<char*>(base) + i * r.chunk, r.chunk);
+        if (e != hipSuccess && first == hipSuccess) first = e;
+        e = hipMemRelease(r.chunks[i]);
+        if (e != hipSuccess && first == hipSuccess) first = e;
+    }
+    const hipError_t e = hipMemAddressFree(base, r.reserved);
+    if (e != hipSuccess && first == hipSuccess) first = e;
+    g_vmem.erase(it);
+    if (first != hipSuccess) (void)hipGetLastError();
+    return static_cast<int>(first);
+}
 
 int ahpc_hip_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream) {
     if (!bytes) return AHPC_OK;

@@ -36,6 +36,10 @@ struct Tuning {
     // 256 (8 wavefronts, one workgroup per CU: one stream of K/V tiles feeds twice the rows); 0 (default) = by shape.
     // (AHPC_FLASH_ROWS)
     std::atomic<int64_t> flash_rows;
+    // KV block pool (host class): 1 (default) = slabs are address ranges that grow in place where the device has virtual
+    // memory management; 0 = plain allocations that grow by reallocation and a device copy.  Read when a pool is
+    // created.  (AHPC_POOL_IN_PLACE)
+    std::atomic<int64_t> pool_in_place;
     Tuning();
 };
 

@@ -47,6 +47,10 @@ SIGNATURES = {
     "ahpc_hip_free": (_ci, [_vp]),
     "ahpc_hip_host_malloc": (_ci, [C.POINTER(_vp), _sz]),
     "ahpc_hip_host_free": (_ci, [_vp]),
+    "ahpc_hip_vmem_granularity": (_ci, [C.POINTER(_sz)]),
+    "ahpc_hip_vmem_reserve": (_ci, [C.POINTER(_vp), _sz, _sz]),
+    "ahpc_hip_vmem_commit": (_ci, [_vp, _sz, C.POINTER(_sz)]),
+    "ahpc_hip_vmem_release": (_ci, [_vp]),
     "ahpc_hip_memcpy_h2d": (_ci, [_vp, _vp, _sz, _vp]),
     "ahpc_hip_memcpy_d2h": (_ci, [_vp, _vp, _sz, _vp]),
     "ahpc_hip_memcpy_d2d": (_ci, [_vp, _vp, _sz, _vp]),
@@ -123,6 +127,30 @@ def get_tuning(name):
     v = _i64()
     _check(load().ahpc_hip_get_tuning(name.encode(), C.byref(v)), "get_tuning")
     return v.value
+
+
+def vmem_granularity():
+    """Bytes address ranges that grow in place are rounded to; 0 = the device has no virtual memory management."""
+    n = _sz(0)
+    _check(load().ahpc_hip_vmem_granularity(C.byref(n)), "vmem_granularity")
+    return n.value
+
+
+def vmem_reserve(nbytes, chunk_bytes):
+    p = _vp()
+    _check(load().ahpc_hip_vmem_reserve(C.byref(p), nbytes, chunk_bytes), "vmem_reserve")
+    return p.value
+
+
+def vmem_commit(base, nbytes):
+    """Backs the first nbytes of the range with memory; returns the bytes now backed."""
+    n = _sz(0)
+    _check(load().ahpc_hip_vmem_commit(base, nbytes, C.byref(n)), "vmem_commit")
+    return n.value
+
+
+def vmem_release(base):
+    _check(load().ahpc_hip_vmem_release(base), "vmem_release")
 
 
 def device_info(device=0):

@@ -21,26 +21,66 @@ KVBlockPool::KVBlockPool(size_t page_tokens, size_t heads, size_t head_dim, Data
         const uint64_t avail = info.free_memory_bytes ? info.free_memory_bytes : info.total_memory_bytes;
         max_bytes_ = static_cast<size_t>(avail / 10 * 9);
     }
+    // Where the device has virtual memory management the slabs are address ranges sized for the whole budget, backed
+    // by physical memory only as far as pages exist: they grow in place.
+    const size_t page_bytes_one = slab_elems_per_page_ * hipsup::dtype_size(dtype_);
+    size_t granularity = 0;
+    int64_t wanted = 1;
+    ahpc_hip_get_tuning("pool_in_place", &wanted);
+    if (wanted != 0 && ahpc_hip_vmem_granularity(&granularity) == 0 && granularity != 0) {
+        const size_t range = std::max<size_t>(max_bytes_ / (2 * page_bytes_one), 1) * page_bytes_one;
+        // memory arrives in chunks of one size per slab: 64 MiB, or more where the budget is large (at most 256 chunks)
+        size_t chunk = size_t(64) << 20;
+        while (chunk * 256 < range) chunk *= 2;
+        void* nk = nullptr;
+        void* nv = nullptr;
+        if (ahpc_hip_vmem_reserve(&nk, range, chunk) == 0 && ahpc_hip_vmem_reserve(&nv, range, chunk) == 0) {
+            k_slab_ = nk;
+            v_slab_ = nv;
+            in_place_ = true;
+        } else {
+            ahpc_hip_vmem_release(nk);
+            ahpc_hip_vmem_release(nv);
+        }
+    }
     std::lock_guard<std::mutex> lock(mutex_);
     create_pages_locked(initial_pages);
 }
 
 KVBlockPool::~KVBlockPool() {
-    ahpc_hip_free(k_slab_);
-    ahpc_hip_free(v_slab_);
+    if (in_place_) {
+        ahpc_hip_vmem_release(k_slab_);
+        ahpc_hip_vmem_release(v_slab_);
+    } else {
+        ahpc_hip_free(k_slab_);
+        ahpc_hip_free(v_slab_);
+    }
 }
 
-// Grows the slabs to hold at least `pages` pages: new allocation of twice the size (at least 64
-// pages), device-to-device copy of what exists, release of the old slabs.
+// Grows the slabs to hold at least `pages` pages.  In place (the usual case): more physical memory is mapped behind
+// the slabs' address ranges, in whole chunks, within the budget; nothing moves, no stream waits, the generation stays
+// what it is.  Without virtual memory management: new allocation of twice
+// the size (at least 64 pages), device-to-device copy of what exists, release of the old slabs.
 void KVBlockPool::reserve_locked(size_t pages) {
     if (pages <= capacity_pages_) return;
     const size_t page_bytes_one = slab_elems_per_page_ * hipsup::dtype_size(dtype_);
-    size_t want = std::max<size_t>(std::max<size_t>(capacity_pages_ * 2, pages), 64);
     const size_t cap_by_budget = max_bytes_ / (2 * page_bytes_one);
-    if (want > cap_by_budget) want = cap_by_budget;
-    if (want < pages)
+    if (pages > cap_by_budget)
         throw MemoryPoolException("KV block pool exhausted: " + std::to_string(pages) + " pages needed, device budget allows " +
                                   std::to_string(cap_by_budget));
+    if (in_place_) {
+        // whole chunks: what a commit gives beyond the request is capacity for later pages
+        size_t got_k = 0, got_v = 0;
+        const int rk = ahpc_hip_vmem_commit(k_slab_, pages * page_bytes_one, &got_k);
+        const int rv = ahpc_hip_vmem_commit(v_slab_, pages * page_bytes_one, &got_v);
+        capacity_pages_ = std::max(capacity_pages_, std::min(std::min(got_k, got_v) / page_bytes_one, cap_by_budget));
+        if (rk != 0 || rv != 0 || capacity_pages_ < pages)
+            throw MemoryPoolException("KV block pool exhausted: the device cannot back " + std::to_string(pages) + " pages (" +
+                                      std::to_string(capacity_pages_) + " backed, status " + std::to_string(rk ? rk : rv) + ")");
+        return;
+    }
+    size_t want = std::max<size_t>(std::max<size_t>(capacity_pages_ * 2, pages), 64);
+    if (want > cap_by_budget) want = cap_by_budget;
     // Old and new slabs exist side by side until the copy is done; when the device cannot hold both, fall back
     // to exactly what is needed, and report what is left as the pool being exhausted (not as a failed call).
     void* nk = nullptr;

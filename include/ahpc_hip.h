@@ -68,9 +68,9 @@ typedef struct ahpc_device_info {
 } ahpc_device_info;
 
 /* Launcher tuning values ("flash_pair_min_tiles", "flash_rows", "decode_waves", "decode_chunk", "decode_matrix_min_group",
- * "bwd_split", "bwd_pair", "mask_pack"): process-wide, each starts from its environment variable (AHPC_FLASH_PAIR_MIN,
- * AHPC_FLASH_ROWS, AHPC_DECODE_WAVES, AHPC_DECODE_CHUNK, AHPC_DECODE_MFMA_MIN_GROUP, AHPC_BWD_SPLIT, AHPC_BWD_PAIR,
- * AHPC_MASK_PACK), which is read once.  No value
+ * "bwd_split", "bwd_pair", "mask_pack", "pool_in_place"): process-wide, each starts from its environment variable
+ * (AHPC_FLASH_PAIR_MIN, AHPC_FLASH_ROWS, AHPC_DECODE_WAVES, AHPC_DECODE_CHUNK, AHPC_DECODE_MFMA_MIN_GROUP, AHPC_BWD_SPLIT,
+ * AHPC_BWD_PAIR, AHPC_MASK_PACK, AHPC_POOL_IN_PLACE), which is read once.  No value
  * changes results; unknown names and negative values are refused.  The reference has no counterpart: its tile sizes
  * sit in PerformanceConfig (src/api/attention_interface.hpp:29-53), which the host classes still honour. */
 int ahpc_hip_set_tuning(const char* name, int64_t value);
@@ -81,6 +81,20 @@ int ahpc_hip_malloc(void** ptr, size_t bytes);
 int ahpc_hip_free(void* ptr);
 int ahpc_hip_host_malloc(void** ptr, size_t bytes);           /* pinned host staging memory */
 int ahpc_hip_host_free(void* ptr);
+/* Device address ranges that grow in place (what the KV block pool's slabs live in): reserve `bytes` of addresses
+ * once, then commit physical memory behind the first `bytes` of the range, as often as needed.  Memory arrives in
+ * chunks of `chunk_bytes` (rounded up to 2 MiB; one size per range, which this runtime's virtual memory management
+ * insists on): committed only ever grows, *committed, when given, receives the bytes now backed - the request
+ * rounded up to whole chunks, or less when the device ran out of memory part-way (then the call returns the
+ * runtime's out-of-memory code and what was committed stays usable).  Pointers into the range never move, nothing
+ * is copied and no stream is synchronised: kernels on other streams keep running while a range grows.
+ * ahpc_hip_vmem_granularity reports 0 on a device without virtual memory management (then reserve returns
+ * AHPC_ERR_NO_DEVICE and callers fall back to ahpc_hip_malloc).  Takes the place of the reference's
+ * grow-by-reallocation of host vectors (PagePool::allocate_new_pages, src/algorithms/paged_attention.cpp:41-48). */
+int ahpc_hip_vmem_granularity(size_t* bytes);
+int ahpc_hip_vmem_reserve(void** base, size_t bytes, size_t chunk_bytes);
+int ahpc_hip_vmem_commit(void* base, size_t bytes, size_t* committed);
+int ahpc_hip_vmem_release(void* base);                        /* unmaps, frees the physical memory and the addresses */
 int ahpc_hip_memcpy_h2d(void* dst, const void* src_host, size_t bytes, void* stream);
 int ahpc_hip_memcpy_d2h(void* dst_host, const void* src, size_t bytes, void* stream);
 int ahpc_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream);

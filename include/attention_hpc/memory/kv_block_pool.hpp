@@ -5,9 +5,11 @@
 // src/algorithms/paged_attention.cpp:11-64) and keeps its allocation order exactly, because page ids
 // end up in the block table and so in every gather index: pages are numbered in creation order,
 // allocate() pops the FRONT of the free queue, an empty queue first grows by `growth` pages, and
-// deallocate() pushes to the BACK.  What is new is where the bytes live: the slab is sized against
-// the GPU's HBM (288 GB on MI355X), grows by doubling (device-to-device copy) when the page count
-// outruns it, and is never touched by the host.  Counters follow the reference's MemoryStats idea
+// deallocate() pushes to the BACK.  What is new is where the bytes live: each slab is a range of device
+// addresses reserved once for the whole budget (sized against the GPU's HBM, 288 GB on MI355X) and backed
+// by physical memory only as far as pages exist; growth maps more memory behind it, in place: slab pointers
+// never move, nothing is copied, no stream waits.  (On a device without virtual memory management the slabs
+// are plain allocations that grow by doubling and a device-to-device copy.)  The host never touches them.  Counters follow the reference's MemoryStats idea
 // (src/memory/memory_pool.hpp:29-53): bytes in use, peak, capacity.
 #pragma once
 
@@ -61,8 +63,10 @@ public:
     void* v_slab() const { return v_slab_; }
     DataType dtype() const { return dtype_; }
     size_t page_tokens() const { return page_tokens_; }
-    // Bumped whenever the slabs move (growth): holders of raw slab pointers must re-read them.
+    // Bumped whenever the slabs move: holders of raw slab pointers must re-read them.  Slabs that grow in place
+    // (grows_in_place()) never move: the generation then stays 0.
     uint64_t generation() const { return generation_; }
+    bool grows_in_place() const { return in_place_; }
 
 private:
     void create_pages_locked(size_t count);
@@ -76,6 +80,7 @@ private:
     size_t capacity_pages_ = 0;
     void* k_slab_ = nullptr;
     void* v_slab_ = nullptr;
+    bool in_place_ = false;
     uint64_t generation_ = 0;
     std::deque<int32_t> free_;
     std::vector<uint8_t> in_use_;

@@ -13,6 +13,7 @@
 #include <functional>
 #include <string>
 #include <atomic>
+#include <chrono>
 #include <thread>
 #include <vector>
 
@@ -20,6 +21,8 @@
 #include "algorithms/paged_attention.hpp"
 #include "api/backend_factory.hpp"
 #include "api/tensor.hpp"
+#include "ahpc_hip.h"
+#include "memory/kv_block_pool.hpp"
 #include "oracle.h"
 
 using namespace attention_hpc;
@@ -1066,6 +1069,189 @@ CASE(Paged_PoolGrowsWhileOtherThreadsAppendAndDecode, true) {
     ahpc_oracle_paged_decode(q.data(), want.data(), k.data(), v.data(), table.data(), &len, nullptr, 1, H, d, P, table.size(),
                              1.0f / std::sqrt((float)d), 2);
     EXPECT(max_abs_diff(out, want) <= 1e-4f);
+}
+
+// ---- KV block pool growth ---------------------------------------------------------------------------------------
+static bool on_cpu_executor() {
+    ahpc_device_info info;
+    return ahpc_hip_device_info(0, &info) == 0 && std::strstr(info.name, "CPU executor") != nullptr;
+}
+
+// Fills pages [0, pages) of a pool from seeded host data through the scatter entry point and returns what was written.
+static void fill_pool_pages(KVBlockPool& pool, size_t pages, size_t H, size_t d, size_t P, std::vector<float>& k, std::vector<float>& v) {
+    const size_t tokens = pages * P;
+    k = normal(tokens * H * d, 123, 2);
+    v = normal(tokens * H * d, 123, 3);
+    std::vector<int32_t> table(pages);
+    for (size_t i = 0; i < pages; ++i) table[i] = (int32_t)i;
+    void *dk = nullptr, *dv = nullptr, *dt = nullptr;
+    EXPECT(ahpc_hip_malloc(&dk, k.size() * 4) == 0 && ahpc_hip_malloc(&dv, v.size() * 4) == 0 && ahpc_hip_malloc(&dt, pages * 4) == 0);
+    ahpc_hip_memcpy_h2d(dk, k.data(), k.size() * 4, nullptr);
+    ahpc_hip_memcpy_h2d(dv, v.data(), v.size() * 4, nullptr);
+    ahpc_hip_memcpy_h2d(dt, table.data(), pages * 4, nullptr);
+    EXPECT(ahpc_hip_kv_scatter(dk, dv, AHPC_F32, pool.k_slab(), pool.v_slab(), (int)pool.dtype(), (const int32_t*)dt, (int64_t)pages,
+                               nullptr, nullptr, 0, 0, (int64_t)tokens, (int64_t)H, (int64_t)d, (int64_t)P, nullptr) == 0);
+    ahpc_hip_stream_synchronize(nullptr);
+    ahpc_hip_free(dk); ahpc_hip_free(dv); ahpc_hip_free(dt);
+}
+
+static void gather_pool_pages(KVBlockPool& pool, size_t pages, size_t H, size_t d, size_t P, std::vector<float>& k, std::vector<float>& v) {
+    const size_t tokens = pages * P;
+    k.assign(tokens * H * d, -1.0f);
+    v.assign(tokens * H * d, -1.0f);
+    std::vector<int32_t> table(pages);
+    for (size_t i = 0; i < pages; ++i) table[i] = (int32_t)i;
+    void *dk = nullptr, *dv = nullptr, *dt = nullptr;
+    EXPECT(ahpc_hip_malloc(&dk, k.size() * 4) == 0 && ahpc_hip_malloc(&dv, v.size() * 4) == 0 && ahpc_hip_malloc(&dt, pages * 4) == 0);
+    ahpc_hip_memcpy_h2d(dt, table.data(), pages * 4, nullptr);
+    EXPECT(ahpc_hip_kv_gather(dk, dv, AHPC_F32, pool.k_slab(), pool.v_slab(), (int)pool.dtype(), (const int32_t*)dt, (int64_t)pages, 0, 0,
+                              (int64_t)tokens, (int64_t)H, (int64_t)d, (int64_t)P, nullptr) == 0);
+    ahpc_hip_memcpy_d2h(k.data(), dk, k.size() * 4, nullptr);
+    ahpc_hip_memcpy_d2h(v.data(), dv, v.size() * 4, nullptr);
+    ahpc_hip_stream_synchronize(nullptr);
+    ahpc_hip_free(dk); ahpc_hip_free(dv); ahpc_hip_free(dt);
+}
+
+CASE(Pool_GrowsInPlace, true) {
+    // Slabs are address ranges backed on demand: growth keeps their addresses and their contents, the generation stays 0,
+    // and the page order is the FIFO order whatever the capacity steps are.
+    size_t granularity = 0;
+    EXPECT(ahpc_hip_vmem_granularity(&granularity) == 0);
+    if (granularity == 0) { std::printf("    (no virtual memory management on this device: skipped)\n"); return; }
+    const size_t H = 2, d = 32, P = 16;
+    KVBlockPool pool(P, H, d, DataType::FLOAT32, 8, 4, size_t(1) << 30);
+    EXPECT(pool.grows_in_place());
+    void* const k0 = pool.k_slab();
+    void* const v0 = pool.v_slab();
+    std::vector<float> k, v, kg, vg;
+    fill_pool_pages(pool, 8, H, d, P, k, v);
+    for (int i = 0; i < 8; ++i) EXPECT(pool.allocate_page() == i);
+    EXPECT(pool.allocate_page() == 8);  // grows by 4
+    EXPECT(pool.get_pool_size() == 12);
+    pool.resize_pool(40000);            // 40000 pages x 4 KiB x 2 slabs = 312 MiB: several chunks (an exception ends the case here)
+    EXPECT(pool.get_pool_size() == 40000 && pool.k_slab() == k0 && pool.v_slab() == v0 && pool.generation() == 0);
+    EXPECT(pool.stats().slab_capacity_pages >= 40000);
+    if (pool.stats().slab_capacity_pages < 40000) return;
+    gather_pool_pages(pool, 8, H, d, P, kg, vg);
+    EXPECT(kg == k && vg == v);
+    // the last page is usable
+    EXPECT(ahpc_hip_memset(static_cast<char*>(pool.k_slab()) + (40000 - 1) * P * H * d * 4, 0, P * H * d * 4, nullptr) == 0);
+    EXPECT(ahpc_hip_stream_synchronize(nullptr) == 0);
+    // the budget is the limit, and running into it loses nothing
+    EXPECT_THROWS(pool.resize_pool((size_t(1) << 30) / (2 * P * H * d * 4) + 1), AttentionError::MEMORY_ALLOCATION_FAILED);
+    EXPECT(pool.get_pool_size() == 40000);
+    gather_pool_pages(pool, 8, H, d, P, kg, vg);
+    EXPECT(kg == k && vg == v);
+}
+
+CASE(Pool_GrowsByCopyWhenInPlaceIsSwitchedOff, true) {
+    // The path of devices without virtual memory management: the slabs move, the generation counts it, contents survive.
+    int64_t before = 1;
+    ahpc_hip_get_tuning("pool_in_place", &before);
+    ahpc_hip_set_tuning("pool_in_place", 0);
+    {
+        const size_t H = 2, d = 32, P = 16;
+        KVBlockPool pool(P, H, d, DataType::FLOAT32, 8, 4, size_t(1) << 28);
+        EXPECT(!pool.grows_in_place());
+        std::vector<float> k, v, kg, vg;
+        fill_pool_pages(pool, 8, H, d, P, k, v);
+        const uint64_t g0 = pool.generation();
+        pool.resize_pool(4000);
+        EXPECT(pool.generation() > g0 && pool.get_pool_size() == 4000);
+        gather_pool_pages(pool, 8, H, d, P, kg, vg);
+        EXPECT(kg == k && vg == v);
+    }
+    ahpc_hip_set_tuning("pool_in_place", before);
+}
+
+CASE(Pool_GrowsPast8GiBWhileDecodeRunsOnAnotherStream, true) {
+    // A decode loop on its own stream keeps reading the first pages of the pool while the pool grows to more than 8 GiB
+    // in place, 64 MiB per slab at a time: every result is bit-identical with the one before the growth, the slabs stay
+    // where they are, and no decode waits for the growth (the longest iteration is printed next to the median).
+    size_t granularity = 0;
+    ahpc_hip_vmem_granularity(&granularity);
+    if (granularity == 0) { std::printf("    (no virtual memory management on this device: skipped)\n"); return; }
+    const bool small = on_cpu_executor();
+    const size_t H = small ? 2 : 8, d = small ? 32 : 128, P = 16, B = small ? 2 : 8, ctx = small ? 64 : 2048;
+    const size_t pages0 = B * ctx / P;
+    const size_t page_bytes = P * H * d * 2;                     // fp16, one slab
+    const size_t target_pages = small ? 4096 : (size_t(9) << 30) / (2 * page_bytes);  // 9 GiB of K + V
+    KVBlockPool pool(P, H, d, DataType::FLOAT16, pages0, 16, size_t(16) << 30);  // (a budget of 16 GiB: chunks of 64 MiB)
+    EXPECT(pool.grows_in_place());
+    std::vector<float> k, v;
+    fill_pool_pages(pool, pages0, H, d, P, k, v);
+    for (size_t i = 0; i < pages0; ++i) pool.allocate_page();
+    std::vector<int32_t> table(pages0), lens(B, (int32_t)ctx);
+    for (size_t i = 0; i < pages0; ++i) table[i] = (int32_t)i;
+    const auto q = normal(B * H * d, 124, 1);
+    void *dq = nullptr, *dout = nullptr, *dt = nullptr, *dl = nullptr, *dws = nullptr, *stream = nullptr;
+    const size_t ws = ahpc_hip_paged_decode_workspace_bytes(B, H, d, ctx, P, 0);
+    EXPECT(ahpc_hip_malloc(&dq, q.size() * 4) == 0 && ahpc_hip_malloc(&dout, q.size() * 4) == 0 && ahpc_hip_malloc(&dt, pages0 * 4) == 0 &&
+           ahpc_hip_malloc(&dl, B * 4) == 0 && ahpc_hip_malloc(&dws, ws ? ws : 16) == 0 && ahpc_hip_stream_create(&stream) == 0);
+    ahpc_hip_memcpy_h2d(dq, q.data(), q.size() * 4, nullptr);
+    ahpc_hip_memcpy_h2d(dt, table.data(), pages0 * 4, nullptr);
+    ahpc_hip_memcpy_h2d(dl, lens.data(), B * 4, nullptr);
+    ahpc_hip_stream_synchronize(nullptr);
+    void* const k0 = pool.k_slab();
+    auto decode = [&](std::vector<float>& out) {
+        const int rc = ahpc_hip_paged_decode(dq, dout, AHPC_F32, pool.k_slab(), pool.v_slab(), AHPC_F16, (const int32_t*)dt, (const int32_t*)dl, nullptr,
+                                             (int64_t)B, (int64_t)H, (int64_t)d, (int64_t)P, (int64_t)(ctx / P), (int64_t)ctx,
+                                             1.0f / std::sqrt((float)d), 0, dws, ws, stream);
+        ahpc_hip_memcpy_d2h(out.data(), dout, out.size() * 4, stream);
+        ahpc_hip_stream_synchronize(stream);
+        return rc;
+    };
+    std::vector<float> want(q.size());
+    EXPECT(decode(want) == 0);
+    std::atomic<bool> stop{false};
+    std::atomic<int> bad{0};
+    std::vector<double> ms;
+    std::thread reader([&] {
+        std::vector<float> out(q.size());
+        while (!stop.load()) {
+            const auto t0 = std::chrono::steady_clock::now();
+            if (decode(out) != 0 || out != want) bad.fetch_add(1);
+            ms.push_back(std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count());
+        }
+    });
+    double grow_ms = 0.0;
+    int steps = 0;
+    std::string grow_error;
+    try {
+        for (size_t total = pages0; total < target_pages;) {
+            total = std::min(target_pages, total + target_pages / 72);
+            const auto t0 = std::chrono::steady_clock::now();
+            pool.resize_pool(total);
+            grow_ms += std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+            ++steps;
+            std::this_thread::sleep_for(std::chrono::microseconds(300));  // (so that decodes fall between the steps)
+        }
+    } catch (const std::exception& e) {
+        grow_error = e.what();
+    }
+    stop.store(true);
+    reader.join();
+    if (!grow_error.empty()) std::printf("    growth failed: %s\n", grow_error.c_str());
+    EXPECT(grow_error.empty());
+    if (!grow_error.empty()) return;  // (nothing behind the backed part of the slabs is touched)
+    EXPECT(bad.load() == 0);
+    EXPECT(pool.k_slab() == k0 && pool.generation() == 0 && pool.get_pool_size() == target_pages);
+    EXPECT(pool.stats().slab_bytes >= target_pages * 2 * page_bytes);
+    // the far end of the grown slabs is real memory
+    EXPECT(ahpc_hip_memset(static_cast<char*>(pool.v_slab()) + (target_pages - 1) * page_bytes, 0, page_bytes, nullptr) == 0);
+    EXPECT(ahpc_hip_stream_synchronize(nullptr) == 0);
+    std::vector<float> after(q.size());
+    EXPECT(decode(after) == 0 && after == want);
+    if (!ms.empty()) {
+        std::vector<double> sorted = ms;
+        std::sort(sorted.begin(), sorted.end());
+        std::printf("    pool grown to %.2f GiB in %d steps, %.2f ms of host time in all; %zu decodes meanwhile: median %.3f ms, longest %.3f ms\n",
+                    pool.stats().slab_bytes / 1073741824.0, steps, grow_ms, ms.size(), sorted[sorted.size() / 2], sorted.back());
+        // growth by reallocation would stop every stream for the copy of gigabytes (tens of milliseconds per step)
+        if (!small) EXPECT(sorted.back() < 10.0 * sorted[sorted.size() / 2] + 2.0);
+    }
+    ahpc_hip_free(dq); ahpc_hip_free(dout); ahpc_hip_free(dt); ahpc_hip_free(dl); ahpc_hip_free(dws);
+    ahpc_hip_stream_destroy(stream);
 }
 
 // ---- main ------------------------------------------------------------------------------------------------------

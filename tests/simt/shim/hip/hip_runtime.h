@@ -157,7 +157,34 @@ inline hipError_t hipGetDeviceProperties(hipDeviceProp_t* p, int) {
     p->clockRate = 1;
     return hipSuccess;
 }
-inline hipError_t hipMalloc(void** p, size_t n) { *p = std::malloc(n); return *p ? hipSuccess : 2; }
+// One allocation can be made to fail (tests of the callers' out-of-memory paths): the countdown is decremented by every
+// device allocation, the one that takes it to zero fails.
+extern int simt_fail_device_alloc_in;
+inline bool simt_alloc_fails() { return simt_fail_device_alloc_in > 0 && --simt_fail_device_alloc_in == 0; }
+inline hipError_t hipMalloc(void** p, size_t n) {
+    if (simt_alloc_fails()) { *p = nullptr; return 2; }
+    *p = std::malloc(n);
+    return *p ? hipSuccess : 2;
+}
+// virtual memory management, emulated with an inaccessible mapping whose front part is made accessible piece by piece
+enum hipDeviceAttribute_t { hipDeviceAttributeVirtualMemoryManagementSupported = 1 };
+inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = 1; return hipSuccess; }
+enum { hipMemAllocationTypePinned = 1, hipMemLocationTypeDevice = 1, hipMemAccessFlagsProtReadWrite = 3 };
+struct hipMemLocation { int type; int id; };
+struct hipMemAllocationProp { int type; hipMemLocation location; };
+struct hipMemAccessDesc { hipMemLocation location; int flags; };
+typedef size_t hipMemGenericAllocationHandle_t;
+hipError_t hipMemAddressReserve(void** p, size_t n, size_t align, void*, unsigned long long);
+hipError_t hipMemAddressFree(void* p, size_t n);
+inline hipError_t hipMemCreate(hipMemGenericAllocationHandle_t* h, size_t n, const hipMemAllocationProp*, unsigned long long) {
+    if (simt_alloc_fails()) return 2;
+    *h = n;
+    return hipSuccess;
+}
+inline hipError_t hipMemRelease(hipMemGenericAllocationHandle_t) { return hipSuccess; }
+hipError_t hipMemMap(void* p, size_t n, size_t, hipMemGenericAllocationHandle_t, unsigned long long);
+hipError_t hipMemUnmap(void* p, size_t n);
+inline hipError_t hipMemSetAccess(void*, size_t, const hipMemAccessDesc*, size_t) { return hipSuccess; }
 inline hipError_t hipFree(void* p) { std::free(p); return hipSuccess; }
 inline hipError_t hipHostMalloc(void** p, size_t n, unsigned) { *p = std::malloc(n); return *p ? hipSuccess : 2; }
 inline hipError_t hipHostFree(void* p) { std::free(p); return hipSuccess; }

@@ -4,6 +4,7 @@
 // scheduler resumes fibers whose condition has become true, visiting wavefronts in a seeded random
 // order so that different interleavings of the wavefronts of a workgroup are exercised.
 #include <hip/hip_runtime.h>
+#include <sys/mman.h>
 #include <ucontext.h>
 
 #include <algorithm>
@@ -695,8 +696,27 @@ void launch(dim3 grid, dim3 block, const std::function<void()>& body) {
 
 }  // namespace simt
 
+// ---- emulated virtual memory management: an inaccessible mapping, made accessible piece by piece ------------------
+int simt_fail_device_alloc_in = 0;
+hipError_t hipMemAddressReserve(void** p, size_t n, size_t, void*, unsigned long long) {
+    void* m = mmap(nullptr, n, PROT_NONE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+    if (m == MAP_FAILED) return 2;
+    *p = m;
+    return hipSuccess;
+}
+hipError_t hipMemAddressFree(void* p, size_t n) { return munmap(p, n) == 0 ? hipSuccess : 1; }
+hipError_t hipMemMap(void* p, size_t n, size_t, hipMemGenericAllocationHandle_t, unsigned long long) {
+    return mprotect(p, n, PROT_READ | PROT_WRITE) == 0 ? hipSuccess : 1;
+}
+hipError_t hipMemUnmap(void* p, size_t n) {
+    madvise(p, n, MADV_DONTNEED);
+    return mprotect(p, n, PROT_NONE) == 0 ? hipSuccess : 1;
+}
+
 // ---- control from the tests (ctypes) ---------------------------------------------------------------
 extern "C" {
+// The n-th device allocation from now on fails (1 = the next one); 0 switches the countdown off.
+void simt_fail_device_alloc(int n) { simt_fail_device_alloc_in = n; }
 // dma_late != 0: direct-to-LDS loads land at the issuing lane's next s_waitcnt instead of at issue.
 // seed: order in which the wavefronts of a workgroup are advanced.
 void simt_configure(int dma_late, uint64_t seed) {
