@@ -169,6 +169,33 @@ __global__ void gather_indices_kernel(const int32_t* __restrict__ table, const i
     offsets[idx] = off;
 }
 
+// Copies whole pages inside the K and V slabs: page from[i] -> page to[i], i < n (blockIdx.y = 0: K, 1: V).  Sources and
+// destinations must be disjoint sets (compaction moves pages in use onto free ones).  Ids outside [0, n_pages) are
+// skipped.
+__global__ __launch_bounds__(256) void kv_move_pages_kernel(unsigned char* __restrict__ k_pool, unsigned char* __restrict__ v_pool,
+                                                            int64_t page_bytes, int64_t n_pages, const int32_t* __restrict__ from,
+                                                            const int32_t* __restrict__ to, int64_t n) {
+    const int64_t i = blockIdx.x;
+    if (i >= n) return;
+    const int64_t src = from[i], dst = to[i];
+    if (src < 0 || dst < 0 || src >= n_pages || dst >= n_pages || src == dst) return;
+    unsigned char* const pool = blockIdx.y == 0 ? k_pool : v_pool;
+    const unsigned char* const s = pool + src * page_bytes;
+    unsigned char* const d = pool + dst * page_bytes;
+    if (((page_bytes | reinterpret_cast<uintptr_t>(pool)) & 15) == 0) {
+        for (int64_t o = (int64_t)threadIdx.x * 16; o < page_bytes; o += 256 * 16)
+            *reinterpret_cast<u32x4*>(d + o) = *reinterpret_cast<const u32x4*>(s + o);
+    } else {
+        for (int64_t o = threadIdx.x; o < page_bytes; o += 256) d[o] = s[o];
+    }
+}
+
+// dst[0..n) = value (a fill in kernel form: callers may be under graph capture)
+__global__ __launch_bounds__(256) void fill_i64_kernel(int64_t* __restrict__ dst, int64_t n, int64_t value) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = value;
+}
+
 // ---------------------------------------------------------------------------------------------
 // decode
 struct DecodeParams {
@@ -330,9 +357,7 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     if (first_page + lane < p.max_pages) my_page = p.table[row * p.max_pages + first_page + lane];
     bool dumps = DUMP && h_raw == 0 && e0 == 0;  // one lane of the launch's first head group
     if constexpr (DUMP) {
-        if (dumps) {  // (index-dump launches are not balanced: every workgroup clears its own fixed range first)
-            const int te = (t0 + p.chunk_tokens) < p.max_len ? (t0 + p.chunk_tokens) : p.max_len;
-            for (int t = t0; t < te; ++t) p.dump_offsets[(int64_t)b * p.max_len + t] = -1;
+        if (dumps) {  // (the launcher has filled the report with -1: tokens nobody addresses stay that way)
             // what a chunk behind a missing page reads never enters the result (the merge stops in front of it):
             // it is not reported either
             for (int pg = 0; pg < first_page && pg < p.max_pages; ++pg)
@@ -929,7 +954,7 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     const bool mfma_shape = (pool_dtype == AHPC_F16 || pool_dtype == AHPC_BF16) && (d == 64 || d == 128 || d == 256) && P == 16 && H_kv <= 65535 &&
                             group <= 32;
     if (qo_dtype < AHPC_F32 || qo_dtype > AHPC_BF16 || pool_dtype < AHPC_F32 || pool_dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
-    if (B <= 0 || B > 65535 || max_len <= 0 || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;
+    if (B <= 0 || B > 65535 || max_len <= 0 || max_len > 0x7FFFFFFFll || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;
     if ((max_len + P - 1) / P > max_pages) return AHPC_ERR_BAD_SHAPE;
     // head dimensions up to 256 in whole 16-byte pieces of the pool's type; the lane-per-element kernel is instantiated
     // for 32, 64, 128 and 256 and takes the smallest that holds d (DecodeParams::d_kernel)
@@ -1000,15 +1025,16 @@ int ahpc_hip_paged_decode_noalloc(const void* q, void* o, int qo_dtype, const vo
                                   const int32_t* block_table, const int32_t* seq_lens, const int32_t* batch_rows, int64_t B,
                                   int64_t H, int64_t H_kv, int64_t d, int64_t P, int64_t max_pages, int64_t max_len,
                                   float scale, int64_t chunk_tokens, void* stream) {
-    // (arguments that are wrong in themselves are reported by the call below, whatever this size comes out as)
-    if (ahpc_hip_paged_decode_workspace_bytes(B, H, d, max_len, P, chunk_tokens) > AHPC_NOALLOC_SCRATCH_BYTES)
-        return AHPC_ERR_SCRATCH_LIMIT;
     void* ptr = nullptr;
     if (int rc = scratch_of_current_device(&ptr)) return rc;
-    // The partials need no clearing between calls: the merge reads, per sequence, exactly the chunks whose
+    // The call below plans the launch and knows what its partials need (with chunk_tokens = 0 usually far less than the
+    // bound ahpc_hip_paged_decode_workspace_bytes gives): it refuses, before launching anything, a plan that does not fit
+    // the array.  The partials need no clearing between calls: the merge reads, per sequence, exactly the chunks whose
     // decode workgroup wrote them in this call (those that start before the sequence's end).
-    return ahpc_hip_paged_decode_gqa(q, o, qo_dtype, k_pool, v_pool, pool_dtype, block_table, seq_lens, batch_rows, B, H, H_kv,
-                                     d, P, max_pages, max_len, scale, chunk_tokens, ptr, AHPC_NOALLOC_SCRATCH_BYTES, stream);
+    const int rc = ahpc_hip_paged_decode_gqa(q, o, qo_dtype, k_pool, v_pool, pool_dtype, block_table, seq_lens, batch_rows, B, H,
+                                             H_kv, d, P, max_pages, max_len, scale, chunk_tokens, ptr, AHPC_NOALLOC_SCRATCH_BYTES,
+                                             stream);
+    return rc == AHPC_ERR_WORKSPACE_TOO_SMALL ? AHPC_ERR_SCRATCH_LIMIT : rc;
 }
 
 int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype, const void* k_pool, const void* v_pool, int pool_dtype,
@@ -1019,19 +1045,37 @@ int ahpc_hip_paged_decode(const void* q, void* o, int qo_dtype, const void* k_po
                                      d, P, max_pages, max_len, scale, chunk_tokens, workspace, workspace_bytes, stream);
 }
 
+int ahpc_hip_kv_move_pages(void* k_pool, void* v_pool, int pool_dtype, int64_t n_pages, const int32_t* from, const int32_t* to,
+                           int64_t n, int64_t H, int64_t d, int64_t P, void* stream) {
+    if (n == 0) return AHPC_OK;
+    if (!k_pool || !v_pool || !from || !to) return AHPC_ERR_NULL_POINTER;
+    if (pool_dtype < AHPC_F32 || pool_dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
+    if (n < 0 || n > 0x7FFFFFFFll || n_pages <= 0 || n_pages > 0x7FFFFFFFll || !dims_ok(H, d, P, 1)) return AHPC_ERR_BAD_SHAPE;
+    const int64_t page_bytes = P * H * d * (pool_dtype == AHPC_F32 ? 4 : 2);
+    hipLaunchKernelGGL(kv_move_pages_kernel, dim3((unsigned)n, 2), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<unsigned char*>(k_pool), static_cast<unsigned char*>(v_pool), page_bytes, n_pages, from, to, n);
+    return static_cast<int>(hipGetLastError());
+}
+
 int ahpc_hip_paged_gather_indices(const int32_t* block_table, const int32_t* seq_lens, const int32_t* batch_rows, int64_t B,
                                   int64_t H, int64_t d, int64_t P, int64_t max_pages, int64_t max_len, int64_t* offsets,
                                   void* stream) {
     if (!block_table || !seq_lens || !offsets) return AHPC_ERR_NULL_POINTER;
-    if (B <= 0 || max_len <= 0 || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;
+    if (B <= 0 || max_len <= 0 || max_len > 0x7FFFFFFFll || !dims_ok(H, d, P, max_pages)) return AHPC_ERR_BAD_SHAPE;
     if ((max_len + P - 1) / P > max_pages) return AHPC_ERR_BAD_SHAPE;
+    if (B > 0x7FFFFFFFll || (B * max_len + 255) / 256 > 0x7FFFFFFFll) return AHPC_ERR_BAD_SHAPE;  // one thread per reported token
     hipStream_t st = static_cast<hipStream_t>(stream);
     if ((d == 32 || d == 64 || d == 128 || d == 256) && B <= 65535 && H <= 65535) {
-        // the decode kernel itself (16-bit pool, one query head per pool head), launched for pool head 0 only,
-        // reports the rows it addresses
+        // the decode kernel itself (16-bit pool, one query head per pool head), launched for pool head 0 only and with
+        // the chunking of a real decode launch (every sequence cut into equal chunks), reports the rows it addresses
         const int64_t chunk = plan_decode(B, H, 1, (H + 3) / 4, max_len, P, 0).chunk;
         const int64_t n_chunks = (max_len + chunk - 1) / chunk;
         if (n_chunks > 65535) return AHPC_ERR_BAD_SHAPE;
+        {
+            const int64_t total = B * max_len;
+            hipLaunchKernelGGL(fill_i64_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, offsets, total, (int64_t)-1);
+            if (hipError_t e = hipGetLastError(); e != hipSuccess) return static_cast<int>(e);
+        }
         DecodeParams p{};
         p.table = block_table; p.seq_lens = seq_lens; p.batch_rows = batch_rows;
         p.dump_offsets = offsets;
@@ -1039,6 +1083,7 @@ int ahpc_hip_paged_gather_indices(const int32_t* block_table, const int32_t* seq
         p.B = (int32_t)B; p.H = (int32_t)H; p.H_kv = (int32_t)H; p.d = (int32_t)d; p.P = (int32_t)P;
         p.d_kernel = (int32_t)d;
         p.chunk_tokens = (int32_t)chunk; p.n_chunks = (int32_t)n_chunks;
+        p.balanced = 1;
         p.max_len = (int32_t)max_len;
         const dim3 grid(1, (unsigned)n_chunks, (unsigned)B), block(64);
 #define AHPC_DUMP(DD)                                                                                                  \

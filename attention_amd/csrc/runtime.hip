@@ -250,6 +250,30 @@ int ahpc_hip_vmem_commit(void* base, size_t bytes, size_t* committed) {
     return AHPC_OK;
 }
 
+int ahpc_hip_vmem_decommit(void* base, size_t keep_bytes, size_t* committed) {
+    std::lock_guard<std::mutex> lock(g_vmem_mu);
+    auto it = g_vmem.find(base);
+    if (it == g_vmem.end()) return AHPC_ERR_NULL_POINTER;
+    VmemRange& r = it->second;
+    const size_t keep = round_up(keep_bytes, r.chunk);
+    hipError_t first = hipSuccess;
+    while (r.committed > keep && !r.chunks.empty()) {
+        char* at = static_cast<char*>(base) + r.committed - r.chunk;
+        hipError_t e = hipMemUnmap(at, r.chunk);
+        if (e != hipSuccess) {  // (still mapped: leave the books as they are)
+            first = e;
+            break;
+        }
+        e = hipMemRelease(r.chunks.back());
+        if (e != hipSuccess && first == hipSuccess) first = e;
+        r.chunks.pop_back();
+        r.committed -= r.chunk;
+    }
+    if (committed) *committed = r.committed;
+    if (first != hipSuccess) (void)hipGetLastError();
+    return static_cast<int>(first);
+}
+
 int ahpc_hip_vmem_release(void* base) {
     if (!base) return AHPC_OK;
     std::lock_guard<std::mutex> lock(g_vmem_mu);

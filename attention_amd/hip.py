@@ -50,7 +50,9 @@ SIGNATURES = {
     "ahpc_hip_vmem_granularity": (_ci, [C.POINTER(_sz)]),
     "ahpc_hip_vmem_reserve": (_ci, [C.POINTER(_vp), _sz, _sz]),
     "ahpc_hip_vmem_commit": (_ci, [_vp, _sz, C.POINTER(_sz)]),
+    "ahpc_hip_vmem_decommit": (_ci, [_vp, _sz, C.POINTER(_sz)]),
     "ahpc_hip_vmem_release": (_ci, [_vp]),
+    "ahpc_hip_kv_move_pages": (_ci, [_vp, _vp, _ci, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "ahpc_hip_memcpy_h2d": (_ci, [_vp, _vp, _sz, _vp]),
     "ahpc_hip_memcpy_d2h": (_ci, [_vp, _vp, _sz, _vp]),
     "ahpc_hip_memcpy_d2d": (_ci, [_vp, _vp, _sz, _vp]),
@@ -82,7 +84,6 @@ SIGNATURES = {
     "ahpc_hip_paged_decode_gqa": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp, _sz, _vp]),
     "ahpc_hip_paged_decode_noalloc": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp]),
     "ahpc_hip_paged_gather_indices": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp]),
-    "ahpc_hip_probe_matrix_rate": (_ci, [_ci, _ci, _i64, _i64, _vp, _sz, C.POINTER(C.c_double), _vp]),
 }
 
 _lib = None
@@ -264,11 +265,3 @@ def paged_decode_noalloc(q, o, qo_dtype, k_pool, v_pool, pool_dtype, table, seq_
 def paged_gather_indices(table, seq_lens, batch_rows, B, H, d, P, max_pages, max_len, offsets, stream=None):
     _check(load().ahpc_hip_paged_gather_indices(table, seq_lens, batch_rows, B, H, d, P, max_pages, max_len, offsets,
                                                stream), "paged_gather_indices")
-
-
-def probe_matrix_rate(dtype, mix, workgroups, iterations, sink, sink_bytes, stream=None):
-    """Launches the matrix-rate calibration kernel; returns the floating-point operations of the launch."""
-    flop = C.c_double(0.0)
-    _check(load().ahpc_hip_probe_matrix_rate(dtype, mix, workgroups, iterations, sink, sink_bytes, C.byref(flop), stream),
-           "probe_matrix_rate")
-    return flop.value

@@ -143,7 +143,56 @@ void KVBlockPool::deallocate_page(int32_t page) {
 
 void KVBlockPool::resize_pool(size_t new_total_pages) {
     std::lock_guard<std::mutex> lock(mutex_);
-    if (new_total_pages > in_use_.size()) create_pages_locked(new_total_pages - in_use_.size());
+    if (new_total_pages > in_use_.size()) {
+        create_pages_locked(new_total_pages - in_use_.size());
+        return;
+    }
+    // shrink: only free pages at the end of the id range can go
+    size_t keep = in_use_.size();
+    while (keep > new_total_pages && !in_use_[keep - 1]) --keep;
+    if (keep == in_use_.size()) return;
+    in_use_.resize(keep);
+    std::deque<int32_t> still;
+    for (int32_t id : free_)
+        if (static_cast<size_t>(id) < keep) still.push_back(id);
+    free_.swap(still);
+    if (in_place_) {
+        // work in flight may still read pages that were released a moment ago
+        check(ahpc_hip_device_synchronize(), "KV pool shrink");
+        const size_t page_bytes_one = slab_elems_per_page_ * hipsup::dtype_size(dtype_);
+        size_t got_k = 0, got_v = 0;
+        const int rk = ahpc_hip_vmem_decommit(k_slab_, keep * page_bytes_one, &got_k);
+        const int rv = ahpc_hip_vmem_decommit(v_slab_, keep * page_bytes_one, &got_v);
+        if (rk == 0 && rv == 0) capacity_pages_ = std::min(got_k, got_v) / page_bytes_one;
+    }
+}
+
+std::vector<std::pair<int32_t, int32_t>> KVBlockPool::plan_compaction() const {
+    std::lock_guard<std::mutex> lock(mutex_);
+    std::vector<std::pair<int32_t, int32_t>> moves;
+    size_t lo = 0;
+    for (size_t hi = in_use_.size(); hi-- > allocated_;) {
+        if (!in_use_[hi]) continue;
+        while (lo < allocated_ && in_use_[lo]) ++lo;
+        if (lo >= allocated_) break;  // (cannot happen: as many free ids below the mark as pages in use beyond it)
+        moves.emplace_back(static_cast<int32_t>(hi), static_cast<int32_t>(lo));
+        ++lo;
+    }
+    return moves;
+}
+
+void KVBlockPool::apply_compaction(const std::vector<std::pair<int32_t, int32_t>>& moves) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    for (const auto& m : moves) {
+        if (m.first < 0 || m.second < 0 || static_cast<size_t>(m.first) >= in_use_.size() ||
+            static_cast<size_t>(m.second) >= in_use_.size() || !in_use_[m.first] || in_use_[m.second])
+            throw AttentionException(AttentionError::INVALID_INPUT, "KVBlockPool: compaction move does not match the pool's state");
+        in_use_[m.first] = 0;
+        in_use_[m.second] = 1;
+    }
+    free_.clear();
+    for (size_t id = 0; id < in_use_.size(); ++id)
+        if (!in_use_[id]) free_.push_back(static_cast<int32_t>(id));
 }
 
 size_t KVBlockPool::get_pool_size() const {

@@ -687,7 +687,49 @@ KVBlockPoolStats PagedAttention::get_pool_stats() const {
     return impl_->pool ? impl_->pool->stats() : KVBlockPoolStats{};
 }
 
-void PagedAttention::compact_pages() {}
+// Re-homes the pages in use onto the lowest page ids (one device launch moves them, then the block table is rewritten)
+// and hands the pool's free tail back: after sequences have come and gone the pages of the survivors are scattered
+// over the whole id range, and only a pool whose high ids are free can shrink.  Pages keep their order inside every
+// sequence; decode results do not change by a bit.  Reference: PagedAttention::compact_pages,
+// src/algorithms/paged_attention.cpp:577-583 (its per-sequence helper is not defined in the reference's sources).
+void PagedAttention::compact_pages() {
+    Impl& m = *impl_;
+    std::lock_guard<std::mutex> run(m.run_mutex);
+    std::lock_guard<std::mutex> lock(m.seq_mutex);
+    if (!m.pool) return;
+    const auto moves = m.pool->plan_compaction();
+    if (!moves.empty()) {
+        std::vector<int32_t> ids(2 * moves.size());
+        std::unordered_map<int32_t, int32_t> new_id;
+        for (size_t i = 0; i < moves.size(); ++i) {
+            ids[i] = moves[i].first;
+            ids[moves.size() + i] = moves[i].second;
+            new_id.emplace(moves[i].first, moves[i].second);
+        }
+        void* d_ids = m.d_rows.reserve(ids.size() * sizeof(int32_t));
+        check(ahpc_hip_memcpy_h2d(d_ids, ids.data(), ids.size() * sizeof(int32_t), m.stream.get()), "compaction move list");
+        const KVBlockPoolStats st = m.pool->stats();
+        check(ahpc_hip_kv_move_pages(m.pool->k_slab(), m.pool->v_slab(), hipsup::dtype_code(m.pool->dtype()),
+                                     static_cast<int64_t>(st.slab_capacity_pages), static_cast<const int32_t*>(d_ids),
+                                     static_cast<const int32_t*>(d_ids) + moves.size(), static_cast<int64_t>(moves.size()),
+                                     static_cast<int64_t>(m.Hkv), static_cast<int64_t>(m.d), static_cast<int64_t>(m.P), m.stream.get()),
+              "compaction page moves");
+        m.stream.sync();  // (the move list lives in host memory until here)
+        for (auto& kv : m.seqs) {
+            Sequence& s = kv.second;
+            for (size_t i = 0; i < s.pages.size(); ++i) {
+                auto it = new_id.find(s.pages[i]);
+                if (it == new_id.end()) continue;
+                s.pages[i] = it->second;
+                m.table[s.row * m.max_pages + i] = it->second;
+            }
+        }
+        m.table_dirty = true;
+        m.pool->apply_compaction(moves);
+    }
+    // the free tail goes back, down to what the configuration starts a pool with
+    m.pool->resize_pool(std::max(m.pool->get_allocated_pages(), m.cfg.initial_page_pool_size));
+}
 void PagedAttention::preload_pages(const std::vector<size_t>&) {}
 
 }  // namespace attention_hpc

@@ -568,27 +568,6 @@ def run_calibration(steps):
     dt = (time.perf_counter() - t0) / steps
     print(json.dumps({"workload": "bf16 matrix product 8192^3 (torch.matmul)", "ms_per_launch": round(dt * 1e3, 4),
                       "TFLOPs": round(2.0 * m ** 3 / dt / 1e12, 1)}))
-    # What "matrix-bound" means on this box: nothing but v_mfma_f32_32x32x16_bf16 on register operands, one and two
-    # wavefronts per SIMD, without and with a softmax's VALU work between the matrix instructions.
-    from attention_amd import hip
-    import ctypes as C
-    sp = C.c_void_p()
-    assert hip.load().ahpc_hip_stream_create(C.byref(sp)) == 0
-    info = hip.device_info(0)
-    for waves in (1, 2):
-        wgs = info.compute_units * waves
-        sink = torch.empty(wgs * 256, dtype=torch.float32, device="cuda")
-        for mix in (0, 1):
-            flop = [0.0]
-
-            def launch():
-                flop[0] = hip.probe_matrix_rate(hip.BF16, mix, wgs, 20000, sink.data_ptr(), sink.numel() * 4, sp.value)
-            _, per = timed_steps(hip, sp.value, launch, max(steps, 3), 2)
-            ms = float(np.mean(per))
-            print(json.dumps({"workload": f"matrix instructions only, bf16, {waves} wavefront(s) per SIMD"
-                              + (", softmax-like VALU mix" if mix else ""), "ms_per_launch": round(ms, 4),
-                              "TFLOPs": round(flop[0] / (ms * 1e-3) / 1e12, 1)}))
-    hip.load().ahpc_hip_stream_destroy(sp.value)
 
 
 def read_sensors():

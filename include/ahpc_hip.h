@@ -94,6 +94,9 @@ int ahpc_hip_host_free(void* ptr);
 int ahpc_hip_vmem_granularity(size_t* bytes);
 int ahpc_hip_vmem_reserve(void** base, size_t bytes, size_t chunk_bytes);
 int ahpc_hip_vmem_commit(void* base, size_t bytes, size_t* committed);
+/* Gives back the physical memory of the chunks that lie wholly behind the first `keep_bytes` of the range (the caller
+ * vouches that no work in flight touches them: synchronise first). */
+int ahpc_hip_vmem_decommit(void* base, size_t keep_bytes, size_t* committed);
 int ahpc_hip_vmem_release(void* base);                        /* unmaps, frees the physical memory and the addresses */
 int ahpc_hip_memcpy_h2d(void* dst, const void* src_host, size_t bytes, void* stream);
 int ahpc_hip_memcpy_d2h(void* dst_host, const void* src, size_t bytes, void* stream);
@@ -278,6 +281,14 @@ int ahpc_hip_kv_gather(void* k_out, void* v_out, int out_dtype,
                        int64_t row, int64_t start, int64_t n,
                        int64_t H, int64_t d, int64_t P, void* stream);
 
+/* Moves whole pages inside the pool: page from[i] -> page to[i] for i < n, K and V slabs alike, in one launch
+ * (from, to: int32[n] in device memory; n_pages = pages the slabs hold; the two id sets must be disjoint; ids outside
+ * the pool are skipped).  What PagedAttention::compact_pages re-homes pages with before it rewrites the block table
+ * (reference: PagedAttention::compact_pages, src/algorithms/paged_attention.cpp:577-583, whose per-sequence helper
+ * is declared at paged_attention.hpp:262 and not defined in the reference's sources). */
+int ahpc_hip_kv_move_pages(void* k_pool, void* v_pool, int pool_dtype, int64_t n_pages, const int32_t* from,
+                           const int32_t* to, int64_t n, int64_t H, int64_t d, int64_t P, void* stream);
+
 /* ---- PagedAttention decode --------------------------------------------------------------------
  * One query token per batch entry attends to all seq_lens[row] cached tokens of its sequence:
  * replaces PagedAttention::forward_batch -> compute_paged_attention,
@@ -325,8 +336,9 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype,
  * ahpc_hip_paged_decode_gqa, without the workspace: the chunk partials live in an array that is part of the
  * library's device code (AHPC_NOALLOC_SCRATCH_BYTES per GPU, held until the process ends).  The call performs no
  * hipMalloc / hipFree and calls no allocating library routine; its first call on a device looks the array's
- * address up (make that call outside a capture).  A call whose partials do not fit
- * (ahpc_hip_paged_decode_workspace_bytes(...) > AHPC_NOALLOC_SCRATCH_BYTES) returns AHPC_ERR_SCRATCH_LIMIT and
+ * address up (make that call outside a capture).  A call whose partials, at the chunk length the launch picks
+ * (with chunk_tokens = 0 far fewer than the bound ahpc_hip_paged_decode_workspace_bytes reports: 64 sequences of up
+ * to 4096 tokens, 32 heads of 128, take 4.3 MB), do not fit AHPC_NOALLOC_SCRATCH_BYTES returns AHPC_ERR_SCRATCH_LIMIT and
  * launches nothing.  Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (different
  * streams, different threads) race; calls on one stream do not.  Nothing in the array has to start at zero. */
 #define AHPC_NOALLOC_SCRATCH_BYTES ((size_t)16 << 20)
@@ -346,18 +358,6 @@ int ahpc_hip_paged_decode_noalloc(const void* q, void* o, int qo_dtype,
 int ahpc_hip_paged_gather_indices(const int32_t* block_table, const int32_t* seq_lens, const int32_t* batch_rows,
                                   int64_t B, int64_t H, int64_t d, int64_t P, int64_t max_pages, int64_t max_len,
                                   int64_t* offsets, void* stream);
-
-/* ---- calibration ------------------------------------------------------------------------------------
- * One launch that does nothing but matrix instructions on register operands: `workgroups` workgroups of 4
- * wavefronts, each wavefront `iterations` x 4 independent v_mfma_f32_32x32x16 of `dtype` (AHPC_F16 / AHPC_BF16);
- * mix = 1 adds the VALU work of a softmax between them (an exponential, two additions, a maximum, a packing
- * conversion and a bit operation per matrix instruction: somewhat more than the flash forward's).  *flop (optional) receives the floating-point operations of the launch;
- * the caller times it (events on `stream`).  sink: workgroups * 256 floats of device memory that receive the
- * accumulators' sums, so that the work cannot be optimised away.  Measures what "matrix-bound" means on the box
- * in hand, next to the published peak.  No counterpart in the reference (its benchmark,
- * benchmarks/benchmark_attention.cpp:129-255, times whole attention calls only). */
-int ahpc_hip_probe_matrix_rate(int dtype, int mix, int64_t workgroups, int64_t iterations, float* sink,
-                               size_t sink_bytes, double* flop, void* stream);
 
 #ifdef __cplusplus
 }

@@ -117,7 +117,9 @@ public:
     // Page ids of a sequence in order (what its block-table row holds); for tests and tooling.
     std::vector<int32_t> get_sequence_pages(size_t sequence_id) const;
 
-    void compact_pages();                                        // no-op: pages never fragment within a sequence
+    // Moves the pages in use onto the lowest page ids (device copy + block-table rewrite) and returns the pool's free
+    // tail to the device; results of later decodes are unchanged bit for bit.
+    void compact_pages();
     void preload_pages(const std::vector<size_t>& sequence_ids); // no-op: the pool is always device-resident
 
 private:

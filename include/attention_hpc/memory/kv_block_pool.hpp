@@ -17,6 +17,7 @@
 #include <cstdint>
 #include <deque>
 #include <mutex>
+#include <utility>
 #include <vector>
 
 #include "api/attention_interface.hpp"
@@ -52,7 +53,16 @@ public:
 
     int32_t allocate_page();             // throws MemoryPoolException when HBM is exhausted
     void deallocate_page(int32_t page);  // unknown / already-free ids are ignored, as in the reference
+    // Grows the pool to `new_total_pages`, or shrinks it: pages at the end of the id range that are free are dropped
+    // (never below the highest page in use; the device is synchronised first and, where slabs grow in place, the
+    // memory of chunks that no longer hold a page goes back to the device).
     void resize_pool(size_t new_total_pages);
+    // Compaction in two steps, for the owner of the block tables.  plan_compaction() lists the moves (from, to) that
+    // bring every page in use below allocated_pages(): pages in use at or beyond that mark, highest first, onto the
+    // free ids below it, lowest first.  After the device copy, apply_compaction(moves) swaps the ids' roles and
+    // rebuilds the free queue in ascending id order.
+    std::vector<std::pair<int32_t, int32_t>> plan_compaction() const;
+    void apply_compaction(const std::vector<std::pair<int32_t, int32_t>>& moves);
 
     size_t get_pool_size() const;
     size_t get_free_pages() const;

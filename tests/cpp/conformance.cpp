@@ -1071,6 +1071,75 @@ CASE(Paged_PoolGrowsWhileOtherThreadsAppendAndDecode, true) {
     EXPECT(max_abs_diff(out, want) <= 1e-4f);
 }
 
+CASE(Paged_CompactPagesRehomesPagesAndShrinksThePool, true) {
+    // Six sequences of three pages each, every other one destroyed: the survivors' pages are scattered over the id range.
+    // compact_pages() moves them onto the lowest ids (on the device), rewrites the block table and drops the pool's free
+    // tail; cache contents and decode results are what they were, bit for bit, and the pool goes on working.
+    PagedAttention pa;
+    AttentionParams p{};
+    p.batch_size = 1; p.sequence_length = 1; p.num_heads = 2; p.head_dimension = 32; p.max_sequence_length = 256;
+    PagedAttentionConfig c;
+    c.initial_page_pool_size = 8;
+    c.page_pool_growth = 4;
+    pa.configure_paged_attention(c);
+    pa.configure(p);
+    const size_t H = 2, d = 32, T = 40;
+    std::vector<size_t> ids;
+    std::vector<std::vector<float>> ks, vs;
+    for (int i = 0; i < 6; ++i) {
+        ids.push_back(pa.create_sequence(64));
+        ks.push_back(normal(T * H * d, 130 + i, 2));
+        vs.push_back(normal(T * H * d, 130 + i, 3));
+        pa.append_kv_cache(ids.back(), ks.back().data(), vs.back().data(), T, DataType::FLOAT32);
+    }
+    for (int i : {0, 2, 4}) pa.destroy_sequence(ids[i]);
+    const std::vector<size_t> keep = {ids[1], ids[3], ids[5]};
+    const auto q = normal(3 * H * d, 140, 1);
+    const TensorShape qs = shape4(1, 1, H, d);
+    auto decode_all = [&]() {
+        std::vector<float> out(3 * H * d);
+        pa.forward_batch(keep, {qs, qs, qs}, {q.data(), q.data() + H * d, q.data() + 2 * H * d}, {qs, qs, qs},
+                         {out.data(), out.data() + H * d, out.data() + 2 * H * d});
+        return out;
+    };
+    const auto before = decode_all();
+    std::vector<std::vector<int32_t>> pages_before;
+    for (size_t id : keep) pages_before.push_back(pa.get_sequence_pages(id));
+    EXPECT(pa.get_pool_stats().total_pages >= 18);
+    int32_t highest = 0;
+    for (auto& pg : pages_before) for (int32_t x : pg) highest = std::max(highest, x);
+    EXPECT(highest >= 9);  // scattered: some page in use lies beyond the count of pages in use
+
+    pa.compact_pages();
+
+    const KVBlockPoolStats st = pa.get_pool_stats();
+    EXPECT(st.allocated_pages == 9 && st.total_pages == 9 && st.free_pages == 0);
+    std::vector<int32_t> seen;
+    for (size_t i = 0; i < keep.size(); ++i) {
+        const auto pg = pa.get_sequence_pages(keep[i]);
+        EXPECT(pg.size() == 3);
+        for (int32_t x : pg) { EXPECT(x >= 0 && x < 9); seen.push_back(x); }
+        std::vector<float> kg(T * H * d), vg(T * H * d);
+        pa.get_kv_cache(keep[i], kg.data(), vg.data(), 0, T, DataType::FLOAT32);
+        EXPECT(kg == ks[2 * i + 1] && vg == vs[2 * i + 1]);
+    }
+    std::sort(seen.begin(), seen.end());
+    EXPECT(std::adjacent_find(seen.begin(), seen.end()) == seen.end() && seen.size() == 9);  // every id once
+    EXPECT(decode_all() == before);
+    // compacting a compact pool changes nothing
+    pa.compact_pages();
+    EXPECT(decode_all() == before && pa.get_pool_stats().total_pages == 9);
+    // the pool goes on: a new sequence takes the next ids (the pool grows again) and appends to a survivor still work
+    const size_t fresh = pa.create_sequence(64);
+    pa.append_kv_cache(fresh, ks[0].data(), vs[0].data(), T, DataType::FLOAT32);
+    const auto pg = pa.get_sequence_pages(fresh);
+    EXPECT(pg.size() == 3 && pg[0] == 9 && pg[1] == 10 && pg[2] == 11);
+    std::vector<float> kg(T * H * d), vg(T * H * d);
+    pa.get_kv_cache(fresh, kg.data(), vg.data(), 0, T, DataType::FLOAT32);
+    EXPECT(kg == ks[0] && vg == vs[0]);
+    EXPECT(decode_all() == before);
+}
+
 // ---- KV block pool growth ---------------------------------------------------------------------------------------
 static bool on_cpu_executor() {
     ahpc_device_info info;
@@ -1140,6 +1209,22 @@ CASE(Pool_GrowsInPlace, true) {
     // the budget is the limit, and running into it loses nothing
     EXPECT_THROWS(pool.resize_pool((size_t(1) << 30) / (2 * P * H * d * 4) + 1), AttentionError::MEMORY_ALLOCATION_FAILED);
     EXPECT(pool.get_pool_size() == 40000);
+    gather_pool_pages(pool, 8, H, d, P, kg, vg);
+    EXPECT(kg == k && vg == v);
+    // shrinking drops the free pages at the end of the id range (the nine in use stay) and gives their chunks back;
+    // growing again maps new memory at the same addresses
+    const size_t bytes_big = pool.stats().slab_bytes;
+    pool.resize_pool(4);
+    EXPECT(pool.get_pool_size() == 9 && pool.get_free_pages() == 0 && pool.k_slab() == k0);
+    EXPECT(pool.stats().slab_bytes < bytes_big && pool.stats().slab_capacity_pages >= 9);
+    gather_pool_pages(pool, 8, H, d, P, kg, vg);
+    EXPECT(kg == k && vg == v);
+    EXPECT(pool.allocate_page() == 9);  // grows by 4 again: ids follow on
+    pool.resize_pool(40000);
+    EXPECT(pool.get_pool_size() == 40000 && pool.k_slab() == k0 && pool.stats().slab_capacity_pages >= 40000);
+    if (pool.stats().slab_capacity_pages < 40000) return;
+    EXPECT(ahpc_hip_memset(static_cast<char*>(pool.v_slab()) + (40000 - 1) * P * H * d * 4, 0, P * H * d * 4, nullptr) == 0);
+    EXPECT(ahpc_hip_stream_synchronize(nullptr) == 0);
     gather_pool_pages(pool, 8, H, d, P, kg, vg);
     EXPECT(kg == k && vg == v);
 }

@@ -75,6 +75,8 @@ def test_paged_decode_argument_checks(lib):
     assert decode(lib, qo=5) == BAD_DTYPE and decode(lib, pool=-2) == BAD_DTYPE
     assert decode(lib, B=0) == BAD_SHAPE and decode(lib, max_len=0) == BAD_SHAPE
     assert decode(lib, max_len=65, max_pages=4) == BAD_SHAPE           # the table row cannot hold that many tokens
+    # lengths are 32-bit in the kernels: a bound beyond that is refused, not truncated
+    assert decode(lib, Pg=4096, max_pages=1 << 20, max_len=(1 << 31) + 4096, chunk=262144, ws=P, ws_bytes=1 << 40) == BAD_SHAPE
     assert decode(lib, d=44) == HEAD_DIM and decode(lib, d=264) == HEAD_DIM   # whole 16-byte pieces of an fp16 row, up to 256
     assert decode(lib, kp=P + 8) == BAD_ALIGNMENT and decode(lib, o=P + 2) == BAD_ALIGNMENT
     assert decode(lib, H=6, Hkv=4) == BAD_SHAPE                        # does not divide
@@ -100,9 +102,14 @@ def test_pool_copy_argument_checks(lib):
     assert sb(P, P, F16, 0, 8 * 64, P, P, F16, P, 4, None, None, None, None, 2, 16, 8, 64, 16, None) == NULL_POINTER
     assert sb(P, P, F16, 0, 100, P, P, F16, P, 4, P, None, None, None, 2, 16, 8, 64, 16, None) == BAD_SHAPE  # rows overlap
     assert sb(P, P, F16, 0, 8 * 64, P, P, 4, P, 4, P, None, None, None, 2, 16, 8, 64, 16, None) == BAD_DTYPE
+    mv = lib.ahpc_hip_kv_move_pages
+    assert mv(P, P, F16, 64, P, P, 0, 8, 64, 16, None) == 0                                        # nothing to move
+    assert mv(P, None, F16, 64, P, P, 3, 8, 64, 16, None) == NULL_POINTER and mv(P, P, F16, 64, None, P, 3, 8, 64, 16, None) == NULL_POINTER
+    assert mv(P, P, 7, 64, P, P, 3, 8, 64, 16, None) == BAD_DTYPE and mv(P, P, F16, 0, P, P, 3, 8, 64, 16, None) == BAD_SHAPE
     gi = lib.ahpc_hip_paged_gather_indices
     assert gi(P, P, None, 2, 8, 64, 16, 4, 64, None, None) == NULL_POINTER
     assert gi(P, P, None, 2, 8, 64, 16, 4, 65, P, None) == BAD_SHAPE
+    assert gi(P, P, None, 2, 8, 64, 4096, 1 << 20, (1 << 31) + 4096, P, None) == BAD_SHAPE
 
 
 def test_error_strings_cover_every_code(lib):
@@ -114,13 +121,3 @@ def test_error_strings_cover_every_code(lib):
         seen.add(text)
     assert len(seen) == 9
     assert hip.error_string(-99) == "unknown error code"
-
-
-def test_calibration_probe_argument_checks(lib):
-    probe = lambda dtype=F16, mix=0, wgs=4, it=10, sink=P, nbytes=4 * 256 * 4: lib.ahpc_hip_probe_matrix_rate(
-        dtype, mix, wgs, it, sink, nbytes, None, None)
-    assert probe(sink=None) == NULL_POINTER
-    assert probe(dtype=0) == BAD_DTYPE and probe(dtype=7) == BAD_DTYPE
-    for bad in (dict(wgs=0), dict(it=0), dict(mix=2), dict(it=1 << 25), dict(wgs=1 << 21)):
-        assert probe(**bad) == BAD_SHAPE, bad
-    assert probe(nbytes=4 * 256 * 4 - 1) == WORKSPACE

@@ -962,21 +962,6 @@ def test_backward_ragged_batch(emu, dtype, d, H, H_kv, causal):
         check_gradients(tuple(g[a:b][None] for g in got), want, dtype)
 
 
-# ---- calibration probe -------------------------------------------------------------------------------------
-@pytest.mark.parametrize("dtype", [O.F16, O.BF16])
-@pytest.mark.parametrize("mix", [0, 1])
-def test_matrix_rate_probe_runs_and_counts_its_work(emu, dtype, mix):
-    """The probe has no result worth checking beyond being finite and written by every lane; its operation count is
-    what the benchmark divides by the measured time."""
-    import ctypes as C
-    wgs, it = 2, 3
-    sink = S.guarded(np.full(wgs * 256, np.nan, np.float32))
-    flop = C.c_double(0.0)
-    assert S.load().ahpc_hip_probe_matrix_rate(dtype, mix, wgs, it, S.ptr(sink), sink.nbytes, C.byref(flop), None) == 0
-    assert np.isfinite(sink).all()
-    assert flop.value == 2.0 * 32 * 32 * 16 * 4 * it * 4 * wgs
-
-
 # ---- decode without a workspace argument ----------------------------------------------------------------------
 def decode_noalloc(emu, q, kp, vp, table, lens, B, H, H_kv, d, P, dtype, scale, chunk):
     dq = dev(q, dtype)

@@ -57,6 +57,16 @@ def test_grouped_heads_and_single_chunk(gpu):
     assert np.array_equal(a, b) and np.abs(b - want).max() <= 2e-2
 
 
+def test_headline_decode_shape_with_the_launchers_own_chunking(gpu):
+    # 64 sequences of 512..4096 tokens, 32 heads of 128: the upper bound of the size query (34 MB) is beyond the
+    # array, what the launch plan really needs (chunks of 1024 tokens: 4.3 MB) is not
+    rng = np.random.default_rng(65)
+    lens = [int(x) for x in rng.integers(512, 4097, 64)]
+    assert gpu.paged_decode_workspace_bytes(64, 32, 128, max(lens), 16, 0) > (16 << 20)
+    a, b, want = both(gpu, 64, 32, 32, 128, 16, lens, 65, O.F16, 0)
+    assert np.isfinite(b).all() and np.array_equal(a, b) and np.abs(b - want).max() <= 2e-2
+
+
 def test_beyond_the_built_in_scratch_is_refused(gpu):
     import torch
     x = torch.zeros(1 << 16, device="cuda")
