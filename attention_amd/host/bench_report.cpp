@@ -9,6 +9,14 @@
 // "gflops" is the reference's figure: B*H*N^2*d*2 over the TOTAL time (:241-242).  --csv FILE also writes the table of
 // examples/performance_comparison.cpp:431-463 (same columns, same precisions).
 //
+// PagedAttention rows follow BM_PagedAttention (benchmarks/benchmark_attention.cpp:336-385, registered at :436-457 for
+// batch 2 x sequence {256, 512, 1024} x heads {4, 8} x head_dim {64, 128}): createPagedAttention -> configure (page
+// size 16, max_sequence_length = 2 x sequence) -> the convenience forward, timed as a whole (temporary sequences, cache
+// append, one decode token per batch entry, release), with bytes_per_second as that benchmark's SetBytesProcessed
+// counts them (4 tensors of B x N x H x d elements).  One figure is added: decode_time_ms, the decode of one token per
+// sequence over caches that are already resident (PagedAttention::forward_batch), which is what a serving loop pays.
+// They go into "paged_results" of the JSON file and a second table of the report.
+//
 // Differences, all forced: the backend is BackendType::HIP; inputs are seeded, not std::random_device.  Two extra
 // JSON fields per row say where the tensors lived: with --device the tensors are resident in HBM (the kernel rate),
 // without it they are host vectors exactly as in the reference and the times include the PCIe copies.
@@ -27,6 +35,7 @@
 
 #include "ahpc_hip.h"
 #include "algorithms/flash_attention.hpp"
+#include "algorithms/paged_attention.hpp"
 #include "api/backend_factory.hpp"
 #include "api/tensor.hpp"
 
@@ -146,6 +155,84 @@ Metrics run_config(size_t B, size_t N, size_t H, size_t d, const Options& opt) {
     return m;
 }
 
+struct PagedResult {
+    size_t B = 0, N = 0, H = 0, d = 0;
+    double forward_time_ms = 0.0, decode_time_ms = 0.0, bytes_per_second = 0.0, decode_kv_bytes_per_second = 0.0;
+    bool success = false;
+    std::string error_message;
+};
+
+// BM_PagedAttention, benchmarks/benchmark_attention.cpp:336-385
+PagedResult run_paged_config(size_t B, size_t N, size_t H, size_t d, const Options& opt) {
+    PagedResult r;
+    r.B = B; r.N = N; r.H = H; r.d = d;
+    try {
+        auto attention = BackendFactory::createPagedAttention(BackendType::HIP);
+        AttentionParams params;
+        params.batch_size = B;
+        params.sequence_length = 1;           // one query token per batch entry
+        params.num_heads = H;
+        params.head_dimension = d;
+        params.max_sequence_length = N * 2;   // "allow for growth", :361
+        params.page_size = 16;
+        attention->configure(params);
+        const size_t n_kv = B * N * H * d, n_q = B * H * d, es = elem_size(opt.dtype);
+        auto q = random_tensor(n_q, opt.dtype, 11), k = random_tensor(n_kv, opt.dtype, 12), v = random_tensor(n_kv, opt.dtype, 13);
+        std::vector<unsigned char> o(n_q * es, 0);
+        const TensorShape q_shape({B, 1, H, d}, opt.dtype, MemoryLayout::ROW_MAJOR), kv_shape({B, N, H, d}, opt.dtype, MemoryLayout::ROW_MAJOR);
+        const void *pq = q.data(), *pk = k.data(), *pv = v.data();
+        void* po = o.data();
+        std::unique_ptr<DeviceTensor> dq, dk, dv, dout;
+        if (opt.device) {
+            dq.reset(new DeviceTensor(q)); dk.reset(new DeviceTensor(k)); dv.reset(new DeviceTensor(v)); dout.reset(new DeviceTensor(o));
+            pq = dq->p; pk = dk->p; pv = dv->p; po = dout->p;
+        }
+        for (int i = 0; i < opt.warmup; ++i) attention->forward(q_shape, pq, kv_shape, pk, kv_shape, pv, q_shape, po);
+        auto t0 = std::chrono::steady_clock::now();
+        for (int i = 0; i < opt.iters; ++i) attention->forward(q_shape, pq, kv_shape, pk, kv_shape, pv, q_shape, po);
+        auto t1 = std::chrono::steady_clock::now();
+        r.forward_time_ms = std::chrono::duration<double, std::milli>(t1 - t0).count() / opt.iters;
+        r.bytes_per_second = (double)(n_kv * es * 4) / (r.forward_time_ms / 1000.0);  // SetBytesProcessed, :381-382
+        // the serving loop's step: caches resident, one token per sequence decoded
+        PagedAttention& pa = dynamic_cast<PagedAttention&>(*attention);
+        std::vector<size_t> ids(B);
+        std::vector<TensorShape> shapes(B, TensorShape({1, 1, H, d}, opt.dtype, MemoryLayout::ROW_MAJOR));
+        std::vector<const void*> qp(B);
+        std::vector<void*> op(B);
+        for (size_t b = 0; b < B; ++b) {
+            ids[b] = pa.create_sequence(N * 2);
+            pa.append_kv_cache(ids[b], static_cast<const unsigned char*>(pk) + b * N * H * d * es,
+                               static_cast<const unsigned char*>(pv) + b * N * H * d * es, N, opt.dtype);
+            qp[b] = static_cast<const unsigned char*>(pq) + b * H * d * es;
+            op[b] = static_cast<unsigned char*>(po) + b * H * d * es;
+        }
+        for (int i = 0; i < opt.warmup; ++i) pa.forward_batch(ids, shapes, qp, shapes, op);
+        t0 = std::chrono::steady_clock::now();
+        for (int i = 0; i < opt.iters; ++i) pa.forward_batch(ids, shapes, qp, shapes, op);
+        t1 = std::chrono::steady_clock::now();
+        r.decode_time_ms = std::chrono::duration<double, std::milli>(t1 - t0).count() / opt.iters;
+        r.decode_kv_bytes_per_second = (double)(2 * n_kv * es) / (r.decode_time_ms / 1000.0);
+        for (size_t id : ids) pa.destroy_sequence(id);
+        r.success = true;
+    } catch (const std::exception& e) {
+        r.error_message = e.what();
+    }
+    return r;
+}
+
+void report_paged(const std::vector<PagedResult>& results) {
+    std::cout << "\n=== PagedAttention (BM_PagedAttention configurations) ===\n";
+    std::cout << std::left << std::setw(12) << "Backend" << std::setw(18) << "Config" << std::setw(15) << "Forward(ms)" << std::setw(15)
+              << "Decode(ms)" << std::setw(16) << "Bytes/s (ref.)" << "KV GB/s (decode)\n";
+    for (const PagedResult& r : results) {
+        if (!r.success) continue;
+        const std::string cfg = std::to_string(r.B) + "x" + std::to_string(r.N) + "x" + std::to_string(r.H) + "x" + std::to_string(r.d);
+        std::cout << std::left << std::setw(12) << "HIP" << std::setw(18) << cfg << std::setw(15) << std::fixed << std::setprecision(3)
+                  << r.forward_time_ms << std::setw(15) << r.decode_time_ms << std::setw(16) << std::scientific << std::setprecision(3)
+                  << r.bytes_per_second << std::fixed << std::setprecision(2) << r.decode_kv_bytes_per_second / 1e9 << "\n";
+    }
+}
+
 const char* dtype_name(DataType t) { return t == DataType::FLOAT32 ? "fp32" : t == DataType::FLOAT16 ? "fp16" : "bf16"; }
 
 void report(const std::vector<Result>& results) {  // GeneratePerformanceReport, :529-620
@@ -169,7 +256,7 @@ void report(const std::vector<Result>& results) {  // GeneratePerformanceReport,
     if (best_gf) std::cout << "Best GFLOPS: HIP with " << std::fixed << std::setprecision(2) << best_gf->m.gflops << " GFLOPS\n";
 }
 
-bool save_json(const std::vector<Result>& results, const Options& opt) {  // SaveResultsToJSON, :625-669
+bool save_json(const std::vector<Result>& results, const std::vector<PagedResult>& paged, const Options& opt) {  // SaveResultsToJSON, :625-669
     std::ofstream f(opt.json);
     if (!f) return false;
     f << "{\n  \"benchmark_results\": [\n";
@@ -191,6 +278,21 @@ bool save_json(const std::vector<Result>& results, const Options& opt) {  // Sav
             f << "      \"error_message\": \"" << r.m.error_message << "\"\n";
         }
         f << "    }" << (i + 1 < results.size() ? "," : "") << "\n";
+    }
+    f << "  ],\n  \"paged_results\": [\n";
+    for (size_t i = 0; i < paged.size(); ++i) {
+        const PagedResult& r = paged[i];
+        f << "    {\n      \"backend\": \"HIP\",\n      \"batch_size\": " << r.B << ",\n      \"sequence_length\": " << r.N
+          << ",\n      \"num_heads\": " << r.H << ",\n      \"head_dimension\": " << r.d << ",\n      \"page_size\": 16,\n";
+        f << "      \"data_type\": \"" << dtype_name(opt.dtype) << "\",\n      \"tensors_resident_on_device\": " << (opt.device ? "true" : "false") << ",\n";
+        f << "      \"success\": " << (r.success ? "true" : "false") << ",\n";
+        if (r.success)
+            f << "      \"forward_time_ms\": " << r.forward_time_ms << ",\n      \"bytes_per_second\": " << r.bytes_per_second
+              << ",\n      \"decode_time_ms\": " << r.decode_time_ms << ",\n      \"decode_kv_bytes_per_second\": "
+              << r.decode_kv_bytes_per_second << "\n";
+        else
+            f << "      \"error_message\": \"" << r.error_message << "\"\n";
+        f << "    }" << (i + 1 < paged.size() ? "," : "") << "\n";
     }
     f << "  ],\n  \"config\": {\n    \"warmup_iterations\": " << opt.warmup << ",\n    \"benchmark_iterations\": " << opt.iters
       << ",\n    \"causal_mask\": " << (opt.causal ? "true" : "false") << "\n  }\n}\n";
@@ -260,7 +362,19 @@ int main(int argc, char** argv) {
                     results.push_back(r);
                 }
     report(results);
-    if (!save_json(results, opt)) {
+    // PagedAttention: the subset BM_PagedAttention is registered for, benchmarks/benchmark_attention.cpp:436-457
+    std::vector<PagedResult> paged;
+    for (size_t N : {256, 512, 1024})
+        for (size_t H : {4, 8})
+            for (size_t d : {64, 128}) {
+                paged.push_back(run_paged_config(2, N, H, d, opt));
+                const PagedResult& r = paged.back();
+                std::cout << "  Testing paged config: batch=2, seq_len=" << N << ", heads=" << H << ", head_dim=" << d;
+                if (r.success) std::cout << " - OK (" << std::fixed << std::setprecision(3) << r.forward_time_ms << "ms)\n";
+                else std::cout << " - FAILED (" << r.error_message << ")\n";
+            }
+    report_paged(paged);
+    if (!save_json(results, paged, opt)) {
         std::cerr << "Failed to open file for writing: " << opt.json << "\n";
         return 1;
     }
@@ -274,5 +388,7 @@ int main(int argc, char** argv) {
     }
     for (const Result& r : results)
         if (!r.m.success) return 1;
+    for (const PagedResult& r : paged)
+        if (!r.success) return 1;
     return 0;
 }

@@ -41,6 +41,17 @@ def test_quick_sweep_writes_reference_shaped_results(tmp_path, args):
         assert row["throughput_tokens_per_sec"] == pytest.approx(B * N / (row["forward_time_ms"] / 1e3), rel=1e-3)
         assert row["theoretical_flops"] == pytest.approx(B * H * N * N * (2 * d + 4), rel=1e-5)
         assert row["tensors_resident_on_device"] is ("--device" in args)
+    # PagedAttention rows: the configurations BM_PagedAttention is registered for (benchmarks/benchmark_attention.cpp:436-457)
+    assert "=== PagedAttention" in r.stdout
+    paged = json.loads(out.read_text())["paged_results"]
+    assert [(p["batch_size"], p["sequence_length"], p["num_heads"], p["head_dimension"]) for p in paged] == [
+        (2, N, H, d) for N in (256, 512, 1024) for H in (4, 8) for d in (64, 128)]
+    es = 4 if "--dtype" not in args else 2
+    for p in paged:
+        assert p["success"] is True and p["page_size"] == 16 and p["forward_time_ms"] > 0 and 0 < p["decode_time_ms"] < p["forward_time_ms"]
+        n = p["batch_size"] * p["sequence_length"] * p["num_heads"] * p["head_dimension"]
+        assert p["bytes_per_second"] == pytest.approx(n * es * 4 / (p["forward_time_ms"] / 1e3), rel=1e-3)
+        assert p["decode_kv_bytes_per_second"] == pytest.approx(2 * n * es / (p["decode_time_ms"] / 1e3), rel=1e-3)
     # the CSV: the reference's header, one row per configuration, the same figures
     with open(table) as f:
         lines = list(csv.reader(f))
