@@ -2,15 +2,19 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <atomic>
 #include <cstdlib>
 #include <mutex>
 
 #include "ahpc_device.hpp"
 #include "flash_fwd_mfma.hpp"
+#include "flash_fwd_wide.hpp"
 #include "flash_fwd_f32_mfma.hpp"
 #include "tuning.hpp"
 
 namespace ahpc {
+
+constexpr int kMaxPersistentDevices = 64;
 
 // ---------------------------------------------------------------------------------------------
 // fp32-FMA kernel: any dtype, any head dimension up to 256, optional dense mask.  One thread owns
@@ -153,26 +157,45 @@ static int dispatch_simple(int dtype, const SimpleParams& p, int64_t B, hipStrea
 }
 
 // ---------------------------------------------------------------------------------------------
-// Query rows per workgroup of the 16-bit forward: the tuning value when it names one, else by shape.  Timed on
-// MI355X over dense shapes from 1x256x32 to 1x32768x32: 256 rows (one K/V tile stream per CU) is 3-8 % faster at d = 128
-// from 2048 tokens on once every CU gets a workgroup, and 4-30 % slower on shorter sequences, smaller launches and at
-// d = 64 (where three 128-row workgroups share a CU).
+// Query rows per workgroup of the 16-bit forward without a mask: 128 (flash_fwd_mfma.hpp, two workgroups per CU) or 256
+// (flash_fwd_wide.hpp, one persistent workgroup per CU: dense launches at d = 64 and 128).  The tuning value when it
+// names one, else by shape.  Timed on MI355X over dense shapes from 1x256x32 to 1x32768x32: 256 rows is 3-8 % faster at
+// d = 128 from 2048 tokens on once every CU gets a workgroup, and 4-30 % slower on shorter sequences, smaller launches
+// and at d = 64 (where three 128-row workgroups share a CU).
 static int flash_rows_for(int D, bool varlen, int64_t B, int64_t N, int64_t H) {
-    if (D == 256) return kFlashRows;  // (one wavefront per SIMD already)
+    if (D == 256 || varlen) return kFlashRows;
     const int64_t t = tuning().flash_rows.load();
     if (t == kFlashRows || t == kFlashWideRows) return (int)t;
-    if (D != 128 || varlen || N < 2048) return kFlashRows;
+    if (D != 128 || N < 2048) return kFlashRows;
     return B * H * ((N + kFlashWideRows - 1) / kFlashWideRows) >= 256 ? kFlashWideRows : kFlashRows;
+}
+
+// Workgroups of a persistent launch: one per CU, a multiple of 8 (a workgroup's block ids then all map to the XCD it
+// runs on), and never more than there are block ids.
+static int persistent_grid(int n_block_ids) {
+    static std::atomic<int> cus[kMaxPersistentDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxPersistentDevices) dev = 0;
+    int n = cus[dev].load();
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8) {
+            (void)hipGetLastError();
+            n = 8;
+        }
+        n -= n % 8;
+        cus[dev].store(n);
+    }
+    return n_block_ids < n ? n_block_ids : n;
 }
 
 template <typename T, int D, bool VARLEN>
 static int launch_mfma(FlashParams p, int64_t B, bool causal, hipStream_t stream) {
-    if constexpr (D != 256) {
+    if constexpr (D != 256 && !VARLEN) {
         if (flash_rows_for(D, VARLEN, B, p.N, p.H) == kFlashWideRows) {
-            if (int rc = flash_plan_launch(p, B, causal, kFlashWideRows, tuning().flash_pair_min_tiles.load(), VARLEN)) return rc;
-            dim3 grid((unsigned)(p.blocks_per_xcd * 8)), block(64 * kFlashWideWaves);
-            if (causal) hipLaunchKernelGGL((flash_fwd_mfma_wide_kernel<T, D, true, VARLEN>), grid, block, 0, stream, p);
-            else hipLaunchKernelGGL((flash_fwd_mfma_wide_kernel<T, D, false, VARLEN>), grid, block, 0, stream, p);
+            if (int rc = flash_plan_launch(p, B, causal, kFlashWideRows, tuning().flash_pair_min_tiles.load(), false)) return rc;
+            dim3 grid((unsigned)persistent_grid(p.n_block_ids)), block(64 * kFlashWideWaves);
+            if (causal) hipLaunchKernelGGL((flash_fwd_wide_kernel<T, D, true>), grid, block, 0, stream, p);
+            else hipLaunchKernelGGL((flash_fwd_wide_kernel<T, D, false>), grid, block, 0, stream, p);
             return static_cast<int>(hipGetLastError());
         }
     }

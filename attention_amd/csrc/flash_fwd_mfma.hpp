@@ -71,12 +71,15 @@ struct FlashParams {
     int32_t n_bh;               // B * H: no workgroup may address a (sequence, head) at or beyond this
     int32_t spread_groups;      // ragged batches: 1 = (sequence, head) pairs are dealt to the 8 XCDs in turn (see flash_work_of_block)
     int32_t blocks_per_xcd;     // ceil(total_blocks / 8)
+    int32_t n_block_ids;        // 8 * blocks_per_xcd: the block ids of the work map (a persistent kernel walks them with a stride)
     float scale_log2;           // scale * log2(e)
 };
 
 constexpr int kFlashThreads = 256;
 constexpr int kFlashRows = 128;  // query rows per workgroup
 constexpr int kFlashKeys = 64;   // keys per tile
+constexpr int kFlashWideWaves = 8;                    // flash_fwd_wide.hpp: eight wavefronts,
+constexpr int kFlashWideRows = 32 * kFlashWideWaves;  // 256 query rows per workgroup
 
 #ifndef AHPC_LDS
 #define AHPC_LDS __attribute__((address_space(3)))
@@ -189,7 +192,8 @@ template <int D> struct FlashTile {
 // Streams one 64-key tile (K or V) from global memory into LDS through a buffer descriptor.
 // `base` = first row of the tile, `nrec` = bytes that may be read from there on (anything beyond reads
 // as zero), off[i] = this lane's byte offset for its i-th instruction, wave_u = wavefront index (uniform).
-// IPW = instructions per wavefront: a tile's instructions are shared out evenly among the workgroup's wavefronts.
+// IPW = instructions per wavefront: a tile's instructions are shared out evenly among the workgroup's wavefronts (four
+// of them here, eight in flash_fwd_wide.hpp).
 template <int D, int IPW = FlashTile<D>::kInstrPerWave>
 __device__ inline void dma_tile(const void* base, unsigned nrec, const int* off, unsigned char* lds_tile, int wave_u) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the descriptor type exists only in the device pass
@@ -279,12 +283,9 @@ struct FlashStatsOut {
 //   MASK == 2: the kernel reads one 64-bit word per query and tile of a packed copy (flash_mask_pack_kernel made it
 //              in front of this launch): a sixteenth of the bytes, one load instead of eight, two registers
 //              instead of 32.
-template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS, int MASK = 0, int WAVES = 4>
+template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS, int MASK = 0>
 __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const FlashStatsOut& st) {
     constexpr bool MASKED = MASK != 0;
-    constexpr int ROWS = 32 * WAVES;  // query rows per workgroup: 32 per wavefront
-    constexpr int IPW = kFlashKeys / (WAVES * FlashTile<D>::kRowsPerInstr);  // tile-request instructions per wavefront and tile
-    static_assert(IPW >= 1 && IPW * WAVES * FlashTile<D>::kRowsPerInstr == kFlashKeys, "a tile's requests divide evenly among the wavefronts");
     static_assert(!(MASKED && (VARLEN || STATS)), "the mask belongs to dense forward launches");
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;  // k-steps of the first product
@@ -333,7 +334,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
     }
     // query tiles of this sequence, and the slots they fill (a ragged batch hands every sequence as many slots as
     // the longest one needs: the surplus exits here, before anything is requested)
-    const int n_q = VARLEN ? (L + ROWS - 1) / ROWS : p.n_qtiles;
+    const int n_q = VARLEN ? (L + kFlashRows - 1) / kFlashRows : p.n_qtiles;
     if (VARLEN && slot >= (p.paired ? (n_q + 1) >> 1 : n_q)) return;
     const T* const gq = static_cast<const T*>(p.q) + base;
     const T* const gk = static_cast<const T*>(p.k) + kv_base;
@@ -345,10 +346,10 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
     const int d_real = (p.d_real > 0 && p.d_real < D) ? p.d_real : D;
 
     // ---- per-lane DMA offsets (bytes from the first row of a tile), fixed for the whole kernel ------
-    int dma_off_k[IPW], dma_off_v[IPW];
+    int dma_off_k[TL::kInstrPerWave], dma_off_v[TL::kInstrPerWave];
 #pragma unroll
-    for (int i = 0; i < IPW; ++i) {
-        const int r = (wave * IPW + i) * TL::kRowsPerInstr + lane / TL::kChunks;
+    for (int i = 0; i < TL::kInstrPerWave; ++i) {
+        const int r = (wave * TL::kInstrPerWave + i) * TL::kRowsPerInstr + lane / TL::kChunks;
         const int pc = lane % TL::kChunks;
         const int ck = pc ^ TL::fk(r), cv = pc ^ TL::fv(r);  // the 8-element chunk of the row that belongs at this lane's place
         dma_off_k[i] = (int)(r * skv * 2) + ((8 * ck < d_real ? ck : 0) << 4);
@@ -361,8 +362,8 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
         // (a tile that starts at or behind the end of the sequence touches no memory and lands as zeros)
         const int64_t rem = k0 < L ? (int64_t)(L - k0 - 1) * skv * 2 + 2 * d_real : 0;  // the last row ends with its own d
         const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
-        dma_tile<D, IPW>(gk + (int64_t)k0 * skv, nrec, dma_off_k, dst_k, wave_u);
-        dma_tile<D, IPW>(gv + (int64_t)k0 * skv, nrec, dma_off_v, dst_v, wave_u);
+        dma_tile<D>(gk + (int64_t)k0 * skv, nrec, dma_off_k, dst_k, wave_u);
+        dma_tile<D>(gv + (int64_t)k0 * skv, nrec, dma_off_v, dst_v, wave_u);
     };
 
     // ---- LDS operand addresses (byte offsets inside a tile) -------------------------------------
@@ -384,11 +385,11 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
     for (int part = 0; part < 2; ++part) {
         const int qt = flash_qtile_of_part(p, n_q, slot, part);
         if (qt < 0) break;
-        const int q_tile0 = qt * ROWS;
+        const int q_tile0 = qt * kFlashRows;
         if (q_tile0 >= L) continue;
 
         int k_end = L;
-        if (CAUSAL) k_end = (q_tile0 + ROWS) < L ? (q_tile0 + ROWS) : L;
+        if (CAUSAL) k_end = (q_tile0 + kFlashRows) < L ? (q_tile0 + kFlashRows) : L;
         const int n_tiles = (k_end + kFlashKeys - 1) / kFlashKeys;
 
         // first tile on its way before anything else
@@ -640,7 +641,7 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                     }
             }
             const float delta = halves_sum(part) * inv;
-            if (half == 0 && qrow < q_tile0 + ROWS) {
+            if (half == 0 && qrow < q_tile0 + kFlashRows) {
                 const int64_t row = (int64_t)bh * st.rows_padded + qrow;
                 const bool live = qrow < L && l > 0.0f;
                 st.neg_lse2[row] = live ? neg_m[0] - __builtin_log2f(l) : -INFINITY;
@@ -683,21 +684,13 @@ inline int flash_plan_launch(FlashParams& p, int64_t B, bool causal, int rows_pe
         if (per_xcd * 8 > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
         p.blocks_per_xcd = (int32_t)per_xcd;
     }
+    p.n_block_ids = p.blocks_per_xcd * 8;
     return AHPC_OK;
 }
 
 template <typename T, int D, bool CAUSAL, bool VARLEN>
 __global__ __launch_bounds__(kFlashThreads, D == 256 ? 1 : 2) void flash_fwd_mfma_kernel(const FlashParams p) {
     flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, false>(p, FlashStatsOut{});
-}
-
-// The same with 8 wavefronts = 256 query rows per workgroup and one workgroup per CU: the CU requests every K/V tile
-// once instead of twice (half the tile-request instructions and half the L2 -> LDS bytes per matrix instruction).
-constexpr int kFlashWideWaves = 8;
-constexpr int kFlashWideRows = 32 * kFlashWideWaves;
-template <typename T, int D, bool CAUSAL, bool VARLEN>
-__global__ __launch_bounds__(64 * kFlashWideWaves, 1) void flash_fwd_mfma_wide_kernel(const FlashParams p) {
-    flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, false, 0, kFlashWideWaves>(p, FlashStatsOut{});
 }
 
 // Dense launches with a mask [B,N,N]: MASK 1 reads the caller's fp32 mask, MASK 2 its packed copy.

@@ -167,7 +167,7 @@ inline hipError_t hipMalloc(void** p, size_t n) {
     return *p ? hipSuccess : 2;
 }
 // virtual memory management, emulated with an inaccessible mapping whose front part is made accessible piece by piece
-enum hipDeviceAttribute_t { hipDeviceAttributeVirtualMemoryManagementSupported = 1 };
+enum hipDeviceAttribute_t { hipDeviceAttributeVirtualMemoryManagementSupported = 1, hipDeviceAttributeMultiprocessorCount = 2 };
 inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = 1; return hipSuccess; }
 enum { hipMemAllocationTypePinned = 1, hipMemLocationTypeDevice = 1, hipMemAccessFlagsProtReadWrite = 3 };
 struct hipMemLocation { int type; int id; };
@@ -230,6 +230,9 @@ inline hipError_t hipGetLastError() { return ::simt::last_error(); }
 #define AHPC_TRACED_LDS_READ_B128(p) ::simt::lds_read_b128((p))
 #define __builtin_amdgcn_permlane32_swap(a, b, fi, bc) ::simt::permlane32_swap((a), (b))
 #define __builtin_amdgcn_ballot_w64(p) ::simt::ballot((p))
+// the lanes of a wavefront meet here (on the GPU they are in step anyway): every lane's LDS writes in front of it are
+// visible to the reads behind it
+#define __builtin_amdgcn_wave_barrier() ((void)::simt::ballot(true))
 #define __builtin_amdgcn_readfirstlane(x) ::simt::readfirstlane((x))
 #define __builtin_amdgcn_readlane(x, l) ::simt::readlane((x), (l))
 #define __builtin_amdgcn_update_dpp(old, src, ctrl, rm, bm, bc) ::simt::update_dpp((old), (src), (ctrl), (rm), (bm), (bc))

@@ -292,29 +292,34 @@ def test_256_row_workgroups_against_oracle_and_128_row_form(gpu, flash_rows, dty
     assert np.array_equal(wide, narrow)
 
 
-def test_256_row_workgroups_ragged_and_grouped_heads(gpu, flash_rows):
+def test_256_row_workgroups_grouped_heads_and_more_block_ids_than_workgroups(gpu, flash_rows):
+    """Grouped K/V heads on the persistent kernel, in a launch whose block ids outnumber the CUs (every workgroup walks
+    several ids, paired tiles included)."""
     import torch
-    from gpu_util import stream_ptr, to_dev, to_host, dev_i32, TOL
+    from gpu_util import stream_ptr, to_dev, to_host, TOL
     flash_rows(256)
-    gpu.set_tuning("flash_pair_min_tiles", 1)
-    try:
-        dtype, H, H_kv, d = O.BF16, 4, 2, 128
-        lens = np.array([700, 1, 256, 1029, 64], np.int32)
-        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
-        T = int(cu[-1])
-        q = O.round_to(O.fill_normal((T, H, d), 77, 1), dtype)
-        k = O.round_to(O.fill_normal((T, H_kv, d), 77, 2), dtype)
-        v = O.round_to(O.fill_normal((T, H_kv, d), 77, 3), dtype)
-        dq, dk, dv = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype)
-        do = torch.full_like(dq, float("nan"))
-        gpu.flash_fwd_varlen_gqa(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), do.data_ptr(), dtype, dev_i32(cu).data_ptr(), len(lens),
-                                 int(lens.max()), H, H_kv, d, H * d, d, H_kv * d, d, 0.1, True, stream_ptr())
-        torch.cuda.synchronize()
-        kr, vr = np.repeat(k, H // H_kv, axis=1), np.repeat(v, H // H_kv, axis=1)
-        want = O.attention_varlen(q, kr, vr, cu, H, d, 0.1, True)
-        assert np.abs(to_host(do) - want).max() <= TOL[dtype]
-    finally:
-        gpu.set_tuning("flash_pair_min_tiles", 1024)
+    dtype, B, N, H, H_kv, d = O.BF16, 3, 1100, 40, 10, 128      # 3 * 40 * 5 = 600 query tiles of 256 rows
+    q = O.round_to(O.fill_normal((B, N, H, d), 78, 1), dtype)
+    k = O.round_to(O.fill_normal((B, N, H_kv, d), 78, 2), dtype)
+    v = O.round_to(O.fill_normal((B, N, H_kv, d), 78, 3), dtype)
+    for causal, pair_min in ((True, 1), (False, 1024)):
+        gpu.set_tuning("flash_pair_min_tiles", pair_min)
+        try:
+            dq, dk, dv = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype)
+            do = torch.full_like(dq, float("nan"))
+            gpu.flash_fwd_gqa(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), do.data_ptr(), dtype, B, N, H, H_kv, d, (N * H * d, H * d, d),
+                              (N * H_kv * d, H_kv * d, d), 0.09, causal, stream_ptr())
+            torch.cuda.synchronize()
+        finally:
+            gpu.set_tuning("flash_pair_min_tiles", 1024)
+        got = to_host(do)
+        assert np.isfinite(got).all()
+        rng = np.random.default_rng(5)
+        rows = np.unique(np.concatenate([rng.integers(0, B * H * N, 200), [0, N - 1, B * H * N - 1, 255, 256, 1099]])).astype(np.int64)
+        kr, vr = np.repeat(k, H // H_kv, axis=2), np.repeat(v, H // H_kv, axis=2)
+        want = O.attention_rows(q, kr, vr, B, N, H, d, 0.09, rows, causal)
+        have = np.stack([got[r // (N * H), r % N, (r // N) % H] for r in rows])
+        assert np.abs(have - want).max() <= TOL[dtype]
 
 
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16])
