@@ -18,6 +18,7 @@
 
 #include "ahpc_device.hpp"
 #include "flash_bwd_mfma.hpp"
+#include "mask_pack.hpp"
 #include "flash_bwd_f32_mfma.hpp"
 #include "tuning.hpp"
 
@@ -410,6 +411,59 @@ static int launch_mfma_dv(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool
     return static_cast<int>(hipGetLastError());
 }
 
+// The same three steps under a dense mask, on its packed copy (dense launches only).
+template <typename T, int D>
+static int launch_mfma_masked_dv(FlashBwdParams p, const PackedMask& pm, int64_t B, int64_t H_kv, bool causal, float* lse2,
+                                 float* delta, hipStream_t stream) {
+    FlashParams f{};
+    f.q = p.q; f.k = p.k; f.v = p.v; f.o = nullptr;
+    f.stride_b = p.stride_b; f.stride_n = p.stride_n; f.stride_h = p.stride_h;
+    f.kv_stride_b = p.kv_stride_b; f.kv_stride_n = p.kv_stride_n; f.kv_stride_h = p.kv_stride_h;
+    f.N = p.N; f.H = p.H; f.kv_group = p.kv_group;
+    f.scale_log2 = p.scale_log2;
+    f.d_real = p.d_real;
+    f.mask_bits = pm.bits;
+    f.mask_kt = pm.tiles;
+    if (int rc = flash_plan_launch(f, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load(), false)) return rc;
+    const FlashStatsOut st{p.d_out, lse2, delta, p.rows_padded};
+    const dim3 block(kFlashThreads);
+    const dim3 grid_stats((unsigned)(f.blocks_per_xcd * 8));
+    FlashBwdParams m = p;
+    m.mask_bits = pm.bits;
+    m.mask_bits_t = pm.bits_t;
+    m.mask_tiles = pm.tiles;
+    m.n_tiles = (p.N + kFlashRows - 1) / kFlashRows;
+    m.paired = (causal && m.n_tiles >= 2 && tuning().bwd_pair.load() != 0) ? 1 : 0;
+    const int64_t units = bwd_units(m);
+    const int64_t total_q = B * p.H * units, total_kv = B * H_kv * units;
+    if (total_q > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
+    m.total_q = (int32_t)total_q; m.per_xcd_q = (int32_t)((total_q + 7) / 8);
+    m.total_kv = (int32_t)total_kv; m.per_xcd_kv = (int32_t)((total_kv + 7) / 8);
+    const dim3 grid_q((unsigned)(m.per_xcd_q * 8)), grid_kv((unsigned)(m.per_xcd_kv * 8));
+    const int64_t choice = tuning().bwd_split.load();
+    const bool split = choice == 0 ? D == 128 : choice == 2;
+    if (causal) {
+        hipLaunchKernelGGL((flash_bwd_stats_masked_mfma_kernel<T, D, true>), grid_stats, block, 0, stream, f, st);
+        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, true, false, true>), grid_q, block, 0, stream, m);
+        if (split) {
+            hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, true, false, 1, true>), grid_kv, block, 0, stream, m);
+            hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, true, false, 2, true>), grid_kv, block, 0, stream, m);
+        } else {
+            hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, true, false, 0, true>), grid_kv, block, 0, stream, m);
+        }
+    } else {
+        hipLaunchKernelGGL((flash_bwd_stats_masked_mfma_kernel<T, D, false>), grid_stats, block, 0, stream, f, st);
+        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, false, false, true>), grid_q, block, 0, stream, m);
+        if (split) {
+            hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, false, false, 1, true>), grid_kv, block, 0, stream, m);
+            hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, false, false, 2, true>), grid_kv, block, 0, stream, m);
+        } else {
+            hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, false, false, 0, true>), grid_kv, block, 0, stream, m);
+        }
+    }
+    return static_cast<int>(hipGetLastError());
+}
+
 template <typename T>
 static int launch_mfma(const FlashBwdParams& p, int64_t B, int64_t H_kv, int d, bool causal, float* lse2, float* delta,
                        hipStream_t stream) {
@@ -531,8 +585,32 @@ static int flash_bwd_any(const void* d_out, const void* q, const void* k, const 
     // head dimensions up to 128 in whole 16-byte pieces; one below 64 or 128 runs on the next kernel (FlashParams::d_real)
     const bool d_ok = d <= 128 && d >= (is16 ? 8 : 4) && d % (is16 ? 8 : 4) == 0;
     const int kernel_d = d <= 64 ? 64 : 128;
-    if (!mask && d_ok && (is16 ? strides_ok : strides4_ok) && aligned16(q) &&
-        aligned16(k) && aligned16(v) && aligned16(d_out) && aligned16(d_q) && aligned16(d_k) && aligned16(d_v)) {
+    const bool tensors_ok = d_ok && (is16 ? strides_ok : strides4_ok) && aligned16(q) && aligned16(k) && aligned16(v) &&
+                            aligned16(d_out) && aligned16(d_q) && aligned16(d_k) && aligned16(d_v);
+    if (mask && is16 && tensors_ok && !cu_seqlens && tuning().mask_pack.load() != 0) {
+        // a dense mask on 16-bit tensors: the matrix-core kernels on the mask's packed copy (both layouts), where that
+        // can be made (not under graph capture, not beyond the library's buffer limit)
+        FlashBwdParams m{};
+        m.q = q; m.k = k; m.v = v; m.d_out = d_out;
+        m.d_q = d_q; m.d_k = d_k; m.d_v = d_v;
+        m.neg_lse2 = p.lse; m.neg_delta = p.delta; m.rows_padded = p.rows_padded;
+        m.stride_b = stride_b; m.stride_n = stride_n; m.stride_h = stride_h;
+        m.kv_stride_b = kv_stride_b; m.kv_stride_n = kv_stride_n; m.kv_stride_h = kv_stride_h;
+        m.N = (int32_t)N; m.H = (int32_t)H; m.kv_group = p.kv_group;
+        m.scale = scale;
+        m.scale_log2 = scale * kLog2e;
+        m.d_real = (int32_t)d;
+        bool launched = false;
+        const int rc = with_packed_mask(mask, B, N, true, st, &launched, [&](const PackedMask& pm) {
+            if (dtype == AHPC_F16)
+                return kernel_d == 64 ? launch_mfma_masked_dv<f16_t, 64>(m, pm, B, H_kv, causal != 0, p.lse, p.delta, st)
+                                      : launch_mfma_masked_dv<f16_t, 128>(m, pm, B, H_kv, causal != 0, p.lse, p.delta, st);
+            return kernel_d == 64 ? launch_mfma_masked_dv<bf16_t, 64>(m, pm, B, H_kv, causal != 0, p.lse, p.delta, st)
+                                  : launch_mfma_masked_dv<bf16_t, 128>(m, pm, B, H_kv, causal != 0, p.lse, p.delta, st);
+        });
+        if (launched || rc != AHPC_OK) return rc;
+    }
+    if (!mask && tensors_ok) {
         FlashBwdParams m{};
         m.q = q; m.k = k; m.v = v; m.d_out = d_out;
         m.d_q = d_q; m.d_k = d_k; m.d_v = d_v;

@@ -38,6 +38,11 @@ struct FlashBwdParams {
     const float* neg_lse2;      // [B*H][rows_padded]: -lse2 and -delta, what the accumulators start from
     const float* neg_delta;
     const int32_t* cu_seqlens;  // ragged batches only
+    // dense mask, packed (masked kernels only; see PackedMask): 64 keys per word and query for the dQ kernel, 64 queries
+    // per word and key for the dK/dV kernels; mask_tiles = ceil(N / 64)
+    const uint64_t* mask_bits;
+    const uint64_t* mask_bits_t;
+    int32_t mask_tiles;
     int64_t rows_padded;
     int64_t stride_b, stride_n, stride_h;           // Q, dO, dQ
     int64_t kv_stride_b, kv_stride_n, kv_stride_h;  // K, V, dK, dV
@@ -121,8 +126,11 @@ __device__ inline void store_row(T* dst_row, const f32x16 (&acc)[MB], int half, 
 }
 
 // grid: 8 * per_xcd_q workgroups, see bwd_work_of_block
-template <typename T, int D, bool CAUSAL, bool VARLEN>
+// MASKED: a dense mask removes keys per query; the lane's word of the packed mask (its query's 64 keys of the tile) is
+// loaded in front of the tile requests and tested bit by bit next to the causal / end-of-sequence test.
+template <typename T, int D, bool CAUSAL, bool VARLEN, bool MASKED = false>
 __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(const FlashBwdParams p) {
+    static_assert(!(MASKED && VARLEN), "the mask belongs to dense launches");
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;
     constexpr int MB = D / 32;
@@ -207,6 +215,7 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
         load_row_operands<T, KS>(qreg, gq + (int64_t)row * sn, half, p.scale_log2, d_real);
         load_row_operands<T, KS>(doreg, gdo + (int64_t)row * sn, half, 1.0f, d_real);
         const int64_t stat = ((int64_t)b * p.H + h) * p.rows_padded + qrow;  // qrow < rows_padded always
+        const uint64_t* const mword = MASKED ? p.mask_bits + (int64_t)b * p.mask_tiles * p.N + row : nullptr;
         f32x16 neg_lse, neg_delta;
         {
             const float a = p.neg_lse2[stat], d0 = p.neg_delta[stat];
@@ -222,7 +231,7 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mb][r] = 0.0f;
 
-        auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int k0) {
+        auto compute_tile = [&](const unsigned char* tile_k, const unsigned char* tile_v, int k0, uint64_t mw) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
                 const int kblock0 = k0 + 32 * kb;
@@ -267,7 +276,7 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
                 f32x16 ds;
                 // the per-element test is needed only where the block meets the diagonal or the end of the sequence
                 // (uniform per wavefront)
-                const bool all_on = kblock0 + 31 < L && (!CAUSAL || kblock0 + 31 <= qw);
+                const bool all_on = !MASKED && kblock0 + 31 < L && (!CAUSAL || kblock0 + 31 <= qw);
                 if (all_on) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) ds[r] = fast_exp2(s[r]) * dp[r];
@@ -275,10 +284,13 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
                     int lim = L - 1;
                     if (CAUSAL) lim = qrow < lim ? qrow : lim;
                     lim -= kblock0 + 4 * half;
+                    // the lane's keys of the block as bits 0.. of one word: key kblock0 + 4*half + off <-> bit off
+                    const uint32_t bits = MASKED ? (uint32_t)(mw >> (32 * kb)) >> (4 * half) : 0xFFFFFFFFu;
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const int off = 8 * (r >> 2) + (r & 3);
-                        ds[r] = off <= lim ? fast_exp2(s[r]) * dp[r] : 0.0f;
+                        const bool on = off <= lim && (!MASKED || ((bits >> off) & 1u));
+                        ds[r] = on ? fast_exp2(s[r]) * dp[r] : 0.0f;
                     }
                 }
                 __builtin_amdgcn_s_setprio(1);
@@ -306,8 +318,14 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
         auto step = [&](unsigned char* cur_k, unsigned char* cur_v, unsigned char* nxt_k, unsigned char* nxt_v, int t) {
             const int k0 = t * kFlashKeys;
             const bool more = t + 1 < n_tiles;
+            uint64_t mw = 0;
+            if constexpr (MASKED) {
+                // in front of the tile requests: loads complete in order, a word requested behind them would wait for the tile
+                mw = mword[(int64_t)t * p.N];
+                __builtin_amdgcn_sched_barrier(0);
+            }
             if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
-            compute_tile(cur_k, cur_v, k0);
+            compute_tile(cur_k, cur_v, k0, mw);
             if (more) {
                 __builtin_amdgcn_s_waitcnt(0);
                 __syncthreads();
@@ -329,8 +347,10 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
 // wavefront per SIMD), 1 = dV only (S and dV: two products, V and dO.V never touched), 2 = dK only (S, dP, dK).  The
 // two partial walks execute five products between them but each fits two wavefronts per SIMD, which hide each
 // other's softmax arithmetic and LDS waits; at d = 128 they are the faster way (the launcher picks).
-template <typename T, int D, bool CAUSAL, bool VARLEN, int PART>
+// MASKED: as in the dQ kernel, with the transposed packed mask (the lane's key, 64 queries per word).
+template <typename T, int D, bool CAUSAL, bool VARLEN, int PART, bool MASKED = false>
 __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_dkv_mfma_kernel(const FlashBwdParams p) {
+    static_assert(!(MASKED && VARLEN), "the mask belongs to dense launches");
     constexpr bool kDoK = PART != 1, kDoV = PART != 2;
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;
@@ -396,6 +416,7 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
         const int kw = k_tile0 + wave * 32;  // first key of this wavefront
         const int key = kw + col;
         const int krow = key < L ? key : L - 1;
+        const uint64_t* const mword = MASKED ? p.mask_bits_t + (int64_t)b * p.mask_tiles * p.N + krow : nullptr;
         u32x4 kreg[KS], vreg[KS];
         load_row_operands<T, KS>(kreg, gk + (int64_t)krow * skv, half, p.scale_log2, d_real);
         if constexpr (kDoK) load_row_operands<T, KS>(vreg, gv + (int64_t)krow * skv, half, 1.0f, d_real);
@@ -436,7 +457,8 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
                 }
             };
 
-            auto compute_tile = [&](const unsigned char* tile_q, const unsigned char* tile_o, const unsigned char* tile_s, int i0) {
+            auto compute_tile = [&](const unsigned char* tile_q, const unsigned char* tile_o, const unsigned char* tile_s, int i0,
+                                    uint64_t mw) {
 #pragma unroll
                 for (int ib = 0; ib < 2; ++ib) {
                     const int iblock0 = i0 + 32 * ib;
@@ -502,7 +524,7 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
                     f32x16 pw, ds;
                     // the per-element tests are needed only where the block meets the diagonal or an end of the sequence
                     // (uniform per wavefront): everywhere else every (query, key) pair of the block counts
-                    const bool all_on = iblock0 + 31 < L && kw + 31 < L && (!CAUSAL || iblock0 >= kw + 31);
+                    const bool all_on = !MASKED && iblock0 + 31 < L && kw + 31 < L && (!CAUSAL || iblock0 >= kw + 31);
                     if (all_on) {
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
@@ -513,10 +535,12 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
                         int first = 0;
                         if (CAUSAL) first = key - (iblock0 + 4 * half);
                         const int last = (key < L ? L : 0) - (iblock0 + 4 * half);  // off < last
+                        // the lane's queries of the block as bits 0.. of one word: query iblock0 + 4*half + off <-> bit off
+                        const uint32_t bits = MASKED ? (uint32_t)(mw >> (32 * ib)) >> (4 * half) : 0xFFFFFFFFu;
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
                             const int off = 8 * (r >> 2) + (r & 3);
-                            const bool on = off >= first && off < last;
+                            const bool on = off >= first && off < last && (!MASKED || ((bits >> off) & 1u));
                             pw[r] = on ? fast_exp2(s[r]) : 0.0f;
                             if constexpr (kDoK) ds[r] = on ? pw[r] * dp[r] : 0.0f;
                         }
@@ -561,8 +585,13 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_
                             unsigned char* nxt_s, int t) {
                 const int i0 = t * kFlashKeys;
                 const bool more = t + 1 < n_tiles;
+                uint64_t mw = 0;
+                if constexpr (MASKED) {
+                    mw = mword[(int64_t)t * p.N];  // (in front of the tile requests, see the dQ kernel)
+                    __builtin_amdgcn_sched_barrier(0);
+                }
                 if (more) dma_both(i0 + kFlashKeys, nxt_q, nxt_o, nxt_s);
-                compute_tile(cur_q, cur_o, cur_s, i0);
+                compute_tile(cur_q, cur_o, cur_s, i0, mw);
                 if (more) {
                     __builtin_amdgcn_s_waitcnt(0);
                     __syncthreads();

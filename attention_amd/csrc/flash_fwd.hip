@@ -4,11 +4,13 @@
 #include <cmath>
 #include <atomic>
 #include <cstdlib>
+#include <functional>
 #include <mutex>
 
 #include "ahpc_device.hpp"
 #include "flash_fwd_mfma.hpp"
 #include "flash_fwd_wide.hpp"
+#include "mask_pack.hpp"
 #include "flash_fwd_f32_mfma.hpp"
 #include "tuning.hpp"
 
@@ -229,9 +231,13 @@ static int dispatch_mfma_masked(const FlashParams& p, int64_t B, int d, bool cau
 // keys of the tile, bit j set = mask[b][query][64 * tile + j] != 0 (keys at or beyond N: clear).  A wavefront takes
 // 64 queries x 64 keys: per query one coalesced 256-byte read and a ballot; lane r keeps the word of query r, and the
 // 64 words leave as one coalesced 512-byte store.  Consecutive wavefronts take consecutive tiles of the same queries.
+// With bits_t given the same pass also writes the transposed layout the backward's dK/dV kernels read: word
+// [(b * n_rb + query block) * N + key] holds the block's 64 queries, bit r set = mask[b][64 * block + r][key] != 0
+// (lane = key collects its own word from the values it loads).
 constexpr int kMaskPackThreads = 256;
 __global__ __launch_bounds__(kMaskPackThreads) void flash_mask_pack_kernel(const float* __restrict__ mask, uint64_t* __restrict__ bits,
-                                                                            int N, int n_kt, int n_rb, int64_t n_units) {
+                                                                            uint64_t* __restrict__ bits_t, int N, int n_kt, int n_rb,
+                                                                            int64_t n_units) {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t unit = (int64_t)blockIdx.x * (kMaskPackThreads / kWave) + (threadIdx.x >> 6);
     if (unit >= n_units) return;
@@ -240,22 +246,24 @@ __global__ __launch_bounds__(kMaskPackThreads) void flash_mask_pack_kernel(const
     const int b = (int)(unit / ((int64_t)n_kt * n_rb));
     const int key = 64 * kt + lane;
     const float* const src = mask + (int64_t)b * N * N + (key < N ? key : 0);
-    uint64_t mine = 0;
+    uint64_t mine = 0, mine_t = 0;
 #pragma unroll 16
     for (int r = 0; r < 64; ++r) {
         const int row = 64 * rb + r;
         const float m = (row < N && key < N) ? __builtin_nontemporal_load(src + (int64_t)row * N) : 0.0f;  // read once
         const uint64_t word = __builtin_amdgcn_ballot_w64(m != 0.0f);
         if (lane == r) mine = word;
+        mine_t |= (uint64_t)(m != 0.0f) << r;
     }
     const int row = 64 * rb + lane;
     if (row < N) bits[((int64_t)b * n_kt + kt) * N + row] = mine;
+    if (bits_t && key < N) bits_t[((int64_t)b * n_rb + rb) * N + key] = mine_t;
 }
 
 // The packed copy of a mask lives in device memory that the library owns: one buffer per device, grown on demand and kept
-// until the process ends (B * N * ceil(N / 64) * 8 bytes: an eighth of a byte per mask element).  Calls on one device
-// share it: `done` is recorded behind the launch that reads it, and the next call's stream waits for it before the
-// buffer is overwritten; the mutex covers the whole of that.
+// until the process ends (B * N * ceil(N / 64) * 8 bytes per layout: an eighth of a byte per mask element).  Calls on one
+// device share it: `done` is recorded behind the last launch that reads it, and the next call's stream waits for it
+// before the buffer is overwritten; the mutex covers the whole of that.
 struct MaskScratch {
     std::mutex mu;
     void* ptr = nullptr;
@@ -266,11 +274,11 @@ constexpr int kMaxDevices = 64;
 constexpr size_t kMaskScratchLimit = size_t(1) << 30;  // larger masks are read in place
 static MaskScratch g_mask_scratch[kMaxDevices];
 
-// Packs `mask` and launches a matrix-core kernel (launch_on_bits) on the packed copy.  AHPC_OK + *launched = false: not possible here
-// (stream under capture, no memory, mask too large), nothing was launched and the caller reads the mask in place.
-template <typename Launch>
-static int forward_on_packed_mask(FlashParams p, const float* mask, int64_t B, hipStream_t stream, bool* launched,
-                                  Launch launch_on_bits) {
+// Packs `mask` (with_transposed: both layouts) and runs launch_on_bits on the packed copy.  AHPC_OK + *launched = false:
+// not possible here (stream under capture, no memory, mask too large), nothing was launched and the caller takes another
+// path.
+int with_packed_mask(const float* mask, int64_t B, int64_t N, bool with_transposed, hipStream_t stream, bool* launched,
+                     const std::function<int(const PackedMask&)>& launch_on_bits) {
     *launched = false;
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
@@ -279,8 +287,9 @@ static int forward_on_packed_mask(FlashParams p, const float* mask, int64_t B, h
     }
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return AHPC_OK;
-    const int64_t N = p.N, n_kt = (N + 63) / 64, n_rb = (N + 63) / 64;
-    const size_t need = (size_t)B * (size_t)n_kt * (size_t)N * sizeof(uint64_t);
+    const int64_t n_kt = (N + 63) / 64, n_rb = (N + 63) / 64;
+    const size_t one = (size_t)B * (size_t)n_kt * (size_t)N * sizeof(uint64_t);
+    const size_t need = with_transposed ? 2 * one : one;
     if (need > kMaskScratchLimit) return AHPC_OK;
     MaskScratch& sc = g_mask_scratch[dev];
     std::lock_guard<std::mutex> lock(sc.mu);
@@ -305,16 +314,29 @@ static int forward_on_packed_mask(FlashParams p, const float* mask, int64_t B, h
     const int64_t n_units = B * n_rb * n_kt;
     const int64_t blocks = (n_units + kMaskPackThreads / kWave - 1) / (kMaskPackThreads / kWave);
     if (blocks > 0x7FFFFFFFll) return AHPC_OK;
+    PackedMask pm{};
+    pm.bits = static_cast<const uint64_t*>(sc.ptr);
+    pm.bits_t = with_transposed ? pm.bits + one / sizeof(uint64_t) : nullptr;
+    pm.tiles = (int32_t)n_kt;
     hipLaunchKernelGGL(flash_mask_pack_kernel, dim3((unsigned)blocks), dim3(kMaskPackThreads), 0, stream, mask,
-                       static_cast<uint64_t*>(sc.ptr), (int)N, (int)n_kt, (int)n_rb, n_units);
+                       const_cast<uint64_t*>(pm.bits), const_cast<uint64_t*>(pm.bits_t), (int)N, (int)n_kt, (int)n_rb, n_units);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return static_cast<int>(e);
-    p.mask = nullptr;
-    p.mask_bits = static_cast<const uint64_t*>(sc.ptr);
-    p.mask_kt = (int32_t)n_kt;
     *launched = true;
-    const int rc = launch_on_bits(p);
+    const int rc = launch_on_bits(pm);
     const hipError_t e = hipEventRecord(sc.done, stream);
     return rc != AHPC_OK ? rc : static_cast<int>(e);
+}
+
+// The forward on a packed mask.
+template <typename Launch>
+static int forward_on_packed_mask(FlashParams p, const float* mask, int64_t B, hipStream_t stream, bool* launched,
+                                  Launch launch_on_bits) {
+    return with_packed_mask(mask, B, p.N, false, stream, launched, [&](const PackedMask& pm) {
+        p.mask = nullptr;
+        p.mask_bits = pm.bits;
+        p.mask_kt = pm.tiles;
+        return launch_on_bits(p);
+    });
 }
 
 template <typename T, bool VARLEN>

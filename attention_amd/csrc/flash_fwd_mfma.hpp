@@ -286,7 +286,8 @@ struct FlashStatsOut {
 template <typename T, int D, bool CAUSAL, bool VARLEN, bool STATS, int MASK = 0>
 __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const FlashStatsOut& st) {
     constexpr bool MASKED = MASK != 0;
-    static_assert(!(MASKED && (VARLEN || STATS)), "the mask belongs to dense forward launches");
+    static_assert(!(MASKED && VARLEN), "the mask belongs to dense launches");
+    static_assert(!(STATS && MASK == 1), "the statistics pass reads the packed mask only");
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;  // k-steps of the first product
     constexpr int MB = D / 32;  // 32-row blocks of O^T
@@ -703,6 +704,12 @@ __global__ __launch_bounds__(kFlashThreads, D == 256 ? 1 : 2) void flash_fwd_mfm
 template <typename T, int D, bool CAUSAL, bool VARLEN>
 __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_stats_mfma_kernel(const FlashParams p, const FlashStatsOut st) {
     flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, true>(p, st);
+}
+// The same under a dense mask (its packed copy).  A query that sees no key gets -lse2 = -inf and -delta = 0, like a row
+// beyond the sequence: every weight of it is exp2(s - inf) = 0 in the backward kernels.
+template <typename T, int D, bool CAUSAL>
+__global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_stats_masked_mfma_kernel(const FlashParams p, const FlashStatsOut st) {
+    flash_fwd_mfma_body<T, D, CAUSAL, false, true, 2>(p, st);
 }
 
 }  // namespace ahpc

@@ -736,6 +736,48 @@ def test_backward_matrix_core_kernels(emu, tuned, dtype, B, N, H, H_kv, d, causa
     check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), dtype)
 
 
+@pytest.mark.parametrize("split,dma_late", [(1, False), (2, True)])
+@pytest.mark.parametrize("dtype,B,N,H,H_kv,d,causal", [
+    (O.BF16, 2, 64, 2, 2, 128, False), (O.F16, 2, 131, 2, 1, 128, True), (O.F16, 1, 300, 2, 2, 64, False),
+    (O.BF16, 2, 200, 4, 2, 64, True), (O.BF16, 1, 3, 2, 2, 128, False), (O.F16, 2, 65, 2, 2, 32, True)])
+def test_backward_matrix_core_kernels_dense_mask(emu, tuned, dtype, B, N, H, H_kv, d, causal, dma_late, split):
+    """fp16/bf16 with a mask [B,N,N]: statistics, dQ, dK and dV on the matrix cores, on the packed copy of the mask in
+    both of its layouts (keys per query for dQ, queries per key for dK and dV).  A query that sees nothing (no gradient
+    reaches or leaves it), a key that nobody sees, queries that see one key, a last tile of 1 to 60 rows."""
+    tuned("bwd_split", split)
+    tuned("bwd_pair", split - 1)
+    q, k, v, do = bwd_inputs(B, N, H, H_kv, d, 35, dtype)
+    mask = (O.fill_uniform((B, N, N), 35, 6) > 0.4).astype(np.float32)
+    mask[0, N // 2, :] = 0.0
+    mask[0, :, N // 3] = 0.0
+    mask[B - 1, N - 1, :] = 0.0
+    mask[B - 1, N - 1, N - 1] = 1.0
+    mask[B - 1, 0, :] = 0.0
+    mask[B - 1, 0, 0] = 1.0
+    scale = 1.0 / np.sqrt(d)
+    S.configure(dma_late, seed=N + d)
+    S.lds_stats(reset=True)
+    try:
+        got = backward(emu, q, k, v, do, dtype, B, N, H, H_kv, d, scale, causal, mask=mask, front=dma_late)
+    finally:
+        S.configure(False, 1)
+    assert S.lds_stats(reset=True)[0] > 0   # the matrix-core kernels ran (the FMA kernels make no traced reads)
+    assert not got[0][0, N // 2].any()
+    assert not got[1][0, N // 3].any() and not got[2][0, N // 3].any()
+    check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv, mask), dtype)
+
+
+def test_backward_dense_mask_without_the_packed_copy_takes_the_plain_kernels(emu, tuned):
+    tuned("mask_pack", 0)
+    B, N, H, d = 1, 70, 2, 64
+    q, k, v, do = bwd_inputs(B, N, H, H, d, 36, O.BF16)
+    mask = (O.fill_uniform((B, N, N), 36, 6) > 0.3).astype(np.float32)
+    S.lds_stats(reset=True)
+    got = backward(emu, q, k, v, do, O.BF16, B, N, H, H, d, 0.125, False, mask=mask)
+    assert S.lds_stats(reset=True)[0] == 0
+    check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, 0.125, False, H, mask), O.BF16)
+
+
 @pytest.mark.parametrize("dma_late", [False, True])
 @pytest.mark.parametrize("B,N,H,H_kv,d,causal", [
     (1, 64, 1, 1, 128, False), (2, 129, 2, 2, 128, True), (1, 300, 2, 2, 64, True), (1, 200, 2, 1, 64, False),
