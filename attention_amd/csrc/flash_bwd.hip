@@ -361,21 +361,23 @@ static int64_t padded_rows(int64_t N) { return (N + kFlashRows - 1) / kFlashRows
 
 // dK and dV: in one walk over the query tiles where that fits two workgroups on a CU (d = 64), in two walks (dV, then
 // dK) where it does not (d = 128); the tuning value bwd_split (0 = by head dimension, 1 = one walk, 2 = two) overrides.
-template <typename T, int D, bool CAUSAL, bool VARLEN>
+// d = 256: always two walks (one walk would need more registers than a wavefront has).
+template <typename T, int D, bool CAUSAL, bool VARLEN, bool MASKED>
 static void launch_dkv(const FlashBwdParams& m, dim3 grid, dim3 block, hipStream_t stream) {
     const int64_t choice = tuning().bwd_split.load();
-    const bool split = choice == 0 ? D == 128 : choice == 2;
+    const bool split = D == 256 || (choice == 0 ? D == 128 : choice == 2);
     if (split) {
-        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, CAUSAL, VARLEN, 1>), grid, block, 0, stream, m);
-        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, CAUSAL, VARLEN, 2>), grid, block, 0, stream, m);
-    } else {
-        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, CAUSAL, VARLEN, 0>), grid, block, 0, stream, m);
+        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, CAUSAL, VARLEN, 1, MASKED>), grid, block, 0, stream, m);
+        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, CAUSAL, VARLEN, 2, MASKED>), grid, block, 0, stream, m);
+    } else if constexpr (D != 256) {
+        hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, CAUSAL, VARLEN, 0, MASKED>), grid, block, 0, stream, m);
     }
 }
 
+// Statistics, dQ, dK and dV.  pm: the packed copy of a dense mask (dense launches only), or null.
 template <typename T, int D, bool VARLEN>
-static int launch_mfma_dv(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool causal, float* lse2, float* delta,
-                          hipStream_t stream) {
+static int launch_mfma_dv(const FlashBwdParams& p, const PackedMask* pm, int64_t B, int64_t H_kv, bool causal, float* lse2,
+                          float* delta, hipStream_t stream) {
     // 1. statistics: the forward kernel with its output kept in registers
     FlashParams f{};
     f.q = p.q; f.k = p.k; f.v = p.v; f.o = nullptr;
@@ -385,11 +387,18 @@ static int launch_mfma_dv(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool
     f.cu_seqlens = p.cu_seqlens;
     f.scale_log2 = p.scale_log2;
     f.d_real = p.d_real;
+    FlashBwdParams m = p;
+    if (pm) {
+        f.mask_bits = pm->bits;
+        f.mask_kt = pm->tiles;
+        m.mask_bits = pm->bits;
+        m.mask_bits_t = pm->bits_t;
+        m.mask_tiles = pm->tiles;
+    }
     if (int rc = flash_plan_launch(f, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load(), VARLEN)) return rc;
     const FlashStatsOut st{p.d_out, lse2, delta, p.rows_padded};
     const dim3 block(kFlashThreads);
     const dim3 grid_stats((unsigned)(f.blocks_per_xcd * 8));
-    FlashBwdParams m = p;
     m.n_tiles = (p.N + kFlashRows - 1) / kFlashRows;
     // causal dense launches: a workgroup takes a long and a short tile of its head, so that all do the same work
     m.paired = (causal && !VARLEN && m.n_tiles >= 2 && tuning().bwd_pair.load() != 0) ? 1 : 0;
@@ -399,80 +408,40 @@ static int launch_mfma_dv(const FlashBwdParams& p, int64_t B, int64_t H_kv, bool
     m.total_q = (int32_t)total_q; m.per_xcd_q = (int32_t)((total_q + 7) / 8);
     m.total_kv = (int32_t)total_kv; m.per_xcd_kv = (int32_t)((total_kv + 7) / 8);
     const dim3 grid_q((unsigned)(m.per_xcd_q * 8)), grid_kv((unsigned)(m.per_xcd_kv * 8));
-    if (causal) {
-        hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, true, VARLEN>), grid_stats, block, 0, stream, f, st);
-        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, true, VARLEN>), grid_q, block, 0, stream, m);
-        launch_dkv<T, D, true, VARLEN>(m, grid_kv, block, stream);
-    } else {
-        hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, false, VARLEN>), grid_stats, block, 0, stream, f, st);
-        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, false, VARLEN>), grid_q, block, 0, stream, m);
-        launch_dkv<T, D, false, VARLEN>(m, grid_kv, block, stream);
-    }
-    return static_cast<int>(hipGetLastError());
-}
-
-// The same three steps under a dense mask, on its packed copy (dense launches only).
-template <typename T, int D>
-static int launch_mfma_masked_dv(FlashBwdParams p, const PackedMask& pm, int64_t B, int64_t H_kv, bool causal, float* lse2,
-                                 float* delta, hipStream_t stream) {
-    FlashParams f{};
-    f.q = p.q; f.k = p.k; f.v = p.v; f.o = nullptr;
-    f.stride_b = p.stride_b; f.stride_n = p.stride_n; f.stride_h = p.stride_h;
-    f.kv_stride_b = p.kv_stride_b; f.kv_stride_n = p.kv_stride_n; f.kv_stride_h = p.kv_stride_h;
-    f.N = p.N; f.H = p.H; f.kv_group = p.kv_group;
-    f.scale_log2 = p.scale_log2;
-    f.d_real = p.d_real;
-    f.mask_bits = pm.bits;
-    f.mask_kt = pm.tiles;
-    if (int rc = flash_plan_launch(f, B, causal, kFlashRows, tuning().flash_pair_min_tiles.load(), false)) return rc;
-    const FlashStatsOut st{p.d_out, lse2, delta, p.rows_padded};
-    const dim3 block(kFlashThreads);
-    const dim3 grid_stats((unsigned)(f.blocks_per_xcd * 8));
-    FlashBwdParams m = p;
-    m.mask_bits = pm.bits;
-    m.mask_bits_t = pm.bits_t;
-    m.mask_tiles = pm.tiles;
-    m.n_tiles = (p.N + kFlashRows - 1) / kFlashRows;
-    m.paired = (causal && m.n_tiles >= 2 && tuning().bwd_pair.load() != 0) ? 1 : 0;
-    const int64_t units = bwd_units(m);
-    const int64_t total_q = B * p.H * units, total_kv = B * H_kv * units;
-    if (total_q > 0x7FFFFFF0ll) return AHPC_ERR_BAD_SHAPE;
-    m.total_q = (int32_t)total_q; m.per_xcd_q = (int32_t)((total_q + 7) / 8);
-    m.total_kv = (int32_t)total_kv; m.per_xcd_kv = (int32_t)((total_kv + 7) / 8);
-    const dim3 grid_q((unsigned)(m.per_xcd_q * 8)), grid_kv((unsigned)(m.per_xcd_kv * 8));
-    const int64_t choice = tuning().bwd_split.load();
-    const bool split = choice == 0 ? D == 128 : choice == 2;
-    if (causal) {
-        hipLaunchKernelGGL((flash_bwd_stats_masked_mfma_kernel<T, D, true>), grid_stats, block, 0, stream, f, st);
-        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, true, false, true>), grid_q, block, 0, stream, m);
-        if (split) {
-            hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, true, false, 1, true>), grid_kv, block, 0, stream, m);
-            hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, true, false, 2, true>), grid_kv, block, 0, stream, m);
+    auto launch = [&](auto causal_c, auto masked_c) {
+        constexpr bool C = decltype(causal_c)::value, M = decltype(masked_c)::value;
+        if constexpr (M && VARLEN) {
+            return;  // (a mask belongs to dense launches: never asked for)
         } else {
-            hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, true, false, 0, true>), grid_kv, block, 0, stream, m);
+            if constexpr (M) hipLaunchKernelGGL((flash_bwd_stats_masked_mfma_kernel<T, D, C>), grid_stats, block, 0, stream, f, st);
+            else hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, C, VARLEN>), grid_stats, block, 0, stream, f, st);
+            hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, C, VARLEN, M>), grid_q, block, 0, stream, m);
+            launch_dkv<T, D, C, VARLEN, M>(m, grid_kv, block, stream);
         }
+    };
+    if (pm && VARLEN) return AHPC_ERR_BAD_SHAPE;
+    if (causal) {
+        if (pm) launch(std::true_type{}, std::true_type{});
+        else launch(std::true_type{}, std::false_type{});
     } else {
-        hipLaunchKernelGGL((flash_bwd_stats_masked_mfma_kernel<T, D, false>), grid_stats, block, 0, stream, f, st);
-        hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, false, false, true>), grid_q, block, 0, stream, m);
-        if (split) {
-            hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, false, false, 1, true>), grid_kv, block, 0, stream, m);
-            hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, false, false, 2, true>), grid_kv, block, 0, stream, m);
-        } else {
-            hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, false, false, 0, true>), grid_kv, block, 0, stream, m);
-        }
+        if (pm) launch(std::false_type{}, std::true_type{});
+        else launch(std::false_type{}, std::false_type{});
     }
     return static_cast<int>(hipGetLastError());
 }
 
 template <typename T>
-static int launch_mfma(const FlashBwdParams& p, int64_t B, int64_t H_kv, int d, bool causal, float* lse2, float* delta,
-                       hipStream_t stream) {
+static int launch_mfma(const FlashBwdParams& p, const PackedMask* pm, int64_t B, int64_t H_kv, int d, bool causal, float* lse2,
+                       float* delta, hipStream_t stream) {
     if (p.cu_seqlens) {
-        if (d == 128) return launch_mfma_dv<T, 128, true>(p, B, H_kv, causal, lse2, delta, stream);
-        if (d == 64) return launch_mfma_dv<T, 64, true>(p, B, H_kv, causal, lse2, delta, stream);
+        if (pm) return AHPC_ERR_BAD_SHAPE;
+        if (d == 128) return launch_mfma_dv<T, 128, true>(p, nullptr, B, H_kv, causal, lse2, delta, stream);
+        if (d == 64) return launch_mfma_dv<T, 64, true>(p, nullptr, B, H_kv, causal, lse2, delta, stream);
+        if (d == 256) return launch_mfma_dv<T, 256, true>(p, nullptr, B, H_kv, causal, lse2, delta, stream);
     } else {
-        if (d == 128) return launch_mfma_dv<T, 128, false>(p, B, H_kv, causal, lse2, delta, stream);
-        if (d == 64) return launch_mfma_dv<T, 64, false>(p, B, H_kv, causal, lse2, delta, stream);
+        if (d == 128) return launch_mfma_dv<T, 128, false>(p, pm, B, H_kv, causal, lse2, delta, stream);
+        if (d == 64) return launch_mfma_dv<T, 64, false>(p, pm, B, H_kv, causal, lse2, delta, stream);
+        if (d == 256) return launch_mfma_dv<T, 256, false>(p, pm, B, H_kv, causal, lse2, delta, stream);
     }
     return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
 }
@@ -582,35 +551,13 @@ static int flash_bwd_any(const void* d_out, const void* q, const void* k, const 
     const bool strides4_ok = !(stride_b % 4) && !(stride_n % 4) && !(stride_h % 4) && !(kv_stride_b % 4) && !(kv_stride_n % 4) &&
                              !(kv_stride_h % 4) && stride_n < (int64_t(1) << 24) && kv_stride_n < (int64_t(1) << 24);
     const bool is16 = dtype == AHPC_F16 || dtype == AHPC_BF16;
-    // head dimensions up to 128 in whole 16-byte pieces; one below 64 or 128 runs on the next kernel (FlashParams::d_real)
-    const bool d_ok = d <= 128 && d >= (is16 ? 8 : 4) && d % (is16 ? 8 : 4) == 0;
-    const int kernel_d = d <= 64 ? 64 : 128;
+    // head dimensions up to 256 (fp32: 128) in whole 16-byte pieces; one below 64, 128 or 256 runs on the next kernel
+    // (FlashParams::d_real)
+    const bool d_ok = d <= (is16 ? 256 : 128) && d >= (is16 ? 8 : 4) && d % (is16 ? 8 : 4) == 0;
+    const int kernel_d = d <= 64 ? 64 : d <= 128 ? 128 : 256;
     const bool tensors_ok = d_ok && (is16 ? strides_ok : strides4_ok) && aligned16(q) && aligned16(k) && aligned16(v) &&
                             aligned16(d_out) && aligned16(d_q) && aligned16(d_k) && aligned16(d_v);
-    if (mask && is16 && tensors_ok && !cu_seqlens && tuning().mask_pack.load() != 0) {
-        // a dense mask on 16-bit tensors: the matrix-core kernels on the mask's packed copy (both layouts), where that
-        // can be made (not under graph capture, not beyond the library's buffer limit)
-        FlashBwdParams m{};
-        m.q = q; m.k = k; m.v = v; m.d_out = d_out;
-        m.d_q = d_q; m.d_k = d_k; m.d_v = d_v;
-        m.neg_lse2 = p.lse; m.neg_delta = p.delta; m.rows_padded = p.rows_padded;
-        m.stride_b = stride_b; m.stride_n = stride_n; m.stride_h = stride_h;
-        m.kv_stride_b = kv_stride_b; m.kv_stride_n = kv_stride_n; m.kv_stride_h = kv_stride_h;
-        m.N = (int32_t)N; m.H = (int32_t)H; m.kv_group = p.kv_group;
-        m.scale = scale;
-        m.scale_log2 = scale * kLog2e;
-        m.d_real = (int32_t)d;
-        bool launched = false;
-        const int rc = with_packed_mask(mask, B, N, true, st, &launched, [&](const PackedMask& pm) {
-            if (dtype == AHPC_F16)
-                return kernel_d == 64 ? launch_mfma_masked_dv<f16_t, 64>(m, pm, B, H_kv, causal != 0, p.lse, p.delta, st)
-                                      : launch_mfma_masked_dv<f16_t, 128>(m, pm, B, H_kv, causal != 0, p.lse, p.delta, st);
-            return kernel_d == 64 ? launch_mfma_masked_dv<bf16_t, 64>(m, pm, B, H_kv, causal != 0, p.lse, p.delta, st)
-                                  : launch_mfma_masked_dv<bf16_t, 128>(m, pm, B, H_kv, causal != 0, p.lse, p.delta, st);
-        });
-        if (launched || rc != AHPC_OK) return rc;
-    }
-    if (!mask && tensors_ok) {
+    if (tensors_ok && (!mask || (is16 && !cu_seqlens && tuning().mask_pack.load() != 0))) {
         FlashBwdParams m{};
         m.q = q; m.k = k; m.v = v; m.d_out = d_out;
         m.d_q = d_q; m.d_k = d_k; m.d_v = d_v;
@@ -622,9 +569,19 @@ static int flash_bwd_any(const void* d_out, const void* q, const void* k, const 
         m.scale = scale;
         m.scale_log2 = scale * kLog2e;
         m.d_real = (int32_t)d;
-        if (dtype == AHPC_F32) return launch_f32_mfma(m, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st);
-        return dtype == AHPC_F16 ? launch_mfma<f16_t>(m, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st)
-                                 : launch_mfma<bf16_t>(m, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st);
+        if (!mask) {
+            if (dtype == AHPC_F32) return launch_f32_mfma(m, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st);
+            return dtype == AHPC_F16 ? launch_mfma<f16_t>(m, nullptr, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st)
+                                     : launch_mfma<bf16_t>(m, nullptr, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st);
+        }
+        // a dense mask on 16-bit tensors: the matrix-core kernels on the mask's packed copy (both layouts), where that
+        // can be made (not under graph capture, not beyond the library's buffer limit)
+        bool launched = false;
+        const int rc = with_packed_mask(mask, B, N, true, st, &launched, [&](const PackedMask& pm) {
+            return dtype == AHPC_F16 ? launch_mfma<f16_t>(m, &pm, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st)
+                                     : launch_mfma<bf16_t>(m, &pm, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st);
+        });
+        if (launched || rc != AHPC_OK) return rc;
     }
     switch (dtype) {
         case AHPC_F32: return launch_simple<float>(p, B, H_kv, st);

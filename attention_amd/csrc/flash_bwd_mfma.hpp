@@ -129,7 +129,7 @@ __device__ inline void store_row(T* dst_row, const f32x16 (&acc)[MB], int half, 
 // MASKED: a dense mask removes keys per query; the lane's word of the packed mask (its query's 64 keys of the tile) is
 // loaded in front of the tile requests and tested bit by bit next to the causal / end-of-sequence test.
 template <typename T, int D, bool CAUSAL, bool VARLEN, bool MASKED = false>
-__global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(const FlashBwdParams p) {
+__global__ __launch_bounds__(kFlashThreads, (D > 128 ? 1 : 2)) void flash_bwd_dq_mfma_kernel(const FlashBwdParams p) {
     static_assert(!(MASKED && VARLEN), "the mask belongs to dense launches");
     typedef FlashTile<D> TL;
     constexpr int KS = D / 16;
@@ -349,7 +349,7 @@ __global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_dq_mfma_kernel(con
 // other's softmax arithmetic and LDS waits; at d = 128 they are the faster way (the launcher picks).
 // MASKED: as in the dQ kernel, with the transposed packed mask (the lane's key, 64 queries per word).
 template <typename T, int D, bool CAUSAL, bool VARLEN, int PART, bool MASKED = false>
-__global__ __launch_bounds__(kFlashThreads, (PART == 0 ? 1 : 2)) void flash_bwd_dkv_mfma_kernel(const FlashBwdParams p) {
+__global__ __launch_bounds__(kFlashThreads, (PART == 0 || D > 128 ? 1 : 2)) void flash_bwd_dkv_mfma_kernel(const FlashBwdParams p) {
     static_assert(!(MASKED && VARLEN), "the mask belongs to dense launches");
     constexpr bool kDoK = PART != 1, kDoV = PART != 2;
     typedef FlashTile<D> TL;

@@ -185,7 +185,7 @@ template <int D> struct FlashTile {
     // and the 4 rows of a transposing read get chunk quads that do not overlap
     __device__ static int fb(int row) {
         const int b0 = row & 1, b1 = (row >> 1) & 1, b2 = (row >> 2) & 1, b3 = (row >> 3) & 1;
-        return D == 128 ? (((b1 ^ b3) << 3) | (b0 << 2) | (b2 << 1) | b1) : (((b1 ^ b0) << 2) | (b2 << 1) | (b3 ^ b0));
+        return D >= 128 ? (((b1 ^ b3) << 3) | (b0 << 2) | (b2 << 1) | b1) : (((b1 ^ b0) << 2) | (b2 << 1) | (b3 ^ b0));
     }
 };
 
@@ -702,13 +702,13 @@ __global__ __launch_bounds__(kFlashThreads, D == 256 ? 1 : 2) void flash_fwd_mfm
 
 // The forward pass with its output kept in registers: writes the softmax statistics the backward needs.
 template <typename T, int D, bool CAUSAL, bool VARLEN>
-__global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_stats_mfma_kernel(const FlashParams p, const FlashStatsOut st) {
+__global__ __launch_bounds__(kFlashThreads, D == 256 ? 1 : 2) void flash_bwd_stats_mfma_kernel(const FlashParams p, const FlashStatsOut st) {
     flash_fwd_mfma_body<T, D, CAUSAL, VARLEN, true>(p, st);
 }
 // The same under a dense mask (its packed copy).  A query that sees no key gets -lse2 = -inf and -delta = 0, like a row
 // beyond the sequence: every weight of it is exp2(s - inf) = 0 in the backward kernels.
 template <typename T, int D, bool CAUSAL>
-__global__ __launch_bounds__(kFlashThreads, 2) void flash_bwd_stats_masked_mfma_kernel(const FlashParams p, const FlashStatsOut st) {
+__global__ __launch_bounds__(kFlashThreads, D == 256 ? 1 : 2) void flash_bwd_stats_masked_mfma_kernel(const FlashParams p, const FlashStatsOut st) {
     flash_fwd_mfma_body<T, D, CAUSAL, false, true, 2>(p, st);
 }
 

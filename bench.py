@@ -413,6 +413,18 @@ def bench_extras(hip, stream, steps, warmup):
                               gv.data_ptr(), hip.BF16, B, N, H, H, d, st, st, sc, True, wsf.data_ptr(), wsb, stream),
         flops=2.5 * 2.0 * B * H * N * N * d)
 
+    # backward with head dimension 256 (half the heads, the same tensor sizes): one workgroup per CU, dK and dV in two walks
+    qw, kw, vw, gow = (randn((B, N, 16, 256), torch.bfloat16) for _ in range(4))
+    gqw, gkw, gvw = torch.empty_like(qw), torch.empty_like(kw), torch.empty_like(vw)
+    stw = (N * 16 * 256, 16 * 256, 256)
+    wsw = torch.empty(hip.flash_bwd_workspace_bytes(B, N, 16) // 4, dtype=torch.float32, device="cuda")
+    run("flash_bwd bf16 causal B=4 N=4096 H=16 d=256",
+        lambda: hip.flash_bwd(gow.data_ptr(), qw.data_ptr(), kw.data_ptr(), vw.data_ptr(), gqw.data_ptr(), gkw.data_ptr(),
+                              gvw.data_ptr(), hip.BF16, B, N, 16, 16, 256, stw, stw, 1.0 / 16.0, True, wsw.data_ptr(),
+                              wsw.numel() * 4, stream),
+        flops=2.5 * 2.0 * B * 16 * N * N * 256)
+    del qw, kw, vw, gow, gqw, gkw, gvw, wsw
+
     # the same backward in fp32 (fp32 matrix-core kernels; dK and dV always in two walks)
     qf, kf, vf, gof = (randn((B, N, H, d), torch.float32) for _ in range(4))
     gqf, gkf, gvf = torch.empty_like(qf), torch.empty_like(kf), torch.empty_like(vf)
@@ -428,6 +440,11 @@ def bench_extras(hip, stream, steps, warmup):
         lambda: hip.flash_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), hip.BF16, B, N, H, d, st, sc, False, stream,
                               dmask.data_ptr()),
         flops=4.0 * B * H * N * N * d)
+    run("flash_bwd bf16 non-causal B=4 N=4096 H=32 d=128 with a dense fp32 mask [B,N,N]",
+        lambda: hip.flash_bwd(go.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), gq.data_ptr(), gk.data_ptr(),
+                              gv.data_ptr(), hip.BF16, B, N, H, H, d, st, st, sc, False, wsf.data_ptr(), wsb, stream,
+                              dmask.data_ptr()),
+        flops=2.5 * 4.0 * B * H * N * N * d)
     del dmask
 
     # ragged fp16 causal batch: 16 sequences, lengths U[128,8192], H=32, d=64 (sigma 0.5)

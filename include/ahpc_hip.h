@@ -209,8 +209,9 @@ int ahpc_hip_flash_block_map(int64_t B, int64_t N, int64_t H, int causal, int64_
  * accumulation throughout; the gradient tensors are fully overwritten, rows that see no key get zeros.
  * workspace: device memory of at least ahpc_hip_flash_bwd_workspace_bytes(B, N, H) bytes, 16-byte aligned,
  * for two floats per (sequence, head, row of a whole 128-row tile); its contents afterwards are unspecified.
- * d <= 128 in whole 16-byte pieces (a multiple of 8 for fp16/bf16, of 4 for fp32) and 16-byte aligned rows run on
- * the matrix cores (fp16/bf16 on 16-bit matrix instructions, fp32 on fp32 ones), everything else on fp32-FMA kernels.
+ * Head dimensions in whole 16-byte pieces (fp16/bf16: a multiple of 8 up to 256; fp32: a multiple of 4 up to 128) with
+ * 16-byte aligned rows run on the matrix cores (fp16/bf16 on 16-bit matrix instructions, fp32 on fp32 ones; kernels exist
+ * for 64, 128 and, 16-bit only, 256, a smaller head dimension runs on the next one), everything else on fp32-FMA kernels.
  * mask: NULL or fp32 [B,N,N] as in the forward.  fp16/bf16 tensors with a mask stay on the matrix cores, on the
  * packed copy of the mask that ahpc_hip_flash_fwd_masked describes (here in two layouts, a quarter of a byte per
  * element; same owner, same limits, same conditions); fp32 tensors with a mask take the fp32-FMA kernels. */

@@ -722,24 +722,27 @@ def test_backward_fp32_kernels_16bit_storage(emu, dtype):
 @pytest.mark.parametrize("dtype", [O.BF16, O.F16])
 @pytest.mark.parametrize("B,N,H,H_kv,d,causal", [
     (1, 64, 1, 1, 128, False), (2, 129, 2, 2, 128, True), (1, 300, 2, 2, 64, True), (1, 200, 2, 1, 64, False),
-    (1, 1, 2, 2, 128, True), (1, 260, 4, 2, 128, True)])
+    (1, 1, 2, 2, 128, True), (1, 260, 4, 2, 128, True), (1, 150, 2, 1, 256, True), (2, 70, 2, 2, 200, False)])
 def test_backward_matrix_core_kernels(emu, tuned, dtype, B, N, H, H_kv, d, causal, dma_late, split):
     tuned("bwd_split", split)   # dK and dV in one walk over the query tiles, or in two (the default at d = 128)
     tuned("bwd_pair", split - 1)  # causal launches: one tile per workgroup (with one walk), a long and a short one (with two)
     q, k, v, do = bwd_inputs(B, N, H, H_kv, d, 34, dtype)
     scale = 1.0 / np.sqrt(d)
     S.configure(dma_late, seed=N + d)
+    S.lds_stats(reset=True)
     try:
         got = backward(emu, q, k, v, do, dtype, B, N, H, H_kv, d, scale, causal, front=dma_late)
     finally:
         S.configure(False, 1)
+    assert S.lds_stats(reset=True)[0] > 0   # the matrix-core kernels ran (the FMA kernels make no traced reads)
     check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv), dtype)
 
 
 @pytest.mark.parametrize("split,dma_late", [(1, False), (2, True)])
 @pytest.mark.parametrize("dtype,B,N,H,H_kv,d,causal", [
     (O.BF16, 2, 64, 2, 2, 128, False), (O.F16, 2, 131, 2, 1, 128, True), (O.F16, 1, 300, 2, 2, 64, False),
-    (O.BF16, 2, 200, 4, 2, 64, True), (O.BF16, 1, 3, 2, 2, 128, False), (O.F16, 2, 65, 2, 2, 32, True)])
+    (O.BF16, 2, 200, 4, 2, 64, True), (O.BF16, 1, 3, 2, 2, 128, False), (O.F16, 2, 65, 2, 2, 32, True),
+    (O.BF16, 1, 140, 2, 1, 256, True), (O.F16, 1, 66, 2, 2, 192, False)])
 def test_backward_matrix_core_kernels_dense_mask(emu, tuned, dtype, B, N, H, H_kv, d, causal, dma_late, split):
     """fp16/bf16 with a mask [B,N,N]: statistics, dQ, dK and dV on the matrix cores, on the packed copy of the mask in
     both of its layouts (keys per query for dQ, queries per key for dK and dV).  A query that sees nothing (no gradient
@@ -818,7 +821,7 @@ def test_backward_smaller_head_dimensions(emu, dtype, d, N, causal, H, H_kv, dma
 
 
 # ---- LDS bank conflicts (model: 64 banks of 4 bytes) --------------------------------------------------------
-@pytest.mark.parametrize("dtype,d", [(O.BF16, 128), (O.F16, 64)])
+@pytest.mark.parametrize("dtype,d", [(O.BF16, 128), (O.F16, 64), (O.BF16, 256)])
 def test_operand_reads_are_free_of_bank_conflicts(emu, dtype, d):
     """Every 16-byte operand read and every transposing read of the matrix-core kernels, forward and backward.
     (The GPU's own conflict counter reads zero for the forward kernel, which is what anchors the model.)"""

@@ -81,9 +81,9 @@ def test_dense_mask(gpu):
 @pytest.mark.parametrize("B,N,H,H_kv,d,causal", [
     (1, 64, 1, 1, 128, False), (2, 129, 2, 2, 128, True), (1, 300, 2, 2, 64, True), (1, 200, 2, 1, 64, False),
     (1, 1, 2, 2, 128, True), (1, 260, 4, 2, 128, True), (2, 1024, 4, 4, 128, True), (1, 517, 3, 3, 64, False),
-    (1, 70, 4, 2, 32, True)])
+    (1, 70, 4, 2, 32, True), (1, 300, 2, 1, 256, True), (2, 517, 2, 2, 200, False), (1, 1024, 4, 4, 256, True)])
 def test_16bit_tensors(gpu, dtype, B, N, H, H_kv, d, causal):
-    # d = 64, 128: matrix-core kernels; d = 32: fp32-FMA kernels with 16-bit storage
+    # matrix-core kernels for 64, 128 and 256 (smaller head dimensions run on the next one)
     q, k, v, do = inputs(B, N, H, H_kv, d, 34, dtype)
     scale = 1.0 / np.sqrt(d)
     got = run_backward(gpu, q, k, v, do, dtype, B, N, H, H_kv, d, scale, causal)
@@ -93,7 +93,7 @@ def test_16bit_tensors(gpu, dtype, B, N, H, H_kv, d, causal):
 @pytest.mark.parametrize("dtype,B,N,H,H_kv,d,causal", [
     (O.BF16, 2, 64, 2, 2, 128, False), (O.F16, 2, 131, 2, 1, 128, True), (O.F16, 1, 300, 2, 2, 64, False),
     (O.BF16, 2, 517, 4, 2, 64, True), (O.BF16, 1, 3, 2, 2, 128, False), (O.F16, 2, 65, 2, 2, 32, True),
-    (O.BF16, 1, 1030, 2, 2, 128, False)])
+    (O.BF16, 1, 1030, 2, 2, 128, False), (O.F16, 1, 300, 2, 1, 256, True), (O.BF16, 2, 130, 2, 2, 192, False)])
 def test_16bit_tensors_dense_mask(gpu, dtype, B, N, H, H_kv, d, causal):
     """fp16/bf16 with a mask [B,N,N]: the matrix-core kernels on the packed copy of the mask.  A query that sees nothing,
     a key that nobody sees, queries that see one key."""
@@ -220,7 +220,7 @@ def test_bad_arguments_are_rejected_without_launch(gpu):
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("dtype,d,H,H_kv", [(O.F16, 64, 4, 4), (O.BF16, 128, 4, 2), (O.F32, 32, 2, 1)])
+@pytest.mark.parametrize("dtype,d,H,H_kv", [(O.F16, 64, 4, 4), (O.BF16, 128, 4, 2), (O.F32, 32, 2, 1), (O.BF16, 256, 2, 1)])
 @pytest.mark.parametrize("causal", [False, True])
 def test_ragged_batch(gpu, dtype, d, H, H_kv, causal):
     """Packed sequences of different lengths: every sequence's gradients equal the dense oracle's on that sequence."""
