@@ -45,7 +45,7 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 # scaled by its reading for a 1 GiB device copy).  The figure is not re-measured by this script: it is read from the
 # committed summary of those runs, together with the kernel it was taken for, and reported as null when that summary
 # is missing or names another kernel.
-PROFILE_FLASH = os.path.join(ROOT, "profiles", "flash_fwd_mfma_bf16_d128_causal_B4_N4096_H32.txt")
+PROFILE_FLASH = os.path.join(ROOT, "profiles", "flash_fwd_wide_bf16_d128_causal_B4_N4096_H32.txt")
 PROFILE_DECODE = os.path.join(ROOT, "profiles", "paged_decode_f16_d128_B64_ctx512-4096.txt")
 
 
@@ -208,13 +208,16 @@ def bench_flash(hip, stream, steps, warmup, cpu):
     value = flops * steps / wall / 1e12
     kern_ms = float(np.mean(per))
     achieved = flops / (kern_ms * 1e-3) / 1e12
-    flash_traffic, flash_traffic_src = traffic_from_profile(PROFILE_FLASH, "flash_fwd_mfma_kernel")
+    # the kernel this shape takes by default (256 query rows per workgroup); the tuning value flash_rows = 128 asks for the other
+    wide = hip.get_tuning("flash_rows") != 128
+    kernel_name = "flash_fwd_wide_kernel" if wide else "flash_fwd_mfma_kernel"
+    flash_traffic, flash_traffic_src = traffic_from_profile(PROFILE_FLASH, kernel_name)
     res = {
         "metric": "FlashAttn fwd TFLOP/s (bf16, N=4096, d=128)", "value": round(value, 2), "unit": "TFLOP/s",
         "ms_per_step": round(wall / steps * 1e3, 4),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": flash_traffic, "traffic_source": flash_traffic_src,
-                     "kernel": "flash_fwd_mfma_kernel<bf16,128,causal>", "kernel_ms_mean": round(kern_ms, 4),
+                     "kernel": kernel_name + "<bf16,128,causal>", "kernel_ms_mean": round(kern_ms, 4),
                      "kernel_ms_median": round(float(np.median(per)), 4), "kernel_ms_min": round(float(np.min(per)), 4), "flop_per_launch": flops},
         "config": {"workload": "flash_fwd bf16 causal B=4 N=4096 H=32 d=128 layout [B,N,H,d], fp32 accumulate, bf16 out"},
     }

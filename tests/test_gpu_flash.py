@@ -322,6 +322,34 @@ def test_256_row_workgroups_grouped_heads_and_more_block_ids_than_workgroups(gpu
         assert np.abs(have - want).max() <= TOL[dtype]
 
 
+def test_256_row_workgroups_one_long_sequence(gpu, flash_rows):
+    """B=1 N=32768 H=8 d=128 bf16 causal (128 query tiles a head, every workgroup walks several): the two forms of the
+    kernel agree bit for bit over the whole output, and sampled rows (first, last, tile edges, random) match the oracle."""
+    import torch
+    from gpu_util import stream_ptr, TOL
+    B, N, H, d = 1, 32768, 8, 128
+    g = torch.Generator(device="cuda").manual_seed(0xA77E0008)
+    q, k, v = (torch.randn((B, N, H, d), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16) for _ in range(3))
+    scale = 1.0 / np.sqrt(d)
+    outs = []
+    for rows in (256, 128):
+        flash_rows(rows)
+        o = torch.full_like(q, float("nan"))
+        gpu.flash_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), O.BF16, B, N, H, d, (N * H * d, H * d, d), scale, True,
+                      stream_ptr())
+        torch.cuda.synchronize()
+        outs.append(o)
+    assert torch.isfinite(outs[0].float()).all()
+    assert torch.equal(outs[0], outs[1])
+    rng = np.random.default_rng(9)
+    rows = np.unique(np.concatenate([rng.integers(0, H * N, 48), [0, 255, 256, N - 1, H * N - 1, 7 * N + 16383]])).astype(np.int64)
+    qh, kh, vh = (t.float().cpu().numpy() for t in (q, k, v))
+    want = O.attention_rows(qh, kh, vh, B, N, H, d, scale, rows, True)
+    got = outs[0].float().cpu().numpy()
+    have = np.stack([got[0, r % N, r // N] for r in rows])
+    assert np.abs(have - want).max() <= TOL[O.BF16]
+
+
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16])
 def test_mfma_closed_forms(gpu, dtype):
     B, N, H, d = 1, 256, 2, 128
