@@ -235,6 +235,7 @@ static int dispatch_mfma_masked(const FlashParams& p, int64_t B, int d, bool cau
 // [(b * n_rb + query block) * N + key] holds the block's 64 queries, bit r set = mask[b][64 * block + r][key] != 0
 // (lane = key collects its own word from the values it loads).
 constexpr int kMaskPackThreads = 256;
+template <bool TRANSPOSED>
 __global__ __launch_bounds__(kMaskPackThreads) void flash_mask_pack_kernel(const float* __restrict__ mask, uint64_t* __restrict__ bits,
                                                                             uint64_t* __restrict__ bits_t, int N, int n_kt, int n_rb,
                                                                             int64_t n_units) {
@@ -253,11 +254,13 @@ __global__ __launch_bounds__(kMaskPackThreads) void flash_mask_pack_kernel(const
         const float m = (row < N && key < N) ? __builtin_nontemporal_load(src + (int64_t)row * N) : 0.0f;  // read once
         const uint64_t word = __builtin_amdgcn_ballot_w64(m != 0.0f);
         if (lane == r) mine = word;
-        mine_t |= (uint64_t)(m != 0.0f) << r;
+        if constexpr (TRANSPOSED) mine_t |= (uint64_t)(m != 0.0f) << r;
     }
     const int row = 64 * rb + lane;
     if (row < N) bits[((int64_t)b * n_kt + kt) * N + row] = mine;
-    if (bits_t && key < N) bits_t[((int64_t)b * n_rb + rb) * N + key] = mine_t;
+    if constexpr (TRANSPOSED) {
+        if (key < N) bits_t[((int64_t)b * n_rb + rb) * N + key] = mine_t;
+    }
 }
 
 // The packed copy of a mask lives in device memory that the library owns: one buffer per device, grown on demand and kept
@@ -318,8 +321,12 @@ int with_packed_mask(const float* mask, int64_t B, int64_t N, bool with_transpos
     pm.bits = static_cast<const uint64_t*>(sc.ptr);
     pm.bits_t = with_transposed ? pm.bits + one / sizeof(uint64_t) : nullptr;
     pm.tiles = (int32_t)n_kt;
-    hipLaunchKernelGGL(flash_mask_pack_kernel, dim3((unsigned)blocks), dim3(kMaskPackThreads), 0, stream, mask,
-                       const_cast<uint64_t*>(pm.bits), const_cast<uint64_t*>(pm.bits_t), (int)N, (int)n_kt, (int)n_rb, n_units);
+    if (with_transposed)
+        hipLaunchKernelGGL(flash_mask_pack_kernel<true>, dim3((unsigned)blocks), dim3(kMaskPackThreads), 0, stream, mask,
+                           const_cast<uint64_t*>(pm.bits), const_cast<uint64_t*>(pm.bits_t), (int)N, (int)n_kt, (int)n_rb, n_units);
+    else
+        hipLaunchKernelGGL(flash_mask_pack_kernel<false>, dim3((unsigned)blocks), dim3(kMaskPackThreads), 0, stream, mask,
+                           const_cast<uint64_t*>(pm.bits), nullptr, (int)N, (int)n_kt, (int)n_rb, n_units);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return static_cast<int>(e);
     *launched = true;
     const int rc = launch_on_bits(pm);
