@@ -256,6 +256,51 @@ CASE(Flash_BackwardCausalGroupedHalf, true) {  // bf16 tensors, causal, 4 query 
                   AttentionError::INVALID_INPUT);
 }
 
+CASE(Flash_BackwardDenseMaskHalfWideHeads, true) {  // fp16 tensors, head dimension 192, dense mask: matrix-core kernels on the packed mask
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    p.sequence_length = 150;
+    p.head_dimension = 192;
+    p.scale_factor = 1.0f / std::sqrt(192.0f);
+    fa.configure(p);
+    const size_t B = p.batch_size, N = p.sequence_length, H = p.num_heads, d = p.head_dimension, n = B * N * H * d;
+    auto q = uniform(n, 14, 1), k = uniform(n, 14, 2), v = uniform(n, 14, 3), go = uniform(n, 14, 7);
+    auto to_f16 = [](std::vector<float>& x) {
+        std::vector<half> y(x.size());
+        for (size_t i = 0; i < x.size(); ++i) {
+            y[i] = half(x[i]);
+            x[i] = static_cast<float>(y[i]);  // the oracle sees the rounded values
+        }
+        return y;
+    };
+    auto hq = to_f16(q), hk = to_f16(k), hv = to_f16(v), hgo = to_f16(go);
+    std::vector<float> mask = uniform(B * N * N, 14, 6, 0.0f, 1.0f);
+    for (float& m : mask) m = m > 0.4f ? 1.0f : 0.0f;
+    for (size_t j = 0; j < N; ++j) mask[(0 * N + 70) * N + j] = 0.0f;  // a query that sees nothing
+    for (size_t i = 0; i < N; ++i) mask[(0 * N + i) * N + 33] = 0.0f;  // a key that nobody sees
+    std::vector<half> gq(n), gk(n), gv(n);
+    const TensorShape s = shape4(B, N, H, d, DataType::FLOAT16);
+    fa.backward(s, hgo.data(), s, hq.data(), s, hk.data(), s, hv.data(), s, gq.data(), s, gk.data(), s, gv.data(), mask.data());
+    std::vector<float> wq(n), wk(n), wv(n);
+    ahpc_oracle_attention_backward(q.data(), k.data(), v.data(), go.data(), wq.data(), wk.data(), wv.data(), B, N, H, H, d,
+                                   p.scale_factor, 0, mask.data(), 4);
+    auto close = [](const std::vector<half>& got, const std::vector<float>& want) {
+        float top = 1.0f, worst = 0.0f;
+        for (float w : want) top = std::max(top, std::fabs(w));
+        for (size_t i = 0; i < want.size(); ++i) worst = std::max(worst, std::fabs(static_cast<float>(got[i]) - want[i]));
+        return worst <= 2e-2f * top;
+    };
+    EXPECT(close(gq, wq) && close(gk, wk) && close(gv, wv));
+    bool dead_query = true, dead_key = true;
+    for (size_t h = 0; h < H; ++h)
+        for (size_t e = 0; e < d; ++e) {
+            dead_query = dead_query && static_cast<float>(gq[((0 * N + 70) * H + h) * d + e]) == 0.0f;
+            dead_key = dead_key && static_cast<float>(gk[((0 * N + 33) * H + h) * d + e]) == 0.0f &&
+                       static_cast<float>(gv[((0 * N + 33) * H + h) * d + e]) == 0.0f;
+        }
+    EXPECT(dead_query && dead_key);
+}
+
 CASE(Flash_BackwardRaggedBatch, true) {  // packed sequences: each one's gradients equal the dense oracle's on it
     FlashAttention fa;
     AttentionParams p = fixture_params();
