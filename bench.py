@@ -150,6 +150,10 @@ def timed_steps(hip, stream, launch, steps, warmup):
     (synchronised on both sides) and an event pair around each launch."""
     import torch
     lib = hip.load()
+    # The workloads' tensors are made on torch's stream and the launches go to a stream of their own, which does not wait
+    # for it: without this, the first launches overlap the kernels that still fill the inputs, and an output tensor that
+    # torch's allocator carved out of a block whose last reader is still pending is written under that reader's feet.
+    torch.cuda.synchronize()
     settle(hip, stream, launch)
     for _ in range(warmup):
         launch()
@@ -625,12 +629,18 @@ def run_sensors(seconds):
     b = torch.randn_like(a)
     src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
     dst = torch.empty_like(src)
+    kz, az = torch.zeros_like(k), torch.zeros_like(a)
     st = (N * H * d, H * d, d)
     work = [
         ("flash_fwd bf16 causal B=4 N=4096 H=32 d=128",
          lambda: hip.flash_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), hip.BF16, B, N, H, d, st, 1.0 / np.sqrt(d), True, None)),
         ("torch.matmul bf16 8192^3", lambda: torch.matmul(a, b)),
         ("1 GiB device copy", lambda: dst.copy_(src)),
+        # The same two matrix workloads on tensors of zeros: the same instructions, far fewer bits that change from one
+        # operand to the next.  What they draw and how they clock shows how much of the N(0,1) figures is the power limit.
+        ("flash_fwd bf16 causal B=4 N=4096 H=32 d=128, K and V all zeros",
+         lambda: hip.flash_fwd(q.data_ptr(), kz.data_ptr(), kz.data_ptr(), o.data_ptr(), hip.BF16, B, N, H, d, st, 1.0 / np.sqrt(d), True, None)),
+        ("torch.matmul bf16 8192^3, both factors all zeros", lambda: torch.matmul(az, az)),
     ]
     print(json.dumps({"workload": "idle", "sensors": read_sensors()}))
     for name, launch in work:
