@@ -359,6 +359,42 @@ static bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr
 
 static int64_t padded_rows(int64_t N) { return (N + kFlashRows - 1) / kFlashRows * kFlashRows; }
 
+// Backward after a forward that kept its row statistics (FlashParams::keep_neg_lse2) and whose output is still there:
+// the statistics pass shrinks to -delta = -dO.O per query row, read from the output tensor.  One row per LPR lanes,
+// 8 elements per lane; writes both arrays the dQ and dK/dV kernels read, padding rows included (-inf, 0).
+constexpr int kDeltaThreads = 256;
+template <typename T, int LPR>
+__global__ __launch_bounds__(kDeltaThreads) void flash_bwd_delta_kernel(const T* __restrict__ d_out, const T* __restrict__ o,
+                                                                         const float* __restrict__ kept, float* __restrict__ neg_lse2,
+                                                                         float* __restrict__ neg_delta, int64_t stride_b,
+                                                                         int64_t stride_n, int64_t stride_h, int N, int H, int d,
+                                                                         int64_t rows_padded, int64_t total_rows) {
+    const int64_t r = (int64_t)blockIdx.x * (kDeltaThreads / LPR) + threadIdx.x / LPR;  // (sequence * H + head) * rows_padded + row
+    const int piece = threadIdx.x % LPR;
+    float part = 0.0f;
+    bool live = false;
+    if (r < total_rows) {
+        const int64_t bh = r / rows_padded;
+        const int row = (int)(r - bh * rows_padded);
+        live = row < N;
+        if (live && 8 * piece < d) {
+            const int64_t b = bh / H, h = bh - b * H;
+            const int64_t off = b * stride_b + (int64_t)row * stride_n + h * stride_h + 8 * piece;
+            const u32x4 a = *reinterpret_cast<const u32x4*>(d_out + off);
+            const u32x4 c = *reinterpret_cast<const u32x4*>(o + off);
+#pragma unroll
+            for (int w = 0; w < 4; ++w) part += lo_f32<T>(a[w]) * lo_f32<T>(c[w]) + hi_f32<T>(a[w]) * hi_f32<T>(c[w]);
+        }
+    }
+    // (every lane of the wavefront takes part in the exchange, rows beyond the end with zeros)
+#pragma unroll
+    for (int step = LPR / 2; step >= 1; step >>= 1) part += __shfl_xor(part, step, kWave);
+    if (piece == 0 && r < total_rows) {
+        neg_lse2[r] = live ? kept[r] : -INFINITY;
+        neg_delta[r] = live ? -part : 0.0f;
+    }
+}
+
 // dK and dV: in one walk over the query tiles where that fits two workgroups on a CU (d = 64), in two walks (dV, then
 // dK) where it does not (d = 128); the tuning value bwd_split (0 = by head dimension, 1 = one walk, 2 = two) overrides.
 // d = 256: always two walks (one walk would need more registers than a wavefront has).
@@ -376,8 +412,8 @@ static void launch_dkv(const FlashBwdParams& m, dim3 grid, dim3 block, hipStream
 
 // Statistics, dQ, dK and dV.  pm: the packed copy of a dense mask (dense launches only), or null.
 template <typename T, int D, bool VARLEN>
-static int launch_mfma_dv(const FlashBwdParams& p, const PackedMask* pm, int64_t B, int64_t H_kv, bool causal, float* lse2,
-                          float* delta, hipStream_t stream) {
+static int launch_mfma_dv(const FlashBwdParams& p, const PackedMask* pm, const void* o_kept, const float* stats_kept, int64_t B,
+                          int64_t H_kv, bool causal, float* lse2, float* delta, hipStream_t stream) {
     // 1. statistics: the forward kernel with its output kept in registers
     FlashParams f{};
     f.q = p.q; f.k = p.k; f.v = p.v; f.o = nullptr;
@@ -413,8 +449,19 @@ static int launch_mfma_dv(const FlashBwdParams& p, const PackedMask* pm, int64_t
         if constexpr (M && VARLEN) {
             return;  // (a mask belongs to dense launches: never asked for)
         } else {
-            if constexpr (M) hipLaunchKernelGGL((flash_bwd_stats_masked_mfma_kernel<T, D, C>), grid_stats, block, 0, stream, f, st);
-            else hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, C, VARLEN>), grid_stats, block, 0, stream, f, st);
+            if (o_kept && stats_kept && !VARLEN) {
+                // the forward kept its row statistics and its output is at hand: no statistics pass
+                constexpr int LPR = D / 8;
+                const int64_t total_rows = B * p.H * p.rows_padded;
+                const int64_t blocks = (total_rows + kDeltaThreads / LPR - 1) / (kDeltaThreads / LPR);
+                hipLaunchKernelGGL((flash_bwd_delta_kernel<T, LPR>), dim3((unsigned)blocks), dim3(kDeltaThreads), 0, stream,
+                                   static_cast<const T*>(p.d_out), static_cast<const T*>(o_kept), stats_kept, lse2, delta,
+                                   p.stride_b, p.stride_n, p.stride_h, (int)p.N, (int)p.H, (int)p.d_real, p.rows_padded, total_rows);
+            } else if constexpr (M) {
+                hipLaunchKernelGGL((flash_bwd_stats_masked_mfma_kernel<T, D, C>), grid_stats, block, 0, stream, f, st);
+            } else {
+                hipLaunchKernelGGL((flash_bwd_stats_mfma_kernel<T, D, C, VARLEN>), grid_stats, block, 0, stream, f, st);
+            }
             hipLaunchKernelGGL((flash_bwd_dq_mfma_kernel<T, D, C, VARLEN, M>), grid_q, block, 0, stream, m);
             launch_dkv<T, D, C, VARLEN, M>(m, grid_kv, block, stream);
         }
@@ -431,17 +478,17 @@ static int launch_mfma_dv(const FlashBwdParams& p, const PackedMask* pm, int64_t
 }
 
 template <typename T>
-static int launch_mfma(const FlashBwdParams& p, const PackedMask* pm, int64_t B, int64_t H_kv, int d, bool causal, float* lse2,
-                       float* delta, hipStream_t stream) {
+static int launch_mfma(const FlashBwdParams& p, const PackedMask* pm, const void* o_kept, const float* stats_kept, int64_t B,
+                       int64_t H_kv, int d, bool causal, float* lse2, float* delta, hipStream_t stream) {
     if (p.cu_seqlens) {
         if (pm) return AHPC_ERR_BAD_SHAPE;
-        if (d == 128) return launch_mfma_dv<T, 128, true>(p, nullptr, B, H_kv, causal, lse2, delta, stream);
-        if (d == 64) return launch_mfma_dv<T, 64, true>(p, nullptr, B, H_kv, causal, lse2, delta, stream);
-        if (d == 256) return launch_mfma_dv<T, 256, true>(p, nullptr, B, H_kv, causal, lse2, delta, stream);
+        if (d == 128) return launch_mfma_dv<T, 128, true>(p, nullptr, nullptr, nullptr, B, H_kv, causal, lse2, delta, stream);
+        if (d == 64) return launch_mfma_dv<T, 64, true>(p, nullptr, nullptr, nullptr, B, H_kv, causal, lse2, delta, stream);
+        if (d == 256) return launch_mfma_dv<T, 256, true>(p, nullptr, nullptr, nullptr, B, H_kv, causal, lse2, delta, stream);
     } else {
-        if (d == 128) return launch_mfma_dv<T, 128, false>(p, pm, B, H_kv, causal, lse2, delta, stream);
-        if (d == 64) return launch_mfma_dv<T, 64, false>(p, pm, B, H_kv, causal, lse2, delta, stream);
-        if (d == 256) return launch_mfma_dv<T, 256, false>(p, pm, B, H_kv, causal, lse2, delta, stream);
+        if (d == 128) return launch_mfma_dv<T, 128, false>(p, pm, o_kept, stats_kept, B, H_kv, causal, lse2, delta, stream);
+        if (d == 64) return launch_mfma_dv<T, 64, false>(p, pm, o_kept, stats_kept, B, H_kv, causal, lse2, delta, stream);
+        if (d == 256) return launch_mfma_dv<T, 256, false>(p, pm, o_kept, stats_kept, B, H_kv, causal, lse2, delta, stream);
     }
     return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
 }
@@ -515,8 +562,9 @@ static int flash_bwd_any(const void* d_out, const void* q, const void* k, const 
                          int dtype, const int32_t* cu_seqlens, int64_t B, int64_t N, int64_t H, int64_t H_kv, int64_t d,
                          int64_t stride_b, int64_t stride_n, int64_t stride_h, int64_t kv_stride_b, int64_t kv_stride_n,
                          int64_t kv_stride_h, float scale, int causal, const float* mask, void* workspace,
-                         size_t workspace_bytes, void* stream) {
+                         size_t workspace_bytes, void* stream, const void* o_kept = nullptr, const float* stats_kept = nullptr) {
     if (!d_out || !q || !k || !v || !d_q || !d_k || !d_v) return AHPC_ERR_NULL_POINTER;
+    if (!o_kept || !stats_kept || !aligned16(o_kept)) o_kept = nullptr, stats_kept = nullptr;  // both or neither
     if (dtype < AHPC_F32 || dtype > AHPC_BF16) return AHPC_ERR_BAD_DTYPE;
     if (B <= 0 || N <= 0 || H <= 0 || d <= 0 || H_kv <= 0) return AHPC_ERR_BAD_SHAPE;
     if (H % H_kv) return AHPC_ERR_BAD_SHAPE;
@@ -571,15 +619,15 @@ static int flash_bwd_any(const void* d_out, const void* q, const void* k, const 
         m.d_real = (int32_t)d;
         if (!mask) {
             if (dtype == AHPC_F32) return launch_f32_mfma(m, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st);
-            return dtype == AHPC_F16 ? launch_mfma<f16_t>(m, nullptr, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st)
-                                     : launch_mfma<bf16_t>(m, nullptr, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st);
+            return dtype == AHPC_F16 ? launch_mfma<f16_t>(m, nullptr, o_kept, stats_kept, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st)
+                                     : launch_mfma<bf16_t>(m, nullptr, o_kept, stats_kept, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st);
         }
         // a dense mask on 16-bit tensors: the matrix-core kernels on the mask's packed copy (both layouts), where that
         // can be made (not under graph capture, not beyond the library's buffer limit)
         bool launched = false;
         const int rc = with_packed_mask(mask, B, N, true, st, &launched, [&](const PackedMask& pm) {
-            return dtype == AHPC_F16 ? launch_mfma<f16_t>(m, &pm, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st)
-                                     : launch_mfma<bf16_t>(m, &pm, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st);
+            return dtype == AHPC_F16 ? launch_mfma<f16_t>(m, &pm, o_kept, stats_kept, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st)
+                                     : launch_mfma<bf16_t>(m, &pm, o_kept, stats_kept, B, H_kv, kernel_d, causal != 0, p.lse, p.delta, st);
         });
         if (launched || rc != AHPC_OK) return rc;
     }
@@ -596,6 +644,21 @@ int ahpc_hip_flash_bwd(const void* d_out, const void* q, const void* k, const vo
                        const float* mask, void* workspace, size_t workspace_bytes, void* stream) {
     return flash_bwd_any(d_out, q, k, v, d_q, d_k, d_v, dtype, nullptr, B, N, H, H_kv, d, stride_b, stride_n, stride_h,
                          kv_stride_b, kv_stride_n, kv_stride_h, scale, causal, mask, workspace, workspace_bytes, stream);
+}
+
+size_t ahpc_hip_flash_row_stats_bytes(int64_t B, int64_t N, int64_t H) {
+    if (B <= 0 || N <= 0 || H <= 0) return 0;
+    return (size_t)B * (size_t)H * (size_t)padded_rows(N) * sizeof(float);
+}
+
+int ahpc_hip_flash_bwd_kept(const void* d_out, const void* q, const void* k, const void* v, const void* o, const float* row_stats,
+                            void* d_q, void* d_k, void* d_v, int dtype, int64_t B, int64_t N, int64_t H, int64_t H_kv, int64_t d,
+                            int64_t stride_b, int64_t stride_n, int64_t stride_h, int64_t kv_stride_b, int64_t kv_stride_n,
+                            int64_t kv_stride_h, float scale, int causal, const float* mask, void* workspace,
+                            size_t workspace_bytes, void* stream) {
+    return flash_bwd_any(d_out, q, k, v, d_q, d_k, d_v, dtype, nullptr, B, N, H, H_kv, d, stride_b, stride_n, stride_h,
+                         kv_stride_b, kv_stride_n, kv_stride_h, scale, causal, mask, workspace, workspace_bytes, stream, o,
+                         row_stats);
 }
 
 int ahpc_hip_flash_bwd_varlen(const void* d_out, const void* q, const void* k, const void* v, void* d_q, void* d_k, void* d_v,

@@ -422,11 +422,14 @@ using namespace ahpc;
 
 extern "C" {
 
-int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N, int64_t H,
+// The dense forward.  row_stats given: the 16-bit matrix-core kernels also write every query row's softmax statistic there
+// (FlashParams::keep_neg_lse2) and *stats_written becomes 1; launches that take other kernels leave it 0.
+static int flash_fwd_dense(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N, int64_t H,
                            int64_t H_kv, int64_t d, int64_t stride_b, int64_t stride_n, int64_t stride_h,
                            int64_t kv_stride_b, int64_t kv_stride_n, int64_t kv_stride_h, float scale, int causal,
-                           const float* mask, void* stream) {
+                           const float* mask, float* row_stats, int* stats_written, void* stream) {
     const Strides sq{stride_b, stride_n, stride_h}, skv{kv_stride_b, kv_stride_n, kv_stride_h};
+    if (stats_written) *stats_written = 0;
     if (int rc = check_dense(q, k, v, o, dtype, B, N, H, H_kv, d, sq, skv)) return rc;
     if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)d);
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -440,9 +443,17 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
         p.N = (int32_t)N; p.H = (int32_t)H; p.kv_group = group;
         p.scale_log2 = scale * kLog2e;
         p.d_real = (int32_t)d;
+        if (row_stats && stats_written) {
+            p.keep_neg_lse2 = row_stats;
+            p.keep_rows = (N + kFlashRows - 1) / kFlashRows * kFlashRows;
+        }
+        auto kept = [&](int rc) {  // (every path below runs a kernel that writes the statistics)
+            if (rc == AHPC_OK && p.keep_neg_lse2) *stats_written = 1;
+            return rc;
+        };
         if (!mask)
-            return dtype == AHPC_F16 ? dispatch_mfma<f16_t, false>(p, B, kernel_head_dim(d), causal != 0, st)
-                                     : dispatch_mfma<bf16_t, false>(p, B, kernel_head_dim(d), causal != 0, st);
+            return kept(dtype == AHPC_F16 ? dispatch_mfma<f16_t, false>(p, B, kernel_head_dim(d), causal != 0, st)
+                                          : dispatch_mfma<bf16_t, false>(p, B, kernel_head_dim(d), causal != 0, st));
         // The mask, by preference, as a packed copy made in front of the launch (every head reads the mask: packed, a
         // sixteenth of the bytes).  Where that is not possible, or switched off, the kernel reads the mask in place,
         // 16 bytes at a time: rows of a multiple of 4 floats and an aligned base; everything else takes the kernel below.
@@ -452,11 +463,11 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
                 return dtype == AHPC_F16 ? dispatch_mfma_masked<f16_t, 2>(pb, B, kernel_head_dim(d), causal != 0, st)
                                          : dispatch_mfma_masked<bf16_t, 2>(pb, B, kernel_head_dim(d), causal != 0, st);
             });
-            if (launched || rc != AHPC_OK) return rc;
+            if (launched || rc != AHPC_OK) return launched ? kept(rc) : rc;
         }
         if (d <= 128 && N % 4 == 0 && aligned16(mask))  // (beyond 128 only the packed mask has a kernel)
-            return dtype == AHPC_F16 ? dispatch_mfma_masked<f16_t, 1>(p, B, kernel_head_dim(d), causal != 0, st)
-                                     : dispatch_mfma_masked<bf16_t, 1>(p, B, kernel_head_dim(d), causal != 0, st);
+            return kept(dtype == AHPC_F16 ? dispatch_mfma_masked<f16_t, 1>(p, B, kernel_head_dim(d), causal != 0, st)
+                                          : dispatch_mfma_masked<bf16_t, 1>(p, B, kernel_head_dim(d), causal != 0, st));
     }
     if (f32_mfma_eligible(dtype, d, q, k, v, o, sq, skv)) {
         FlashParams p{};
@@ -478,6 +489,24 @@ int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o,
     }
     SimpleParams p{q, k, v, o, nullptr, mask, sq.b, sq.n, sq.h, skv.b, skv.n, skv.h, (int32_t)N, (int32_t)H, (int32_t)d, group, scale, causal ? 1 : 0};
     return dispatch_simple<false>(dtype, p, B, st);
+}
+
+int ahpc_hip_flash_fwd_gqa(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N, int64_t H,
+                           int64_t H_kv, int64_t d, int64_t stride_b, int64_t stride_n, int64_t stride_h,
+                           int64_t kv_stride_b, int64_t kv_stride_n, int64_t kv_stride_h, float scale, int causal,
+                           const float* mask, void* stream) {
+    return flash_fwd_dense(q, k, v, o, dtype, B, N, H, H_kv, d, stride_b, stride_n, stride_h, kv_stride_b, kv_stride_n,
+                           kv_stride_h, scale, causal, mask, nullptr, nullptr, stream);
+}
+
+int ahpc_hip_flash_fwd_keep(const void* q, const void* k, const void* v, void* o, int dtype, int64_t B, int64_t N, int64_t H,
+                            int64_t H_kv, int64_t d, int64_t stride_b, int64_t stride_n, int64_t stride_h,
+                            int64_t kv_stride_b, int64_t kv_stride_n, int64_t kv_stride_h, float scale, int causal,
+                            const float* mask, float* row_stats, int* stats_written, void* stream) {
+    if (!row_stats || !stats_written) return AHPC_ERR_NULL_POINTER;
+    if ((reinterpret_cast<uintptr_t>(row_stats) & 3u) != 0) return AHPC_ERR_BAD_ALIGNMENT;
+    return flash_fwd_dense(q, k, v, o, dtype, B, N, H, H_kv, d, stride_b, stride_n, stride_h, kv_stride_b, kv_stride_n,
+                           kv_stride_h, scale, causal, mask, row_stats, stats_written, stream);
 }
 
 int ahpc_hip_flash_block_map(int64_t B, int64_t N, int64_t H, int causal, int64_t capacity, int64_t* n_blocks,

@@ -73,6 +73,11 @@ struct FlashParams {
     int32_t blocks_per_xcd;     // ceil(total_blocks / 8)
     int32_t n_block_ids;        // 8 * blocks_per_xcd: the block ids of the work map (a persistent kernel walks them with a stride)
     float scale_log2;           // scale * log2(e)
+    // Dense launches may keep the softmax statistic of every query row for a later backward: -log2 of the row's sum of
+    // exp2(scale_log2 * q.k) over its visible keys (-inf for a row that sees none), at [(b * H + h) * keep_rows + row].
+    // Null: nothing is kept.
+    float* keep_neg_lse2;
+    int64_t keep_rows;          // rows per (sequence, head) of that array: N rounded up to whole 128-row tiles
 };
 
 constexpr int kFlashThreads = 256;
@@ -659,6 +664,10 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                                           pack2<T>(a[4 * g4 + 2] * inv, a[4 * g4 + 3] * inv)};
                     if (32 * mb + 8 * g4 + 4 * half < d_real) *reinterpret_cast<u32x2*>(dst + 32 * mb + 8 * g4) = w;
                 }
+            if constexpr (!VARLEN) {
+                if (p.keep_neg_lse2 != nullptr && half == 0)
+                    p.keep_neg_lse2[(int64_t)bh * p.keep_rows + qrow] = l > 0.0f ? neg_m[0] - __builtin_log2f(l) : -INFINITY;
+            }
         }
         __syncthreads();  // the next query tile's first DMA reuses the buffers
     }

@@ -102,7 +102,7 @@ __global__ __launch_bounds__(64 * kFlashWideWaves, 1) void flash_fwd_wide_kernel
     const T* gk = nullptr;
     const T* gv = nullptr;
     T* go = nullptr;
-    int q_tile0 = 0, n_tiles = 0, qw = 0, qw_u = 0, qrow = 0;
+    int q_tile0 = 0, n_tiles = 0, qw = 0, qw_u = 0, qrow = 0, cur_bh = 0;
     u32x4 qreg[KS];  // raw Q rows between `request` and the start of the tile, scaled operands afterwards
 
     auto dma_one = [&](const T* g, const int* off, int k0, unsigned char* dst) {
@@ -127,6 +127,7 @@ __global__ __launch_bounds__(64 * kFlashWideWaves, 1) void flash_fwd_wide_kernel
         gk = static_cast<const T*>(p.k) + kv_base;
         gv = static_cast<const T*>(p.v) + kv_base;
         go = static_cast<T*>(p.o) + base;
+        cur_bh = it.bh;
         q_tile0 = it.qt * ROWS;
         int k_end = L;
         if (CAUSAL) k_end = (q_tile0 + ROWS) < L ? (q_tile0 + ROWS) : L;
@@ -317,6 +318,7 @@ __global__ __launch_bounds__(64 * kFlashWideWaves, 1) void flash_fwd_wide_kernel
         // ---- the next query tile's requests leave before this one is written out ----------------------------------
         T* const out = go;
         const int out_row0 = qw;  // first output row of this wavefront
+        const int out_bh = cur_bh;
         Item next;
         const bool more = advance(next);
         if (more) request(next);
@@ -328,6 +330,8 @@ __global__ __launch_bounds__(64 * kFlashWideWaves, 1) void flash_fwd_wide_kernel
         {
             const float l = halves_sum(l_run);
             const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+            if (p.keep_neg_lse2 != nullptr && half == 0 && out_row0 + col < L)  // (FlashParams::keep_neg_lse2)
+                p.keep_neg_lse2[(int64_t)out_bh * p.keep_rows + out_row0 + col] = l > 0.0f ? neg_m[0] - __builtin_log2f(l) : -INFINITY;
             unsigned char* const mine = lds_out + wave_u * (32 * RB);
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)

@@ -72,6 +72,9 @@ SIGNATURES = {
     "ahpc_hip_flash_block_map": (_ci, [_i64, _i64, _i64, _ci, _i64, C.POINTER(_i64), _vp, _vp, _vp]),
     "ahpc_hip_flash_bwd_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "ahpc_hip_flash_bwd": (_ci, [_vp] * 7 + [_ci] + [_i64] * 11 + [_f32, _ci, _vp, _vp, _sz, _vp]),
+    "ahpc_hip_flash_row_stats_bytes": (_sz, [_i64, _i64, _i64]),
+    "ahpc_hip_flash_fwd_keep": (_ci, [_vp, _vp, _vp, _vp, _ci] + [_i64] * 11 + [_f32, _ci, _vp, _vp, C.POINTER(_ci), _vp]),
+    "ahpc_hip_flash_bwd_kept": (_ci, [_vp] * 9 + [_ci] + [_i64] * 11 + [_f32, _ci, _vp, _vp, _sz, _vp]),
     "ahpc_hip_flash_bwd_varlen": (_ci, [_vp] * 7 + [_ci, _vp] + [_i64] * 9 + [_f32, _ci, _vp, _sz, _vp]),
     "ahpc_hip_flash_fwd_masked": (_ci, [_vp, _vp, _vp, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp, _vp]),
     "ahpc_hip_flash_fwd_varlen": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ci, _vp]),
@@ -197,6 +200,28 @@ def flash_bwd(d_out, q, k, v, d_q, d_k, d_v, dtype, B, N, H, H_kv, d, strides, k
     kb, kn, kh = kv_strides
     _check(load().ahpc_hip_flash_bwd(d_out, q, k, v, d_q, d_k, d_v, dtype, B, N, H, H_kv, d, sb, sn, sh, kb, kn, kh, scale,
                                     int(causal), mask, workspace, workspace_bytes, stream), "flash_bwd")
+
+
+def flash_row_stats_bytes(B, N, H):
+    return load().ahpc_hip_flash_row_stats_bytes(B, N, H)
+
+
+def flash_fwd_keep(q, k, v, o, dtype, B, N, H, H_kv, d, strides, kv_strides, scale, causal, row_stats, stream=None, mask=None):
+    """The dense forward that also keeps its row statistics for flash_bwd_kept; returns True when it did."""
+    sb, sn, sh = strides
+    kb, kn, kh = kv_strides
+    written = _ci(0)
+    _check(load().ahpc_hip_flash_fwd_keep(q, k, v, o, dtype, B, N, H, H_kv, d, sb, sn, sh, kb, kn, kh, scale, int(causal), mask,
+                                         row_stats, C.byref(written), stream), "flash_fwd_keep")
+    return bool(written.value)
+
+
+def flash_bwd_kept(d_out, q, k, v, o, row_stats, d_q, d_k, d_v, dtype, B, N, H, H_kv, d, strides, kv_strides, scale, causal,
+                   workspace, workspace_bytes, stream=None, mask=None):
+    sb, sn, sh = strides
+    kb, kn, kh = kv_strides
+    _check(load().ahpc_hip_flash_bwd_kept(d_out, q, k, v, o, row_stats, d_q, d_k, d_v, dtype, B, N, H, H_kv, d, sb, sn, sh, kb, kn,
+                                         kh, scale, int(causal), mask, workspace, workspace_bytes, stream), "flash_bwd_kept")
 
 
 def flash_bwd_varlen(d_out, q, k, v, d_q, d_k, d_v, dtype, cu_seqlens, n_seqs, max_len, H, H_kv, d, stride_t, stride_h,

@@ -420,6 +420,23 @@ def bench_extras(hip, stream, steps, warmup):
                               gv.data_ptr(), hip.BF16, B, N, H, H, d, st, st, sc, True, wsf.data_ptr(), wsb, stream),
         flops=2.5 * 2.0 * B * H * N * N * d)
 
+    # the same backward after a forward that kept its row statistics (ahpc_hip_flash_fwd_keep / _bwd_kept: an extension of
+    # the reference's interface): no statistics launch, eight products instead of ten
+    rs = torch.empty(hip.flash_row_stats_bytes(B, N, H) // 4, dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    kept = hip.flash_fwd_keep(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), hip.BF16, B, N, H, H, d, st, st, sc, True,
+                              rs.data_ptr(), stream)
+    assert hip.load().ahpc_hip_stream_synchronize(stream) == 0 and kept
+    run("flash_bwd bf16 causal B=4 N=4096 H=32 d=128 on the forward's kept row statistics and output",
+        lambda: hip.flash_bwd_kept(go.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), rs.data_ptr(),
+                                   gq.data_ptr(), gk.data_ptr(), gv.data_ptr(), hip.BF16, B, N, H, H, d, st, st, sc, True,
+                                   wsf.data_ptr(), wsb, stream),
+        flops=2.5 * 2.0 * B * H * N * N * d)
+    run("flash_fwd bf16 causal B=4 N=4096 H=32 d=128 keeping its row statistics",
+        lambda: hip.flash_fwd_keep(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), hip.BF16, B, N, H, H, d, st, st, sc, True,
+                                   rs.data_ptr(), stream),
+        flops=2.0 * B * H * N * N * d)
+
     # backward with head dimension 256 (half the heads, the same tensor sizes): one workgroup per CU, dK and dV in two walks
     qw, kw, vw, gow = (randn((B, N, 16, 256), torch.bfloat16) for _ in range(4))
     gqw, gkw, gvw = torch.empty_like(qw), torch.empty_like(kw), torch.empty_like(vw)

@@ -236,6 +236,37 @@ int ahpc_hip_flash_bwd_varlen(const void* d_out, const void* q, const void* k, c
                               float scale, int causal,
                               void* workspace, size_t workspace_bytes, void* stream);
 
+/* Forward and backward as a pair, for callers that run both on the same tensors (training): the forward keeps one float
+ * per query row, the statistic its online softmax ends with (OnlineSoftmaxState::max_val / sum_exp,
+ * src/algorithms/flash_attention.hpp:50-57, as -log2 of the row's sum of exp2(scale * log2(e) * q.k)), and the backward reads
+ * it and the forward's output instead of recomputing both: its statistics launch, two of the backward's ten matrix products,
+ * shrinks to one pass over dO and O.  The reference's backward has no such inputs
+ * (FlashAttention::backward, src/algorithms/flash_attention.cpp:114-174, takes dO, Q, K, V only); the pair is an extension
+ * of that interface.
+ *   ahpc_hip_flash_row_stats_bytes(B, N, H): size of row_stats (4-byte aligned device memory).
+ *   ahpc_hip_flash_fwd_keep: ahpc_hip_flash_fwd_gqa that also fills row_stats.  *stats_written = 1 when the launch did
+ *     (fp16 / bf16 tensors on the matrix-core kernels), 0 when it ran on kernels that keep nothing (fp32, unaligned
+ *     tensors): the backward must then be called without them.
+ *   ahpc_hip_flash_bwd_kept: ahpc_hip_flash_bwd with o (the forward's output, layout and strides of Q) and row_stats, both
+ *     as that forward left them for the same q, k, v, mask, scale and causal flag; anything else computes wrong gradients
+ *     without notice.  o = NULL or row_stats = NULL: exactly ahpc_hip_flash_bwd.  Launches the matrix-core kernels cannot
+ *     take ignore both and recompute. */
+size_t ahpc_hip_flash_row_stats_bytes(int64_t B, int64_t N, int64_t H);
+int ahpc_hip_flash_fwd_keep(const void* q, const void* k, const void* v, void* o, int dtype,
+                            int64_t B, int64_t N, int64_t H, int64_t H_kv, int64_t d,
+                            int64_t stride_b, int64_t stride_n, int64_t stride_h,
+                            int64_t kv_stride_b, int64_t kv_stride_n, int64_t kv_stride_h,
+                            float scale, int causal, const float* mask,
+                            float* row_stats, int* stats_written, void* stream);
+int ahpc_hip_flash_bwd_kept(const void* d_out, const void* q, const void* k, const void* v,
+                            const void* o, const float* row_stats,
+                            void* d_q, void* d_k, void* d_v, int dtype,
+                            int64_t B, int64_t N, int64_t H, int64_t H_kv, int64_t d,
+                            int64_t stride_b, int64_t stride_n, int64_t stride_h,
+                            int64_t kv_stride_b, int64_t kv_stride_n, int64_t kv_stride_h,
+                            float scale, int causal, const float* mask,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- paged KV pool ---------------------------------------------------------------------------
  * Pool layout: K and V are separate slabs  [page][slot 0..P-1][head][d]  (the layout
  * update_kv_cache_kernel writes, src/backends/cuda/cuda_kernels.cu:547-556).

@@ -770,6 +770,96 @@ def test_backward_matrix_core_kernels_dense_mask(emu, tuned, dtype, B, N, H, H_k
     check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv, mask), dtype)
 
 
+def forward_keep_backward_kept(emu, q, k, v, do, dtype, B, N, H, H_kv, d, scale, causal, mask=None, front=False, shift=0.0):
+    """Forward that keeps its row statistics, then the backward that uses them: (output, kept statistics or None, gradients)."""
+    dq_, dk_, dv_, ddo = dev(q, dtype, front), dev(k, dtype, front), dev(v, dtype, front), dev(do, dtype, front)
+    o = S.guarded(S.empty_storage((B, N, H, d), dtype), front)
+    dm = None if mask is None else S.guarded(mask, front)
+    stats = S.guarded(np.full(emu.flash_row_stats_bytes(B, N, H) // 4, np.nan, np.float32), front)
+    st, kst = (N * H * d, H * d, d), (N * H_kv * d, H_kv * d, d)
+    written = emu.flash_fwd_keep(S.ptr(dq_), S.ptr(dk_), S.ptr(dv_), S.ptr(o), dtype, B, N, H, H_kv, d, st, kst, scale, causal,
+                                 S.ptr(stats), None, None if dm is None else S.ptr(dm))
+    gq = S.guarded(S.empty_storage((B, N, H, d), dtype), front)
+    gk = S.guarded(S.empty_storage((B, N, H_kv, d), dtype), front)
+    gv = S.guarded(S.empty_storage((B, N, H_kv, d), dtype), front)
+    ws_bytes = emu.flash_bwd_workspace_bytes(B, N, H)
+    ws = S.guarded(np.full(ws_bytes // 4, np.nan, np.float32), front)
+    if shift:
+        stats += np.float32(shift)
+    emu.flash_bwd_kept(S.ptr(ddo), S.ptr(dq_), S.ptr(dk_), S.ptr(dv_), S.ptr(o) if written else None,
+                       S.ptr(stats) if written else None, S.ptr(gq), S.ptr(gk), S.ptr(gv), dtype, B, N, H, H_kv, d, st, kst, scale,
+                       causal, S.ptr(ws), ws_bytes, None, None if dm is None else S.ptr(dm))
+    rows = (N + 127) // 128 * 128
+    kept = np.array(stats).reshape(B, H, rows)[:, :, :N] if written else None
+    return S.from_storage(o, dtype), kept, tuple(S.from_storage(x, dtype) for x in (gq, gk, gv))
+
+
+def row_statistics(q, k, B, N, H, H_kv, d, scale, causal, mask=None):
+    """-log2 of every query row's sum of exp2(scale * log2(e) * q.k) over its visible keys, in double precision."""
+    g = H // H_kv
+    out = np.empty((B, H, N))
+    for b in range(B):
+        for h in range(H):
+            s = (q[b, :, h].astype(np.float64) @ k[b, :, h // g].astype(np.float64).T) * scale
+            vis = np.ones((N, N), bool)
+            if causal:
+                vis &= np.tril(np.ones((N, N), bool))
+            if mask is not None:
+                vis &= mask[b] != 0
+            with np.errstate(divide="ignore"):
+                m = np.where(vis, s, -np.inf).max(axis=1, keepdims=True)
+                m = np.where(np.isfinite(m), m, 0.0)
+                out[b, h] = -(m[:, 0] + np.log(np.where(vis, np.exp(s - m), 0.0).sum(axis=1))) / np.log(2.0)
+    return out
+
+
+@pytest.mark.parametrize("rows", [128, 256])
+@pytest.mark.parametrize("dtype,B,N,H,H_kv,d,causal,masked", [
+    (O.BF16, 2, 300, 2, 2, 128, True, False), (O.F16, 1, 150, 4, 2, 64, False, False), (O.BF16, 1, 260, 2, 1, 128, False, True),
+    (O.F16, 2, 70, 2, 2, 96, True, True), (O.BF16, 1, 140, 2, 2, 256, True, False)])
+def test_backward_with_the_forward_s_kept_statistics(emu, tuned, rows, dtype, B, N, H, H_kv, d, causal, masked):
+    """The forward keeps -log2 of every row's softmax sum (both forms of the kernel), the backward reads it and the
+    forward's output instead of running its statistics pass: the kept values against a double-precision computation, the
+    gradients against the oracle's, rows that see no key included."""
+    tuned("flash_rows", rows)
+    q, k, v, do = bwd_inputs(B, N, H, H_kv, d, 41, dtype)
+    mask = None
+    if masked:
+        mask = (O.fill_uniform((B, N, N), 41, 6) > 0.4).astype(np.float32)
+        mask[0, N // 2, :] = 0.0
+    scale = 1.0 / np.sqrt(d)
+    S.lds_stats(reset=True)
+    out, kept, got = forward_keep_backward_kept(emu, q, k, v, do, dtype, B, N, H, H_kv, d, scale, causal, mask, front=rows == 256)
+    assert S.lds_stats(reset=True)[0] > 0
+    assert kept is not None
+    want_stats = row_statistics(q, k, B, N, H, H_kv, d, scale, causal, mask)
+    live = np.isfinite(want_stats)
+    assert np.array_equal(np.isfinite(kept), live)
+    assert np.abs(kept[live] - want_stats[live]).max() <= 2e-2   # (scores from 16-bit operands scaled before the product)
+    rep = H // H_kv
+    assert np.abs(out - O.attention(q, np.repeat(k, rep, axis=2), np.repeat(v, rep, axis=2), B, N, H, d, scale, causal, mask=mask)).max() <= TOL[dtype]
+    check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv, mask), dtype)
+
+
+def test_backward_really_reads_the_kept_statistics(emu):
+    """Statistics shifted by one (every weight halved) halve dV: the backward used what it was given, not its own pass."""
+    B, N, H, d = 1, 200, 2, 128
+    q, k, v, do = bwd_inputs(B, N, H, H, d, 43, O.BF16)
+    _, _, good = forward_keep_backward_kept(emu, q, k, v, do, O.BF16, B, N, H, H, d, 0.09, True)
+    _, _, half = forward_keep_backward_kept(emu, q, k, v, do, O.BF16, B, N, H, H, d, 0.09, True, shift=-1.0)
+    assert np.abs(half[2] - 0.5 * good[2]).max() <= 1e-2 * max(1.0, np.abs(good[2]).max())
+
+
+def test_kept_statistics_are_not_written_by_kernels_that_keep_none(emu):
+    """fp32 tensors run on kernels that keep nothing: the forward says so, and the backward without them is the plain one."""
+    B, N, H, d = 1, 40, 2, 64
+    q, k, v, do = bwd_inputs(B, N, H, H, d, 42, O.F32)
+    out, kept, got = forward_keep_backward_kept(emu, q, k, v, do, O.F32, B, N, H, H, d, 0.125, True)
+    assert kept is None
+    assert np.abs(out - O.attention(q, k, v, B, N, H, d, 0.125, True)).max() <= 1e-4
+    check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, 0.125, True, H), O.F32)
+
+
 def test_backward_dense_mask_without_the_packed_copy_takes_the_plain_kernels(emu, tuned):
     tuned("mask_pack", 0)
     B, N, H, d = 1, 70, 2, 64

@@ -151,6 +151,92 @@ def test_16bit_dense_mask_runs_at_matrix_core_speed(gpu):
     assert ms_masked <= 4 * ms_plain
 
 
+def run_kept(hip, q, k, v, do, dtype, B, N, H, H_kv, d, scale, causal, mask=None):
+    """Forward that keeps its row statistics, backward that uses them: (output, statistics were kept, gradients)."""
+    import torch
+    from gpu_util import to_dev, to_host, stream_ptr
+    tq, tk, tv, tdo = (to_dev(x, dtype) for x in (q, k, v, do))
+    to = torch.full_like(tq, float("nan"))
+    gq, gk, gv = torch.full_like(tq, float("nan")), torch.full_like(tk, float("nan")), torch.full_like(tv, float("nan"))
+    tm = None if mask is None else torch.from_numpy(mask).cuda()
+    stats = torch.full((hip.flash_row_stats_bytes(B, N, H) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    ws_bytes = hip.flash_bwd_workspace_bytes(B, N, H)
+    ws = torch.full((ws_bytes // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    st, kst = (N * H * d, H * d, d), (N * H_kv * d, H_kv * d, d)
+    mp = None if tm is None else tm.data_ptr()
+    kept = hip.flash_fwd_keep(tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), to.data_ptr(), dtype, B, N, H, H_kv, d, st, kst, scale,
+                              causal, stats.data_ptr(), stream_ptr(), mp)
+    hip.flash_bwd_kept(tdo.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), to.data_ptr() if kept else None,
+                       stats.data_ptr() if kept else None, gq.data_ptr(), gk.data_ptr(), gv.data_ptr(), dtype, B, N, H, H_kv, d, st,
+                       kst, scale, causal, ws.data_ptr(), ws_bytes, stream_ptr(), mp)
+    torch.cuda.synchronize()
+    return to_host(to), kept, (to_host(gq), to_host(gk), to_host(gv))
+
+
+@pytest.mark.parametrize("dtype,B,N,H,H_kv,d,causal,masked", [
+    (O.BF16, 2, 300, 2, 2, 128, True, False), (O.F16, 1, 150, 4, 2, 64, False, False), (O.BF16, 1, 260, 2, 1, 128, False, True),
+    (O.F16, 2, 70, 2, 2, 96, True, True), (O.BF16, 1, 140, 2, 2, 256, True, False), (O.BF16, 2, 2048, 8, 8, 128, True, False),
+    (O.F16, 1, 2304, 16, 4, 128, False, False), (O.F32, 1, 40, 2, 2, 64, True, False)])
+def test_backward_with_the_forward_s_kept_statistics(gpu, dtype, B, N, H, H_kv, d, causal, masked):
+    """ahpc_hip_flash_fwd_keep + ahpc_hip_flash_bwd_kept: output and gradients against the oracle (the 2048- and 2304-token
+    cases take the 256-row forward); fp32 tensors keep nothing and fall back to the plain backward."""
+    from gpu_util import TOL
+    q, k, v, do = inputs(B, N, H, H_kv, d, 44, dtype)
+    mask = None
+    if masked:
+        mask = (O.fill_uniform((B, N, N), 44, 6) > 0.4).astype(np.float32)
+        mask[0, N // 2, :] = 0.0
+    scale = 1.0 / np.sqrt(d)
+    out, kept, got = run_kept(gpu, q, k, v, do, dtype, B, N, H, H_kv, d, scale, causal, mask)
+    assert kept == (dtype != O.F32)
+    rep = H // H_kv
+    want = O.attention(q, np.repeat(k, rep, axis=2), np.repeat(v, rep, axis=2), B, N, H, d, scale, causal, mask=mask)
+    assert np.abs(out - want).max() <= TOL[dtype]
+    check(got, O.attention_backward(q, k, v, do, B, N, H, d, scale, causal, H_kv, mask), dtype)
+
+
+def test_kept_statistics_headline_shape_timing(gpu):
+    """B=4 N=4096 H=32 d=128 bf16 causal: the backward on kept statistics agrees with the plain one and is faster."""
+    import torch
+    from gpu_util import stream_ptr
+    B, N, H, d = 4, 4096, 32, 128
+    g = torch.Generator(device="cuda").manual_seed(0xA77E000A)
+    tq, tk, tv, tdo = (torch.randn((B, N, H, d), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+                       for _ in range(4))
+    to = torch.empty_like(tq)
+    stats = torch.empty(gpu.flash_row_stats_bytes(B, N, H) // 4, dtype=torch.float32, device="cuda")
+    ws_bytes = gpu.flash_bwd_workspace_bytes(B, N, H)
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device="cuda")
+    st = (N * H * d, H * d, d)
+    scale = 1.0 / np.sqrt(d)
+    assert gpu.flash_fwd_keep(tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), to.data_ptr(), O.BF16, B, N, H, H, d, st, st, scale, True,
+                              stats.data_ptr(), stream_ptr())
+
+    def run(kept):
+        out = tuple(torch.full_like(tq, float("nan")) for _ in range(3))
+        def call():
+            gpu.flash_bwd_kept(tdo.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), to.data_ptr() if kept else None,
+                               stats.data_ptr() if kept else None, *(t.data_ptr() for t in out), O.BF16, B, N, H, H, d, st, st,
+                               scale, True, ws.data_ptr(), ws_bytes, stream_ptr())
+        for _ in range(5):
+            call()
+        torch.cuda.synchronize()
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        for _ in range(10):
+            call()
+        t1.record()
+        torch.cuda.synchronize()
+        return out, t0.elapsed_time(t1) / 10
+
+    plain, ms_plain = run(False)
+    kept, ms_kept = run(True)
+    print(f"backward B=4 N=4096 H=32 d=128 bf16 causal: {ms_plain:.3f} ms recomputing the statistics, {ms_kept:.3f} ms on kept ones")
+    for a, b in zip(plain, kept):
+        assert (a.float() - b.float()).abs().max().item() <= 2e-2 * max(1.0, a.float().abs().max().item())
+    assert ms_kept < ms_plain
+
+
 def test_closed_forms_16bit(gpu):
     B, N, H, d = 1, 256, 2, 128
     q, k, v, do = inputs(B, N, H, H, d, 35, O.BF16)
