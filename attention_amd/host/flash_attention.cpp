@@ -17,6 +17,22 @@ struct FlashAttention::Impl {
     hipsup::Stream stream;
     hipsup::DeviceBuffer dq, dk, dv, dout, dmask, dcu;
     hipsup::DeviceBuffer ddo, gq, gk, gv, ws;  // backward: staged dO, gradients, statistics workspace
+    // What the last forward() left for a backward() on the same tensors (FlashAttentionConfig::keep_forward_statistics):
+    // the row statistics, the device address of its output, and what identifies the call.
+    hipsup::DeviceBuffer row_stats;
+    struct Kept {
+        bool valid = false;
+        const void* q = nullptr;
+        const void* k = nullptr;
+        const void* v = nullptr;
+        const void* mask = nullptr;
+        const void* out_on_device = nullptr;
+        size_t N = 0;
+        DataType type = DataType::FLOAT32;
+        int causal = 0;
+        float scale = 0.0f;
+        bool bhnd = false;
+    } kept;
     std::vector<std::pair<std::string, double>> profile;
 };
 
@@ -42,6 +58,7 @@ void FlashAttention::configure(const AttentionParams& params, const PerformanceC
     if (n < 1) throw AttentionException(AttentionError::BACKEND_NOT_AVAILABLE, "no HIP device");
     current_params_ = params;
     current_perf_config_ = perf_config;
+    impl_->kept.valid = false;
     if (perf_config.enable_profiling) profiling_enabled_ = true;
     impl_->configured = true;
 }
@@ -50,6 +67,7 @@ void FlashAttention::configure_flash_attention(const FlashAttentionConfig& flash
     if (flash_config.apply_dropout && flash_config.dropout_probability > 0.0f)
         throw AttentionException(AttentionError::UNSUPPORTED_OPERATION, "dropout is not supported (forward inference only)");
     impl_->cfg = flash_config;
+    impl_->kept.valid = false;
 }
 
 static size_t kv_heads(const AttentionParams& p) { return p.key_value_heads ? p.key_value_heads : p.num_heads; }
@@ -126,9 +144,24 @@ void FlashAttention::forward(const TensorShape& qs, const void* q, const TensorS
         kb = (int64_t)(N * Hkv * d); kn = (int64_t)(Hkv * d); kh = sh;
     }
     const int dt = hipsup::dtype_code(qs.data_type);
+    impl_->kept.valid = false;
     if (profiling_enabled_) timer.start(st);
-    check(ahpc_hip_flash_fwd_gqa(dq, dk, dv, dout, dt, (int64_t)B, (int64_t)N, (int64_t)H, (int64_t)Hkv, (int64_t)d, sb, sn,
-                                 sh, kb, kn, kh, scale, causal, dmask, st), "flash forward");
+    if (impl_->cfg.keep_forward_statistics) {
+        float* stats = static_cast<float*>(impl_->row_stats.reserve(ahpc_hip_flash_row_stats_bytes((int64_t)B, (int64_t)N, (int64_t)H)));
+        int written = 0;
+        check(ahpc_hip_flash_fwd_keep(dq, dk, dv, dout, dt, (int64_t)B, (int64_t)N, (int64_t)H, (int64_t)Hkv, (int64_t)d, sb, sn,
+                                      sh, kb, kn, kh, scale, causal, dmask, stats, &written, st), "flash forward");
+        if (written) {
+            Impl::Kept& kp = impl_->kept;
+            kp.valid = true;
+            kp.q = q; kp.k = k; kp.v = v; kp.mask = mask;
+            kp.out_on_device = dout;
+            kp.N = N; kp.type = qs.data_type; kp.causal = causal; kp.scale = scale; kp.bhnd = impl_->cfg.tensor_layout_bhnd;
+        }
+    } else {
+        check(ahpc_hip_flash_fwd_gqa(dq, dk, dv, dout, dt, (int64_t)B, (int64_t)N, (int64_t)H, (int64_t)Hkv, (int64_t)d, sb, sn,
+                                     sh, kb, kn, kh, scale, causal, dmask, st), "flash forward");
+    }
     if (profiling_enabled_) timer.stop(st);
     if (!out_on_device) check(ahpc_hip_memcpy_d2h(o, dout, bytes, st), "copy from device");
     impl_->stream.sync();
@@ -165,6 +198,7 @@ void FlashAttention::forward_varlen(const TensorShape& shape, const void* q, con
     if ((size_t)cu_seqlens[n_seqs] != shape.dimensions[0])
         throw AttentionException(AttentionError::INVALID_INPUT, "cu_seqlens must end at total_tokens");
     if (max_len == 0) return;
+    impl_->kept.valid = false;  // (the output staging buffer is about to be reused)
     void* st = impl_->stream.get();
     const size_t Hkv = kv_heads(current_params_);
     const size_t bytes = shape.total_bytes(), kv_bytes = bytes / H * Hkv;
@@ -241,9 +275,16 @@ void FlashAttention::backward(const TensorShape& gos, const void* go, const Tens
         sb = (int64_t)(N * H * d); sn = (int64_t)(H * d); sh = (int64_t)d;
         kb = (int64_t)(N * Hkv * d); kn = (int64_t)(Hkv * d); kh = sh;
     }
+    // the forward's statistics and output, if this is the backward of the last forward()
+    const Impl::Kept& kp = impl_->kept;
+    const bool same = impl_->cfg.keep_forward_statistics && kp.valid && kp.q == q && kp.k == k && kp.v == v && kp.mask == mask &&
+                      kp.N == N && kp.type == qs.data_type && kp.causal == causal && kp.scale == scale &&
+                      kp.bhnd == impl_->cfg.tensor_layout_bhnd;
     if (profiling_enabled_) timer.start(st);
-    check(ahpc_hip_flash_bwd(d_go, d_q, d_k, d_v, d_gq, d_gk, d_gv, hipsup::dtype_code(qs.data_type), (int64_t)B, (int64_t)N,
-                             (int64_t)H, (int64_t)Hkv, (int64_t)d, sb, sn, sh, kb, kn, kh, scale, causal, dmask, ws, ws_bytes, st),
+    check(ahpc_hip_flash_bwd_kept(d_go, d_q, d_k, d_v, same ? kp.out_on_device : nullptr,
+                                  same ? static_cast<const float*>(impl_->row_stats.get()) : nullptr, d_gq, d_gk, d_gv,
+                                  hipsup::dtype_code(qs.data_type), (int64_t)B, (int64_t)N, (int64_t)H, (int64_t)Hkv, (int64_t)d, sb,
+                                  sn, sh, kb, kn, kh, scale, causal, dmask, ws, ws_bytes, st),
           "flash backward");
     if (profiling_enabled_) timer.stop(st);
     if (!gq_dev) check(ahpc_hip_memcpy_d2h(gq, d_gq, bytes, st), "copy from device");

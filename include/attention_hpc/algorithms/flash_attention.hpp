@@ -33,6 +33,12 @@ struct FlashAttentionConfig {
     // Addition: tensors are indexed [B,H,N,d] (as the reference's own test oracle does,
     // tests/test_flash_attention.cpp:46) instead of the declared [B,N,H,d].
     bool tensor_layout_bhnd = false;
+    // Addition, for callers that run forward() and then backward() on the same tensors (training): forward() keeps its
+    // softmax statistic per query row and where its output lives on the device, and a backward() whose query, key, value
+    // and mask pointers, shapes and settings are those of that forward() reads them instead of recomputing both (a fifth
+    // less time).  The caller promises that those tensors' contents, and the output if it was given as a device pointer,
+    // have not changed in between; any other backward() recomputes as usual.
+    bool keep_forward_statistics = false;
 };
 
 // The merge rule shared by key tiles, split contexts and (in principle) devices.

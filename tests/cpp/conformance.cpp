@@ -301,6 +301,48 @@ CASE(Flash_BackwardDenseMaskHalfWideHeads, true) {  // fp16 tensors, head dimens
     EXPECT(dead_query && dead_key);
 }
 
+CASE(Flash_BackwardOnKeptForwardStatistics, true) {  // keep_forward_statistics: backward() of the last forward() skips its statistics pass
+    FlashAttention fa;
+    AttentionParams p = fixture_params();
+    p.sequence_length = 300;
+    p.head_dimension = 128;
+    p.causal_mask = true;
+    p.scale_factor = 1.0f / std::sqrt(128.0f);
+    fa.configure(p);
+    FlashAttentionConfig c;
+    c.keep_forward_statistics = true;
+    fa.configure_flash_attention(c);
+    const size_t B = p.batch_size, N = p.sequence_length, H = p.num_heads, d = p.head_dimension, n = B * N * H * d;
+    auto q = uniform(n, 15, 1), k = uniform(n, 15, 2), v = uniform(n, 15, 3), go = uniform(n, 15, 7);
+    auto to_bf16 = [](std::vector<float>& x) {
+        std::vector<bfloat16> y(x.size());
+        for (size_t i = 0; i < x.size(); ++i) {
+            y[i] = bfloat16(x[i]);
+            x[i] = static_cast<float>(y[i]);
+        }
+        return y;
+    };
+    auto hq = to_bf16(q), hk = to_bf16(k), hv = to_bf16(v), hgo = to_bf16(go);
+    std::vector<bfloat16> out(n), gq(n), gk(n), gv(n), gq2(n), gk2(n), gv2(n);
+    const TensorShape s = shape4(B, N, H, d, DataType::BFLOAT16);
+    fa.forward(s, hq.data(), s, hk.data(), s, hv.data(), s, out.data());
+    fa.backward(s, hgo.data(), s, hq.data(), s, hk.data(), s, hv.data(), s, gq.data(), s, gk.data(), s, gv.data());
+    std::vector<float> wq(n), wk(n), wv(n);
+    ahpc_oracle_attention_backward(q.data(), k.data(), v.data(), go.data(), wq.data(), wk.data(), wv.data(), B, N, H, H, d,
+                                   p.scale_factor, 1, nullptr, 4);
+    auto close = [](const std::vector<bfloat16>& got, const std::vector<float>& want) {
+        float top = 1.0f, worst = 0.0f;
+        for (float w : want) top = std::max(top, std::fabs(w));
+        for (size_t i = 0; i < want.size(); ++i) worst = std::max(worst, std::fabs(static_cast<float>(got[i]) - want[i]));
+        return worst <= 2e-2f * top;
+    };
+    EXPECT(close(gq, wq) && close(gk, wk) && close(gv, wv));
+    // a backward for other tensors (another query pointer) must not use what the forward kept: same values, new address
+    std::vector<bfloat16> hq_copy = hq;
+    fa.backward(s, hgo.data(), s, hq_copy.data(), s, hk.data(), s, hv.data(), s, gq2.data(), s, gk2.data(), s, gv2.data());
+    EXPECT(close(gq2, wq) && close(gk2, wk) && close(gv2, wv));
+}
+
 CASE(Flash_BackwardRaggedBatch, true) {  // packed sequences: each one's gradients equal the dense oracle's on it
     FlashAttention fa;
     AttentionParams p = fixture_params();
