@@ -259,7 +259,7 @@ CASE(Flash_BackwardCausalGroupedHalf, true) {  // bf16 tensors, causal, 4 query 
 CASE(Flash_BackwardDenseMaskHalfWideHeads, true) {  // fp16 tensors, head dimension 192, dense mask: matrix-core kernels on the packed mask
     FlashAttention fa;
     AttentionParams p = fixture_params();
-    p.sequence_length = 150;
+    p.sequence_length = 90;
     p.head_dimension = 192;
     p.scale_factor = 1.0f / std::sqrt(192.0f);
     fa.configure(p);
@@ -304,7 +304,7 @@ CASE(Flash_BackwardDenseMaskHalfWideHeads, true) {  // fp16 tensors, head dimens
 CASE(Flash_BackwardOnKeptForwardStatistics, true) {  // keep_forward_statistics: backward() of the last forward() skips its statistics pass
     FlashAttention fa;
     AttentionParams p = fixture_params();
-    p.sequence_length = 300;
+    p.sequence_length = 160;
     p.head_dimension = 128;
     p.causal_mask = true;
     p.scale_factor = 1.0f / std::sqrt(128.0f);
