@@ -185,6 +185,20 @@ __global__ __launch_bounds__(kFlashThreads, (D > 128 ? 1 : 2)) void flash_bwd_dq
         dma_tile<D>(gk + (int64_t)k0 * skv, nrec, dma_off, dst_k, wave_u);
         dma_tile<D>(gv + (int64_t)k0 * skv, nrec, dma_off, dst_v, wave_u);
     };
+    // The tiles behind the first are requested one per step, in order: their addresses and the bytes that remain behind
+    // them advance by a tile per request instead of being worked out from the tile number (64-bit products) every step.
+    const int64_t tile_elems = (int64_t)kFlashKeys * skv;
+    const T* k_next = nullptr;
+    const T* v_next = nullptr;
+    int64_t rem_next = 0;
+    auto dma_next = [&](unsigned char* dst_k, unsigned char* dst_v) {
+        const unsigned nrec = rem_next <= 0 ? 0u : rem_next > 0xffffffffll ? 0xffffffffu : (unsigned)rem_next;
+        dma_tile<D>(k_next, nrec, dma_off, dst_k, wave_u);
+        dma_tile<D>(v_next, nrec, dma_off, dst_v, wave_u);
+        k_next += tile_elems;
+        v_next += tile_elems;
+        rem_next -= 2 * tile_elems;
+    };
 
     int row_off[KS];
 #pragma unroll
@@ -207,6 +221,9 @@ __global__ __launch_bounds__(kFlashThreads, (D > 128 ? 1 : 2)) void flash_bwd_dq
         if (CAUSAL) k_end = (q_tile0 + kFlashRows) < L ? (q_tile0 + kFlashRows) : L;
         const int n_tiles = (k_end + kFlashKeys - 1) / kFlashKeys;
         dma_both(0, lds_k0, lds_v0);
+        k_next = gk + tile_elems;
+        v_next = gv + tile_elems;
+        rem_next = (int64_t)(L - kFlashKeys - 1) * skv * 2 + 2 * d_real;
 
         const int qw = q_tile0 + wave * 32;
         const int qrow = qw + col;
@@ -324,7 +341,7 @@ __global__ __launch_bounds__(kFlashThreads, (D > 128 ? 1 : 2)) void flash_bwd_dq
                 mw = mword[(int64_t)t * p.N];
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
+            if (more) dma_next(nxt_k, nxt_v);
             compute_tile(cur_k, cur_v, k0, mw);
             if (more) {
                 __builtin_amdgcn_s_waitcnt(0);
@@ -455,6 +472,22 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 || D > 128 ? 1 : 2)) void
                     dma_dword(lse2 + i0, nst, 4 * lane, dst_s);
                     dma_dword(delta + i0, nst, 4 * lane, dst_s + 256);
                 }
+            };
+            // (the tiles behind the first: addresses and remaining bytes advance by a tile per request, as in the dQ kernel)
+            const int64_t tile_elems = (int64_t)kFlashKeys * sn;
+            int64_t off_next = (int64_t)(t_begin + 1) * tile_elems;  // (an element count: Q and dO share it)
+            int64_t rem_next = (int64_t)(L - (t_begin + 1) * kFlashKeys - 1) * sn * 2 + 2 * d_real;
+            auto dma_next = [&](int i0, unsigned char* dst_q, unsigned char* dst_o, unsigned char* dst_s) {
+                const unsigned nrec = rem_next <= 0 ? 0u : rem_next > 0xffffffffll ? 0xffffffffu : (unsigned)rem_next;
+                dma_tile<D>(gq + off_next, nrec, dma_off, dst_q, wave_u);
+                dma_tile<D>(gdo + off_next, nrec, dma_off, dst_o, wave_u);
+                if (wave_u == 0) {
+                    const unsigned nst = rem_next > 0 ? 256u : 0u;
+                    dma_dword(lse2 + i0, nst, 4 * lane, dst_s);
+                    dma_dword(delta + i0, nst, 4 * lane, dst_s + 256);
+                }
+                off_next += tile_elems;
+                rem_next -= 2 * tile_elems;
             };
 
             auto compute_tile = [&](const unsigned char* tile_q, const unsigned char* tile_o, const unsigned char* tile_s, int i0,
@@ -590,7 +623,7 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 || D > 128 ? 1 : 2)) void
                     mw = mword[(int64_t)t * p.N];  // (in front of the tile requests, see the dQ kernel)
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                if (more) dma_both(i0 + kFlashKeys, nxt_q, nxt_o, nxt_s);
+                if (more) dma_next(i0 + kFlashKeys, nxt_q, nxt_o, nxt_s);
                 compute_tile(cur_q, cur_o, cur_s, i0, mw);
                 if (more) {
                     __builtin_amdgcn_s_waitcnt(0);

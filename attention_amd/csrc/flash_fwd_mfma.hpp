@@ -371,6 +371,20 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
         dma_tile<D>(gk + (int64_t)k0 * skv, nrec, dma_off_k, dst_k, wave_u);
         dma_tile<D>(gv + (int64_t)k0 * skv, nrec, dma_off_v, dst_v, wave_u);
     };
+    // The tiles behind the first are requested one per step, in order: their addresses and the bytes that remain behind
+    // them advance by a tile per request instead of being worked out from the tile number (64-bit products) every step.
+    const int64_t tile_elems = (int64_t)kFlashKeys * skv;
+    const T* k_next = nullptr;
+    const T* v_next = nullptr;
+    int64_t rem_next = 0;
+    auto dma_next = [&](unsigned char* dst_k, unsigned char* dst_v) {
+        const unsigned nrec = rem_next <= 0 ? 0u : rem_next > 0xffffffffll ? 0xffffffffu : (unsigned)rem_next;
+        dma_tile<D>(k_next, nrec, dma_off_k, dst_k, wave_u);
+        dma_tile<D>(v_next, nrec, dma_off_v, dst_v, wave_u);
+        k_next += tile_elems;
+        v_next += tile_elems;
+        rem_next -= 2 * tile_elems;
+    };
 
     // ---- LDS operand addresses (byte offsets inside a tile) -------------------------------------
     // K: lane reads row (32*kb + col), logical chunk 2*ks + half
@@ -400,6 +414,9 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
 
         // first tile on its way before anything else
         dma_both(0, lds_k0, lds_v0);
+        k_next = gk + tile_elems;
+        v_next = gv + tile_elems;
+        rem_next = (int64_t)(L - kFlashKeys - 1) * skv * 2 + 2 * d_real;
 
         // ---- Q^T operands, pre-multiplied by c = scale*log2(e), kept for the whole query tile --------
         const int qw = q_tile0 + wave * 32;  // first query row of this wavefront
@@ -589,6 +606,15 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                         vf[g + 1][mb][1] = TrRead<T>::load(tile_v + v_off[mb] + (16 * (g + 1) + 8) * RB);
                     }
                     make_pb(g + 1);
+                    // the order of issue: behind every matrix instruction two operand reads for the next 16 keys and a
+                    // share of their exponentials (left to itself the compiler bunches the matrix instructions)
+                    constexpr int kValuPerMfma = D >= 256 ? 2 : D == 128 ? 4 : 8;
+#pragma unroll
+                    for (int i = 0; i < MB; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // matrix instruction
+                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);             // LDS reads
+                        __builtin_amdgcn_sched_group_barrier(0x402, kValuPerMfma, 0);  // vector arithmetic, exponentials included
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -608,9 +634,9 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                 if constexpr (MASK == 1) load_mask(mk, k0);
                 else mw = mword[(int64_t)t * p.N];
                 __builtin_amdgcn_sched_barrier(0);
-                dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
+                dma_next(nxt_k, nxt_v);
             } else {
-                if (more) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
+                if (more) dma_next(nxt_k, nxt_v);
             }
             // a wavefront whose queries all precede this tile has nothing to add
             if (!(CAUSAL && k0 > qw + 31)) compute_tile(cur_k, cur_v, k0, mk, mw);

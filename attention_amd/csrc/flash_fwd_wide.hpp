@@ -115,6 +115,20 @@ __global__ __launch_bounds__(64 * kFlashWideWaves, 1) void flash_fwd_wide_kernel
         dma_one(gk, dma_off_k, k0, dst_k);
         dma_one(gv, dma_off_v, k0, dst_v);
     };
+    // The tiles from the third on are requested one per step, in order: their addresses and the bytes that remain behind
+    // them advance by a tile per request instead of being worked out from the tile number (64-bit products) every time.
+    const int64_t tile_elems = (int64_t)kFlashKeys * skv;
+    const T* k_next = nullptr;
+    const T* v_next = nullptr;
+    int64_t rem_next = 0;
+    auto dma_next = [&](unsigned char* dst_k, unsigned char* dst_v) {
+        const unsigned nrec = rem_next <= 0 ? 0u : rem_next > 0xffffffffll ? 0xffffffffu : (unsigned)rem_next;
+        dma_tile<D, IPW>(k_next, nrec, dma_off_k, dst_k, wave_u);
+        dma_tile<D, IPW>(v_next, nrec, dma_off_v, dst_v, wave_u);
+        k_next += tile_elems;
+        v_next += tile_elems;
+        rem_next -= 2 * tile_elems;
+    };
     // Everything a query tile needs before its first product: addresses, the first two K/V tiles on their way into the
     // four buffers (all free: every wavefront is behind the barrier of the previous tile's last step), its Q rows on
     // their way into registers.
@@ -134,6 +148,9 @@ __global__ __launch_bounds__(64 * kFlashWideWaves, 1) void flash_fwd_wide_kernel
         n_tiles = (k_end + kFlashKeys - 1) / kFlashKeys;
         dma_both(0, lds_k0, lds_v0);
         dma_both(n_tiles > 1 ? kFlashKeys : L, lds_k1, lds_v1);
+        k_next = gk + 2 * tile_elems;
+        v_next = gv + 2 * tile_elems;
+        rem_next = (int64_t)(L - 2 * kFlashKeys - 1) * skv * 2 + 2 * d_real;
         qw = q_tile0 + wave * 32;
         qw_u = q_tile0 + wave_u * 32;
         qrow = qw + col;
@@ -289,6 +306,14 @@ __global__ __launch_bounds__(64 * kFlashWideWaves, 1) void flash_fwd_wide_kernel
                         vf[g + 1][mb][1] = TrRead<T>::load(tile_v + v_off[mb] + (16 * (g + 1) + 8) * RB);
                     }
                     make_pb(g + 1);
+                    // the order of issue: behind every matrix instruction two operand reads for the next 16 keys and a
+                    // share of their exponentials (left to itself the compiler bunches the matrix instructions)
+#pragma unroll
+                    for (int i = 0; i < MB; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // matrix instruction
+                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // LDS reads
+                        __builtin_amdgcn_sched_group_barrier(0x402, 4, 0);  // vector arithmetic, exponentials included
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -300,7 +325,7 @@ __global__ __launch_bounds__(64 * kFlashWideWaves, 1) void flash_fwd_wide_kernel
         // walk starts); every step ends with a wait and a barrier, the last one too: behind it the buffers are free.
         auto step = [&](unsigned char* cur_k, unsigned char* cur_v, unsigned char* nxt_k, unsigned char* nxt_v, int t) {
             const int k0 = t * kFlashKeys;
-            if (t > 0 && t + 1 < n_tiles) dma_both(k0 + kFlashKeys, nxt_k, nxt_v);
+            if (t > 0 && t + 1 < n_tiles) dma_next(nxt_k, nxt_v);
             // a wavefront whose queries all precede this tile has nothing to add
             if (!(CAUSAL && k0 > qw_u + 31)) compute_tile(cur_k, cur_v, k0);
             __builtin_amdgcn_s_waitcnt(0);
