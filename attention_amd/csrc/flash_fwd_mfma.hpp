@@ -589,6 +589,11 @@ __device__ __forceinline__ void flash_fwd_mfma_body(const FlashParams& p, const 
                     pb[g][w] = pack2<T>(p0, p1);
                     sum += p0 + p1;  // plain adds co-issue with the matrix pipe; v_dot2 does not
                 }
+#if defined(__HIP_DEVICE_COMPILE__)
+                // the additions stay with their group of keys (left alone, the compiler sinks all of them behind the last
+                // matrix instruction, where nothing overlaps them)
+                asm volatile("" : "+v"(sum));
+#endif
             };
             make_pb(0);
             set_priority(true);

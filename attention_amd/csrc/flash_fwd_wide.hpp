@@ -289,6 +289,11 @@ __global__ __launch_bounds__(64 * kFlashWideWaves, 1) void flash_fwd_wide_kernel
                     pb[g][w] = pack2<T>(p0, p1);
                     sum += p0 + p1;
                 }
+#if defined(__HIP_DEVICE_COMPILE__)
+                // the additions stay with their group of keys (left alone, the compiler sinks all of them behind the last
+                // matrix instruction, where nothing overlaps them)
+                asm volatile("" : "+v"(sum));
+#endif
             };
             make_pb(0);
             set_priority(true);
