@@ -105,18 +105,9 @@ __global__ __launch_bounds__(64 * kFlashWideWaves, 1) void flash_fwd_wide_kernel
     int q_tile0 = 0, n_tiles = 0, qw = 0, qw_u = 0, qrow = 0, cur_bh = 0;
     u32x4 qreg[KS];  // raw Q rows between `request` and the start of the tile, scaled operands afterwards
 
-    auto dma_one = [&](const T* g, const int* off, int k0, unsigned char* dst) {
-        // (a tile that starts at or behind the end of the sequence touches no memory and lands as zeros)
-        const int64_t rem = k0 < L ? (int64_t)(L - k0 - 1) * skv * 2 + 2 * d_real : 0;  // the last row ends with its own d
-        const unsigned nrec = rem > 0xffffffffll ? 0xffffffffu : (unsigned)rem;
-        dma_tile<D, IPW>(g + (int64_t)k0 * skv, nrec, off, dst, wave_u);
-    };
-    auto dma_both = [&](int k0, unsigned char* dst_k, unsigned char* dst_v) {
-        dma_one(gk, dma_off_k, k0, dst_k);
-        dma_one(gv, dma_off_v, k0, dst_v);
-    };
-    // The tiles from the third on are requested one per step, in order: their addresses and the bytes that remain behind
-    // them advance by a tile per request instead of being worked out from the tile number (64-bit products) every time.
+    // The K/V tiles of a query tile are requested in order, one per call: the addresses and the bytes that remain behind them
+    // (the descriptor's bound: rows behind the sequence's end read as zeros) advance by a tile per request instead of being
+    // worked out from the tile number (64-bit products) every time.
     const int64_t tile_elems = (int64_t)kFlashKeys * skv;
     const T* k_next = nullptr;
     const T* v_next = nullptr;
@@ -146,11 +137,11 @@ __global__ __launch_bounds__(64 * kFlashWideWaves, 1) void flash_fwd_wide_kernel
         int k_end = L;
         if (CAUSAL) k_end = (q_tile0 + ROWS) < L ? (q_tile0 + ROWS) : L;
         n_tiles = (k_end + kFlashKeys - 1) / kFlashKeys;
-        dma_both(0, lds_k0, lds_v0);
-        dma_both(n_tiles > 1 ? kFlashKeys : L, lds_k1, lds_v1);
-        k_next = gk + 2 * tile_elems;
-        v_next = gv + 2 * tile_elems;
-        rem_next = (int64_t)(L - 2 * kFlashKeys - 1) * skv * 2 + 2 * d_real;
+        k_next = gk;
+        v_next = gv;
+        rem_next = (int64_t)(L - 1) * skv * 2 + 2 * d_real;  // the last row ends with its own d
+        dma_next(lds_k0, lds_v0);
+        dma_next(lds_k1, lds_v1);  // (a tile that starts at or behind the end of the sequence touches no memory and lands as zeros)
         qw = q_tile0 + wave * 32;
         qw_u = q_tile0 + wave_u * 32;
         qrow = qw + col;
