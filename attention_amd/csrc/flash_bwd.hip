@@ -8,7 +8,7 @@
 //                  dQ_i = scale * sum_j dS_ij k_j,
 //   3. dK, dV      a workgroup owns key rows and walks the queries: dV_j = sum_i P_ij dO_i,
 //                  dK_j = scale * sum_i dS_ij q_i  (summed over the query heads of a K/V head);
-//                  on the matrix cores at d = 128 as one walk for dV and one for dK (launch_dkv).
+//                  on the matrix cores, dK and dV in one walk over the query tiles up to d = 128 (launch_dkv).
 // with P_ij = exp(scale q_i.k_j - lse_i).  Nothing is accumulated through atomics, so results do not depend
 // on launch order.  The statistics live in the caller's workspace: two floats per (sequence, head, row).
 #include <hip/hip_runtime.h>
@@ -395,13 +395,16 @@ __global__ __launch_bounds__(kDeltaThreads) void flash_bwd_delta_kernel(const T*
     }
 }
 
-// dK and dV: in one walk over the query tiles where that fits two workgroups on a CU (d = 64), in two walks (dV, then
-// dK) where it does not (d = 128); the tuning value bwd_split (0 = by head dimension, 1 = one walk, 2 = two) overrides.
-// d = 256: always two walks (one walk would need more registers than a wavefront has).
+// dK and dV: in one walk over the query tiles (four matrix products per tile) up to d = 128, in two walks (dV, then dK:
+// five products) at d = 256, where one walk would need more registers than a wavefront has.  At d = 128 the one walk
+// runs at one wavefront per SIMD (324 registers) and takes 5 % more cycles than the two walks at two per SIMD; on
+// N(0,1) inputs, where the board sits at its power limit and the clock follows the energy spent, it is the faster of
+// the two by 4-15 % at every shape timed (fewer products), and it is one launch less.  The tuning value bwd_split
+// (0 = this choice, 1 = one walk, 2 = two) overrides.
 template <typename T, int D, bool CAUSAL, bool VARLEN, bool MASKED>
 static void launch_dkv(const FlashBwdParams& m, dim3 grid, dim3 block, hipStream_t stream) {
     const int64_t choice = tuning().bwd_split.load();
-    const bool split = D == 256 || (choice == 0 ? D == 128 : choice == 2);
+    const bool split = D == 256 || choice == 2;
     if (split) {
         hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, CAUSAL, VARLEN, 1, MASKED>), grid, block, 0, stream, m);
         hipLaunchKernelGGL((flash_bwd_dkv_mfma_kernel<T, D, CAUSAL, VARLEN, 2, MASKED>), grid, block, 0, stream, m);

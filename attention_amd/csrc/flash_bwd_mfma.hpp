@@ -363,7 +363,8 @@ __global__ __launch_bounds__(kFlashThreads, (D > 128 ? 1 : 2)) void flash_bwd_dq
 // PART: 0 = dK and dV in one walk over the query tiles (four products per tile; at d = 128 that is 324 registers, one
 // wavefront per SIMD), 1 = dV only (S and dV: two products, V and dO.V never touched), 2 = dK only (S, dP, dK).  The
 // two partial walks execute five products between them but each fits two wavefronts per SIMD, which hide each
-// other's softmax arithmetic and LDS waits; at d = 128 they are the faster way (the launcher picks).
+// other's softmax arithmetic and LDS waits: 5 % fewer cycles at d = 128, and still the slower way on inputs that hold
+// the board at its power limit, where four products beat five (the launcher picks).
 // MASKED: as in the dQ kernel, with the transposed packed mask (the lane's key, 64 queries per word).
 template <typename T, int D, bool CAUSAL, bool VARLEN, int PART, bool MASKED = false>
 __global__ __launch_bounds__(kFlashThreads, (PART == 0 || D > 128 ? 1 : 2)) void flash_bwd_dkv_mfma_kernel(const FlashBwdParams p) {

@@ -22,8 +22,8 @@ struct Tuning {
     // query head per pool head the lane-per-element kernel stays ahead by 1-2 %.  Groups of 9 to 32 exist on the
     // matrix-core kernels only.  (AHPC_DECODE_MFMA_MIN_GROUP)
     std::atomic<int64_t> decode_matrix_min_group;
-    // backward: dK and dV in one walk over the query tiles (1), in two (2), or by head dimension (0, the default:
-    // two at d = 128).  (AHPC_BWD_SPLIT)
+    // backward: dK and dV in one walk over the query tiles (1), in two (2), or the launcher's choice (0, the default:
+    // one walk up to d = 128, two at d = 256).  (AHPC_BWD_SPLIT)
     std::atomic<int64_t> bwd_split;
     // forward with a dense mask on the matrix-core kernel: 1 (default) = the mask is packed to one bit per element in
     // front of the launch, into device memory the library keeps; 0 = the kernel reads the caller's fp32 mask in place

@@ -409,8 +409,8 @@ def bench_extras(hip, stream, steps, warmup):
     del qf, kf, vf, of
 
     # backward at the headline shape.  FLOP by the usual convention: 2.5 x the forward's (five products
-    # against two); the four launches here execute ten, because the interface passes neither the forward
-    # output nor its softmax statistics and they are recomputed, and dK and dV each recompute the scores.
+    # against two); the three launches here execute nine, because the interface passes neither the forward
+    # output nor its softmax statistics and they are recomputed, and the dK/dV walk recomputes the scores as dQ does.
     go = randn((B, N, H, d), torch.bfloat16)
     gq, gk, gv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     wsb = hip.flash_bwd_workspace_bytes(B, N, H)
@@ -421,7 +421,7 @@ def bench_extras(hip, stream, steps, warmup):
         flops=2.5 * 2.0 * B * H * N * N * d)
 
     # the same backward after a forward that kept its row statistics (ahpc_hip_flash_fwd_keep / _bwd_kept: an extension of
-    # the reference's interface): no statistics launch, eight products instead of ten
+    # the reference's interface): no statistics launch, seven products instead of nine
     rs = torch.empty(hip.flash_row_stats_bytes(B, N, H) // 4, dtype=torch.float32, device="cuda")
     torch.cuda.synchronize()
     kept = hip.flash_fwd_keep(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), hip.BF16, B, N, H, H, d, st, st, sc, True,

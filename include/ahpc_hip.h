@@ -239,7 +239,7 @@ int ahpc_hip_flash_bwd_varlen(const void* d_out, const void* q, const void* k, c
 /* Forward and backward as a pair, for callers that run both on the same tensors (training): the forward keeps one float
  * per query row, the statistic its online softmax ends with (OnlineSoftmaxState::max_val / sum_exp,
  * src/algorithms/flash_attention.hpp:50-57, as -log2 of the row's sum of exp2(scale * log2(e) * q.k)), and the backward reads
- * it and the forward's output instead of recomputing both: its statistics launch, two of the backward's ten matrix products,
+ * it and the forward's output instead of recomputing both: its statistics launch, two of the backward's nine matrix products,
  * shrinks to one pass over dO and O.  The reference's backward has no such inputs
  * (FlashAttention::backward, src/algorithms/flash_attention.cpp:114-174, takes dO, Q, K, V only); the pair is an extension
  * of that interface.

@@ -724,7 +724,7 @@ def test_backward_fp32_kernels_16bit_storage(emu, dtype):
     (1, 64, 1, 1, 128, False), (2, 129, 2, 2, 128, True), (1, 300, 2, 2, 64, True), (1, 200, 2, 1, 64, False),
     (1, 1, 2, 2, 128, True), (1, 260, 4, 2, 128, True), (1, 150, 2, 1, 256, True), (2, 70, 2, 2, 200, False)])
 def test_backward_matrix_core_kernels(emu, tuned, dtype, B, N, H, H_kv, d, causal, dma_late, split):
-    tuned("bwd_split", split)   # dK and dV in one walk over the query tiles, or in two (the default at d = 128)
+    tuned("bwd_split", split)   # dK and dV in one walk over the query tiles (the default up to d = 128), or in two
     tuned("bwd_pair", split - 1)  # causal launches: one tile per workgroup (with one walk), a long and a short one (with two)
     q, k, v, do = bwd_inputs(B, N, H, H_kv, d, 34, dtype)
     scale = 1.0 / np.sqrt(d)
