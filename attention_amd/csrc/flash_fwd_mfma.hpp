@@ -211,11 +211,17 @@ __device__ inline void dma_tile(const void* base, unsigned nrec, const int* off,
 }
 
 // One direct-to-LDS load instruction on its own: lane i's 16 bytes at base + off (bytes; anything not inside
-// [0, nrec) reads as zero) land at lds + 16*i.
-__device__ inline void dma_instr(const void* base, unsigned nrec, int off, unsigned char* lds) {
+// [0, nrec) reads as zero) land at lds + 16*i.  AUX = the instruction's cache policy bits (2: non-temporal).
+template <int AUX = 0> __device__ inline void dma_instr(const void* base, unsigned nrec, int off, unsigned char* lds) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the descriptor type exists only in the device pass
     const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, nrec, 0x00020000);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (AHPC_LDS void*)lds, 16, off, 0, 0, 0);
+#if defined(AHPC_TRACED_LDS_READ_B128)  // the CPU executor: LDS is host memory
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (AHPC_LDS void*)lds, 16, off, 0, 0, AUX);
+#else
+    // (the LDS address is the low half of the generic one; taking it as a number spares the scalar unit the
+    // null test that the pointer conversion carries)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (AHPC_LDS void*)(uintptr_t)(uint32_t)(uintptr_t)lds, 16, off, 0, 0, AUX);
+#endif
 #endif
 }
 

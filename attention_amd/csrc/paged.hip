@@ -273,6 +273,48 @@ template <int N> __device__ __forceinline__ void load_qo_vec(const void* base, i
     }
 }
 
+// The query operands of the matrix-core decode kernels: KS pieces of 8 consecutive elements (piece ks starts at element
+// i0 + ks * step), requested together and converted later.  With the element type tested per piece, every load would be
+// followed by its own wait: KS memory round trips in a row in front of a wavefront's first tile.
+template <int KS> struct QRaw { u32x4 w[KS][2]; };  // 16-bit types use w[ks][0] only
+
+template <int KS> __device__ __forceinline__ void q_request(QRaw<KS>& r, const void* q, int dtype, int64_t i0, int step) {
+    if (dtype == AHPC_F32) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int v = 0; v < 2; ++v) r.w[ks][v] = reinterpret_cast<const u32x4*>(static_cast<const float*>(q) + i0 + ks * step)[v];
+    } else {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) r.w[ks][0] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(q) + i0 + ks * step);
+    }
+}
+
+// The pieces as pairs of T (the pool's 16-bit type), each element multiplied by c.
+template <typename T, int KS> __device__ __forceinline__ void q_convert(const QRaw<KS>& r, int dtype, float c, u32x4 (&out)[KS]) {
+    if (dtype == AHPC_F32) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                // (through named words: the bit cast of a vector's element expression reads element 0 with this compiler)
+                const uint32_t lo = r.w[ks][w >> 1][2 * (w & 1)], hi = r.w[ks][w >> 1][2 * (w & 1) + 1];
+                out[ks][w] = pack2<T>(__builtin_bit_cast(float, lo) * c, __builtin_bit_cast(float, hi) * c);
+            }
+    } else {
+        const bool is_f16 = dtype == AHPC_F16;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t x = r.w[ks][0][w];
+                const float lo = is_f16 ? lo_f32<f16_t>(x) : lo_f32<bf16_t>(x);
+                const float hi = is_f16 ? hi_f32<f16_t>(x) : hi_f32<bf16_t>(x);
+                out[ks][w] = pack2<T>(lo * c, hi * c);
+            }
+    }
+}
+
 template <int N> __device__ __forceinline__ void store_qo_vec(void* base, int dtype, int64_t i, const float (&x)[N]) {
     if (dtype == AHPC_F32) {
         f32x4* dst = reinterpret_cast<f32x4*>(static_cast<float*>(base) + i);
@@ -661,10 +703,33 @@ static int64_t fit_chunk(int64_t chunk, int64_t P) {
 struct DecodePlan { int64_t chunk; int waves; };
 
 static DecodePlan plan_decode(int64_t B, int64_t H_kv, int64_t group, int64_t row_waves, int64_t max_len, int64_t P,
-                              int64_t requested, bool matrix_kernel = false) {
+                              int64_t requested, bool matrix_kernel = false, int wide_max_waves = 0) {
     DecodePlan plan{requested, (int)tuning().decode_waves.load()};
     if (plan.waves < 0 || plan.waves > 8) plan.waves = 0;
     if (plan.chunk <= 0) plan.chunk = tuning().decode_chunk.load();
+    if (wide_max_waves > 0) {
+        // The kernel for groups of 17 to 32 query heads: a workgroup of W wavefronts per (pool head, chunk), two tile
+        // slots of LDS per wavefront (W = 4 fills a CU at d = 128).  Timed with 32 query heads over one pool head, d =
+        // 128: a launch with more workgroups than the CUs hold at once is bound by the stream, and single wavefronts on
+        // the longest chunks win (five to a CU, each at its own point of its chunk, few partials: B = 64 with contexts
+        // U[16384,32768] 0.158 ms at W = 1, 0.169 at 2, 0.190 at 4).  A launch that fits the CUs in one round is bound
+        // by the time of one workgroup, and W wavefronts that share a chunk's tiles out shorten that (B = 8 with the
+        // same contexts: 0.042 ms at 256 tokens and W = 1, 0.030 at 1024 and W = 4; B = 16 with contexts U[512,4096]:
+        // 0.021 -> 0.017 ms).
+        const auto wgs = [&](int64_t chunk) { return B * H_kv * ((max_len + chunk - 1) / chunk); };
+        int waves = wgs(1024) > 512 ? 1 : wgs(1024) > 256 ? 2 : 4;
+        if (waves > wide_max_waves) waves = wide_max_waves;
+        if (plan.chunk > 0) {
+            plan.chunk = fit_chunk(plan.chunk, P);
+            if (!plan.waves) plan.waves = plan.chunk >= 256 ? waves : plan.chunk >= 128 ? (waves < 2 ? waves : 2) : 1;  // two tiles and more per wavefront
+            return plan;
+        }
+        int64_t chunk = 1024;
+        while (waves > 1 && chunk > 256 && wgs(chunk) < 256) chunk /= 2;
+        plan.chunk = fit_chunk(chunk, P);
+        if (!plan.waves) plan.waves = waves;
+        return plan;
+    }
     if (plan.chunk > 0) {
         plan.chunk = fit_chunk(plan.chunk, P);
         if (!plan.waves) plan.waves = 2;
@@ -735,15 +800,30 @@ static int launch_decode_dp(const DecodeParams& base, dim3 grid, dim3 block, hip
     return AHPC_OK;
 }
 
-// Matrix-core kernel for grouped heads: one wavefront per (pool head, chunk, batch entry).
-template <typename T>
-static int launch_decode_mfma(const DecodeParams& p, hipStream_t st) {
-    const dim3 grid((unsigned)p.H_kv, (unsigned)p.n_chunks, (unsigned)p.B), block(64);
-    if (p.d == 128) hipLaunchKernelGGL((paged_decode_mfma_kernel<T, 128>), grid, block, 0, st, p);
-    else if (p.d == 64) hipLaunchKernelGGL((paged_decode_mfma_kernel<T, 64>), grid, block, 0, st, p);
-    else if (p.d == 256) hipLaunchKernelGGL((paged_decode_mfma_kernel<T, 256>), grid, block, 0, st, p);
-    else return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
+// Matrix-core kernel for groups of 17 to 32 query heads: a workgroup of 1, 2 or 4 wavefronts per (pool head, chunk,
+// batch entry); the wavefronts share the chunk's tiles out and merge their results in LDS.
+template <typename T, int D>
+static int launch_decode_mfma_d(const DecodeParams& p, int waves, hipStream_t st) {
+    constexpr int kMaxW = D <= 128 ? 4 : 2;  // a wavefront's two tile slots take 256 * D bytes of LDS
+    int w = waves >= 4 ? 4 : waves >= 2 ? 2 : 1;
+    if (w > kMaxW) w = kMaxW;
+    const dim3 grid((unsigned)p.H_kv, (unsigned)p.n_chunks, (unsigned)p.B), block(64 * w);
+    if (w == 4) {
+        if constexpr (kMaxW >= 4) hipLaunchKernelGGL((paged_decode_mfma_kernel<T, D, 4>), grid, block, 0, st, p);
+    } else if (w == 2) {
+        hipLaunchKernelGGL((paged_decode_mfma_kernel<T, D, 2>), grid, block, 0, st, p);
+    } else {
+        hipLaunchKernelGGL((paged_decode_mfma_kernel<T, D, 1>), grid, block, 0, st, p);
+    }
     return static_cast<int>(hipGetLastError());
+}
+
+template <typename T>
+static int launch_decode_mfma(const DecodeParams& p, int waves, hipStream_t st) {
+    if (p.d == 128) return launch_decode_mfma_d<T, 128>(p, waves, st);
+    if (p.d == 64) return launch_decode_mfma_d<T, 64>(p, waves, st);
+    if (p.d == 256) return launch_decode_mfma_d<T, 256>(p, waves, st);
+    return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
 }
 
 // Matrix-core kernel for groups of up to 16 query heads: a wavefront per (pool head, chunk, batch entry), up to 8
@@ -970,7 +1050,8 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     const int hpw = 64 / lph;
     const int64_t matrix_from = tuning().decode_matrix_min_group.load();
     const bool use_mfma = mfma_shape && (group > 8 || group >= matrix_from);
-    const DecodePlan plan = plan_decode(B, H_kv, group < 8 ? group : 8, (H_kv + hpw - 1) / hpw, max_len, P, chunk_tokens, use_mfma);
+    const DecodePlan plan = plan_decode(B, H_kv, group < 8 ? group : 8, (H_kv + hpw - 1) / hpw, max_len, P, chunk_tokens, use_mfma,
+                                        use_mfma && group > 16 ? (d <= 128 ? 4 : 2) : 0);
     const int64_t chunk = plan.chunk;
     const int waves = plan.waves;
     const int64_t n_chunks = (max_len + chunk - 1) / chunk;
@@ -1006,7 +1087,7 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     if (use_mfma && group <= 16) {
         rc = pool_dtype == AHPC_F16 ? launch_decode_group<f16_t>(p, st) : launch_decode_group<bf16_t>(p, st);
     } else if (use_mfma) {
-        rc = pool_dtype == AHPC_F16 ? launch_decode_mfma<f16_t>(p, st) : launch_decode_mfma<bf16_t>(p, st);
+        rc = pool_dtype == AHPC_F16 ? launch_decode_mfma<f16_t>(p, waves, st) : launch_decode_mfma<bf16_t>(p, waves, st);
     } else
     switch (pool_dtype) {
         case AHPC_F32: rc = launch_decode_d<float>(p, grid, block, st); break;

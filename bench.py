@@ -514,6 +514,9 @@ def bench_extras(hip, stream, steps, warmup):
     # multi-query decode (32 query heads over one pool head): the matrix-core kernel
     decode_case("paged_decode (matrix-core kernel) fp16 B=64 H=32 over 1 pool head d=128 page=16 context U[512,4096]",
                 dict(DECODE), 32, 1, hip.F16, torch.float16)
+    # the same with long contexts: 814 MB instead of 82 MB, enough for the stream to set the time
+    decode_case("paged_decode (matrix-core kernel) fp16 B=64 H=32 over 1 pool head d=128 page=16 context U[16384,32768]",
+                dict(DECODE, lo=16384, hi=32768), 32, 1, hip.F16, torch.float16)
 
     # prefill -> cache hand-off: K and V of the headline prefill into the pool, one launch
     P = 16

@@ -460,6 +460,28 @@ def test_decode_grouped_heads(emu, tuned, G, matrix_from):
         assert np.abs(got - want).max() <= 2e-2
 
 
+@pytest.mark.parametrize("G,H_kv,d,dtype", [(32, 1, 128, O.F16), (24, 2, 64, O.BF16), (17, 1, 128, O.BF16)])
+@pytest.mark.parametrize("waves", [1, 2, 4])
+def test_decode_wide_groups(emu, tuned, G, H_kv, d, dtype, waves):
+    # groups of 17 to 32 query heads run on the matrix-core kernel with tiles of 32 tokens (two pages, one descriptor
+    # pair per page): sequences that end inside a page, inside a tile's first page and on a tile's border, one chunk
+    # and several; workgroups of 1, 2 and 4 wavefronts that share a chunk's tiles out (with fewer tiles than
+    # wavefronts, and with none at all) and merge in LDS
+    tuned("decode_waves", waves)
+    B, P = 4, 16
+    H = G * H_kv
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [70, 5, 64, 300], 29, dtype)
+    q = O.round_to(O.fill_normal((B, H, d), 29, 1), dtype)
+    scale = 1.0 / np.sqrt(d)
+    rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
+    want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
+    kp, vp, table = poison_unused(kp, vp, table, lens, P, H_kv, d, wild_page=1 << 24)
+    for chunk in (0, 32, 48, 160):
+        got = decode(emu, q, kp, vp, table, lens, None, B, H, H_kv, d, P, dtype, dtype, scale, chunk)
+        assert np.isfinite(got).all()
+        assert np.abs(got - want).max() <= 2e-2, f"chunk={chunk}"
+
+
 def test_decode_empty_sequence_and_batch_rows(emu):
     B, H, d, P = 4, 4, 64, 16
     q, kp, vp, table, lens, _, _ = build_problem(B, H, d, P, [40, 7, 90, 16], 41, O.BF16)

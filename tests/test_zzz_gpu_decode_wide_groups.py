@@ -55,6 +55,37 @@ def test_matrix_core_decode_equals_repeated_heads(gpu, G, dtype, d, matrix_kerne
         assert np.abs(got - want).max() <= 2e-2, (chunk, qo)
 
 
+@pytest.mark.parametrize("waves", [1, 2, 4])
+@pytest.mark.parametrize("G,H_kv,d,dtype", [(32, 1, 128, O.F16), (24, 2, 64, O.BF16), (17, 1, 256, O.BF16), (32, 3, 128, O.BF16)])
+def test_wide_groups_workgroup_widths(gpu, G, H_kv, d, dtype, waves):
+    """Groups of 17 to 32 query heads in workgroups of 1, 2 and 4 wavefronts (at d = 256: 1 and 2) that share a chunk's
+    tiles out and merge in LDS: chunks with fewer tiles than wavefronts, with one tile more than a multiple, a sequence
+    that ends on a tile's border, an empty one, and a page that is missing inside a chunk."""
+    B, P = 6, 16
+    H = G * H_kv
+    _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [1500, 33, 1024, 7, 2049, 300], 31, dtype)
+    lens = lens.copy()
+    lens[3] = 0
+    q = O.round_to(O.fill_normal((B, H, d), 31, 1), dtype)
+    scale = 1.0 / np.sqrt(d)
+    rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
+    holed = table.copy()
+    holed[5, 9] = -1           # sequence 5 ends in front of its tenth page: 144 tokens
+    want = O.paged_decode(q, rep(kp), rep(vp), holed, lens, None, B, H, d, P, scale)
+    kp, vp, _ = poison_unused(kp, vp, table, lens, P, H_kv, d)
+    table = holed
+    before = gpu.get_tuning("decode_waves")
+    gpu.set_tuning("decode_waves", waves)
+    try:
+        for chunk in (0, 1024, 288, 64):
+            got = run(gpu, q, kp, vp, table, lens, B, H, H_kv, d, P, dtype, dtype, scale, chunk)
+            assert np.isfinite(got).all()
+            assert np.all(got[3] == 0.0)
+            assert np.abs(got - want).max() <= 2e-2, chunk
+    finally:
+        gpu.set_tuning("decode_waves", before)
+
+
 @pytest.mark.parametrize("H_kv,G,d,dtype", [(8, 4, 128, O.F16), (5, 2, 64, O.BF16), (1, 16, 128, O.BF16), (3, 8, 64, O.F16)])
 def test_page_ring_of_the_group_kernel(gpu, H_kv, G, d, dtype):
     """8, 4, 2 and 1 pool heads side by side in a workgroup of the page-by-page kernel, chunks of several trips round its
