@@ -725,7 +725,7 @@ static DecodePlan plan_decode(int64_t B, int64_t H_kv, int64_t group, int64_t ro
             return plan;
         }
         int64_t chunk = 1024;
-        while (waves > 1 && chunk > 256 && wgs(chunk) < 256) chunk /= 2;
+        while (waves > 1 && chunk > 256 && wgs(chunk) < 256 && (max_len + chunk / 2 - 1) / (chunk / 2) <= 64) chunk /= 2;
         plan.chunk = fit_chunk(chunk, P);
         if (!plan.waves) plan.waves = waves;
         return plan;
@@ -737,8 +737,10 @@ static DecodePlan plan_decode(int64_t B, int64_t H_kv, int64_t group, int64_t ro
     }
     if (matrix_kernel) {
         // one wavefront per pool head and chunk, bound by the stream like the case below
+        // (a sequence in more than 64 chunks costs more in the merge, which walks them one wavefront per head, than
+        // the shorter chunks gain: one sequence of 30 000 tokens, 32 heads over 8: 0.050 ms in chunks of 128, 0.034 in 512)
         int64_t chunk = 1024;
-        while (chunk > 128 && B * ((max_len + chunk - 1) / chunk) * H_kv < 1024) chunk /= 2;
+        while (chunk > 128 && B * ((max_len + chunk - 1) / chunk) * H_kv < 1024 && (max_len + chunk / 2 - 1) / (chunk / 2) <= 64) chunk /= 2;
         plan.chunk = fit_chunk(chunk, P);
         if (!plan.waves) plan.waves = 2;  // (unused by those kernels)
         return plan;
@@ -747,8 +749,11 @@ static DecodePlan plan_decode(int64_t B, int64_t H_kv, int64_t group, int64_t ro
         // One query head per pool head is pure streaming: the longest chunks that still leave about four
         // wavefronts for every CU (timed on B=1..256, contexts 128..131072: chunks of 1024 tokens win wherever
         // they leave >= 1024 wavefronts; shorter chunks pay in partials and in part-filled requests).
+        // (and no more than 64 chunks to a sequence: the merge walks them one wavefront per head, and beyond that it
+        // costs more than the shorter chunks gain: one sequence of 30 000 tokens, 32 heads, 0.105 ms in chunks of 128,
+        // 0.091 in 512)
         int64_t chunk = 1024;
-        while (chunk > 128 && B * ((max_len + chunk - 1) / chunk) * row_waves < 1024) chunk /= 2;
+        while (chunk > 128 && B * ((max_len + chunk - 1) / chunk) * row_waves < 1024 && (max_len + chunk / 2 - 1) / (chunk / 2) <= 64) chunk /= 2;
         plan.chunk = fit_chunk(chunk, P);
         if (!plan.waves) {
             // Whole token rows per workgroup (8 wavefronts read 8 consecutive KiB and more) when such workgroups
@@ -829,9 +834,19 @@ static int launch_decode_mfma(const DecodeParams& p, int waves, hipStream_t st) 
 // Matrix-core kernel for groups of up to 16 query heads: a wavefront per (pool head, chunk, batch entry), up to 8
 // pool heads side by side in a workgroup.
 template <typename T, int D>
-static int launch_decode_group_d(const DecodeParams& p, hipStream_t st) {
+static int launch_decode_group_d(const DecodeParams& p, int waves_wanted, hipStream_t st) {
     // (at d = 256 a wavefront's two page slots take 32 KiB of LDS: four wavefronts at most)
-    const int w = (p.H_kv >= 8 && D <= 128) ? 8 : p.H_kv >= 4 ? 4 : p.H_kv >= 2 ? 2 : 1;
+    int w = (p.H_kv >= 8 && D <= 128) ? 8 : p.H_kv >= 4 ? 4 : p.H_kv >= 2 ? 2 : 1;
+    // A CU draws about 25 GB/s however many wavefronts ask, so a launch with fewer workgroups than CUs is bound by the
+    // CUs it reaches: narrower workgroups then, until the launch has one for every CU.  (32 query heads over 8 pool
+    // heads, d = 128, contexts U[512,4096]: B = 32 0.086 ms on 8 wavefronts, 0.059 on 4 or 2; B = 16 0.052 -> 0.035;
+    // B = 4 0.021 -> 0.017; from B = 64 on whole token rows per workgroup win by 5 %.)
+    // (the tuning value decode_waves, when set, says how wide instead)
+    if (waves_wanted > 0) {
+        while (w > waves_wanted) w /= 2;
+    } else {
+        while (w > 1 && (int64_t)p.B * p.n_chunks * ((p.H_kv + w - 1) / w) < 256) w /= 2;
+    }
     const dim3 grid((unsigned)((p.H_kv + w - 1) / w), (unsigned)p.n_chunks, (unsigned)p.B), block(64 * w);
     switch (w) {
         case 8:
@@ -845,10 +860,10 @@ static int launch_decode_group_d(const DecodeParams& p, hipStream_t st) {
 }
 
 template <typename T>
-static int launch_decode_group(const DecodeParams& p, hipStream_t st) {
-    if (p.d == 128) return launch_decode_group_d<T, 128>(p, st);
-    if (p.d == 64) return launch_decode_group_d<T, 64>(p, st);
-    if (p.d == 256) return launch_decode_group_d<T, 256>(p, st);
+static int launch_decode_group(const DecodeParams& p, int waves_wanted, hipStream_t st) {
+    if (p.d == 128) return launch_decode_group_d<T, 128>(p, waves_wanted, st);
+    if (p.d == 64) return launch_decode_group_d<T, 64>(p, waves_wanted, st);
+    if (p.d == 256) return launch_decode_group_d<T, 256>(p, waves_wanted, st);
     return AHPC_ERR_UNSUPPORTED_HEAD_DIM;
 }
 
@@ -1085,7 +1100,8 @@ int ahpc_hip_paged_decode_gqa(const void* q, void* o, int qo_dtype, const void* 
     dim3 grid((unsigned)head_groups, (unsigned)n_chunks, (unsigned)B), block(64 * waves);
     int rc;
     if (use_mfma && group <= 16) {
-        rc = pool_dtype == AHPC_F16 ? launch_decode_group<f16_t>(p, st) : launch_decode_group<bf16_t>(p, st);
+        const int wanted = (int)tuning().decode_waves.load();
+        rc = pool_dtype == AHPC_F16 ? launch_decode_group<f16_t>(p, wanted, st) : launch_decode_group<bf16_t>(p, wanted, st);
     } else if (use_mfma) {
         rc = pool_dtype == AHPC_F16 ? launch_decode_mfma<f16_t>(p, waves, st) : launch_decode_mfma<bf16_t>(p, waves, st);
     } else

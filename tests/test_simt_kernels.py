@@ -953,6 +953,7 @@ def test_operand_reads_are_free_of_bank_conflicts(emu, dtype, d):
 @pytest.mark.parametrize("G", [4, 8, 16, 32])
 def test_decode_grouped_heads_matrix_core_kernel(emu, G, dtype, d, tuned):
     tuned("decode_matrix_min_group", 4)   # groups of 4 and 8 take this kernel only when asked to
+    tuned("decode_waves", 8)              # the widest workgroups (a launch this small would get single wavefronts)
     B, H_kv, P = 4, 2, 16
     H = G * H_kv
     _, kp, vp, table, lens, _, _ = build_problem(B, H_kv, d, P, [70, 5, 129, 32], 23, dtype)

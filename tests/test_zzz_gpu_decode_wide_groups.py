@@ -99,15 +99,19 @@ def test_page_ring_of_the_group_kernel(gpu, H_kv, G, d, dtype):
     rep = lambda pool: np.repeat(pool.reshape(-1, H_kv, d), G, axis=1).reshape(-1)
     want = O.paged_decode(q, rep(kp), rep(vp), table, lens, None, B, H, d, P, scale)
     kp, vp, table = poison_unused(kp, vp, table, lens, P, H_kv, d)
-    before = gpu.get_tuning("decode_matrix_min_group")
+    before = gpu.get_tuning("decode_matrix_min_group"), gpu.get_tuning("decode_waves")
     gpu.set_tuning("decode_matrix_min_group", 2)
     try:
-        for chunk in (1024, 96, 0):
-            got = run(gpu, q, kp, vp, table, lens, B, H, H_kv, d, P, dtype, dtype, scale, chunk)
-            assert np.isfinite(got).all()
-            assert np.abs(got - want).max() <= 2e-2, chunk
+        # (a launch this small would get single wavefronts: 8 asks for the widest workgroup the pool's heads fill)
+        for waves in (8, 0):
+            gpu.set_tuning("decode_waves", waves)
+            for chunk in (1024, 96, 0):
+                got = run(gpu, q, kp, vp, table, lens, B, H, H_kv, d, P, dtype, dtype, scale, chunk)
+                assert np.isfinite(got).all()
+                assert np.abs(got - want).max() <= 2e-2, (waves, chunk)
     finally:
-        gpu.set_tuning("decode_matrix_min_group", before)
+        gpu.set_tuning("decode_matrix_min_group", before[0])
+        gpu.set_tuning("decode_waves", before[1])
 
 
 def test_both_kernels_agree_for_groups_of_four(gpu):
