@@ -511,6 +511,9 @@ def bench_extras(hip, stream, steps, warmup):
                 dict(B=8, H=32, d=128, P=16, lo=16384, hi=32768, seed=0xA77E0004), 32, 32, hip.BF16, torch.bfloat16)
     decode_case("paged_decode fp16 B=64 H=32 over 8 pool heads d=128 page=16 context U[512,4096]",
                 dict(DECODE), 32, 8, hip.F16, torch.float16)
+    # the same at a quarter of the batch: a launch with fewer workgroups than CUs, which gets narrower workgroups
+    decode_case("paged_decode fp16 B=16 H=32 over 8 pool heads d=128 page=16 context U[512,4096]",
+                dict(DECODE, B=16), 32, 8, hip.F16, torch.float16)
     # multi-query decode (32 query heads over one pool head): the matrix-core kernel
     decode_case("paged_decode (matrix-core kernel) fp16 B=64 H=32 over 1 pool head d=128 page=16 context U[512,4096]",
                 dict(DECODE), 32, 1, hip.F16, torch.float16)
