@@ -364,7 +364,8 @@ __global__ __launch_bounds__(kFlashThreads, (D > 128 ? 1 : 2)) void flash_bwd_dq
 // wavefront per SIMD), 1 = dV only (S and dV: two products, V and dO.V never touched), 2 = dK only (S, dP, dK).  The
 // two partial walks execute five products between them but each fits two wavefronts per SIMD, which hide each
 // other's softmax arithmetic and LDS waits: 5 % fewer cycles at d = 128, and still the slower way on inputs that hold
-// the board at its power limit, where four products beat five (the launcher picks).
+// the board at its power limit, where four products beat five (the launcher picks).  The one walk overlaps its own
+// vector arithmetic with its matrix products by pipelining the two blocks of a tile (see compute_tile).
 // MASKED: as in the dQ kernel, with the transposed packed mask (the lane's key, 64 queries per word).
 template <typename T, int D, bool CAUSAL, bool VARLEN, int PART, bool MASKED = false>
 __global__ __launch_bounds__(kFlashThreads, (PART == 0 || D > 128 ? 1 : 2)) void flash_bwd_dkv_mfma_kernel(const FlashBwdParams p) {
@@ -493,6 +494,148 @@ __global__ __launch_bounds__(kFlashThreads, (PART == 0 || D > 128 ? 1 : 2)) void
 
             auto compute_tile = [&](const unsigned char* tile_q, const unsigned char* tile_o, const unsigned char* tile_s, int i0,
                                     uint64_t mw) {
+                if constexpr (PART == 0 && !MASKED) {
+                    // Both blocks of 32 queries in full (no end of the sequence, no diagonal in either), which is almost
+                    // every tile of a long sequence.  This kernel runs one wavefront per SIMD, so nobody else fills the
+                    // matrix pipe while a block's exponentials and products P.dP run (some 100 vector instructions
+                    // between 16 + 16 matrix instructions).  The two blocks are therefore laid out as a pipeline:
+                    //     first products (S, dP) of block 0
+                    //     first products of block 1   among   the exponentials of block 0
+                    //     second products (dV, dK) of block 0   among   the exponentials of block 1
+                    //     second products of block 1
+                    // (the same arithmetic in the same order per element: results are bit for bit those of the loop below).
+                    if (i0 + 63 < L && kw + 31 < L && (!CAUSAL || i0 >= kw + 31)) {
+                        f32x16 s0, dp0, s1, dp1;
+#pragma unroll
+                        for (int g4 = 0; g4 < 4; ++g4) {
+                            const f32x4 a0 = *reinterpret_cast<const f32x4*>(tile_s + 4 * (8 * g4 + 4 * half));
+                            const f32x4 d0 = *reinterpret_cast<const f32x4*>(tile_s + 256 + 4 * (8 * g4 + 4 * half));
+                            const f32x4 a1 = *reinterpret_cast<const f32x4*>(tile_s + 4 * (32 + 8 * g4 + 4 * half));
+                            const f32x4 d1 = *reinterpret_cast<const f32x4*>(tile_s + 256 + 4 * (32 + 8 * g4 + 4 * half));
+#pragma unroll
+                            for (int x = 0; x < 4; ++x) {
+                                s0[4 * g4 + x] = a0[x];
+                                dp0[4 * g4 + x] = d0[x];
+                                s1[4 * g4 + x] = a1[x];
+                                dp1[4 * g4 + x] = d1[x];
+                            }
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                        __builtin_amdgcn_s_setprio(1);
+                        u32x2 ot[2][MB][2], qt[2][MB][2];
+                        auto request_tr = [&](int row0, int g2) __attribute__((always_inline)) {
+#pragma unroll
+                            for (int mb = 0; mb < MB; ++mb) {
+                                ot[g2][mb][0] = TrRead<T>::load(tile_o + row0 * RB + tr_off[mb][0]);
+                                ot[g2][mb][1] = TrRead<T>::load(tile_o + row0 * RB + tr_off[mb][1]);
+                                qt[g2][mb][0] = TrRead<T>::load(tile_q + row0 * RB + tr_off[mb][0]);
+                                qt[g2][mb][1] = TrRead<T>::load(tile_q + row0 * RB + tr_off[mb][1]);
+                            }
+                        };
+                        auto second_products = [&](int row0, const f32x16& pw, const f32x16& ds) __attribute__((always_inline)) {
+#pragma unroll
+                            for (int g2 = 0; g2 < 2; ++g2) {
+                                if (g2 == 0) request_tr(row0 + 16, 1);
+                                const u32x4 bp = pack_operand<T>(pw, 8 * g2);
+#pragma unroll
+                                for (int mb = 0; mb < MB; ++mb)
+                                    acc_v[mb] = mfma_32x32x16<T>(u32x4{ot[g2][mb][0][0], ot[g2][mb][0][1], ot[g2][mb][1][0], ot[g2][mb][1][1]}, bp, acc_v[mb]);
+                                const u32x4 bs = pack_operand<T>(ds, 8 * g2);
+#pragma unroll
+                                for (int mb = 0; mb < MB; ++mb)
+                                    acc_k[mb] = mfma_32x32x16<T>(u32x4{qt[g2][mb][0][0], qt[g2][mb][0][1], qt[g2][mb][1][0], qt[g2][mb][1][1]}, bs, acc_k[mb]);
+                                __builtin_amdgcn_sched_barrier(0);
+                            }
+                        };
+                        constexpr int kAhead = 2;  // (3 and 4 steps ahead time the same)
+                        request_tr(0, 0);
+                        {   // first products of block 0
+                            u32x4 aq[KS], ao[KS];
+#pragma unroll
+                            for (int ks = 0; ks < KS; ++ks) {
+                                aq[ks] = lds_read_b128(tile_q + row_off[ks]);
+                                ao[ks] = lds_read_b128(tile_o + row_off[ks]);
+                            }
+#pragma unroll
+                            for (int ks = 0; ks < KS; ++ks) {
+                                s0 = mfma_32x32x16<T>(aq[ks], kreg[ks], s0);
+                                dp0 = mfma_32x32x16<T>(ao[ks], vreg[ks], dp0);
+                            }
+                            __builtin_amdgcn_sched_group_barrier(0x100, 4 * MB + 2 * kAhead, 0);
+#pragma unroll
+                            for (int i = 0; i < KS - kAhead; ++i) {
+                                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                            }
+#pragma unroll
+                            for (int i = 0; i < kAhead; ++i) __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                        f32x16 pw0, ds0;
+                        {   // first products of block 1 among the exponentials of block 0
+                            u32x4 aq[KS], ao[KS];
+#pragma unroll
+                            for (int ks = 0; ks < KS; ++ks) {
+                                aq[ks] = lds_read_b128(tile_q + 32 * RB + row_off[ks]);
+                                ao[ks] = lds_read_b128(tile_o + 32 * RB + row_off[ks]);
+                            }
+#pragma unroll
+                            for (int ks = 0; ks < KS; ++ks) {
+                                s1 = mfma_32x32x16<T>(aq[ks], kreg[ks], s1);
+                                dp1 = mfma_32x32x16<T>(ao[ks], vreg[ks], dp1);
+                            }
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) {
+                                pw0[r] = fast_exp2(s0[r]);
+                                ds0[r] = pw0[r] * dp0[r];
+                            }
+                            __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+#pragma unroll
+                            for (int i = 0; i < KS - kAhead; ++i) {
+                                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x402, 32 / KS, 0);
+                            }
+#pragma unroll
+                            for (int i = 0; i < kAhead; ++i) {
+                                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x402, 32 / KS, 0);
+                            }
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                        // second products of block 0 among the exponentials of block 1
+                        f32x16 pw1, ds1;
+#pragma unroll
+                        for (int g2 = 0; g2 < 2; ++g2) {
+                            if (g2 == 0) request_tr(16, 1);
+                            const u32x4 bp = pack_operand<T>(pw0, 8 * g2);
+#pragma unroll
+                            for (int mb = 0; mb < MB; ++mb)
+                                acc_v[mb] = mfma_32x32x16<T>(u32x4{ot[g2][mb][0][0], ot[g2][mb][0][1], ot[g2][mb][1][0], ot[g2][mb][1][1]}, bp, acc_v[mb]);
+                            const u32x4 bs = pack_operand<T>(ds0, 8 * g2);
+#pragma unroll
+                            for (int mb = 0; mb < MB; ++mb)
+                                acc_k[mb] = mfma_32x32x16<T>(u32x4{qt[g2][mb][0][0], qt[g2][mb][0][1], qt[g2][mb][1][0], qt[g2][mb][1][1]}, bs, acc_k[mb]);
+#pragma unroll
+                            for (int r = 8 * g2; r < 8 * g2 + 8; ++r) {
+                                pw1[r] = fast_exp2(s1[r]);
+                                ds1[r] = pw1[r] * dp1[r];
+                            }
+                            if (g2 == 1) request_tr(32, 0);  // block 1's first 16 queries (the registers of block 0's are free)
+                            __builtin_amdgcn_sched_group_barrier(0x402, 4, 0);
+#pragma unroll
+                            for (int i = 0; i < 2 * MB; ++i) {
+                                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x100, 4 * MB / (2 * MB), 0);
+                                __builtin_amdgcn_sched_group_barrier(0x402, 5, 0);
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                        second_products(32, pw1, ds1);
+                        __builtin_amdgcn_s_setprio(0);
+                        return;
+                    }
+                }
 #pragma unroll
                 for (int ib = 0; ib < 2; ++ib) {
                     const int iblock0 = i0 + 32 * ib;

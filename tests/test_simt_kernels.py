@@ -740,7 +740,7 @@ def test_backward_fp32_kernels_16bit_storage(emu, dtype):
     check_gradients(got, O.attention_backward(q, k, v, do, B, N, H, d, 0.2, True, H_kv), dtype)
 
 
-@pytest.mark.parametrize("split,dma_late", [(1, False), (2, True)])
+@pytest.mark.parametrize("split,dma_late", [(1, False), (2, True), (1, True)])
 @pytest.mark.parametrize("dtype", [O.BF16, O.F16])
 @pytest.mark.parametrize("B,N,H,H_kv,d,causal", [
     (1, 64, 1, 1, 128, False), (2, 129, 2, 2, 128, True), (1, 300, 2, 2, 64, True), (1, 200, 2, 1, 64, False),
